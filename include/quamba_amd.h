@@ -1,0 +1,262 @@
+/*
+ * quamba_amd.h - C ABI of libquamba_amd.so: quantized Mamba mixer kernels for AMD MI355X (gfx950).
+ *
+ * Every entry point takes a parameter block of plain pointers, sizes, element strides and scales,
+ * plus the HIP stream (hipStream_t passed as void*) on which the kernels are enqueued.  The
+ * library never allocates, never synchronises and keeps no mutable global state, so calls are
+ * re-entrant and can be captured into HIP graphs.  All pointers are device pointers unless said
+ * otherwise.  Strides count elements, not bytes.  Return value: QA_OK (0) or a negative QaStatus.
+ *
+ * Each entry point names the interface of the reference (enyac-group/Quamba, paths relative to
+ * its root) that it replaces.
+ */
+#ifndef QUAMBA_AMD_H
+#define QUAMBA_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum QaStatus {
+    QA_OK = 0,
+    QA_ERR_NULL = -1,        /* a required pointer is null */
+    QA_ERR_SHAPE = -2,       /* a size is out of the supported range */
+    QA_ERR_STRIDE = -3,      /* a stride / alignment requirement is violated */
+    QA_ERR_UNSUPPORTED = -4, /* valid request the library has no kernel for */
+    QA_ERR_LAUNCH = -5       /* the HIP runtime refused the launch */
+} QaStatus;
+
+/* Human-readable text for a status code (static storage). */
+const char* qa_status_string(int status);
+/* ABI version, bumped on any incompatible change of the structs below. */
+int qa_abi_version(void);
+/* Last HIP error code seen by a failed launch on this thread (0 if none). */
+int qa_last_hip_error(void);
+
+/* ------------------------------------------------------------------------------------------
+ * Mamba1 int8 depthwise causal conv1d (+ optional SiLU) with int8 requantisation.
+ * Replaces quant_causal_conv1d_cuda.fwd / .update
+ *   (csrc/causal_conv1d/quant_causal_conv1d.cpp:76-164, :167-226; parameter block
+ *    csrc/causal_conv1d/causal_conv1d.h:9-55).
+ * ---------------------------------------------------------------------------------------- */
+typedef struct QaConvParams {
+    int32_t batch, dim, seqlen, width;   /* width in [2,4] */
+    int32_t silu_activation;             /* 0 / 1 */
+    int32_t reserved0;
+    /* x, out: int8 (batch, dim, seqlen).  Either seqlen-contiguous (x_l_stride == 1) or
+     * channel-contiguous (x_c_stride == 1); out uses its own strides. */
+    int64_t x_batch_stride, x_c_stride, x_l_stride;
+    int64_t out_batch_stride, out_c_stride, out_l_stride;
+    int64_t weight_c_stride, weight_width_stride;   /* weight int8 (dim, width) */
+    /* update only: conv_state int8 (batch, dim, state_len), state_len == width or width-1 */
+    int64_t conv_state_batch_stride, conv_state_c_stride, conv_state_l_stride;
+    int32_t conv_state_len;
+    int32_t reserved1;
+    const int8_t* x;
+    const int8_t* weight;
+    const int8_t* bias;        /* int8 (dim) or null */
+    int8_t* out;
+    int8_t* conv_state;        /* update only, modified in place */
+    float scale_x, scale_w, scale_b, scale_out;
+} QaConvParams;
+
+int qa_causal_conv1d_fwd(const QaConvParams* p, void* stream);
+int qa_causal_conv1d_update(const QaConvParams* p, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Mamba1 int8 selective scan, forward over a sequence.
+ * Replaces quant_sscan_cuda.fwd (csrc/selective_scan/quant_sscan.cpp:122-265; parameter block
+ * csrc/selective_scan/quant_sscan.h:26-86).  Differences kept deliberate: the output is written
+ * directly in (batch, seqlen, dim) order (the reference transposes afterwards, quant_sscan.cpp:262),
+ * and the last state can be returned as fp32 and/or int8.
+ * Scales are device pointers to one fp32 each, exactly as the reference passes them.
+ * ---------------------------------------------------------------------------------------- */
+typedef struct QaSScanParams {
+    int32_t batch, dim, seqlen, dstate;  /* dstate <= 256 */
+    int32_t n_groups;                    /* B/C groups, dim % n_groups == 0 */
+    int32_t delta_softplus;
+    /* u, delta, z: int8 (batch, dim, seqlen), seqlen-contiguous */
+    int64_t u_batch_stride, u_d_stride;
+    int64_t delta_batch_stride, delta_d_stride;
+    int64_t z_batch_stride, z_d_stride;
+    /* B, C: int8 (batch, n_groups, dstate, seqlen), seqlen-contiguous */
+    int64_t B_batch_stride, B_group_stride, B_dstate_stride;
+    int64_t C_batch_stride, C_group_stride, C_dstate_stride;
+    int64_t A_d_stride, A_dstate_stride;             /* A_log int8 (dim, dstate) */
+    /* out: fp16, element (b, l, d) at b*out_batch_stride + l*out_l_stride + d*out_d_stride */
+    int64_t out_batch_stride, out_l_stride, out_d_stride;
+    const int8_t* u;
+    const int8_t* delta;
+    const int8_t* A_log;
+    const int8_t* B;
+    const int8_t* C;
+    const int8_t* D;           /* int8 (dim) or null */
+    const int8_t* delta_bias;  /* int8 (dim) or null */
+    const int8_t* z;           /* or null */
+    const float* scale_u;
+    const float* scale_delta;
+    const float* scale_A;
+    const float* scale_B;
+    const float* scale_C;
+    const float* scale_D;          /* required iff D */
+    const float* scale_delta_bias; /* required iff delta_bias */
+    const float* scale_z;          /* required iff z */
+    const float* scale_ssm_state;  /* required iff last_state_i8 */
+    void* out;                     /* fp16 */
+    int8_t* last_state_i8;         /* int8 (batch, dim, dstate) contiguous, or null */
+    float* last_state_f32;         /* fp32 (batch, dim, dstate) contiguous, or null */
+} QaSScanParams;
+
+int qa_sscan_fwd(const QaSScanParams* p, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Single-token recurrent state update (decode step), Mamba1 (nheads == 1, headdim == d_inner)
+ * and Mamba2 (nheads x headdim).
+ * Replaces quant_sscan_update_triton / quamba2_sscan_update_triton
+ *   (quamba/triton/selective_state_update.py:129-227, :365-478).
+ * The state is either int8 with a scale (reference behaviour: dequantise, update, requantise in
+ * place) or fp32 (updated in place, no requantisation).
+ * ---------------------------------------------------------------------------------------- */
+typedef struct QaSsmUpdateParams {
+    int32_t batch, nheads, dim, dstate;  /* dim = channels per head */
+    int32_t ngroups;                     /* B/C groups, nheads % ngroups == 0 */
+    int32_t dt_softplus;
+    int32_t state_is_fp32;               /* 0: int8 state + state_scale, 1: fp32 state */
+    int32_t dt_bias_is_fp16;             /* 0: int8 dt_bias + scale (Mamba1), 1: fp16 dt_bias (Mamba2) */
+    /* grouped state scales (Mamba2 head/dim groups); 0 groups = one scalar state scale */
+    int32_t nhead_groups, ndim_groups;
+    int64_t state_batch_stride, state_head_stride, state_dim_stride, state_dstate_stride;
+    int64_t x_batch_stride, x_head_stride, x_dim_stride;
+    int64_t dt_batch_stride, dt_head_stride, dt_dim_stride;      /* stride 0 = broadcast */
+    int64_t dt_bias_head_stride, dt_bias_dim_stride;
+    int64_t A_head_stride, A_dim_stride, A_dstate_stride;
+    int64_t B_batch_stride, B_group_stride, B_dstate_stride;
+    int64_t C_batch_stride, C_group_stride, C_dstate_stride;
+    int64_t D_head_stride, D_dim_stride;
+    int64_t z_batch_stride, z_head_stride, z_dim_stride;
+    int64_t out_batch_stride, out_head_stride, out_dim_stride;
+    void* state;               /* int8 or fp32, in place */
+    const int8_t* x;
+    const int8_t* dt;
+    const void* dt_bias;       /* int8 or fp16 or null */
+    const int8_t* A_log;
+    const int8_t* B;
+    const int8_t* C;
+    const int8_t* D;           /* or null */
+    const int8_t* z;           /* or null */
+    const float* x_scale;      /* one fp32, or [ngroups, nhead_groups, ndim_groups] when grouped */
+    const float* dt_scale;
+    const float* dt_bias_scale; /* int8 dt_bias only */
+    const float* A_log_scale;
+    const float* state_scale;  /* one fp32, or [ngroups, nhead_groups, ndim_groups, dstate] when grouped */
+    const float* B_scale;      /* one fp32, or [ngroups] when grouped */
+    const float* C_scale;
+    const float* D_scale;
+    const float* z_scale;
+    const int32_t* x_head_group_range; /* [ngroups, nhead_groups] cumulative end indices, grouped only */
+    const int32_t* x_dim_group_range;  /* [ngroups, nhead_groups, ndim_groups] */
+    void* out;                 /* fp16 (batch, nheads, dim) */
+} QaSsmUpdateParams;
+
+int qa_ssm_state_update(const QaSsmUpdateParams* p, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * W8A8 GEMM with scale epilogue:  D[m,n] = cast( s_a[m|0] * ( s_b[n|0] * float(sum_k a[m,k] w[n,k]) ) )
+ * Replaces quant_linear_cuda.cutlass_scaled_mm_dq / cutlass_scaled_mv_dq / w8a8o8_gemv
+ *   (csrc/linear/quant_linear_fwd_kernel.cuh:356-401, quant_linear_fwd_gemv_kernel.cuh:96-134).
+ * Both operands are K-contiguous: a is (M,K) with row stride lda; w is (N,K) with row stride ldw
+ * (the reference's column-major (K,N) "b" operand is the same memory).
+ * ---------------------------------------------------------------------------------------- */
+typedef enum QaOutType { QA_OUT_I8 = 0, QA_OUT_F16 = 1 } QaOutType;
+typedef enum QaRound { QA_ROUND_RNE = 0, QA_ROUND_HALF_AWAY = 1 } QaRound;
+
+typedef struct QaGemmW8A8Params {
+    int32_t m, n, k;
+    int32_t out_type;      /* QaOutType */
+    int32_t round_mode;    /* QaRound, int8 output only */
+    int32_t a_scale_numel; /* 1 or m */
+    int32_t w_scale_numel; /* 1 or n */
+    int32_t reserved0;
+    int64_t lda, ldw, ldd; /* element strides between rows of a, w, d (d is (M,N) row-major) */
+    const int8_t* a;
+    const int8_t* w;
+    const float* a_scale;  /* device */
+    const float* w_scale;  /* device */
+    void* d;               /* int8 or fp16 */
+} QaGemmW8A8Params;
+
+int qa_gemm_w8a8(const QaGemmW8A8Params* p, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * W4A8 GEMM (int4 weights, group-wise fp16 scales, int8 activations).
+ * Replaces quant_linear_cuda.w4a8o8_gemm / w4a8o16_gemm
+ *   (csrc/linear/marlin_qqq_gemm_kernel.cuh:1187-1314, marlin_qqq_gemm_kernel_o8.cuh).
+ * Weights are held in this library's own packing (see qa_w4a8_pack_weights); arithmetic is the
+ * reference's: w8 = rne((q4-8) * s_group) as int8, int32 accumulation, out = (acc*s_ch[n])*s_tok[m|0].
+ * ---------------------------------------------------------------------------------------- */
+typedef struct QaGemmW4A8Params {
+    int32_t m, n, k;
+    int32_t group_size;      /* 128, or -1 for per-channel (w8 = 16 * (q4 - 8)) */
+    int32_t out_type;        /* QaOutType */
+    int32_t tok_scale_numel; /* 1 or m */
+    int32_t output_transpose;/* 0: d is (M,N); 1: d is (N,M) */
+    int32_t reserved0;
+    int64_t lda, ldd;
+    const int8_t* a;         /* (M,K) */
+    const uint8_t* w_packed; /* (N, K/2): two 4-bit codes per byte, low nibble = even k */
+    const void* s_group;     /* fp16 (K/group_size, N) or null when per-channel */
+    const float* s_channel;  /* fp32 (N) */
+    const float* s_token;    /* fp32 (1) or (M) */
+    void* d;
+} QaGemmW4A8Params;
+
+int qa_gemm_w4a8(const QaGemmW4A8Params* p, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Mamba2 quantized SSD chunk scan (prefill).
+ * Replaces _quant_mamba_chunk_scan_combined_fwd / _quamba2_mamba_chunk_scan_combined_fwd
+ *   (quamba/triton/quant_ssd_combined.py:11-81, :84-166).
+ * Workspace is supplied by the caller (size from qa_ssd_workspace_bytes).
+ * ---------------------------------------------------------------------------------------- */
+typedef struct QaSsdParams {
+    int32_t batch, seqlen, nheads, headdim, dstate, ngroups, chunk_size;
+    int32_t dt_softplus;
+    int32_t dt_is_fp32;          /* 0: int8 dt + dt_scale + fp16 dt_bias; 1: fp32 dt already processed */
+    int32_t D_has_hdim;          /* D is (nheads, headdim) instead of (nheads) */
+    int32_t nhead_groups, ndim_groups;  /* 0 = per-tensor x scale */
+    int32_t final_state_is_fp32; /* 1: fp32 final states, 0: int8 with state scale */
+    int32_t reserved0;
+    float dt_min, dt_max;        /* clamp after softplus */
+    const int8_t* x;             /* (batch, seqlen, nheads, headdim) contiguous */
+    const void* dt;              /* int8 or fp32 (batch, seqlen, nheads) contiguous */
+    const int8_t* A_log;         /* (nheads) */
+    const int8_t* B;             /* (batch, seqlen, ngroups, dstate) contiguous */
+    const int8_t* C;
+    const int8_t* D;             /* or null */
+    const int8_t* z;             /* (batch, seqlen, nheads, headdim) or null */
+    const void* dt_bias;         /* fp16 (nheads) or null */
+    const float* x_scale;        /* (1) or [ngroups, nhead_groups, ndim_groups] */
+    const float* dt_scale;
+    const float* A_log_scale;
+    const float* B_scale;        /* (1) or [ngroups] */
+    const float* C_scale;
+    const float* D_scale;
+    const float* z_scale;
+    const float* state_scale;    /* (1) or [ngroups, nhead_groups, ndim_groups, dstate] */
+    const int32_t* x_head_group_range;
+    const int32_t* x_dim_group_range;
+    void* out;                   /* fp16 (batch, seqlen, nheads, headdim) */
+    void* final_states;          /* fp32 or int8 (batch, nheads, headdim, dstate), or null */
+    void* workspace;
+    int64_t workspace_bytes;
+} QaSsdParams;
+
+int64_t qa_ssd_workspace_bytes(const QaSsdParams* p);
+int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* QUAMBA_AMD_H */

@@ -1,0 +1,166 @@
+"""CPU oracle for the quantized Mamba mixer path (numpy in, numpy out).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by __graft_entry__.smoke() and by bench.py's
+cpu_baseline leg, never by quamba_amd/.  The arithmetic lives in qoracle.c (a C restatement of
+the reference kernels, each function citing the file:line it follows); this module builds it
+with gcc and wraps it with ctypes.  ``naive`` holds independent float64 / integer forms used to
+pin the restatement itself.
+
+Parity status: every function below is pinned by the checks in tests/test_oracle_*.py (closed
+forms, float64 brute force, integer matmul, library routines).  The reference holds no golden
+vectors for this path and its kernels (CUDA / Triton-CUDA) cannot be built or run here, so the
+exact low-order bits of the reference binaries are not a target.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libqoracle.so")
+_lib = None
+
+_i8p = np.ctypeslib.ndpointer(np.int8, flags="C_CONTIGUOUS")
+_f32p = np.ctypeslib.ndpointer(np.float32, flags="C_CONTIGUOUS")
+_i32p = np.ctypeslib.ndpointer(np.int32, flags="C_CONTIGUOUS")
+
+
+def build(force=False):
+    src = os.path.join(_HERE, "qoracle.c")
+    if force or not os.path.exists(_LIB_PATH) or os.path.getmtime(src) > os.path.getmtime(_LIB_PATH):
+        subprocess.run(["make", "-C", _HERE, "-B", "libqoracle.so"], check=True, capture_output=True)
+    return _LIB_PATH
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        _lib = C.CDLL(_LIB_PATH)
+        _lib.qo_expf.restype = C.c_float
+        _lib.qo_expf.argtypes = [C.c_float]
+        _lib.qo_sat8_half_away.argtypes = [C.c_float]
+        _lib.qo_sat8_rne.argtypes = [C.c_float]
+    return _lib
+
+
+def _opt(a, dtype=np.int8):
+    if a is None:
+        return None
+    return np.ascontiguousarray(a, dtype=dtype).ctypes.data_as(C.c_void_p)
+
+
+def _req(a, dtype=np.int8):
+    a = np.ascontiguousarray(a, dtype=dtype)
+    return a, a.ctypes.data_as(C.c_void_p)
+
+
+def _f(v):
+    return C.c_float(float(np.float32(v)))
+
+
+def expf(x):
+    """The deterministic exp of the int8-output ops, elementwise on a float32 array."""
+    x = np.asarray(x, dtype=np.float32)
+    out = np.empty_like(x)
+    l = lib()
+    flat_in, flat_out = x.reshape(-1), out.reshape(-1)
+    for i in range(flat_in.size):
+        flat_out[i] = l.qo_expf(C.c_float(float(flat_in[i])))
+    return out
+
+
+def conv1d_fwd(x, weight, bias, s_x, s_w, s_b, s_out, silu=True, tapwise=False):
+    """x int8 (B,D,L), weight int8 (D,k), bias int8 (D) or None -> int8 (B,D,L)."""
+    x, xp = _req(x)
+    weight, wp = _req(weight)
+    B, D, L = x.shape
+    out = np.empty_like(x)
+    keep = _opt(bias)
+    lib().qo_conv1d_fwd(xp, wp, keep, out.ctypes.data_as(C.c_void_p), B, D, L, weight.shape[1],
+                        _f(s_x), _f(s_w), _f(s_b), _f(s_out), int(silu), int(tapwise))
+    return out
+
+
+def conv1d_update(x, state, weight, bias, s_x, s_w, s_b, s_out, silu=True):
+    """x int8 (B,D); state int8 (B,D,S) with S in {k, k-1}.  Returns (out int8 (B,D), new state)."""
+    x, xp = _req(x)
+    weight, wp = _req(weight)
+    state = np.array(state, dtype=np.int8, order="C", copy=True)
+    B, D = x.shape
+    out = np.empty_like(x)
+    lib().qo_conv1d_update(xp, state.ctypes.data_as(C.c_void_p), wp, _opt(bias), out.ctypes.data_as(C.c_void_p),
+                           B, D, weight.shape[1], state.shape[2], _f(s_x), _f(s_w), _f(s_b), _f(s_out), int(silu))
+    return out, state
+
+
+def sscan_fwd(u, delta, A_log, B, C_, D=None, delta_bias=None, z=None, *, s_u, s_delta, s_A, s_B, s_C,
+              s_D=0.0, s_db=0.0, s_z=0.0, s_state=1.0, softplus=True):
+    """u/delta/z int8 (B,D,L); A_log int8 (D,N); B,C int8 (B,G,N,L) or (B,N,L).
+    Returns (y float32 (B,L,D) before the fp16 cast, last state int8 (B,D,N), last state fp32)."""
+    u, up = _req(u)
+    delta, dp = _req(delta)
+    A_log, ap = _req(A_log)
+    B = np.asarray(B)
+    C_ = np.asarray(C_)
+    if B.ndim == 3:
+        B = B[:, None]
+    if C_.ndim == 3:
+        C_ = C_[:, None]
+    B, bp = _req(B)
+    C_, cp = _req(C_)
+    batch, dim, L = u.shape
+    N = A_log.shape[1]
+    G = B.shape[1]
+    y = np.empty((batch, L, dim), np.float32)
+    st8 = np.empty((batch, dim, N), np.int8)
+    st32 = np.empty((batch, dim, N), np.float32)
+    lib().qo_sscan_fwd(up, dp, ap, bp, cp, _opt(D), _opt(delta_bias), _opt(z),
+                       _f(s_u), _f(s_delta), _f(s_A), _f(s_B), _f(s_C), _f(s_D), _f(s_db), _f(s_z), _f(s_state),
+                       batch, dim, L, N, G, int(softplus),
+                       y.ctypes.data_as(C.c_void_p), st8.ctypes.data_as(C.c_void_p), st32.ctypes.data_as(C.c_void_p))
+    return y, st8, st32
+
+
+def sscan_update(state, x, dt, A_log, B, C_, D=None, dt_bias=None, z=None, *, s_x, s_dt, s_A, s_B, s_C,
+                 s_D=0.0, s_db=0.0, s_z=0.0, s_state=1.0, softplus=True):
+    """state int8 or float32 (B,D,N) (not modified; the new state is returned); x, dt, z int8 (B,D);
+    B, C int8 (B,N).  Returns (y float32 (B,D), new state)."""
+    x, xp = _req(x)
+    dt, dp = _req(dt)
+    A_log, ap = _req(A_log)
+    B, bp = _req(B)
+    C_, cp = _req(C_)
+    batch, dim = x.shape
+    N = A_log.shape[1]
+    y = np.empty((batch, dim), np.float32)
+    state = np.array(state, order="C", copy=True)
+    if state.dtype == np.float32:
+        s8, s32 = None, state.ctypes.data_as(C.c_void_p)
+    else:
+        assert state.dtype == np.int8
+        s8, s32 = state.ctypes.data_as(C.c_void_p), None
+    lib().qo_sscan_update(s8, s32, xp, dp, ap, bp, cp, _opt(D), _opt(dt_bias), _opt(z),
+                          _f(s_x), _f(s_dt), _f(s_A), _f(s_B), _f(s_C), _f(s_D), _f(s_db), _f(s_z), _f(s_state),
+                          batch, dim, N, int(softplus), y.ctypes.data_as(C.c_void_p))
+    return y, state
+
+
+def gemm_w8a8(a, w, s_a, s_b, round_half_away=False):
+    """a int8 (M,K), w int8 (N,K), s_a fp32 (1|M), s_b fp32 (1|N).
+    Returns (acc int32 (M,N), fp32 value before the cast, int8 cast)."""
+    a, ap = _req(a)
+    w, wp = _req(w)
+    s_a = np.ascontiguousarray(np.asarray(s_a, np.float32).reshape(-1))
+    s_b = np.ascontiguousarray(np.asarray(s_b, np.float32).reshape(-1))
+    M, K = a.shape
+    N = w.shape[0]
+    acc = np.empty((M, N), np.int32)
+    f = np.empty((M, N), np.float32)
+    q = np.empty((M, N), np.int8)
+    lib().qo_gemm_w8a8(ap, wp, s_a.ctypes.data_as(C.c_void_p), s_a.size, s_b.ctypes.data_as(C.c_void_p), s_b.size,
+                       M, N, K, int(round_half_away), acc.ctypes.data_as(C.c_void_p),
+                       f.ctypes.data_as(C.c_void_p), q.ctypes.data_as(C.c_void_p))
+    return acc, f, q

@@ -1,0 +1,260 @@
+/*
+ * qoracle.c - CPU restatement of the reference's quantized Mamba mixer arithmetic.
+ *
+ * TEST INFRASTRUCTURE ONLY.  Nothing in the product (quamba_amd/) may link, load or call this
+ * file; it is the checker the GPU kernels are compared with, and the CPU baseline bench.py times.
+ *
+ * Every function follows the reference kernel named above it (paths relative to the root of
+ * enyac-group/Quamba), operation for operation in fp32, on dense row-major arrays.
+ * Where the CUDA compiler contracts a*b+c into one FMA (its default), the FMA is written out.
+ * Compile with -ffp-contract=off so no other contraction happens.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <string.h>
+
+/* ---------------------------------------------------------------------------------------------
+ * exp used by the int8-output ops.  The reference calls expf under --use_fast_math, whose low
+ * bits are not reproducible off its GPU; this build defines exp as the following fixed fp32
+ * sequence (Cody-Waite reduction by ln2 in two FMAs, degree-7 Taylor polynomial in Horner form,
+ * exact scaling by 2^n), so that results are reproducible bit for bit.  tests pin it to libm's
+ * expf within 2 ulp.
+ * ------------------------------------------------------------------------------------------- */
+float qo_expf(float x) {
+    if (x > 88.0f) return INFINITY;
+    if (x < -87.0f) return 0.0f;
+    float n = rintf(x * 1.44269504088896341f);
+    float r = fmaf(n, -0.693145751953125f, x);
+    r = fmaf(n, -1.42860682030941723e-6f, r);
+    float p = 1.0f / 5040.0f;
+    p = fmaf(p, r, 1.0f / 720.0f);
+    p = fmaf(p, r, 1.0f / 120.0f);
+    p = fmaf(p, r, 1.0f / 24.0f);
+    p = fmaf(p, r, 1.0f / 6.0f);
+    p = fmaf(p, r, 0.5f);
+    p = fmaf(p, r, 1.0f);
+    p = fmaf(p, r, 1.0f);
+    int e = (int)n;
+    uint32_t bits = (uint32_t)(e + 127) << 23;
+    float s;
+    memcpy(&s, &bits, 4);
+    return p * s;
+}
+
+/* roundf = half away from zero, then clamp to int8 (quant_causal_conv1d_fwd_kernel.cuh:149-150) */
+static int8_t sat8_half_away(float v) {
+    float r = roundf(v);
+    r = fmaxf(r, -128.0f);
+    r = fminf(r, 127.0f);
+    return (int8_t)(int)r;
+}
+
+/* rint = half to even, then clamp (quamba/triton/quant_ssm_states.py:43) */
+static int8_t sat8_rne(float v) {
+    float r = rintf(v);
+    r = fmaxf(r, -128.0f);
+    r = fminf(r, 127.0f);
+    return (int8_t)(int)r;
+}
+
+int qo_sat8_half_away(float v) { return sat8_half_away(v); }
+int qo_sat8_rne(float v) { return sat8_rne(v); }
+
+static float conv_finish(float v, float s_out, int silu) {
+    if (silu) v = v / (1.0f + qo_expf(-v));      /* quant_causal_conv1d_fwd_kernel.cuh:139-144 */
+    return v / s_out;                            /* :149 */
+}
+
+/*
+ * Causal depthwise conv forward on x int8 (batch, dim, seqlen), weight int8 (dim, width).
+ * tapwise == 0: seqlen-contiguous kernel, quant_causal_conv1d_fwd_kernel.cuh:57-157
+ *     out_tmp = sum_w W[w] * x[t-(width-1-w)]  (fp32, exact integers), v = s_wx*out_tmp + bias (:130-136)
+ * tapwise == 1: channel-contiguous kernel, quant_causal_conv1d_fwd_kernel.cuh:340-375
+ *     v = s_b*bias; v += s_wx * W[w] * x[..] per tap (:356-362)
+ */
+void qo_conv1d_fwd(const int8_t* x, const int8_t* weight, const int8_t* bias, int8_t* out,
+                   int batch, int dim, int seqlen, int width,
+                   float s_x, float s_w, float s_b, float s_out, int silu, int tapwise) {
+    const float s_wx = s_w * s_x;                                           /* :62 */
+    for (int b = 0; b < batch; ++b) {
+        for (int d = 0; d < dim; ++d) {
+            const int8_t* xr = x + ((int64_t)b * dim + d) * seqlen;
+            int8_t* orow = out + ((int64_t)b * dim + d) * seqlen;
+            const int8_t* w = weight + (int64_t)d * width;
+            const float bias_f = bias ? (float)bias[d] * s_b : 0.0f;        /* :80-81 */
+            for (int t = 0; t < seqlen; ++t) {
+                float v;
+                if (!tapwise) {
+                    float acc = 0.0f;
+                    for (int k = 0; k < width; ++k) {
+                        const int ti = t - (width - 1 - k);
+                        const float xv = ti >= 0 ? (float)xr[ti] : 0.0f;
+                        acc += (float)w[k] * xv;                            /* exact in fp32 */
+                    }
+                    v = fmaf(s_wx, acc, bias_f);
+                } else {
+                    v = bias_f;
+                    for (int k = 0; k < width; ++k) {
+                        const int ti = t - (width - 1 - k);
+                        const float xv = ti >= 0 ? (float)xr[ti] : 0.0f;
+                        v = fmaf(s_wx * (float)w[k], xv, v);
+                    }
+                }
+                orow[t] = sat8_half_away(conv_finish(v, s_out, silu));
+            }
+        }
+    }
+}
+
+/*
+ * Single-step conv update, quant_causal_conv1d_update_kernel.cuh:34-75.
+ * x int8 (batch, dim); state int8 (batch, dim, state_len) shifted in place; state_len is width
+ * (the reference's layout: slot 0 is dropped) or width-1 (only the live history).
+ */
+void qo_conv1d_update(const int8_t* x, int8_t* state, const int8_t* weight, const int8_t* bias, int8_t* out,
+                      int batch, int dim, int width, int state_len,
+                      float s_x, float s_w, float s_b, float s_out, int silu) {
+    const int drop = state_len - (width - 1);
+    for (int b = 0; b < batch; ++b) {
+        for (int d = 0; d < dim; ++d) {
+            int8_t* st = state + ((int64_t)b * dim + d) * state_len;
+            const int8_t* w = weight + (int64_t)d * width;
+            int8_t xs[8];
+            for (int i = 0; i < width - 1; ++i) xs[i] = st[i + drop];       /* :59-62 */
+            xs[width - 1] = x[(int64_t)b * dim + d];
+            for (int i = 0; i < state_len; ++i) st[i] = xs[i + (width - state_len)];   /* :63-66 */
+            float v = bias ? (float)bias[d] * s_b : 0.0f;
+            for (int i = 0; i < width; ++i) {
+                v = fmaf(s_w * s_x * (float)w[i], (float)xs[i], v);         /* :68-70 */
+            }
+            out[(int64_t)b * dim + d] = sat8_half_away(conv_finish(v, s_out, silu));
+        }
+    }
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * Mamba1 selective scan forward, quant_sscan_fwd_kernel.cuh:110-293.
+ * u, delta, z int8 (batch, dim, seqlen); A_log int8 (dim, dstate); B, C int8 (batch, groups,
+ * dstate, seqlen); D, delta_bias int8 (dim) or NULL.  y fp32 (batch, seqlen, dim) holds the value
+ * the kernel converts to fp16 (:272 / :285; the transposition is quant_sscan.cpp:262).
+ * The recurrence is evaluated sequentially (the kernel's block scan differs only in association).
+ * state_i8 / state_f32 (batch, dim, dstate) receive the state after the last step (:240-241).
+ * ------------------------------------------------------------------------------------------- */
+static float softplus20(float v) { return v <= 20.0f ? log1pf(expf(v)) : v; }   /* :160 */
+
+void qo_sscan_fwd(const int8_t* u, const int8_t* delta, const int8_t* A_log, const int8_t* B, const int8_t* C,
+                  const int8_t* D, const int8_t* delta_bias, const int8_t* z,
+                  float s_u, float s_delta, float s_A, float s_B, float s_C, float s_D, float s_db, float s_z,
+                  float s_state, int batch, int dim, int seqlen, int dstate, int groups, int softplus,
+                  float* y, int8_t* state_i8, float* state_f32) {
+    const int per_group = dim / groups;
+    for (int b = 0; b < batch; ++b) {
+        for (int d = 0; d < dim; ++d) {
+            const int g = d / per_group;
+            const int8_t* ur = u + ((int64_t)b * dim + d) * seqlen;
+            const int8_t* dr = delta + ((int64_t)b * dim + d) * seqlen;
+            const int8_t* zr = z ? z + ((int64_t)b * dim + d) * seqlen : 0;
+            const float D_f = D ? s_D * (float)D[d] : 0.0f;                          /* :115-118 */
+            const float db = delta_bias ? s_db * (float)delta_bias[d] : 0.0f;        /* :121-128 */
+            float h[256];
+            float A[256];
+            for (int n = 0; n < dstate; ++n) {
+                h[n] = 0.0f;
+                A[n] = -expf(s_A * (float)A_log[(int64_t)d * dstate + n]);           /* :173 */
+            }
+            for (int t = 0; t < seqlen; ++t) {
+                const float u_val = s_u * (float)ur[t];                              /* :157 */
+                float dt = fmaf(s_delta, (float)dr[t], db);                          /* :158 */
+                if (softplus) dt = softplus20(dt);
+                const float du = dt * u_val;                                         /* :162 */
+                float acc = D_f * u_val;                                             /* :163 */
+                for (int n = 0; n < dstate; ++n) {
+                    const int64_t bc = (((int64_t)b * groups + g) * dstate + n) * seqlen + t;
+                    const float a = expf(dt * A[n]);                                 /* :219 */
+                    const float bb = s_B * (float)B[bc] * du;                        /* :221 */
+                    h[n] = fmaf(a, h[n], bb);                    /* quant_sscan_common.h:124-127 */
+                    acc = fmaf(h[n], s_C * (float)C[bc], acc);                       /* :246-249 */
+                }
+                if (zr) {
+                    const float zv = s_z * (float)zr[t];
+                    acc = acc * zv / (1.0f + expf(-zv));                             /* :271-272 */
+                }
+                y[((int64_t)b * seqlen + t) * dim + d] = acc;
+            }
+            for (int n = 0; n < dstate; ++n) {
+                const int64_t si = ((int64_t)b * dim + d) * dstate + n;
+                if (state_f32) state_f32[si] = h[n];
+                if (state_i8) state_i8[si] = sat8_half_away(h[n] / s_state);         /* :240-241 */
+            }
+        }
+    }
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * Single-step state update, quamba/triton/selective_state_update.py:83-126 (Mamba1 layout:
+ * one head, per-tensor scales).  state int8 (batch, dim, dstate) is dequantised, updated and
+ * requantised in place with rint((h*1e2)/(s*1e2)) (:119); with state_f32 != NULL the fp32 state
+ * is used instead and kept un-quantised.  y fp32 (batch, dim) is the value stored as fp16 and is
+ * computed from the un-requantised state (:121).
+ * ------------------------------------------------------------------------------------------- */
+void qo_sscan_update(int8_t* state_i8, float* state_f32, const int8_t* x, const int8_t* dt, const int8_t* A_log,
+                     const int8_t* B, const int8_t* C, const int8_t* D, const int8_t* dt_bias, const int8_t* z,
+                     float s_x, float s_dt, float s_A, float s_B, float s_C, float s_D, float s_db, float s_z,
+                     float s_state, int batch, int dim, int dstate, int softplus, float* y) {
+    for (int b = 0; b < batch; ++b) {
+        for (int d = 0; d < dim; ++d) {
+            const int64_t i = (int64_t)b * dim + d;
+            const float xv = s_x * (float)x[i];                                       /* :83 */
+            float dtv = s_dt * (float)dt[i];                                          /* :87 */
+            if (dt_bias) dtv += s_db * (float)dt_bias[d];                             /* :90 */
+            if (softplus) dtv = softplus20(dtv);                                      /* :94 */
+            float acc = 0.0f;
+            for (int n = 0; n < dstate; ++n) {
+                const int64_t si = i * dstate + n;
+                float h = state_f32 ? state_f32[si] : s_state * (float)state_i8[si];  /* :85 */
+                const float A = -expf(s_A * (float)A_log[(int64_t)d * dstate + n]);   /* :96 */
+                const float dA = expf(A * dtv);                                       /* :97 */
+                const float Bv = s_B * (float)B[(int64_t)b * dstate + n];             /* :106 */
+                const float Cv = s_C * (float)C[(int64_t)b * dstate + n];             /* :107 */
+                const float dB = Bv * dtv;                                            /* :114 */
+                h = h * dA + dB * xv;                                                 /* :118 */
+                if (state_f32) state_f32[si] = h;
+                else state_i8[si] = sat8_rne((h * 1e2f) / (s_state * 1e2f));          /* :119 */
+                acc += h * Cv;                                                        /* :121 */
+            }
+            if (D) acc += xv * (s_D * (float)D[d]);                                   /* :122-123 */
+            if (z) {
+                const float zv = s_z * (float)z[i];
+                acc *= zv * (1.0f / (1.0f + expf(-zv)));                              /* :124-125 */
+            }
+            y[i] = acc;
+        }
+    }
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * W8A8 GEMM, csrc/linear/quant_linear_fwd_kernel.cuh:63-130:
+ *   acc = int32 sum_k a[m,k]*w[n,k];  d = s_a[m|0] * (s_b[n|0] * float(acc))  (:85-97)
+ * out_f32 receives the fp32 value before the final cast; out_i8 its int8 cast (round to nearest
+ * even, saturating, :98-100).  round_half_away selects the GEMV epilogue's roundf
+ * (quant_linear_fwd_gemv_kernel.cuh:56-60).
+ * ------------------------------------------------------------------------------------------- */
+void qo_gemm_w8a8(const int8_t* a, const int8_t* w, const float* s_a, int s_a_numel, const float* s_b,
+                  int s_b_numel, int m, int n, int k, int round_half_away, int32_t* acc_out, float* out_f32,
+                  int8_t* out_i8) {
+    for (int i = 0; i < m; ++i) {
+        for (int j = 0; j < n; ++j) {
+            int32_t acc = 0;
+            const int8_t* ar = a + (int64_t)i * k;
+            const int8_t* wr = w + (int64_t)j * k;
+            for (int kk = 0; kk < k; ++kk) acc += (int32_t)ar[kk] * (int32_t)wr[kk];
+            const float sa = s_a[s_a_numel == 1 ? 0 : i];
+            const float sb = s_b[s_b_numel == 1 ? 0 : j];
+            const float v = sa * (sb * (float)acc);
+            const int64_t o = (int64_t)i * n + j;
+            if (acc_out) acc_out[o] = acc;
+            if (out_f32) out_f32[o] = v;
+            if (out_i8) out_i8[o] = round_half_away ? sat8_half_away(v) : sat8_rne(v);
+        }
+    }
+}

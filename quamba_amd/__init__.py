@@ -1,0 +1,3 @@
+"""quamba_amd: MI355X-native (gfx950) kernels behind the Quamba quantized Mamba mixer modules."""
+from .conv import QCausalConv1D  # noqa: F401
+from .sscan import QSScan, quant_selective_scan_fn  # noqa: F401

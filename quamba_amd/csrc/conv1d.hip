@@ -1,0 +1,222 @@
+// int8 depthwise causal conv1d (+SiLU) with int8 requantisation, forward and single-step update.
+//
+// Arithmetic follows the reference kernels op for op:
+//   forward, seqlen-contiguous  csrc/causal_conv1d/quant_causal_conv1d_fwd_kernel.cuh:57-157
+//       v = fma(s_w*s_x, sum_w W[d,w]*x[t-(k-1-w)], s_b*bias[d])
+//   forward, channel-contiguous csrc/causal_conv1d/quant_causal_conv1d_fwd_kernel.cuh:267-383
+//       v = s_b*bias[d];  v = fma((s_w*s_x)*W[d,w], x[..], v) per tap
+//   update                      csrc/causal_conv1d/quant_causal_conv1d_update_kernel.cuh:26-76
+//       same tap-wise order, after shifting the rolling state in place
+//   then v = v / (1 + exp(-v)) if silu, q = sat8(round_half_away(v / s_out)).
+// The kernel is memory-shaped: one 16-byte load and one 16-byte store per 16 outputs, the 3-byte
+// causal halo comes from one extra aligned dword, and the four taps are one packed int8 dot
+// product (exact, so equal to the reference's fp32 accumulation of integer products).
+#include "qa_common.hpp"
+
+namespace qa {
+namespace {
+
+constexpr int kConvThreads = 256;
+
+__device__ __forceinline__ int8_t conv_epilogue(float v, float s_out, int silu) {
+    if (silu) v = v / (1.0f + exp_det(-v));
+    return sat8_half_away(v / s_out);
+}
+
+// packed taps for sdot4: byte j of the window holds x[t-3+j]; tap for x[t-(k-1-w)] is W[w],
+// so byte j pairs with W[j-(4-k)] (zero for j < 4-k).
+__device__ __forceinline__ uint32_t pack_taps(const int8_t* w, int64_t wstride, int width) {
+    uint32_t packed = 0;
+    for (int j = 0; j < 4; ++j) {
+        const int wi = j - (4 - width);
+        const uint32_t b = wi >= 0 ? static_cast<uint8_t>(w[wi * wstride]) : 0u;
+        packed |= b << (8 * j);
+    }
+    return packed;
+}
+
+__device__ __forceinline__ int dot4(uint32_t a, uint32_t b) {
+    return __builtin_amdgcn_sdot4(static_cast<int>(a), static_cast<int>(b), 0, false);
+}
+
+// One thread = 16 consecutive time steps of one (batch, channel) row.  Rows are 16-byte aligned
+// (checked on the host); a ragged tail (seqlen % 16) is handled bytewise by the row's last thread.
+__global__ __launch_bounds__(kConvThreads) void conv_fwd_rows_kernel(QaConvParams p, int segs) {
+    const int64_t idx = static_cast<int64_t>(blockIdx.x) * kConvThreads + threadIdx.x;
+    const int64_t nrows = static_cast<int64_t>(p.batch) * p.dim;
+    if (idx >= nrows * segs) return;
+    const int seg = static_cast<int>(idx % segs);
+    const int64_t row = idx / segs;
+    const int c = static_cast<int>(row % p.dim);
+    const int b = static_cast<int>(row / p.dim);
+    const int8_t* x = p.x + b * p.x_batch_stride + c * p.x_c_stride;
+    int8_t* out = p.out + b * p.out_batch_stride + c * p.out_c_stride;
+
+    const uint32_t taps = pack_taps(p.weight + c * p.weight_c_stride, p.weight_width_stride, p.width);
+    const float s_wx = p.scale_w * p.scale_x;
+    const float bias_f = p.bias ? static_cast<float>(p.bias[c]) * p.scale_b : 0.0f;
+
+    const int t0 = seg * 16;
+    const int remaining = p.seqlen - t0;
+    uint32_t w[5];   // w[0] = x[t0-4 .. t0-1], w[1..4] = x[t0 .. t0+15]
+    w[0] = seg > 0 ? *reinterpret_cast<const uint32_t*>(x + t0 - 4) : 0u;
+    if (remaining >= 16) {
+        const uint4 v = *reinterpret_cast<const uint4*>(x + t0);
+        w[1] = v.x; w[2] = v.y; w[3] = v.z; w[4] = v.w;
+    } else {
+        w[1] = w[2] = w[3] = w[4] = 0u;
+        for (int i = 0; i < remaining; ++i) {
+            w[1 + (i >> 2)] |= static_cast<uint32_t>(static_cast<uint8_t>(x[t0 + i])) << (8 * (i & 3));
+        }
+    }
+    uint32_t o[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        uint32_t packed = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            // window ending at element 4q+j: bytes (4q+j-3 .. 4q+j) of the stream starting at w[1]
+            const uint32_t win = j == 3 ? w[q + 1] : __builtin_amdgcn_alignbyte(w[q + 1], w[q], j + 1);
+            const float acc = static_cast<float>(dot4(win, taps));
+            const float v = __builtin_fmaf(s_wx, acc, bias_f);
+            const int8_t r = conv_epilogue(v, p.scale_out, p.silu_activation);
+            packed |= static_cast<uint32_t>(static_cast<uint8_t>(r)) << (8 * j);
+        }
+        o[q] = packed;
+    }
+    if (remaining >= 16) {
+        *reinterpret_cast<uint4*>(out + t0) = make_uint4(o[0], o[1], o[2], o[3]);
+    } else {
+        for (int i = 0; i < remaining; ++i) {
+            out[t0 + i] = static_cast<int8_t>((o[i >> 2] >> (8 * (i & 3))) & 0xff);
+        }
+    }
+}
+
+// Any strides, one thread per output element.  kTapWise selects the channel-contiguous op order.
+// Lanes run along the contiguous dimension chosen by the host (lanes_along_l).
+template <bool kTapWise>
+__global__ __launch_bounds__(kConvThreads) void conv_fwd_generic_kernel(QaConvParams p, int lanes_along_l) {
+    const int64_t idx = static_cast<int64_t>(blockIdx.x) * kConvThreads + threadIdx.x;
+    const int64_t total = static_cast<int64_t>(p.batch) * p.dim * p.seqlen;
+    if (idx >= total) return;
+    int b, c, t;
+    if (lanes_along_l) {
+        t = static_cast<int>(idx % p.seqlen);
+        c = static_cast<int>((idx / p.seqlen) % p.dim);
+        b = static_cast<int>(idx / (static_cast<int64_t>(p.seqlen) * p.dim));
+    } else {
+        c = static_cast<int>(idx % p.dim);
+        t = static_cast<int>((idx / p.dim) % p.seqlen);
+        b = static_cast<int>(idx / (static_cast<int64_t>(p.seqlen) * p.dim));
+    }
+    const int8_t* x = p.x + b * p.x_batch_stride + c * p.x_c_stride;
+    const int8_t* w = p.weight + c * p.weight_c_stride;
+    const float s_wx = p.scale_w * p.scale_x;
+    const float bias_f = p.bias ? static_cast<float>(p.bias[c]) * p.scale_b : 0.0f;
+    float v;
+    if (kTapWise) {
+        v = bias_f;
+        for (int k = 0; k < p.width; ++k) {
+            const int ti = t - (p.width - 1 - k);
+            const float xv = ti >= 0 ? static_cast<float>(x[ti * p.x_l_stride]) : 0.0f;
+            const float wv = static_cast<float>(w[k * p.weight_width_stride]);
+            v = __builtin_fmaf(s_wx * wv, xv, v);
+        }
+    } else {
+        int acc = 0;
+        for (int k = 0; k < p.width; ++k) {
+            const int ti = t - (p.width - 1 - k);
+            const int xv = ti >= 0 ? x[ti * p.x_l_stride] : 0;
+            acc += xv * static_cast<int>(w[k * p.weight_width_stride]);
+        }
+        v = __builtin_fmaf(s_wx, static_cast<float>(acc), bias_f);
+    }
+    p.out[b * p.out_batch_stride + c * p.out_c_stride + t * p.out_l_stride] =
+        conv_epilogue(v, p.scale_out, p.silu_activation);
+}
+
+// Decode step: one thread per (batch, channel); lanes along channels so x/out are coalesced.
+__global__ __launch_bounds__(kConvThreads) void conv_update_kernel(QaConvParams p) {
+    const int64_t idx = static_cast<int64_t>(blockIdx.x) * kConvThreads + threadIdx.x;
+    if (idx >= static_cast<int64_t>(p.batch) * p.dim) return;
+    const int c = static_cast<int>(idx % p.dim);
+    const int b = static_cast<int>(idx / p.dim);
+    int8_t* st = p.conv_state + b * p.conv_state_batch_stride + c * p.conv_state_c_stride;
+    const int8_t* w = p.weight + c * p.weight_c_stride;
+    const int width = p.width;
+    const int slen = p.conv_state_len;            // width (slot 0 is dropped) or width-1
+    const int drop = slen - (width - 1);          // 1 or 0
+    int8_t xs[4];
+    for (int i = 0; i < width - 1; ++i) xs[i] = st[(i + drop) * p.conv_state_l_stride];
+    xs[width - 1] = p.x[b * p.x_batch_stride + c * p.x_c_stride];
+    for (int i = 0; i < slen; ++i) st[i * p.conv_state_l_stride] = xs[i + (width - slen)];
+    const float s_wx = p.scale_w * p.scale_x;
+    float v = p.bias ? static_cast<float>(p.bias[c]) * p.scale_b : 0.0f;
+    for (int i = 0; i < width; ++i) {
+        const float wv = static_cast<float>(w[i * p.weight_width_stride]);
+        v = __builtin_fmaf(s_wx * wv, static_cast<float>(xs[i]), v);
+    }
+    p.out[b * p.out_batch_stride + c * p.out_c_stride] = conv_epilogue(v, p.scale_out, p.silu_activation);
+}
+
+int validate_common(const QaConvParams* p) {
+    if (!p || !p->x || !p->weight || !p->out) return QA_ERR_NULL;
+    if (p->batch < 0 || p->dim < 0 || p->seqlen < 0) return QA_ERR_SHAPE;
+    if (p->width < 2 || p->width > 4) return QA_ERR_SHAPE;
+    return QA_OK;
+}
+
+}  // namespace
+}  // namespace qa
+
+extern "C" int qa_causal_conv1d_fwd(const QaConvParams* p, void* stream_) {
+    using namespace qa;
+    int st = validate_common(p);
+    if (st != QA_OK) return st;
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const int64_t total = static_cast<int64_t>(p->batch) * p->dim * p->seqlen;
+    if (total == 0) return QA_OK;
+    const bool l_contig = p->x_l_stride == 1 || p->seqlen == 1;
+    const bool c_contig = p->x_c_stride == 1 || p->dim == 1;
+    if (!l_contig && !c_contig) return QA_ERR_STRIDE;
+    const bool channel_last = !l_contig || (p->x_c_stride == 1 && p->x_l_stride > 1);
+    if (!channel_last) {
+        const bool rows_ok = p->out_l_stride == 1 && aligned16(p->x) && aligned16(p->out) &&
+                             p->x_batch_stride % 16 == 0 && p->x_c_stride % 16 == 0 &&
+                             p->out_batch_stride % 16 == 0 && p->out_c_stride % 16 == 0;
+        if (rows_ok) {
+            const int segs = (p->seqlen + 15) / 16;
+            const int64_t threads = static_cast<int64_t>(p->batch) * p->dim * segs;
+            const int64_t blocks = (threads + kConvThreads - 1) / kConvThreads;
+            if (blocks > 0x7fffffffLL) return QA_ERR_SHAPE;
+            hipLaunchKernelGGL(conv_fwd_rows_kernel, dim3(static_cast<unsigned>(blocks)), dim3(kConvThreads), 0,
+                               stream, *p, segs);
+            return check_launch();
+        }
+    }
+    const int64_t blocks = (total + kConvThreads - 1) / kConvThreads;
+    if (blocks > 0x7fffffffLL) return QA_ERR_SHAPE;
+    if (channel_last) {
+        hipLaunchKernelGGL(conv_fwd_generic_kernel<true>, dim3(static_cast<unsigned>(blocks)), dim3(kConvThreads),
+                           0, stream, *p, 0);
+    } else {
+        hipLaunchKernelGGL(conv_fwd_generic_kernel<false>, dim3(static_cast<unsigned>(blocks)), dim3(kConvThreads),
+                           0, stream, *p, 1);
+    }
+    return check_launch();
+}
+
+extern "C" int qa_causal_conv1d_update(const QaConvParams* p, void* stream_) {
+    using namespace qa;
+    int st = validate_common(p);
+    if (st != QA_OK) return st;
+    if (!p->conv_state) return QA_ERR_NULL;
+    if (p->conv_state_len != p->width && p->conv_state_len != p->width - 1) return QA_ERR_SHAPE;
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const int64_t total = static_cast<int64_t>(p->batch) * p->dim;
+    if (total == 0) return QA_OK;
+    const int64_t blocks = (total + kConvThreads - 1) / kConvThreads;
+    hipLaunchKernelGGL(conv_update_kernel, dim3(static_cast<unsigned>(blocks)), dim3(kConvThreads), 0, stream, *p);
+    return check_launch();
+}

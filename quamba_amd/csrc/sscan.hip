@@ -1,0 +1,455 @@
+// Mamba1 int8 selective scan: forward over a sequence, and the single-token state update.
+//
+// Arithmetic (reference csrc/selective_scan/quant_sscan_fwd_kernel.cuh:110-293):
+//   u = s_u q_u;  dt = softplus20(s_dt q_dt + s_db q_db[d]);  A[n] = -exp(s_A q_Alog[d,n])
+//   h[n] = exp(dt A[n]) h[n] + (s_B q_B[n,t]) (dt u);  y = D u + sum_n h[n] (s_C q_C[n,t]);  y *= silu(s_z q_z)
+// Output fp16 (tolerance, not bits): exp runs on the hardware exp2 with A pre-multiplied by log2(e).
+//
+// Mapping for gfx950.  The recurrence is sequential in time and costs one transcendental plus four
+// multiply-adds per (channel, step, state), which is more VALU time than the bytes cost HBM time,
+// so the kernel walks time once, keeps the state in registers and never recomputes:
+//   * a lane owns one channel and NPL of its states; NSPLIT neighbouring lanes share a channel
+//     (their partial dot products meet in a cross-lane add), so the number of waves can be raised
+//     without a second pass over time;
+//   * u / dt / z rows are staged through LDS in tiles of T steps with 16-byte global loads, rows
+//     padded so the per-lane dword reads are bank-conflict free;
+//   * B and C (shared by every channel of a batch entry) are converted to fp32 and scaled once per
+//     workgroup and read from LDS as 16-byte broadcasts;
+//   * the fp16 output is staged through LDS so each time step is written as one contiguous run of
+//     channels in the (batch, seqlen, dim) tensor - no transposition pass afterwards;
+//   * global loads of tile i+1 are issued before the arithmetic of tile i and held in registers
+//     until the tile has been consumed, then written to LDS.
+#include "qa_common.hpp"
+
+namespace qa {
+namespace {
+
+constexpr float kLog2e = 1.44269504088896341f;
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+
+// softplus with the reference's threshold; log1p evaluated so that small exp(x) keeps full
+// relative accuracy (series below 2^-6, log2 above).
+__device__ __forceinline__ float softplus20(float x) {
+    if (x > 20.0f) return x;
+    const float e = fast_exp2(x * kLog2e);
+    const float series = e * __builtin_fmaf(e, __builtin_fmaf(e, __builtin_fmaf(e, -0.25f, 1.0f / 3.0f), -0.5f), 1.0f);
+    const float big = fast_log2(1.0f + e) * 0.693147180559945309f;
+    return e < 0.015625f ? series : big;
+}
+
+__device__ __forceinline__ float silu_gate(float z) {
+    return z * fast_rcp(1.0f + fast_exp2(-z * kLog2e));
+}
+
+__device__ __forceinline__ float i8_of(uint32_t word, int j) {
+    return static_cast<float>(static_cast<int8_t>((word >> (8 * j)) & 0xffu));
+}
+
+// 16 bytes starting at row[t]; bytes at or beyond t_end read as zero.
+__device__ __forceinline__ uint4 load16(const int8_t* row, int t, int t_end, bool vec) {
+    if (vec && t + 16 <= t_end) return *reinterpret_cast<const uint4*>(row + t);
+    uint32_t w[4] = {0u, 0u, 0u, 0u};
+    for (int i = 0; i < 16; ++i) {
+        if (t + i < t_end) w[i >> 2] |= static_cast<uint32_t>(static_cast<uint8_t>(row[t + i])) << (8 * (i & 3));
+    }
+    return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+template <int NPL, int NSPLIT, int T, int WAVES>
+struct ScanCfg {
+    static constexpr int kThreads = 64 * WAVES;
+    static constexpr int kCh = kThreads / NSPLIT;          // channels per workgroup
+    static constexpr int kNP = NPL * NSPLIT;               // padded state count
+    static constexpr int kRow = T + 4;                     // staged row pitch in bytes
+    static constexpr int kInPieces = (kCh * T / 16 + kThreads - 1) / kThreads;       // per tensor
+    static constexpr int kBcPieces = (2 * kNP * T / 16 + kThreads - 1) / kThreads;
+    static constexpr int kOutPitch = kCh + 8;              // halves; keeps rows 16-byte aligned
+};
+
+template <int NPL, int NSPLIT, int T, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void sscan_fwd_kernel(QaSScanParams p, int vec_in, int vec_bc, int vec_out) {
+    using Cfg = ScanCfg<NPL, NSPLIT, T, WAVES>;
+    constexpr int kThreads = Cfg::kThreads, kCh = Cfg::kCh, kNP = Cfg::kNP, kRow = Cfg::kRow;
+    constexpr int kInPieces = Cfg::kInPieces, kBcPieces = Cfg::kBcPieces, kOutPitch = Cfg::kOutPitch;
+    constexpr int kPiecesPerRow = T / 16;
+
+    __shared__ __attribute__((aligned(16))) uint32_t s_in[3][kCh * kRow / 4];
+    __shared__ __attribute__((aligned(16))) float s_bc[T][2][kNP];
+    __shared__ __attribute__((aligned(16))) __half s_out[T][kOutPitch];
+
+    const int tid = threadIdx.x;
+    const int c_local = tid / NSPLIT;
+    const int slice = tid % NSPLIT;
+    const int c0 = blockIdx.x * kCh;
+    const int b = blockIdx.y;
+    const int c = c0 + c_local;
+    const bool c_ok = c < p.dim;
+    const int cc = c_ok ? c : p.dim - 1;                   // clamped channel for parameter loads
+    const int g = c0 / (p.dim / p.n_groups);
+    const bool has_z = p.z != nullptr;
+    const int L = p.seqlen;
+
+    const float s_u = *p.scale_u, s_dt = *p.scale_delta, s_A = *p.scale_A, s_B = *p.scale_B, s_C = *p.scale_C;
+    const float s_z = has_z ? *p.scale_z : 0.0f;
+    const float D_f = p.D ? *p.scale_D * static_cast<float>(p.D[cc]) : 0.0f;
+    const float db = p.delta_bias ? *p.scale_delta_bias * static_cast<float>(p.delta_bias[cc]) : 0.0f;
+
+    float A2[NPL], h[NPL];
+#pragma unroll
+    for (int j = 0; j < NPL; ++j) {
+        const int n = slice * NPL + j;
+        h[j] = 0.0f;
+        A2[j] = n < p.dstate
+                    ? -expf(s_A * static_cast<float>(p.A_log[cc * p.A_d_stride + n * p.A_dstate_stride])) * kLog2e
+                    : 0.0f;
+    }
+
+    const int8_t* in_base[3] = {p.u + b * p.u_batch_stride, p.delta + b * p.delta_batch_stride,
+                                has_z ? p.z + b * p.z_batch_stride : nullptr};
+    const int64_t in_dstride[3] = {p.u_d_stride, p.delta_d_stride, p.z_d_stride};
+    const int8_t* bc_base[2] = {p.B + b * p.B_batch_stride + g * p.B_group_stride,
+                                p.C + b * p.C_batch_stride + g * p.C_group_stride};
+    const int64_t bc_nstride[2] = {p.B_dstate_stride, p.C_dstate_stride};
+    const float bc_scale[2] = {s_B, s_C};
+
+    uint4 r_in[3][kInPieces];
+    uint4 r_bc[kBcPieces];
+
+    auto issue_loads = [&](int t0) {
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            if (k == 2 && !has_z) break;
+#pragma unroll
+            for (int i = 0; i < kInPieces; ++i) {
+                const int piece = tid + i * kThreads;
+                const int row = piece / kPiecesPerRow, col = piece % kPiecesPerRow;
+                uint4 v = make_uint4(0u, 0u, 0u, 0u);
+                if (piece < kCh * kPiecesPerRow && c0 + row < p.dim) {
+                    v = load16(in_base[k] + (c0 + row) * in_dstride[k], t0 + col * 16, L, vec_in);
+                }
+                r_in[k][i] = v;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kBcPieces; ++i) {
+            const int piece = tid + i * kThreads;
+            const int which = piece / (kNP * kPiecesPerRow);
+            const int rem = piece % (kNP * kPiecesPerRow);
+            const int n = rem / kPiecesPerRow, col = rem % kPiecesPerRow;
+            uint4 v = make_uint4(0u, 0u, 0u, 0u);
+            if (which < 2 && n < p.dstate) {
+                v = load16(bc_base[which] + n * bc_nstride[which], t0 + col * 16, L, vec_bc);
+            }
+            r_bc[i] = v;
+        }
+    };
+
+    auto stage = [&]() {
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            if (k == 2 && !has_z) break;
+#pragma unroll
+            for (int i = 0; i < kInPieces; ++i) {
+                const int piece = tid + i * kThreads;
+                if (piece < kCh * kPiecesPerRow) {
+                    const int row = piece / kPiecesPerRow, col = piece % kPiecesPerRow;
+                    uint32_t* dst = &s_in[k][(row * kRow + col * 16) / 4];
+                    dst[0] = r_in[k][i].x; dst[1] = r_in[k][i].y; dst[2] = r_in[k][i].z; dst[3] = r_in[k][i].w;
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kBcPieces; ++i) {
+            const int piece = tid + i * kThreads;
+            const int which = piece / (kNP * kPiecesPerRow);
+            if (which < 2) {
+                const int rem = piece % (kNP * kPiecesPerRow);
+                const int n = rem / kPiecesPerRow, col = rem % kPiecesPerRow;
+                const uint32_t w[4] = {r_bc[i].x, r_bc[i].y, r_bc[i].z, r_bc[i].w};
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    s_bc[col * 16 + e][which][n] = bc_scale[which] * i8_of(w[e >> 2], e & 3);
+                }
+            }
+        }
+    };
+
+    const int n_tiles = (L + T - 1) / T;
+    issue_loads(0);
+    stage();
+    __syncthreads();
+
+    for (int tile = 0; tile < n_tiles; ++tile) {
+        const int t0 = tile * T;
+        const int nt = min(T, L - t0);
+        if (tile + 1 < n_tiles) issue_loads(t0 + T);
+
+        const uint32_t* su = &s_in[0][c_local * kRow / 4];
+        const uint32_t* sd = &s_in[1][c_local * kRow / 4];
+        const uint32_t* sz = &s_in[2][c_local * kRow / 4];
+        for (int tq = 0; tq < T / 4; ++tq) {
+            if (tq * 4 >= nt) break;
+            const uint32_t u4 = su[tq], d4 = sd[tq];
+            const uint32_t z4 = has_z ? sz[tq] : 0u;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int t = tq * 4 + j;
+                if (t >= nt) break;
+                const float u_val = s_u * i8_of(u4, j);
+                float dt = __builtin_fmaf(s_dt, i8_of(d4, j), db);
+                if (p.delta_softplus) dt = softplus20(dt);
+                const float du = dt * u_val;
+                const float4* bf = reinterpret_cast<const float4*>(&s_bc[t][0][slice * NPL]);
+                const float4* cf = reinterpret_cast<const float4*>(&s_bc[t][1][slice * NPL]);
+                float acc = 0.0f;
+#pragma unroll
+                for (int q = 0; q < NPL / 4; ++q) {
+                    const float4 Bv = bf[q];
+                    const float4 Cv = cf[q];
+                    const float Bs[4] = {Bv.x, Bv.y, Bv.z, Bv.w};
+                    const float Cs[4] = {Cv.x, Cv.y, Cv.z, Cv.w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int n = q * 4 + e;
+                        const float a = fast_exp2(dt * A2[n]);
+                        h[n] = __builtin_fmaf(a, h[n], Bs[e] * du);
+                        acc = __builtin_fmaf(h[n], Cs[e], acc);
+                    }
+                }
+#pragma unroll
+                for (int m = 1; m < NSPLIT; m <<= 1) acc += __shfl_xor(acc, m);
+                float y = __builtin_fmaf(D_f, u_val, acc);
+                if (has_z) y *= silu_gate(s_z * i8_of(z4, j));
+                if (slice == 0) s_out[t][c_local] = __float2half(y);
+            }
+        }
+        __syncthreads();   // s_out complete; everyone is done reading the staged tile
+
+        // write the tile's output rows: (t, kCh channels) contiguous along channels
+        {
+            constexpr int kChunk = kCh >= 8 ? 8 : kCh;
+            constexpr int kChunksPerRow = kCh / kChunk;
+            __half* out_b = static_cast<__half*>(p.out) + b * p.out_batch_stride;
+            for (int piece = tid; piece < nt * kChunksPerRow; piece += kThreads) {
+                const int t = piece / kChunksPerRow, ch8 = (piece % kChunksPerRow) * kChunk;
+                __half* dst = out_b + (t0 + t) * p.out_l_stride + (c0 + ch8) * p.out_d_stride;
+                if (kChunk == 8 && vec_out && c0 + ch8 + 8 <= p.dim) {
+                    *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(&s_out[t][ch8]);
+                } else {
+                    for (int e = 0; e < kChunk; ++e) {
+                        if (c0 + ch8 + e < p.dim) dst[e * p.out_d_stride] = s_out[t][ch8 + e];
+                    }
+                }
+            }
+        }
+        if (tile + 1 < n_tiles) stage();
+        __syncthreads();
+    }
+
+    if (c_ok) {
+        const int64_t base = (static_cast<int64_t>(b) * p.dim + c) * p.dstate;
+        const float s_state = p.last_state_i8 ? *p.scale_ssm_state : 1.0f;
+#pragma unroll
+        for (int j = 0; j < NPL; ++j) {
+            const int n = slice * NPL + j;
+            if (n < p.dstate) {
+                if (p.last_state_f32) p.last_state_f32[base + n] = h[j];
+                if (p.last_state_i8) p.last_state_i8[base + n] = sat8_half_away(h[j] / s_state);
+            }
+        }
+    }
+}
+
+template <int NPL, int NSPLIT, int T, int WAVES>
+int launch_fwd(const QaSScanParams& p, hipStream_t stream, int vec_in, int vec_bc, int vec_out) {
+    using Cfg = ScanCfg<NPL, NSPLIT, T, WAVES>;
+    if (p.n_groups > 1 && (p.dim / p.n_groups) % Cfg::kCh != 0) return QA_ERR_UNSUPPORTED;
+    dim3 grid((p.dim + Cfg::kCh - 1) / Cfg::kCh, p.batch);
+    hipLaunchKernelGGL((sscan_fwd_kernel<NPL, NSPLIT, T, WAVES>), grid, dim3(Cfg::kThreads), 0, stream, p, vec_in,
+                       vec_bc, vec_out);
+    return check_launch();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Single-token update.  LPR lanes share one (batch, head, channel) row, four states per lane, so
+// consecutive lanes touch consecutive 16-byte (fp32 state) or 4-byte (int8 state) pieces.
+// Reference: quamba/triton/selective_state_update.py:83-126 and :303-362.
+// ---------------------------------------------------------------------------------------------
+template <int LPR>
+__global__ __launch_bounds__(256) void ssm_update_kernel(QaSsmUpdateParams p) {
+    const int64_t gid = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    const int64_t row = gid / LPR;
+    const int sub = static_cast<int>(gid % LPR);
+    const int64_t nrows = static_cast<int64_t>(p.batch) * p.nheads * p.dim;
+    const bool row_ok = row < nrows;
+    const int64_t r = row_ok ? row : nrows - 1;
+    const int d = static_cast<int>(r % p.dim);
+    const int hd = static_cast<int>((r / p.dim) % p.nheads);
+    const int b = static_cast<int>(r / (static_cast<int64_t>(p.dim) * p.nheads));
+    const int heads_per_group = p.nheads / p.ngroups;
+    const int g = hd / heads_per_group;
+
+    const bool grouped = p.nhead_groups > 0;
+    float x_scale, B_scale, C_scale;
+    const float* state_scale_row;      // grouped: [dstate] scales of this (g, hg, dg)
+    if (grouped) {
+        int hg = 0, dg = 0;
+        const int hrel = hd % heads_per_group;
+        for (int j = 0; j < p.nhead_groups; ++j) hg += hrel >= p.x_head_group_range[g * p.nhead_groups + j] ? 1 : 0;
+        hg = min(hg, p.nhead_groups - 1);
+        const int32_t* dr = p.x_dim_group_range + (g * p.nhead_groups + hg) * p.ndim_groups;
+        for (int j = 0; j < p.ndim_groups; ++j) dg += d >= dr[j] ? 1 : 0;
+        dg = min(dg, p.ndim_groups - 1);
+        const int sidx = (g * p.nhead_groups + hg) * p.ndim_groups + dg;
+        x_scale = p.x_scale[sidx];
+        state_scale_row = p.state_is_fp32 ? nullptr : p.state_scale + static_cast<int64_t>(sidx) * p.dstate;
+        B_scale = p.B_scale[g];
+        C_scale = p.C_scale[g];
+    } else {
+        x_scale = *p.x_scale;
+        state_scale_row = nullptr;
+        B_scale = *p.B_scale;
+        C_scale = *p.C_scale;
+    }
+    const float s_state = (!grouped && !p.state_is_fp32) ? *p.state_scale : 1.0f;
+    const float requant_k = grouped ? 1e6f : 1e2f;
+
+    const float xv = x_scale * static_cast<float>(p.x[b * p.x_batch_stride + hd * p.x_head_stride + d * p.x_dim_stride]);
+    float dt = *p.dt_scale * static_cast<float>(p.dt[b * p.dt_batch_stride + hd * p.dt_head_stride + d * p.dt_dim_stride]);
+    if (p.dt_bias) {
+        const int64_t bi = hd * p.dt_bias_head_stride + d * p.dt_bias_dim_stride;
+        dt += p.dt_bias_is_fp16 ? __half2float(static_cast<const __half*>(p.dt_bias)[bi])
+                                : *p.dt_bias_scale * static_cast<float>(static_cast<const int8_t*>(p.dt_bias)[bi]);
+    }
+    if (p.dt_softplus) dt = dt <= 20.0f ? log1pf(expf(dt)) : dt;
+    const float A_scale = *p.A_log_scale;
+
+    float acc = 0.0f;
+    const int64_t st_base = b * p.state_batch_stride + hd * p.state_head_stride + d * p.state_dim_stride;
+    const int8_t* Bp = p.B + b * p.B_batch_stride + g * p.B_group_stride;
+    const int8_t* Cp = p.C + b * p.C_batch_stride + g * p.C_group_stride;
+    const int8_t* Ap = p.A_log + hd * p.A_head_stride + d * p.A_dim_stride;
+    for (int n0 = sub * 4; n0 < p.dstate; n0 += LPR * 4) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int n = n0 + e;
+            if (n >= p.dstate) break;
+            const int64_t si = st_base + n * p.state_dstate_stride;
+            const float sc = state_scale_row ? state_scale_row[n] : s_state;
+            float hv = p.state_is_fp32 ? static_cast<const float*>(p.state)[si]
+                                       : sc * static_cast<float>(static_cast<const int8_t*>(p.state)[si]);
+            const float A = -expf(A_scale * static_cast<float>(Ap[n * p.A_dstate_stride]));
+            const float dA = expf(A * dt);
+            const float Bv = B_scale * static_cast<float>(Bp[n * p.B_dstate_stride]);
+            const float Cv = C_scale * static_cast<float>(Cp[n * p.C_dstate_stride]);
+            hv = hv * dA + (Bv * dt) * xv;
+            if (row_ok) {
+                if (p.state_is_fp32) static_cast<float*>(p.state)[si] = hv;
+                else static_cast<int8_t*>(p.state)[si] = sat8_rne((hv * requant_k) / (sc * requant_k));
+            }
+            acc += hv * Cv;
+        }
+    }
+#pragma unroll
+    for (int m = 1; m < LPR; m <<= 1) acc += __shfl_xor(acc, m);
+    if (row_ok && sub == 0) {
+        if (p.D) acc += xv * (*p.D_scale * static_cast<float>(p.D[hd * p.D_head_stride + d * p.D_dim_stride]));
+        if (p.z) {
+            const float zv = *p.z_scale * static_cast<float>(p.z[b * p.z_batch_stride + hd * p.z_head_stride + d * p.z_dim_stride]);
+            acc *= zv * (1.0f / (1.0f + expf(-zv)));
+        }
+        static_cast<__half*>(p.out)[b * p.out_batch_stride + hd * p.out_head_stride + d * p.out_dim_stride] =
+            __float2half(acc);
+    }
+}
+
+template <int LPR>
+int launch_update(const QaSsmUpdateParams& p, hipStream_t stream) {
+    const int64_t threads = static_cast<int64_t>(p.batch) * p.nheads * p.dim * LPR;
+    const int64_t blocks = (threads + 255) / 256;
+    if (blocks > 0x7fffffffLL) return QA_ERR_SHAPE;
+    hipLaunchKernelGGL(ssm_update_kernel<LPR>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, p);
+    return check_launch();
+}
+
+}  // namespace
+}  // namespace qa
+
+// Variant override for tuning runs: QA_SSCAN_VARIANT = "<nsplit>x<waves>" (e.g. "4x2").
+static int sscan_variant_from_env(int* nsplit, int* waves) {
+    const char* s = getenv("QA_SSCAN_VARIANT");
+    if (!s) return 0;
+    return sscanf(s, "%dx%d", nsplit, waves) == 2;
+}
+
+extern "C" int qa_sscan_fwd(const QaSScanParams* p, void* stream_) {
+    using namespace qa;
+    if (!p || !p->u || !p->delta || !p->A_log || !p->B || !p->C || !p->out) return QA_ERR_NULL;
+    if (!p->scale_u || !p->scale_delta || !p->scale_A || !p->scale_B || !p->scale_C) return QA_ERR_NULL;
+    if ((p->D && !p->scale_D) || (p->delta_bias && !p->scale_delta_bias) || (p->z && !p->scale_z)) return QA_ERR_NULL;
+    if (p->last_state_i8 && !p->scale_ssm_state) return QA_ERR_NULL;
+    if (p->batch < 0 || p->dim < 0 || p->seqlen < 0 || p->dstate < 1 || p->dstate > 256) return QA_ERR_SHAPE;
+    if (p->n_groups < 1 || (p->dim > 0 && p->dim % p->n_groups != 0)) return QA_ERR_SHAPE;
+    if (p->batch == 0 || p->dim == 0) return QA_OK;
+    if (p->batch > 65535) return QA_ERR_SHAPE;
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+
+    auto ok16 = [](const void* ptr, std::initializer_list<int64_t> strides) {
+        if (!aligned16(ptr)) return 0;
+        for (int64_t s : strides) if (s % 16 != 0) return 0;
+        return 1;
+    };
+    int vec_in = ok16(p->u, {p->u_batch_stride, p->u_d_stride}) && ok16(p->delta, {p->delta_batch_stride, p->delta_d_stride});
+    if (p->z) vec_in = vec_in && ok16(p->z, {p->z_batch_stride, p->z_d_stride});
+    const int vec_bc = ok16(p->B, {p->B_batch_stride, p->B_group_stride, p->B_dstate_stride}) &&
+                       ok16(p->C, {p->C_batch_stride, p->C_group_stride, p->C_dstate_stride});
+    const int vec_out = p->out_d_stride == 1 && aligned16(p->out) && p->out_batch_stride % 8 == 0 &&
+                        p->out_l_stride % 8 == 0;
+
+    const int N = p->dstate;
+    if (N <= 16) {
+        int nsplit = 0, waves = 0;
+        if (!sscan_variant_from_env(&nsplit, &waves)) {
+            // enough waves to give every SIMD of the chip (1024) a few, else split the states
+            const int64_t rows = static_cast<int64_t>(p->batch) * p->dim;
+            nsplit = rows >= 4 * 65536 ? 1 : rows >= 2 * 65536 ? 2 : 4;
+            waves = 1;
+        }
+        if (nsplit == 1 && waves == 1) return launch_fwd<16, 1, 64, 1>(*p, stream, vec_in, vec_bc, vec_out);
+        if (nsplit == 2 && waves == 1) return launch_fwd<8, 2, 64, 1>(*p, stream, vec_in, vec_bc, vec_out);
+        if (nsplit == 2 && waves == 2) return launch_fwd<8, 2, 64, 2>(*p, stream, vec_in, vec_bc, vec_out);
+        if (nsplit == 4 && waves == 1) return launch_fwd<4, 4, 64, 1>(*p, stream, vec_in, vec_bc, vec_out);
+        if (nsplit == 4 && waves == 2) return launch_fwd<4, 4, 64, 2>(*p, stream, vec_in, vec_bc, vec_out);
+        if (nsplit == 4 && waves == 4) return launch_fwd<4, 4, 64, 4>(*p, stream, vec_in, vec_bc, vec_out);
+        return QA_ERR_UNSUPPORTED;
+    }
+    if (N <= 32) return launch_fwd<8, 4, 64, 1>(*p, stream, vec_in, vec_bc, vec_out);
+    if (N <= 64) return launch_fwd<8, 8, 32, 1>(*p, stream, vec_in, vec_bc, vec_out);
+    if (N <= 128) return launch_fwd<8, 16, 16, 1>(*p, stream, vec_in, vec_bc, vec_out);
+    return launch_fwd<16, 16, 16, 1>(*p, stream, vec_in, vec_bc, vec_out);
+}
+
+extern "C" int qa_ssm_state_update(const QaSsmUpdateParams* p, void* stream_) {
+    using namespace qa;
+    if (!p || !p->state || !p->x || !p->dt || !p->A_log || !p->B || !p->C || !p->out) return QA_ERR_NULL;
+    if (!p->x_scale || !p->dt_scale || !p->A_log_scale || !p->B_scale || !p->C_scale) return QA_ERR_NULL;
+    if (!p->state_is_fp32 && !p->state_scale) return QA_ERR_NULL;
+    if ((p->D && !p->D_scale) || (p->z && !p->z_scale)) return QA_ERR_NULL;
+    if (p->dt_bias && !p->dt_bias_is_fp16 && !p->dt_bias_scale) return QA_ERR_NULL;
+    if (p->nhead_groups > 0 && (!p->x_head_group_range || !p->x_dim_group_range || p->ndim_groups < 1)) return QA_ERR_NULL;
+    if (p->batch < 0 || p->nheads < 1 || p->dim < 0 || p->dstate < 1 || p->dstate > 256) return QA_ERR_SHAPE;
+    if (p->ngroups < 1 || p->nheads % p->ngroups != 0) return QA_ERR_SHAPE;
+    if (p->batch == 0 || p->dim == 0) return QA_OK;
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const int N = p->dstate;
+    if (N <= 4) return launch_update<1>(*p, stream);
+    if (N <= 8) return launch_update<2>(*p, stream);
+    if (N <= 16) return launch_update<4>(*p, stream);
+    if (N <= 32) return launch_update<8>(*p, stream);
+    if (N <= 64) return launch_update<16>(*p, stream);
+    if (N <= 128) return launch_update<32>(*p, stream);
+    return launch_update<64>(*p, stream);
+}

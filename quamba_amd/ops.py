@@ -1,0 +1,288 @@
+"""Functional operator layer: one Python function per extension entry point of the reference,
+with the reference's argument order and error behaviour, each forwarding to the C ABI of
+libquamba_amd.so on the tensor's device and torch's current stream.
+
+Reference interfaces mirrored here:
+  quant_causal_conv1d_cuda.fwd / .update   csrc/causal_conv1d/quant_causal_conv1d.cpp:76-226
+  quant_sscan_cuda.fwd                     csrc/selective_scan/quant_sscan.cpp:122-265
+  quant_sscan_update_triton                quamba/triton/selective_state_update.py:129-227
+  quant_linear_cuda.cutlass_scaled_mm_dq   csrc/linear/quant_linear_fwd_kernel.cuh:356-378
+"""
+import ctypes as C
+
+import torch
+
+from . import _lib
+from ._lib import ptr
+
+
+def _require(cond, msg):
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _require_gpu(t, name):
+    _require(t.is_cuda, f"{name} must be a GPU tensor (quamba_amd has no CPU path)")
+
+
+# ----------------------------------------------------------------------------------------------
+# causal conv1d
+# ----------------------------------------------------------------------------------------------
+def causal_conv1d_fwd(x, scale_x, weight, scale_w, scale_out, scale_b, bias=None, seq_idx=None,
+                      initial_states=None, final_states_out=None, silu_activation=True):
+    """int8 (batch, dim, seqlen) -> int8 of the same shape and strides."""
+    _require(x.dtype == torch.int8 and weight.dtype == torch.int8, "x and weight must be int8")
+    _require_gpu(x, "x")
+    _require_gpu(weight, "weight")
+    _require(x.dim() == 3, "x must have shape (batch, dim, seqlen)")
+    batch, dim, seqlen = x.shape
+    width = weight.shape[-1]
+    _require(tuple(weight.shape) == (dim, width), "weight must have shape (dim, width)")
+    _require(x.stride(2) == 1 or x.stride(1) == 1, "x must be contiguous along seqlen or along channels")
+    _require(2 <= width <= 4, "causal_conv1d only supports width between 2 and 4")
+    if bias is not None:
+        _require(bias.dtype == torch.int8 and bias.is_cuda and tuple(bias.shape) == (dim,) and bias.stride(-1) == 1,
+                 "bias must be a contiguous int8 GPU tensor of shape (dim,)")
+    if seq_idx is not None:
+        raise NotImplementedError("No implementation for seq_idx")
+    if initial_states is not None:
+        raise NotImplementedError("No implementation for initial_states")
+    if final_states_out is not None:
+        raise NotImplementedError("No implementation for final_states_out")
+    out = torch.empty_like(x)  # preserves strides for dense (possibly permuted) inputs
+    if out.stride() != x.stride():
+        out = torch.empty_strided(x.shape, x.stride(), dtype=x.dtype, device=x.device)
+    p = _lib.QaConvParams()
+    p.batch, p.dim, p.seqlen, p.width = batch, dim, seqlen, width
+    p.silu_activation = int(bool(silu_activation))
+    p.x_batch_stride, p.x_c_stride, p.x_l_stride = x.stride()
+    p.out_batch_stride, p.out_c_stride, p.out_l_stride = out.stride()
+    p.weight_c_stride, p.weight_width_stride = weight.stride()
+    p.x, p.weight, p.bias, p.out = ptr(x), ptr(weight), ptr(bias), ptr(out)
+    p.scale_x, p.scale_w, p.scale_b, p.scale_out = float(scale_x), float(scale_w), float(scale_b), float(scale_out)
+    with torch.cuda.device(x.device):
+        st = _lib.lib().qa_causal_conv1d_fwd(C.byref(p), _lib.current_stream(x.device))
+    _lib.check(st, "causal_conv1d_fwd")
+    return out
+
+
+def causal_conv1d_update(x, conv_state, scale_x, weight, scale_w, scale_out, scale_b, bias=None,
+                         silu_activation=True):
+    """One decode step: x int8 (batch, dim); conv_state int8 (batch, dim, width) or
+    (batch, dim, width-1), shifted in place."""
+    _require(x.dtype == torch.int8 and weight.dtype == torch.int8 and conv_state.dtype == torch.int8,
+             "x, weight and conv_state must be int8")
+    for t, n in ((x, "x"), (conv_state, "conv_state"), (weight, "weight")):
+        _require_gpu(t, n)
+    _require(x.dim() == 2, "x must have shape (batch, dim)")
+    batch, dim = x.shape
+    width = weight.shape[-1]
+    _require(tuple(weight.shape) == (dim, width), "weight must have shape (dim, width)")
+    _require(2 <= width <= 4, "causal_conv1d only supports width between 2 and 4")
+    _require(conv_state.dim() == 3 and tuple(conv_state.shape[:2]) == (batch, dim)
+             and conv_state.shape[2] in (width, width - 1),
+             "conv_state must have shape (batch, dim, width) or (batch, dim, width-1)")
+    if bias is not None:
+        _require(bias.dtype == torch.int8 and bias.is_cuda and tuple(bias.shape) == (dim,) and bias.stride(-1) == 1,
+                 "bias must be a contiguous int8 GPU tensor of shape (dim,)")
+    out = torch.empty_like(x)
+    p = _lib.QaConvParams()
+    p.batch, p.dim, p.seqlen, p.width = batch, dim, 1, width
+    p.silu_activation = int(bool(silu_activation))
+    p.x_batch_stride, p.x_c_stride, p.x_l_stride = x.stride(0), x.stride(1), 1
+    p.out_batch_stride, p.out_c_stride, p.out_l_stride = out.stride(0), out.stride(1), 1
+    p.weight_c_stride, p.weight_width_stride = weight.stride()
+    p.conv_state_batch_stride, p.conv_state_c_stride, p.conv_state_l_stride = conv_state.stride()
+    p.conv_state_len = conv_state.shape[2]
+    p.x, p.weight, p.bias, p.out, p.conv_state = ptr(x), ptr(weight), ptr(bias), ptr(out), ptr(conv_state)
+    p.scale_x, p.scale_w, p.scale_b, p.scale_out = float(scale_x), float(scale_w), float(scale_b), float(scale_out)
+    with torch.cuda.device(x.device):
+        st = _lib.lib().qa_causal_conv1d_update(C.byref(p), _lib.current_stream(x.device))
+    _lib.check(st, "causal_conv1d_update")
+    return out
+
+
+# ----------------------------------------------------------------------------------------------
+# Mamba1 selective scan
+# ----------------------------------------------------------------------------------------------
+def _scale1(t, name):
+    _require(t is not None and t.dtype == torch.float32 and t.is_cuda and t.numel() == 1,
+             f"{name} must be a one-element fp32 GPU tensor")
+    return t
+
+
+def sscan_fwd(u, scale_u, delta, scale_delta, A, scale_A, B, scale_B, C, scale_C, scale_ssm_state,
+              D=None, scale_D=None, z=None, scale_z=None, delta_bias=None, scale_delta_bias=None,
+              delta_softplus=False, state_dtype=torch.int8):
+    """Selective scan over int8 inputs.
+
+    u, delta, z: int8 (batch, dim, seqlen) with unit stride along seqlen; A: int8 (dim, dstate) holding
+    A_log; B, C: int8 (batch, n_groups, dstate, seqlen).  Returns (out fp16 (batch, seqlen, dim),
+    x) where x is the state after the last step: int8 (batch, dim, 1, dstate) by default (the
+    reference's per-chunk state tensor, one chunk) or fp32 with ``state_dtype=torch.float32``.
+    """
+    _require(u.dtype == torch.int8 and A.dtype == torch.int8, "u and A must be int8")
+    _require(delta.dtype == torch.int8 and B.dtype == torch.int8 and C.dtype == torch.int8,
+             "delta, B and C must be int8")
+    for t, n in ((u, "u"), (delta, "delta"), (A, "A"), (B, "B"), (C, "C")):
+        _require_gpu(t, n)
+    if B.dim() < 3 or C.dim() < 3:
+        raise NotImplementedError("Must be input-dependent B and C")
+    _require(u.dim() == 3, "u must have shape (batch, dim, seqlen)")
+    batch, dim, seqlen = u.shape
+    dstate = A.shape[1]
+    _require(dstate <= 256, "quant_sscan only supports state dimension <= 256")
+    _require(tuple(delta.shape) == (batch, dim, seqlen), "delta must have shape (batch, dim, seqlen)")
+    _require(tuple(A.shape) == (dim, dstate), "A must have shape (dim, dstate)")
+    n_groups = B.shape[1]
+    _require(tuple(B.shape) == (batch, n_groups, dstate, seqlen) and tuple(C.shape) == tuple(B.shape),
+             "B and C must have shape (batch, n_groups, dstate, seqlen)")
+    for t, n in ((u, "u"), (delta, "delta"), (B, "B"), (C, "C")):
+        _require(t.stride(-1) == 1 or t.size(-1) == 1, f"{n} must have unit stride along seqlen")
+    for s, n in ((scale_u, "scale_u"), (scale_delta, "scale_delta"), (scale_A, "scale_A"), (scale_B, "scale_B"),
+                 (scale_C, "scale_C")):
+        _scale1(s, n)
+    p = _lib.QaSScanParams()
+    if D is not None:
+        _require(D.dtype == torch.int8 and D.is_cuda and tuple(D.shape) == (dim,) and D.stride(-1) == 1,
+                 "D must be a contiguous int8 GPU tensor of shape (dim,)")
+        _scale1(scale_D, "scale_D")
+        p.D, p.scale_D = ptr(D), ptr(scale_D)
+    if delta_bias is not None:
+        _require(delta_bias.dtype == torch.int8 and delta_bias.is_cuda and tuple(delta_bias.shape) == (dim,)
+                 and delta_bias.stride(-1) == 1, "delta_bias must be a contiguous int8 GPU tensor of shape (dim,)")
+        _scale1(scale_delta_bias, "scale_delta_bias")
+        p.delta_bias, p.scale_delta_bias = ptr(delta_bias), ptr(scale_delta_bias)
+    if z is not None:
+        _require(z.dtype == torch.int8 and z.is_cuda and tuple(z.shape) == (batch, dim, seqlen),
+                 "z must be an int8 GPU tensor of shape (batch, dim, seqlen)")
+        _require(z.stride(-1) == 1 or z.size(-1) == 1, "z must have unit stride along seqlen")
+        _scale1(scale_z, "scale_z")
+        p.z, p.scale_z = ptr(z), ptr(scale_z)
+        p.z_batch_stride, p.z_d_stride = z.stride(0), z.stride(1)
+    out = torch.empty((batch, seqlen, dim), dtype=torch.float16, device=u.device)
+    x = torch.empty((batch, dim, 1, dstate), dtype=state_dtype, device=u.device)
+    if state_dtype == torch.int8:
+        _scale1(scale_ssm_state, "scale_ssm_state")
+        p.last_state_i8, p.scale_ssm_state = ptr(x), ptr(scale_ssm_state)
+    else:
+        _require(state_dtype == torch.float32, "state_dtype must be torch.int8 or torch.float32")
+        p.last_state_f32 = ptr(x)
+    p.batch, p.dim, p.seqlen, p.dstate, p.n_groups = batch, dim, seqlen, dstate, n_groups
+    p.delta_softplus = int(bool(delta_softplus))
+    p.u_batch_stride, p.u_d_stride = u.stride(0), u.stride(1)
+    p.delta_batch_stride, p.delta_d_stride = delta.stride(0), delta.stride(1)
+    p.B_batch_stride, p.B_group_stride, p.B_dstate_stride = B.stride(0), B.stride(1), B.stride(2)
+    p.C_batch_stride, p.C_group_stride, p.C_dstate_stride = C.stride(0), C.stride(1), C.stride(2)
+    p.A_d_stride, p.A_dstate_stride = A.stride(0), A.stride(1)
+    p.out_batch_stride, p.out_l_stride, p.out_d_stride = out.stride()
+    p.u, p.delta, p.A_log, p.B, p.C, p.out = ptr(u), ptr(delta), ptr(A), ptr(B), ptr(C), ptr(out)
+    p.scale_u, p.scale_delta, p.scale_A = ptr(scale_u), ptr(scale_delta), ptr(scale_A)
+    p.scale_B, p.scale_C = ptr(scale_B), ptr(scale_C)
+    with torch.cuda.device(u.device):
+        st = _lib.lib().qa_sscan_fwd(C.byref(p), _lib.current_stream(u.device))
+    _lib.check(st, "sscan_fwd")
+    return out, x
+
+
+
+def sscan_update(state, q_x, x_scale, q_dt, dt_scale, q_A_log, A_log_scale, ssm_state_scale, q_B, B_scale,
+                 q_C, C_scale, q_D=None, D_scale=None, q_z=None, z_scale=None, dt_bias=None, dt_bias_scale=None,
+                 dt_softplus=False, x_head_group_range=None, x_dim_group_range=None):
+    """One recurrence step; ``state`` (int8 with ssm_state_scale, or fp32) is updated in place.
+
+    Shapes as quamba/triton/selective_state_update.py:129-160: state (batch, dim, dstate) or
+    (batch, nheads, dim, dstate); q_x, q_dt, q_z (batch, dim) or (batch, nheads, dim); q_A_log
+    (dim, dstate) or (nheads, dim, dstate); q_B, q_C (batch, dstate) or (batch, ngroups, dstate);
+    q_D, dt_bias (dim) or (nheads, dim).  dt_bias is int8 with dt_bias_scale, or fp16/fp32 without.
+    With x_head_group_range / x_dim_group_range the scales are the grouped ones of
+    quamba2_sscan_update_triton (:365-478).  Returns out fp16 shaped like q_x.
+    """
+    has_heads = state.dim() > 3
+    if state.dim() == 3:
+        state = state.unsqueeze(1)
+    q_x = q_x.unsqueeze(1) if q_x.dim() == 2 else q_x
+    q_dt = q_dt.unsqueeze(1) if q_dt.dim() == 2 else q_dt
+    q_A_log = q_A_log.unsqueeze(0) if q_A_log.dim() == 2 else q_A_log
+    q_B = q_B.unsqueeze(1) if q_B.dim() == 2 else q_B
+    q_C = q_C.unsqueeze(1) if q_C.dim() == 2 else q_C
+    if q_D is not None and q_D.dim() == 1:
+        q_D = q_D.unsqueeze(0)
+    if q_z is not None and q_z.dim() == 2:
+        q_z = q_z.unsqueeze(1)
+    if dt_bias is not None and dt_bias.dim() == 1:
+        dt_bias = dt_bias.unsqueeze(0)
+    batch, nheads, dim, dstate = state.shape
+    ngroups = q_B.shape[1]
+    _require(state.dtype in (torch.int8, torch.float32), "state must be int8 or fp32")
+    _require_gpu(state, "state")
+    _require(tuple(q_x.shape) == (batch, nheads, dim), "x must have shape (batch, [nheads,] dim)")
+    _require(tuple(q_dt.shape) == tuple(q_x.shape), "dt must have the shape of x")
+    _require(tuple(q_A_log.shape) == (nheads, dim, dstate), "A_log must have shape ([nheads,] dim, dstate)")
+    _require(nheads % ngroups == 0, "nheads must be divisible by ngroups")
+    _require(tuple(q_B.shape) == (batch, ngroups, dstate) and tuple(q_C.shape) == tuple(q_B.shape),
+             "B and C must have shape (batch, [ngroups,] dstate)")
+    for t in (q_x, q_dt, q_A_log, q_B, q_C):
+        _require(t.dtype == torch.int8 and t.is_cuda, "x, dt, A_log, B and C must be int8 GPU tensors")
+    _require(dstate <= 256, "state dimension must be <= 256")
+    out = torch.empty(q_x.shape, dtype=torch.float16, device=q_x.device)
+    p = _lib.QaSsmUpdateParams()
+    p.batch, p.nheads, p.dim, p.dstate, p.ngroups = batch, nheads, dim, dstate, ngroups
+    p.dt_softplus = int(bool(dt_softplus))
+    p.state_is_fp32 = int(state.dtype == torch.float32)
+    (p.state_batch_stride, p.state_head_stride, p.state_dim_stride, p.state_dstate_stride) = state.stride()
+    p.x_batch_stride, p.x_head_stride, p.x_dim_stride = q_x.stride()
+    p.dt_batch_stride, p.dt_head_stride, p.dt_dim_stride = q_dt.stride()
+    p.A_head_stride, p.A_dim_stride, p.A_dstate_stride = q_A_log.stride()
+    p.B_batch_stride, p.B_group_stride, p.B_dstate_stride = q_B.stride()
+    p.C_batch_stride, p.C_group_stride, p.C_dstate_stride = q_C.stride()
+    p.out_batch_stride, p.out_head_stride, p.out_dim_stride = out.stride()
+    p.state, p.x, p.dt, p.A_log, p.B, p.C, p.out = (ptr(state), ptr(q_x), ptr(q_dt), ptr(q_A_log), ptr(q_B),
+                                                   ptr(q_C), ptr(out))
+    keep = []
+
+    def f32(t):
+        t = t.to(device=q_x.device, dtype=torch.float32).contiguous()
+        keep.append(t)
+        return ptr(t)
+
+    p.x_scale, p.dt_scale, p.A_log_scale = f32(x_scale), f32(dt_scale), f32(A_log_scale)
+    p.B_scale, p.C_scale = f32(B_scale), f32(C_scale)
+    if not p.state_is_fp32:
+        p.state_scale = f32(ssm_state_scale)
+    if x_head_group_range is not None:
+        _require(x_head_group_range.dtype == torch.int32 and x_dim_group_range.dtype == torch.int32,
+                 "group ranges must be int32")
+        _require(x_head_group_range.dim() == 2 and x_dim_group_range.dim() == 3,
+                 "x_head_group_range must be [ngroups, nhead_groups], x_dim_group_range [ngroups, nhead_groups, ndim_groups]")
+        p.nhead_groups, p.ndim_groups = x_head_group_range.shape[1], x_dim_group_range.shape[2]
+        _require(x_scale.numel() == ngroups * p.nhead_groups * p.ndim_groups, "x_scale has the wrong number of groups")
+        if not p.state_is_fp32:
+            _require(tuple(ssm_state_scale.shape) == (ngroups, p.nhead_groups, p.ndim_groups, dstate),
+                     "ssm_state_scale must be [ngroups, nhead_groups, ndim_groups, dstate]")
+        hr, dr = x_head_group_range.contiguous(), x_dim_group_range.contiguous()
+        keep += [hr, dr]
+        p.x_head_group_range, p.x_dim_group_range = ptr(hr), ptr(dr)
+    if q_D is not None:
+        _require(tuple(q_D.shape) == (nheads, dim) and q_D.dtype == torch.int8, "D must be int8 ([nheads,] dim)")
+        p.D, p.D_scale = ptr(q_D), f32(D_scale)
+        p.D_head_stride, p.D_dim_stride = q_D.stride()
+    if q_z is not None:
+        _require(tuple(q_z.shape) == tuple(q_x.shape) and q_z.dtype == torch.int8, "z must be int8 shaped like x")
+        p.z, p.z_scale = ptr(q_z), f32(z_scale)
+        p.z_batch_stride, p.z_head_stride, p.z_dim_stride = q_z.stride()
+    if dt_bias is not None:
+        _require(tuple(dt_bias.shape) == (nheads, dim), "dt_bias must have shape ([nheads,] dim)")
+        if dt_bias.dtype == torch.int8:
+            p.dt_bias_scale = f32(dt_bias_scale)
+        else:
+            if dt_bias.dtype != torch.float16:
+                dt_bias = dt_bias.to(torch.float16)
+                keep.append(dt_bias)
+            p.dt_bias_is_fp16 = 1
+        p.dt_bias = ptr(dt_bias)
+        p.dt_bias_head_stride, p.dt_bias_dim_stride = dt_bias.stride()
+    with torch.cuda.device(q_x.device):
+        st = _lib.lib().qa_ssm_state_update(C.byref(p), _lib.current_stream(q_x.device))
+    _lib.check(st, "ssm_state_update")
+    return out if has_heads else out.squeeze(1)

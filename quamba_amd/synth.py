@@ -1,0 +1,117 @@
+"""Seeded synthetic inputs shaped like the quantized Mamba mixer's tensors (numpy, CPU).
+
+Activations are N(0,1) with 1% of the channels scaled 20x (outlier channels), quantised to int8
+with one symmetric absmax scale per tensor; dt is drawn so that softplus(dt + dt_bias) lies in
+[1e-3, 1e-1]; A_log = log(U[1,16]); D = 1.  One generator per tensor name, so changing one shape
+does not perturb the other tensors.
+"""
+import zlib
+
+import numpy as np
+
+
+def rng_for(seed, name):
+    return np.random.default_rng([seed, zlib.crc32(name.encode())])
+
+
+def quantize_absmax(x, n_bits=8):
+    """Symmetric per-tensor quantisation: returns (int8 array, float32 scale)."""
+    qmax = 2 ** (n_bits - 1) - 1
+    s = np.float32(max(float(np.abs(x).max()), 1e-5) / qmax)
+    q = np.clip(np.rint(x / s), -qmax - 1, qmax).astype(np.int8)
+    return q, s
+
+
+def activations(shape, channel_axis, seed, name, outliers=True):
+    """float32 N(0,1) with ceil(1%) outlier channels along channel_axis scaled by 20."""
+    g = rng_for(seed, name)
+    x = g.standard_normal(shape, dtype=np.float32)
+    if outliers:
+        nch = shape[channel_axis]
+        k = max(1, int(np.ceil(0.01 * nch)))
+        idx = g.permutation(nch)[:k]
+        sl = [slice(None)] * len(shape)
+        sl[channel_axis] = idx
+        x[tuple(sl)] *= 20.0
+    return x
+
+
+def softplus(x):
+    return np.where(x <= 20.0, np.log1p(np.exp(np.minimum(x, 20.0))), x)
+
+
+def inv_softplus(y):
+    return y + np.log(-np.expm1(-y))
+
+
+def conv_weights(dim, width, seed, bias=True):
+    """int8 depthwise conv taps and bias with their per-tensor scales."""
+    g = rng_for(seed, "conv_w")
+    w = g.uniform(-0.5, 0.5, (dim, width)).astype(np.float32)
+    qw, sw = quantize_absmax(w)
+    if not bias:
+        return qw, sw, None, np.float32(1.0)
+    b = rng_for(seed, "conv_b").uniform(-0.5, 0.5, (dim,)).astype(np.float32)
+    qb, sb = quantize_absmax(b)
+    return qw, sw, qb, sb
+
+
+def conv_output_scale(qx, sx, qw, sw, qb, sb, silu=True):
+    """Output scale = max |act(conv(x))| / 127 from a float64 evaluation of the dequantised conv."""
+    B, D, L = qx.shape
+    k = qw.shape[1]
+    x = qx.astype(np.float64) * float(sx)
+    w = qw.astype(np.float64) * float(sw)
+    acc = np.zeros((B, D, L))
+    for j in range(k):
+        shift = k - 1 - j
+        if shift < L:
+            acc[:, :, shift:] += w[None, :, j, None] * x[:, :, :L - shift]
+    if qb is not None:
+        acc += (qb.astype(np.float64) * float(sb))[None, :, None]
+    if silu:
+        acc = acc / (1.0 + np.exp(-acc))
+    return np.float32(max(float(np.abs(acc).max()), 1e-5) / 127.0)
+
+
+def mamba1_scan_inputs(batch, seqlen, dim, dstate, seed=1234, with_z=True):
+    """Quantised inputs of the Mamba1 selective scan: dict of int8 arrays and float32 scales.
+
+    u, dt, z: (batch, dim, seqlen); B, C: (batch, dstate, seqlen); A_log: (dim, dstate);
+    D, dt_bias: (dim).
+    """
+    out = {}
+    u = activations((batch, dim, seqlen), 1, seed, "u")
+    out["u"], out["s_u"] = quantize_absmax(u)
+    g = rng_for(seed, "dt")
+    dt_target = np.exp(g.uniform(np.log(1e-3), np.log(1e-1), (batch, dim, seqlen))).astype(np.float32)
+    dt_init = np.exp(rng_for(seed, "dt_bias").uniform(np.log(1e-3), np.log(1e-1), (dim,))).astype(np.float32)
+    dt_bias = inv_softplus(dt_init.astype(np.float64)).astype(np.float32)
+    dt_raw = (inv_softplus(dt_target.astype(np.float64)) - dt_bias[None, :, None]).astype(np.float32)
+    out["dt"], out["s_dt"] = quantize_absmax(dt_raw)
+    out["dt_bias"], out["s_db"] = quantize_absmax(dt_bias)
+    A_log = np.log(rng_for(seed, "A").uniform(1.0, 16.0, (dim, dstate))).astype(np.float32)
+    out["A_log"], out["s_A"] = quantize_absmax(A_log)
+    out["D"], out["s_D"] = quantize_absmax(np.ones((dim,), np.float32))
+    Bm = activations((batch, dstate, seqlen), 1, seed, "B", outliers=False)
+    Cm = activations((batch, dstate, seqlen), 1, seed, "C", outliers=False)
+    out["B"], out["s_B"] = quantize_absmax(Bm)
+    out["C"], out["s_C"] = quantize_absmax(Cm)
+    if with_z:
+        z = activations((batch, dim, seqlen), 1, seed, "z")
+        out["z"], out["s_z"] = quantize_absmax(z)
+    else:
+        out["z"], out["s_z"] = None, np.float32(0.0)
+    return out
+
+
+def linear_weights(out_features, in_features, seed, name="w", per_channel=True):
+    """int8 weights (N,K) ~ N(0, 1/sqrt(K)) with per-output-channel (or per-tensor) scales."""
+    g = rng_for(seed, name)
+    w = (g.standard_normal((out_features, in_features), dtype=np.float32) / np.sqrt(in_features)).astype(np.float32)
+    if per_channel:
+        s = np.maximum(np.abs(w).max(axis=1), 1e-5).astype(np.float32) / np.float32(127.0)
+        q = np.clip(np.rint(w / s[:, None]), -128, 127).astype(np.int8)
+        return q, s.astype(np.float32), w
+    q, s = quantize_absmax(w)
+    return q, np.array([s], np.float32), w

@@ -1,0 +1,183 @@
+"""GPU parity of the Mamba1 selective scan (forward and single-step update) against the CPU oracle.
+fp16 outputs: rtol 1e-2 / atol 1e-2; fp32 state: 1e-3 relative; int8 state: at most one step off."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from quamba_amd import QSScan, ops, synth
+
+pytestmark = pytest.mark.gpu
+
+RTOL = ATOL = 1e-2
+STATE_REL = 1e-3
+
+
+def _t(a, dev):
+    return None if a is None else torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+
+def _s(v, dev):
+    return torch.tensor([float(v)], dtype=torch.float32, device=dev)
+
+
+def _oracle(d, s_state):
+    return oracle.sscan_fwd(d["u"], d["dt"], d["A_log"], d["B"], d["C"], d["D"], d["dt_bias"], d["z"],
+                            s_u=d["s_u"], s_delta=d["s_dt"], s_A=d["s_A"], s_B=d["s_B"], s_C=d["s_C"],
+                            s_D=d["s_D"], s_db=d["s_db"], s_z=d["s_z"], s_state=s_state)
+
+
+def _gpu(d, dev, s_state, state_dtype):
+    return ops.sscan_fwd(
+        _t(d["u"], dev), _s(d["s_u"], dev), _t(d["dt"], dev), _s(d["s_dt"], dev), _t(d["A_log"], dev), _s(d["s_A"], dev),
+        _t(d["B"][:, None], dev), _s(d["s_B"], dev), _t(d["C"][:, None], dev), _s(d["s_C"], dev), _s(s_state, dev),
+        _t(d["D"], dev), _s(d["s_D"], dev), _t(d["z"], dev), _s(d["s_z"], dev) if d["z"] is not None else None,
+        _t(d["dt_bias"], dev), _s(d["s_db"], dev), True, state_dtype=state_dtype)
+
+
+def _check(y_gpu, y_ref):
+    y16 = y_ref.astype(np.float16).astype(np.float32)
+    got = y_gpu.float().cpu().numpy()
+    np.testing.assert_allclose(got, y16, rtol=RTOL, atol=ATOL)
+    r2 = np.sum((got - y_ref) ** 2) / max(np.sum(y_ref ** 2), 1e-30)
+    assert r2 < 1e-5
+
+
+# (batch, seqlen, dim, dstate): 130m/2.8b-shaped rows, ragged lengths, channel tails, wide states
+SHAPES = [(1, 512, 1536, 16), (2, 33, 1536, 16), (2, 89, 100, 16), (1, 1, 64, 16), (2, 2048 + 7, 96, 16),
+          (2, 130, 72, 8), (1, 200, 40, 32), (1, 100, 24, 64), (1, 70, 8, 128), (1, 40, 6, 256)]
+
+
+@pytest.mark.parametrize("B,L,D,N", SHAPES)
+def test_fwd_matches_oracle(dev, B, L, D, N):
+    d = synth.mamba1_scan_inputs(B, L, D, N, seed=L + D)
+    y_ref, st8_ref, st32_ref = _oracle(d, s_state=1.0)
+    s_state = max(float(np.abs(st32_ref).max()), 1e-5) / 127.0
+    _, st8_ref, _ = _oracle(d, s_state=s_state)
+    y, x32 = _gpu(d, dev, s_state, torch.float32)
+    assert y.shape == (B, L, D) and y.dtype == torch.float16 and x32.shape == (B, D, 1, N)
+    _check(y, y_ref)
+    got32 = x32[:, :, 0].cpu().numpy()
+    assert np.abs(got32 - st32_ref).max() <= STATE_REL * np.abs(st32_ref).max()
+    y2, x8 = _gpu(d, dev, s_state, torch.int8)
+    assert torch.equal(y, y2)
+    diff = np.abs(x8[:, :, 0].cpu().numpy().astype(int) - st8_ref.astype(int))
+    assert diff.max() <= 1 and (diff != 0).mean() < 0.02
+
+
+@pytest.mark.parametrize("variant", ["1x1", "2x1", "2x2", "4x1", "4x2", "4x4"])
+def test_every_lane_mapping_gives_the_same_answer(dev, variant, monkeypatch):
+    monkeypatch.setenv("QA_SSCAN_VARIANT", variant)
+    d = synth.mamba1_scan_inputs(2, 300, 200, 16, seed=21)
+    y_ref, _, st32_ref = _oracle(d, s_state=1.0)
+    y, x32 = _gpu(d, dev, 1.0, torch.float32)
+    _check(y, y_ref)
+    assert np.abs(x32[:, :, 0].cpu().numpy() - st32_ref).max() <= STATE_REL * np.abs(st32_ref).max()
+
+
+def test_fwd_without_z_d_and_bias(dev):
+    d = synth.mamba1_scan_inputs(2, 77, 48, 16, seed=4, with_z=False)
+    d["D"] = None
+    d["dt_bias"] = None
+    y_ref, _, _ = _oracle(d, 1.0)
+    y, _ = _gpu(d, dev, 1.0, torch.float32)
+    _check(y, y_ref)
+
+
+def test_fwd_on_strided_mixer_views(dev):
+    # x and z are the halves of in_proj's [2D][B][L] output viewed as (B, D, L); dt has its own buffer
+    B, L, D, N = 2, 256, 128, 16
+    d = synth.mamba1_scan_inputs(B, L, D, N, seed=8)
+    buf = torch.zeros((2 * D, B, L), dtype=torch.int8, device=dev).transpose(0, 1)
+    u, z = buf[:, :D], buf[:, D:]
+    u.copy_(_t(d["u"], dev))
+    z.copy_(_t(d["z"], dev))
+    dt = torch.zeros((D, B, L), dtype=torch.int8, device=dev).transpose(0, 1)
+    dt.copy_(_t(d["dt"], dev))
+    y, _ = ops.sscan_fwd(u, _s(d["s_u"], dev), dt, _s(d["s_dt"], dev), _t(d["A_log"], dev), _s(d["s_A"], dev),
+                         _t(d["B"][:, None], dev), _s(d["s_B"], dev), _t(d["C"][:, None], dev), _s(d["s_C"], dev),
+                         _s(1.0, dev), _t(d["D"], dev), _s(d["s_D"], dev), z, _s(d["s_z"], dev),
+                         _t(d["dt_bias"], dev), _s(d["s_db"], dev), True, state_dtype=torch.float32)
+    _check(y, _oracle(d, 1.0)[0])
+
+
+def test_fwd_unaligned_rows(dev):
+    B, L, D, N = 2, 50, 20, 16               # row pitch 50: no 16-byte alignment anywhere
+    d = synth.mamba1_scan_inputs(B, L, D, N, seed=12)
+    y, _ = _gpu(d, dev, 1.0, torch.float32)
+    _check(y, _oracle(d, 1.0)[0])
+
+
+@pytest.mark.parametrize("B,D,N,fp32_state", [(1, 1536, 16, False), (64, 5120, 16, True), (3, 100, 16, False),
+                                              (2, 64, 128, True), (2, 30, 8, False)])
+def test_update_matches_oracle_over_several_steps(dev, B, D, N, fp32_state):
+    steps = 5
+    d = synth.mamba1_scan_inputs(B, steps, D, N, seed=D + N)
+    g = np.random.default_rng(D)
+    if fp32_state:
+        st_ref = (0.1 * g.standard_normal((B, D, N))).astype(np.float32)
+        s_state = 1.0
+    else:
+        st_ref = g.integers(-128, 128, (B, D, N)).astype(np.int8)
+        s_state = 0.004
+    st = _t(st_ref.copy(), dev)
+    A, Dq, db = _t(d["A_log"], dev), _t(d["D"], dev), _t(d["dt_bias"], dev)
+    for t in range(steps):
+        y_ref, st_ref = oracle.sscan_update(st_ref, d["u"][:, :, t], d["dt"][:, :, t], d["A_log"], d["B"][:, :, t],
+                                            d["C"][:, :, t], d["D"], d["dt_bias"], d["z"][:, :, t],
+                                            s_x=d["s_u"], s_dt=d["s_dt"], s_A=d["s_A"], s_B=d["s_B"], s_C=d["s_C"],
+                                            s_D=d["s_D"], s_db=d["s_db"], s_z=d["s_z"], s_state=s_state)
+        y = ops.sscan_update(st, _t(d["u"][:, :, t], dev), _s(d["s_u"], dev), _t(d["dt"][:, :, t], dev),
+                             _s(d["s_dt"], dev), A, _s(d["s_A"], dev), _s(s_state, dev), _t(d["B"][:, :, t], dev),
+                             _s(d["s_B"], dev), _t(d["C"][:, :, t], dev), _s(d["s_C"], dev), Dq, _s(d["s_D"], dev),
+                             _t(d["z"][:, :, t], dev), _s(d["s_z"], dev), db, _s(d["s_db"], dev), True)
+        np.testing.assert_allclose(y.float().cpu().numpy(), y_ref.astype(np.float16).astype(np.float32),
+                                   rtol=RTOL, atol=ATOL)
+        got = st.cpu().numpy()
+        if fp32_state:
+            assert np.abs(got - st_ref).max() <= STATE_REL * np.abs(st_ref).max()
+        else:
+            diff = np.abs(got.astype(int) - st_ref.astype(int))
+            assert diff.max() <= 1 and (diff != 0).mean() < 0.01
+            st_ref = got.copy()              # follow the GPU's state so a one-step tie does not compound
+
+
+def test_module_forward_then_update_continue_the_same_sequence(dev):
+    B, L, D, N = 2, 64, 96, 16
+    d = synth.mamba1_scan_inputs(B, L + 4, D, N, seed=31)
+    A_log = torch.from_numpy(d["A_log"].astype(np.float32) * d["s_A"]).to(dev)
+    q = QSScan.from_fp16(N, D, A_log, D=torch.ones(D, device=dev),
+                         dt_bias=torch.from_numpy(d["dt_bias"].astype(np.float32) * d["s_db"]).to(dev),
+                         ssm_state_scale=torch.tensor(1.0), u_scale=torch.tensor(float(d["s_u"])),
+                         dt_scale=torch.tensor(float(d["s_dt"])), B_scale=torch.tensor(float(d["s_B"])),
+                         C_scale=torch.tensor(float(d["s_C"])), z_scale=torch.tensor(float(d["s_z"])))
+    assert q.A_log.dtype == torch.int8 and q.A_log.shape == (D, N) and q.u_scale.dtype == torch.float32
+    np.testing.assert_array_equal(q.A_log.cpu().numpy(), d["A_log"])
+    full = {k: (v[..., :] if isinstance(v, np.ndarray) else v) for k, v in d.items()}
+    y_all, _, _ = _oracle(full, 1.0)
+    cut = lambda a: _t(a[:, :, :L], dev)
+    y, state = q(cut(d["u"]), cut(d["dt"]), cut(d["B"]), cut(d["C"]), z=cut(d["z"]), return_last_state=True,
+                 state_dtype=torch.float32)
+    assert state.shape == (B, D, N)
+    _check(y, y_all[:, :L])
+    state = state.contiguous()
+    for t in range(L, L + 4):
+        yt, state = q.update(state, _t(d["u"][:, :, t], dev), _t(d["dt"][:, :, t], dev), _t(d["B"][:, :, t], dev),
+                             _t(d["C"][:, :, t], dev), z=_t(d["z"][:, :, t], dev))
+        np.testing.assert_allclose(yt.float().cpu().numpy(), y_all[:, t].astype(np.float16).astype(np.float32),
+                                   rtol=RTOL, atol=ATOL)
+
+
+def test_errors(dev):
+    d = synth.mamba1_scan_inputs(1, 16, 8, 16, seed=1)
+    args = lambda **o: dict(dict(u=_t(d["u"], dev), B=_t(d["B"][:, None], dev)), **o)
+    with pytest.raises(NotImplementedError, match="input-dependent"):
+        ops.sscan_fwd(_t(d["u"], dev), _s(1, dev), _t(d["dt"], dev), _s(1, dev), _t(d["A_log"], dev), _s(1, dev),
+                      _t(d["B"][0], dev), _s(1, dev), _t(d["C"][0], dev), _s(1, dev), _s(1, dev))
+    with pytest.raises(RuntimeError, match="int8"):
+        ops.sscan_fwd(_t(d["u"], dev).float(), _s(1, dev), _t(d["dt"], dev), _s(1, dev), _t(d["A_log"], dev),
+                      _s(1, dev), _t(d["B"][:, None], dev), _s(1, dev), _t(d["C"][:, None], dev), _s(1, dev), _s(1, dev))
+    big_A = torch.zeros((8, 300), dtype=torch.int8, device=dev)
+    with pytest.raises(RuntimeError, match="<= 256"):
+        ops.sscan_fwd(_t(d["u"], dev), _s(1, dev), _t(d["dt"], dev), _s(1, dev), big_A, _s(1, dev),
+                      _t(d["B"][:, None], dev), _s(1, dev), _t(d["C"][:, None], dev), _s(1, dev), _s(1, dev))
