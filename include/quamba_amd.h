@@ -170,6 +170,7 @@ int qa_ssm_state_update(const QaSsmUpdateParams* p, void* stream);
  * (the reference's column-major (K,N) "b" operand is the same memory).
  * ---------------------------------------------------------------------------------------- */
 typedef enum QaOutType { QA_OUT_I8 = 0, QA_OUT_F16 = 1 } QaOutType;
+/* QA_ROUND_HALF_AWAY selects the rule of w8a8o8_gemv: d = sat8(roundf((s_w[n] * s_a[m|0]) * float(acc))) */
 typedef enum QaRound { QA_ROUND_RNE = 0, QA_ROUND_HALF_AWAY = 1 } QaRound;
 
 typedef struct QaGemmW8A8Params {
@@ -178,6 +179,9 @@ typedef struct QaGemmW8A8Params {
     int32_t round_mode;    /* QaRound, int8 output only */
     int32_t a_scale_numel; /* 1 or m */
     int32_t w_scale_numel; /* 1 or n */
+    int32_t use_alpha;     /* 1: d = cast(alpha * float(acc)) with the host scalar below (the GEMV
+                              rule of cutlass_scaled_mv_dq); the scale pointers are then ignored */
+    float alpha;
     int32_t reserved0;
     int64_t lda, ldw, ldd; /* element strides between rows of a, w, d (d is (M,N) row-major) */
     const int8_t* a;

@@ -250,7 +250,8 @@ void qo_gemm_w8a8(const int8_t* a, const int8_t* w, const float* s_a, int s_a_nu
             for (int kk = 0; kk < k; ++kk) acc += (int32_t)ar[kk] * (int32_t)wr[kk];
             const float sa = s_a[s_a_numel == 1 ? 0 : i];
             const float sb = s_b[s_b_numel == 1 ? 0 : j];
-            const float v = sa * (sb * (float)acc);
+            /* GEMM epilogue :85-97; GEMV: scale = s_a*s_b first (quant_linear_fwd_gemv_kernel.cuh:56-58) */
+            const float v = round_half_away ? (sb * sa) * (float)acc : sa * (sb * (float)acc);
             const int64_t o = (int64_t)i * n + j;
             if (acc_out) acc_out[o] = acc;
             if (out_f32) out_f32[o] = v;

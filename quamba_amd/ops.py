@@ -8,7 +8,7 @@ Reference interfaces mirrored here:
   quant_sscan_update_triton                quamba/triton/selective_state_update.py:129-227
   quant_linear_cuda.cutlass_scaled_mm_dq   csrc/linear/quant_linear_fwd_kernel.cuh:356-378
 """
-import ctypes as C
+import ctypes as ct
 
 import torch
 
@@ -61,7 +61,7 @@ def causal_conv1d_fwd(x, scale_x, weight, scale_w, scale_out, scale_b, bias=None
     p.x, p.weight, p.bias, p.out = ptr(x), ptr(weight), ptr(bias), ptr(out)
     p.scale_x, p.scale_w, p.scale_b, p.scale_out = float(scale_x), float(scale_w), float(scale_b), float(scale_out)
     with torch.cuda.device(x.device):
-        st = _lib.lib().qa_causal_conv1d_fwd(C.byref(p), _lib.current_stream(x.device))
+        st = _lib.lib().qa_causal_conv1d_fwd(ct.byref(p), _lib.current_stream(x.device))
     _lib.check(st, "causal_conv1d_fwd")
     return out
 
@@ -97,7 +97,7 @@ def causal_conv1d_update(x, conv_state, scale_x, weight, scale_w, scale_out, sca
     p.x, p.weight, p.bias, p.out, p.conv_state = ptr(x), ptr(weight), ptr(bias), ptr(out), ptr(conv_state)
     p.scale_x, p.scale_w, p.scale_b, p.scale_out = float(scale_x), float(scale_w), float(scale_b), float(scale_out)
     with torch.cuda.device(x.device):
-        st = _lib.lib().qa_causal_conv1d_update(C.byref(p), _lib.current_stream(x.device))
+        st = _lib.lib().qa_causal_conv1d_update(ct.byref(p), _lib.current_stream(x.device))
     _lib.check(st, "causal_conv1d_update")
     return out
 
@@ -180,7 +180,7 @@ def sscan_fwd(u, scale_u, delta, scale_delta, A, scale_A, B, scale_B, C, scale_C
     p.scale_u, p.scale_delta, p.scale_A = ptr(scale_u), ptr(scale_delta), ptr(scale_A)
     p.scale_B, p.scale_C = ptr(scale_B), ptr(scale_C)
     with torch.cuda.device(u.device):
-        st = _lib.lib().qa_sscan_fwd(C.byref(p), _lib.current_stream(u.device))
+        st = _lib.lib().qa_sscan_fwd(ct.byref(p), _lib.current_stream(u.device))
     _lib.check(st, "sscan_fwd")
     return out, x
 
@@ -283,6 +283,63 @@ def sscan_update(state, q_x, x_scale, q_dt, dt_scale, q_A_log, A_log_scale, ssm_
         p.dt_bias = ptr(dt_bias)
         p.dt_bias_head_stride, p.dt_bias_dim_stride = dt_bias.stride()
     with torch.cuda.device(q_x.device):
-        st = _lib.lib().qa_ssm_state_update(C.byref(p), _lib.current_stream(q_x.device))
+        st = _lib.lib().qa_ssm_state_update(ct.byref(p), _lib.current_stream(q_x.device))
     _lib.check(st, "ssm_state_update")
     return out if has_heads else out.squeeze(1)
+
+
+# ----------------------------------------------------------------------------------------------
+# W8A8 linear
+# ----------------------------------------------------------------------------------------------
+def _gemm_w8a8(c, a, w_nk, a_scales, b_scales, alpha=None, round_half_away=False):
+    """c (M,N) row-major <- a (M,K) x w_nk (N,K)^T, both K-contiguous."""
+    _require(a.dtype == torch.int8 and w_nk.dtype == torch.int8, "a and b must be int8")
+    for t, n in ((a, "a"), (w_nk, "b"), (c, "c")):
+        _require_gpu(t, n)
+    _require(c.dtype in (torch.int8, torch.float16), "c must be int8 or fp16")
+    M, K = a.shape
+    N = w_nk.shape[0]
+    _require(w_nk.shape[1] == K and tuple(c.shape) == (M, N), "shape mismatch: c (M,N) = a (M,K) x b (K,N)")
+    _require(a.stride(1) == 1 and c.stride(1) == 1, "a and c must be row-major")
+    _require(w_nk.stride(1) == 1, "b must be column-major (K contiguous)")
+    _require(a.stride(0) % 16 == 0 and w_nk.stride(0) % 16 == 0 and K % 16 == 0,
+             "row strides of a and b and K must be multiples of 16")
+    p = _lib.QaGemmW8A8Params()
+    p.m, p.n, p.k = M, N, K
+    p.out_type = _lib.QA_OUT_I8 if c.dtype == torch.int8 else _lib.QA_OUT_F16
+    p.round_mode = _lib.QA_ROUND_HALF_AWAY if round_half_away else _lib.QA_ROUND_RNE
+    p.lda, p.ldw, p.ldd = a.stride(0), w_nk.stride(0), c.stride(0)
+    p.a, p.w, p.d = ptr(a), ptr(w_nk), ptr(c)
+    if alpha is not None:
+        p.use_alpha, p.alpha = 1, float(alpha)
+    else:
+        for s, n, full in ((a_scales, "a_scales", M), (b_scales, "b_scales", N)):
+            _require(s.dtype == torch.float32 and s.is_cuda and s.is_contiguous(), f"{n} must be contiguous fp32 on the GPU")
+            _require(s.numel() in (1, full), f"{n} must have 1 or {full} elements")
+        p.a_scale, p.w_scale = ptr(a_scales), ptr(b_scales)
+        p.a_scale_numel, p.w_scale_numel = a_scales.numel(), b_scales.numel()
+    with torch.cuda.device(a.device):
+        st = _lib.lib().qa_gemm_w8a8(ct.byref(p), _lib.current_stream(a.device))
+    _lib.check(st, "gemm_w8a8")
+    return c
+
+
+def scaled_mm_dq(c, a, b, a_scales, b_scales):
+    """c = cast(a_scales * (b_scales * (a @ b))) with a int8 (M,K) row-major, b int8 (K,N) column-major
+    (b.stride(0) == 1), scales fp32 with 1 or M / 1 or N elements; c int8 (round-half-even,
+    saturating) or fp16, written in place.  Interface of cutlass_scaled_mm_dq."""
+    _require(b.dim() == 2 and b.stride(0) == 1, "b must be column-major")
+    return _gemm_w8a8(c, a, b.t(), a_scales, b_scales)
+
+
+def scaled_mv_dq(y, w, x, alpha, beta=0.0):
+    """y (1,N) = cast(alpha * (x (1,K) @ w (N,K)^T)); interface of cutlass_scaled_mv_dq (beta must be 0)."""
+    _require(float(beta) == 0.0, "beta != 0 is not supported")
+    return _gemm_w8a8(y, x, w, None, None, alpha=alpha)
+
+
+def w8a8o8_gemv(y, w, x, b_scales, a_scale):
+    """y (1,N) int8 = sat8(roundf(b_scales[n] * a_scale * (x @ w^T))); interface of w8a8o8_gemv.
+    The reference multiplies b_scales[n] * a_scale first (quant_linear_fwd_gemv_kernel.cuh:56-60); the two scale
+    operands are therefore passed swapped so that the same product is formed."""
+    return _gemm_w8a8(y, x, w, a_scale, b_scales, round_half_away=True)
