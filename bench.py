@@ -1,0 +1,246 @@
+"""Benchmark of the quantized Mamba1 mixer prefill hot path on one MI355X.
+
+One step = one pass of the path over one batch of synthetic input, at the Mamba1-2.8b prefill
+shape (batch 8, seqlen 2048, d_model 2560, d_inner 5120, d_state 16, conv width 4):
+
+    in_proj   W8A8 GEMM  [2560 -> 10240], int8 out, seqlen-last layout  (x | z halves)
+    conv1d    int8 depthwise causal conv + SiLU + requant on the x half
+    sscan     int8 selective scan with z gating, fp16 out (batch, seqlen, d_inner), fp32 last state
+    out_proj  W8A8 GEMM  [5120 -> 2560], fp16 out
+
+Inputs are resident in HBM before the timed region.  dt, B and C (produced by x_proj / dt_proj in
+the full layer) and out_proj's int8 input (produced by the Hadamard-quantise op) are synthetic
+tensors of the right shape and layout.  Prints one JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+from quamba_amd import QCausalConv1D, W8A8B8O8Linear, W8A8B16O16Linear, ops, synth  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
+INT8_PEAK_TOPS = 5000.0     # MI355X dense int8 MFMA
+
+CFG = dict(batch=8, seqlen=2048, d_model=2560, d_inner=5120, d_state=16, dt_rank=160, d_conv=4)
+
+
+def _t(a, dev):
+    return None if a is None else torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+
+def _s(v, dev):
+    return torch.tensor([float(v)], dtype=torch.float32, device=dev)
+
+
+class Mixer:
+    """Holds the resident tensors of one mixer and runs the four kernels in order."""
+
+    def __init__(self, dev, batch, seqlen, cfg=CFG, seed=1234):
+        self.dev = dev
+        B, L = batch, seqlen
+        D, dm, N, k = cfg["d_inner"], cfg["d_model"], cfg["d_state"], cfg["d_conv"]
+        self.B, self.L, self.D, self.dm, self.N = B, L, D, dm, N
+        g = synth.rng_for(seed, "hidden")
+        # hidden states after the (out-of-scope) int8 RMSNorm: outlier channels, per-tensor scale
+        hid = synth.activations((B * L, dm), 1, seed, "hidden")
+        q_hid, s_hid = synth.quantize_absmax(hid)
+        self.hidden = _t(q_hid, dev).view(B, L, dm)
+
+        w_in_q, w_in_s, _ = synth.linear_weights(2 * D, dm, seed, "in_proj", per_channel=False)
+        self.in_proj = W8A8B8O8Linear(dm, 2 * D, device=dev)
+        self.in_proj.weight = _t(w_in_q, dev).t()
+        s_xz = 0.04                                          # int8 scale of in_proj's output
+        self.in_proj.a = torch.tensor([[float(s_hid) / s_xz]], dtype=torch.float32, device=dev)
+        self.in_proj.b = torch.tensor([[float(w_in_s[0])]], dtype=torch.float32, device=dev)
+
+        qw, sw, qb, sb = synth.conv_weights(D, k, seed)
+        self.conv = QCausalConv1D(D, D, k, groups=D, device=dev)
+        self.conv.weight, self.conv.bias = _t(qw, dev), _t(qb, dev)
+        self.conv.weight_scale, self.conv.bias_scale = float(sw), float(sb)
+        self.conv.input_scale, self.conv.output_scale = s_xz, 0.03
+
+        sc = synth.mamba1_scan_inputs(1, 8, D, N, seed=seed)    # parameters only (A_log, D, dt_bias + scales)
+        self.A_log, self.Dq, self.dt_bias = _t(sc["A_log"], dev), _t(sc["D"], dev), _t(sc["dt_bias"], dev)
+        self.s_A, self.s_D, self.s_db = _s(sc["s_A"], dev), _s(sc["s_D"], dev), _s(sc["s_db"], dev)
+        self.s_u, self.s_z = _s(self.conv.output_scale, dev), _s(s_xz, dev)
+        # dt as dt_proj.to_seqlen_last leaves it: (B, D, L) view of a [D][B][L] buffer
+        dt_target = np.exp(g.uniform(np.log(1e-3), np.log(1e-1), (D, B, L))).astype(np.float32)
+        dt_bias_f = sc["dt_bias"].astype(np.float32) * sc["s_db"]
+        dt_raw = synth.inv_softplus(dt_target.astype(np.float64)) - dt_bias_f[:, None, None]
+        q_dt, s_dt = synth.quantize_absmax(dt_raw.astype(np.float32))
+        self.dt = _t(q_dt, dev).transpose(0, 1)
+        self.s_dt = _s(s_dt, dev)
+        qB, sB = synth.quantize_absmax(synth.activations((B, 1, N, L), 2, seed, "B", outliers=False))
+        qC, sC = synth.quantize_absmax(synth.activations((B, 1, N, L), 2, seed, "C", outliers=False))
+        self.Bm, self.Cm, self.s_B, self.s_C = _t(qB, dev), _t(qC, dev), _s(sB, dev), _s(sC, dev)
+        self.s_state = _s(1.0, dev)
+
+        w_out_q, w_out_s, _ = synth.linear_weights(dm, D, seed, "out_proj", per_channel=False)
+        self.out_proj = W8A8B16O16Linear(D, dm, device=dev)
+        self.out_proj.weight = _t(w_out_q, dev).t()
+        self.out_proj.a = torch.tensor([[0.02]], dtype=torch.float32, device=dev)
+        self.out_proj.b = torch.tensor([[float(w_out_s[0])]], dtype=torch.float32, device=dev)
+        y_q, _ = synth.quantize_absmax(synth.activations((B * L, D), 1, seed, "y_had"))
+        self.y_q = _t(y_q, dev).view(B, L, D)
+
+    def step(self, events=None):
+        rec = (lambda i: events[i].record()) if events is not None else (lambda i: None)
+        rec(0)
+        xz = self.in_proj.to_seqlen_last(self.hidden)              # (B, 2D, L), strides (L, B*L, 1)
+        rec(1)
+        x, z = xz[:, :self.D], xz[:, self.D:]
+        xc = self.conv(x)
+        rec(2)
+        y, state = ops.sscan_fwd(xc, self.s_u, self.dt, self.s_dt, self.A_log, self.s_A, self.Bm, self.s_B,
+                                 self.Cm, self.s_C, self.s_state, self.Dq, self.s_D, z, self.s_z, self.dt_bias,
+                                 self.s_db, True, state_dtype=torch.float32)
+        rec(3)
+        out = self.out_proj(self.y_q)
+        rec(4)
+        return xz, xc, y, state, out
+
+
+def kernel_table(B, L, cfg=CFG):
+    """Algorithmic (compulsory) bytes and ops of one launch of each kernel."""
+    D, dm, N, k = cfg["d_inner"], cfg["d_model"], cfg["d_state"], cfg["d_conv"]
+    M = B * L
+    return [
+        dict(name="in_proj_w8a8_gemm", bound="mfma", ops=2.0 * M * dm * 2 * D, bytes=M * dm + dm * 2 * D + M * 2 * D),
+        dict(name="causal_conv1d_fwd", bound="hbm", bytes=2.0 * B * D * L + D * (k + 1)),
+        dict(name="sscan_fwd", bound="hbm", bytes=3.0 * B * D * L + 2 * B * N * L + 2 * B * D * L + 4 * B * D * N + D * (N + 2)),
+        dict(name="out_proj_w8a8_gemm", bound="mfma", ops=2.0 * M * D * dm, bytes=M * D + D * dm + 2 * M * dm),
+    ]
+
+
+def cpu_baseline(dev_mixer, seconds_budget=30.0):
+    """Times the CPU oracle (conv, scan: C restatement with OpenMP) and an fp32 torch.matmul on the
+    dequantised GEMM operands, on a batch-1 slice of the same workload, on the host's cores."""
+    import oracle
+    m = dev_mixer
+    threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    torch.set_num_threads(threads)
+    L, D, dm, N = m.L, m.D, m.dm, m.N
+    hid = m.hidden[:1].cpu().float().view(L, dm)
+    w_in = m.in_proj.weight.t().cpu().float()
+    y_q = m.y_q[:1].cpu().float().view(L, D)
+    w_out = m.out_proj.weight.t().cpu().float()
+    x8 = np.ascontiguousarray(np.random.default_rng(0).integers(-128, 128, (1, D, L)).astype(np.int8))
+    z8 = np.ascontiguousarray(np.random.default_rng(1).integers(-128, 128, (1, D, L)).astype(np.int8))
+    dt8 = np.ascontiguousarray(m.dt[:1].cpu().numpy())
+    B8, C8 = m.Bm[:1].cpu().numpy(), m.Cm[:1].cpu().numpy()
+    A, Dq, db = m.A_log.cpu().numpy(), m.Dq.cpu().numpy(), m.dt_bias.cpu().numpy()
+    qw, qb = m.conv.weight.cpu().numpy(), m.conv.bias.cpu().numpy()
+    sc = lambda t: float(t.item())
+
+    def one_pass():
+        (hid @ w_in.t())
+        xc = oracle.conv1d_fwd(x8, qw, qb, m.conv.input_scale, m.conv.weight_scale, m.conv.bias_scale,
+                               m.conv.output_scale)
+        oracle.sscan_fwd(xc, dt8, A, B8, C8, Dq, db, z8, s_u=sc(m.s_u), s_delta=sc(m.s_dt), s_A=sc(m.s_A),
+                         s_B=sc(m.s_B), s_C=sc(m.s_C), s_D=sc(m.s_D), s_db=sc(m.s_db), s_z=sc(m.s_z))
+        (y_q @ w_out.t())
+
+    one_pass()                                        # warm-up
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        one_pass()
+        reps += 1
+        el = time.perf_counter() - t0
+        if reps >= 3 and (el > 0.5 * seconds_budget or reps >= 20):
+            break
+        if el > seconds_budget:
+            break
+    per_pass = (time.perf_counter() - t0) / reps
+    return dict(value=L / per_pass, unit="tokens/s", cores=threads, kind="port",
+                sample=f"batch 1 of {m.B} (seqlen {L}, same weights and shapes), {reps} passes after 1 warm-up; "
+                       "conv and scan: C oracle with OpenMP; GEMMs: fp32 torch.matmul on dequantised operands")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--batch", type=int, default=CFG["batch"])
+    ap.add_argument("--seqlen", type=int, default=CFG["seqlen"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--traffic-json", default=os.path.join(ROOT, "profiles", "traffic.json"),
+                    help="HBM bytes per launch measured with rocprofv3 --pmc (written by hand from profiles/)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU only: this build has no multi-GPU path (run with --gpus 1)")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    mixer = Mixer(dev, args.batch, args.seqlen)
+    B, L = args.batch, args.seqlen
+
+    for _ in range(args.warmup):
+        mixer.step()
+    torch.cuda.synchronize()
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        mixer.step(ev[i])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+
+    kernels = kernel_table(B, L)
+    for j, kinfo in enumerate(kernels):
+        dur_ms = float(np.mean([ev[i][j].elapsed_time(ev[i][j + 1]) for i in range(args.steps)]))
+        kinfo["avg_us"] = dur_ms * 1e3
+        if kinfo["bound"] == "hbm":
+            kinfo.update(achieved=kinfo["bytes"] / dur_ms / 1e6, peak=HBM_PEAK_GBS, unit="GB/s")
+        else:
+            kinfo.update(achieved=kinfo["ops"] / dur_ms / 1e9, peak=INT8_PEAK_TOPS, unit="TFLOP/s")
+        kinfo["frac"] = kinfo["achieved"] / kinfo["peak"]
+    traffic = {}
+    if os.path.exists(args.traffic_json):
+        traffic = json.load(open(args.traffic_json))
+    dom = max(kernels, key=lambda k: k["avg_us"])
+    roofline = dict(kernel=dom["name"], bound=dom["bound"], achieved=round(dom["achieved"], 2), peak=dom["peak"],
+                    unit=dom["unit"], frac=round(dom["frac"], 4), traffic=traffic.get(dom["name"]),
+                    avg_us=round(dom["avg_us"], 2))
+    per_kernel = [dict(kernel=k["name"], bound=k["bound"], avg_us=round(k["avg_us"], 2), achieved=round(k["achieved"], 2),
+                       unit=k["unit"], peak=k["peak"], frac=round(k["frac"], 4), traffic=traffic.get(k["name"]))
+                  for k in kernels]
+
+    line = {
+        "metric": "quantized mixer prefill tokens/s on 1 MI355X; % HBM peak (scan) / % int8 MFMA (GEMM)",
+        "value": round(B * L / (ms_per_step / 1e3), 1),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8",
+        "data": "synthetic",
+        "config": {"workload": "Mamba1-2.8b quantized prefill mixer: in_proj W8A8 -> conv1d int8 -> selective scan int8 "
+                               "(z gate, fp16 out, fp32 state) -> out_proj W8A8",
+                   "batch": B, "seq_len": L, "d_model": CFG["d_model"], "d_inner": CFG["d_inner"],
+                   "d_state": CFG["d_state"], "d_conv": CFG["d_conv"], "tokens_per_step": B * L},
+        "roofline": roofline,
+        "kernels": per_kernel,
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(mixer)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

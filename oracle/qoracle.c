@@ -76,6 +76,7 @@ void qo_conv1d_fwd(const int8_t* x, const int8_t* weight, const int8_t* bias, in
                    int batch, int dim, int seqlen, int width,
                    float s_x, float s_w, float s_b, float s_out, int silu, int tapwise) {
     const float s_wx = s_w * s_x;                                           /* :62 */
+#pragma omp parallel for collapse(2) schedule(static)
     for (int b = 0; b < batch; ++b) {
         for (int d = 0; d < dim; ++d) {
             const int8_t* xr = x + ((int64_t)b * dim + d) * seqlen;
@@ -148,6 +149,7 @@ void qo_sscan_fwd(const int8_t* u, const int8_t* delta, const int8_t* A_log, con
                   float s_state, int batch, int dim, int seqlen, int dstate, int groups, int softplus,
                   float* y, int8_t* state_i8, float* state_f32) {
     const int per_group = dim / groups;
+#pragma omp parallel for collapse(2) schedule(static)
     for (int b = 0; b < batch; ++b) {
         for (int d = 0; d < dim; ++d) {
             const int g = d / per_group;
