@@ -1,0 +1,299 @@
+// Shared int8-MFMA GEMM core for the W8A8 and W4A8 linears (gfx950).
+//
+//   acc[m,n] = sum_k a[m,k] * w[n,k]   (int32)      a: (M,K) int8, K-contiguous
+//   d[m,n]   = cast(s_row[m|0] * (s_col[n|0] * float(acc)))          w: (N,K) int8, K-contiguous (W8A8)
+//                                                                       or 4-bit codes + group scales (W4A8)
+// Structure: WGM x WGN waves per workgroup, each wave TM x TN tiles of v_mfma_i32_32x32x32_i8; block
+// tile (WGM*TM*32) x (WGN*TN*32) x 128 k-bytes.  The k extent of 128 bytes is one full cache line
+// per operand row: measured on MI355X, 64-byte row pieces halve the L1 load rate.  Operand tiles live
+// in LDS as rows of eight 16-byte chunks, the chunk index XOR-swizzled with bits 1..3 of the row
+// (measured conflict-free for the 32-row x 16-byte fragment reads).  int8 operands go global -> LDS
+// directly (buffer_load ... lds, 16 bytes per lane, out-of-range lanes deliver zeros), so no
+// registers are spent on staging and the next tile is in flight while the current one is multiplied.
+// The 4-bit operand passes through registers, is expanded to int8 there and stored to the same
+// layout.  The weight fragment is the MFMA "A" operand, so a lane ends up with four consecutive
+// output columns of one row; the epilogue scales, converts, stages through LDS (privately per wave)
+// and writes 16-byte pieces of output rows (or of output columns for the transposed layout).
+#pragma once
+#include "qa_common.hpp"
+
+namespace qa {
+namespace gemm {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+constexpr int kBK = 128;                 // k-bytes per tile row
+constexpr int kChunks = kBK / 16;        // 16-byte chunks per tile row
+constexpr int kRsrcFlags = 0x00020000;   // raw buffer, 32-bit data format
+
+__device__ __forceinline__ int swz(int row, int chunk) { return chunk ^ ((row >> 1) & 7); }
+
+// s_waitcnt immediate for "at most n vector-memory operations outstanding" (gfx9 encoding),
+// leaving the LDS/scalar and export counters unconstrained.
+__host__ __device__ constexpr int vmcnt_imm(int n) { return (n & 0xf) | ((n >> 4) << 14) | (0x7 << 4) | (0xf << 8); }
+
+// round (half-even or half-away) and saturate to int8, returned in the low byte of an int
+__device__ __forceinline__ int quant8(float v, int round_mode) {
+    const float r = round_mode == QA_ROUND_RNE ? __builtin_rintf(v) : __builtin_roundf(v);
+    // med3 returns -128 for NaN inputs as min(max(r,-128),127) would
+    return static_cast<int>(__builtin_amdgcn_fmed3f(r, -128.0f, 127.0f));
+}
+
+struct Epilogue {
+    const float* row_scale;   // s_row, numel 1 or M (unused with use_alpha)
+    const float* col_scale;   // s_col, numel 1 or N
+    int row_numel, col_numel;
+    int use_alpha;            // d = cast(alpha * acc)
+    float alpha;
+    int round_mode;           // QaRound
+    int64_t ldd;
+    void* d;
+};
+
+template <int TM, int TN, int WGM, int WGN, int STAGES>
+struct Cfg {
+    static constexpr int kWaves = WGM * WGN;
+    static constexpr int kThreads = 64 * kWaves;
+    static constexpr int kBM = WGM * TM * 32;
+    static constexpr int kBN = WGN * TN * 32;
+    static constexpr int kAInstr = kBM * kChunks / kThreads;   // direct-to-LDS loads per thread per tile
+    static constexpr int kWInstr = kBN * kChunks / kThreads;
+    static constexpr int kStageBytes = (kBM + kBN) * kBK;
+    static constexpr int kLdsBytes = STAGES * kStageBytes;
+};
+
+// Raw buffer descriptor (base, stride 0, num_records bytes) held in four scalar registers.
+__device__ __forceinline__ v4i make_rsrc(const void* base, int num_bytes) {
+    const uint64_t addr = reinterpret_cast<uint64_t>(base);
+    v4i r;
+    r.x = __builtin_amdgcn_readfirstlane(static_cast<int>(addr & 0xffffffffu));
+    r.y = __builtin_amdgcn_readfirstlane(static_cast<int>((addr >> 32) & 0xffffu));
+    r.z = __builtin_amdgcn_readfirstlane(num_bytes);
+    r.w = __builtin_amdgcn_readfirstlane(kRsrcFlags);
+    return r;
+}
+
+// 16 bytes per lane from buffer offset `voff` straight into LDS at lds_addr + lane*16 (lds_addr is
+// wave-uniform); lanes whose offset is outside the buffer deliver zeros.  Written as assembly so
+// that the vector-memory counter stays under this kernel's control: a tile's loads stay in flight
+// during the arithmetic and are waited for with an explicit s_waitcnt just before the barrier.
+__device__ __forceinline__ void buffer_load_lds_b128(v4i rsrc, uint32_t lds_addr, int voff) {
+    asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                 :
+                 : "s"(lds_addr), "v"(voff), "s"(rsrc)
+                 : "memory");
+}
+
+__device__ __forceinline__ uint4 buffer_load_b128(v4i rsrc, int voff) {
+    uint4 v;
+    asm volatile("buffer_load_dwordx4 %0, %1, %2, 0 offen" : "=v"(v) : "v"(voff), "s"(rsrc) : "memory");
+    return v;
+}
+
+__device__ __forceinline__ uint32_t lds_offset_of(const void* p) {
+    return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)p));
+}
+
+// Per-lane addressing of one int8 operand tile (ROWS x 128 bytes) for the direct-to-LDS loads:
+// instruction g = j*waves + wave fills LDS bytes [g*1024, +1024) of the tile, lane l the slot
+// g*64 + l = (row, physical chunk); the lane fetches the logical chunk that the swizzle maps there.
+template <int INSTR>
+struct TileLoader {
+    int voff[INSTR];     // byte offset at k0 = 0 (0x70000000 for rows outside the matrix)
+    int kc[INSTR];       // k offset of the chunk inside the tile
+    template <int WAVES>
+    __device__ __forceinline__ void init(int row0, int rows_total, int64_t ld, int wave, int lane) {
+#pragma unroll
+        for (int j = 0; j < INSTR; ++j) {
+            const int slot = (j * WAVES + wave) * 64 + lane, row = slot / kChunks, c = swz(row, slot % kChunks);
+            kc[j] = c * 16;
+            voff[j] = row0 + row < rows_total ? static_cast<int>((row0 + row) * ld) + c * 16 : 0x70000000;
+        }
+    }
+    template <int WAVES>
+    __device__ __forceinline__ void issue(v4i rsrc, int k0, int k_end, uint32_t dst, int wave) const {
+#pragma unroll
+        for (int j = 0; j < INSTR; ++j) {
+            const int off = (k0 + kc[j] < k_end) ? voff[j] + k0 : 0x7ffffff0;
+            buffer_load_lds_b128(rsrc, dst + (j * WAVES + wave) * 1024, off);
+        }
+    }
+};
+
+// Accumulates one 128-byte k tile: sa / sw point at this wave's rows of the staged operands.
+// Fragments of step kk+1 are requested before the multiplications of step kk are issued.
+template <int TM, int TN>
+__device__ __forceinline__ void mma_tile(const uint8_t* sa, const uint8_t* sw, int frow, int fhalf,
+                                         v16i (&acc)[TN][TM]) {
+    v4i fa[2][TM], fw[2][TN];
+    auto fetch = [&](int kk, int buf) {
+#pragma unroll
+        for (int i = 0; i < TN; ++i) {
+            const int row = i * 32 + frow;
+            fw[buf][i] = *reinterpret_cast<const v4i*>(sw + row * kBK + swz(row, kk * 2 + fhalf) * 16);
+        }
+#pragma unroll
+        for (int j = 0; j < TM; ++j) {
+            const int row = j * 32 + frow;
+            fa[buf][j] = *reinterpret_cast<const v4i*>(sa + row * kBK + swz(row, kk * 2 + fhalf) * 16);
+        }
+    };
+    fetch(0, 0);
+#pragma unroll
+    for (int kk = 0; kk < kBK / 32; ++kk) {
+        if (kk + 1 < kBK / 32) fetch(kk + 1, (kk + 1) & 1);
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+#pragma unroll
+            for (int j = 0; j < TM; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fw[kk & 1][i], fa[kk & 1][j], acc[i][j], 0, 0, 0);
+    }
+}
+
+// Orders this wave's LDS writes before its later LDS reads (the staging area is private to the
+// wave, and one wave's LDS operations execute in order, so no workgroup barrier is needed).
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// In acc[i][j] lane l holds output row m = j*32 + (l & 31) and, in register r, column
+// n = i*32 + 8*(r/4) + 4*(l/32) + (r%4).
+// FLEX = false compiles the common rule only (d = cast_rne(s_row * (s_col * acc))); FLEX = true also
+// honours use_alpha and the round-half-away GEMV rule at run time.  TRANS selects the (N,M) output.
+template <int TM, int TN, int OUT, bool FLEX, bool TRANS>
+__device__ __forceinline__ void epilogue(const Epilogue& e, v16i (&acc)[TN][TM], uint8_t* lds, int m, int n,
+                                         int wave_m0, int wave_n0, int wave, int lane) {
+    constexpr int kElt = OUT == QA_OUT_I8 ? 1 : 2;
+    const int frow = lane & 31, fhalf = lane >> 5;
+    const bool vec_ok = (e.ldd * kElt) % 16 == 0 && aligned16(e.d);
+    const bool use_alpha = FLEX && e.use_alpha;
+    const bool away = FLEX && e.round_mode == QA_ROUND_HALF_AWAY;
+    const int round_mode = FLEX ? e.round_mode : QA_ROUND_RNE;
+
+    // this lane's column scales: 4 consecutive columns per (i, q), loaded once
+    float s_col[TN][4][4];
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const int nn = wave_n0 + i * 32 + 8 * q + 4 * fhalf + t;
+                s_col[i][q][t] = use_alpha ? 1.0f : e.col_scale[e.col_numel == 1 ? 0 : min(nn, n - 1)];
+            }
+    float s_row[TM];
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+        const int mm = wave_m0 + j * 32 + frow;
+        s_row[j] = use_alpha ? e.alpha : e.row_scale[e.row_numel == 1 ? 0 : min(mm, m - 1)];
+    }
+    auto scaled = [&](int i, int j, int q, int t) -> float {
+        const float accf = static_cast<float>(acc[i][j][q * 4 + t]);
+        if (use_alpha) return s_row[j] * accf;
+        // GEMV rule (round-half-away mode): the two scales are multiplied first
+        return away ? (s_col[i][q][t] * s_row[j]) * accf : s_row[j] * (s_col[i][q][t] * accf);
+    };
+
+    if (!TRANS) {
+        constexpr int kPitch = TN * 32 * kElt + 16;
+        uint8_t* stg = lds + wave * (32 * kPitch);
+#pragma unroll
+        for (int j = 0; j < TM; ++j) {
+#pragma unroll
+            for (int i = 0; i < TN; ++i) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int nl = i * 32 + 8 * q + 4 * fhalf;
+                    const float v0 = scaled(i, j, q, 0), v1 = scaled(i, j, q, 1);
+                    const float v2 = scaled(i, j, q, 2), v3 = scaled(i, j, q, 3);
+                    if (OUT == QA_OUT_I8) {
+                        const uint32_t b0 = quant8(v0, round_mode) & 0xff, b1 = quant8(v1, round_mode) & 0xff;
+                        const uint32_t b2 = quant8(v2, round_mode) & 0xff, b3 = quant8(v3, round_mode);
+                        *reinterpret_cast<uint32_t*>(stg + frow * kPitch + nl) = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+                    } else {
+                        __half2 lo = __floats2half2_rn(v0, v1), hi = __floats2half2_rn(v2, v3);
+                        uint2 pk;
+                        pk.x = *reinterpret_cast<uint32_t*>(&lo);
+                        pk.y = *reinterpret_cast<uint32_t*>(&hi);
+                        *reinterpret_cast<uint2*>(stg + frow * kPitch + nl * 2) = pk;
+                    }
+                }
+            }
+            wave_lds_sync();
+            constexpr int kPiecesPerRow = TN * 32 * kElt / 16;
+#pragma unroll
+            for (int piece = lane; piece < 32 * kPiecesPerRow; piece += 64) {
+                const int r = piece / kPiecesPerRow, cb = (piece % kPiecesPerRow) * 16;
+                const int mm2 = wave_m0 + j * 32 + r;
+                const int nn = wave_n0 + cb / kElt;
+                if (mm2 >= m || nn >= n) continue;
+                uint8_t* dst = static_cast<uint8_t*>(e.d) + (static_cast<int64_t>(mm2) * e.ldd + nn) * kElt;
+                const uint4 val = *reinterpret_cast<const uint4*>(stg + r * kPitch + cb);
+                if (vec_ok && nn + 16 / kElt <= n) {
+                    *reinterpret_cast<uint4*>(dst) = val;
+                } else {
+                    const uint8_t* src = reinterpret_cast<const uint8_t*>(&val);
+                    const int nbytes = min(16, (n - nn) * kElt);
+                    for (int t = 0; t < nbytes; ++t) dst[t] = src[t];
+                }
+            }
+            wave_lds_sync();
+        }
+    } else {
+        // transposed output d[n][m]: stage 32 columns n x (TM*32) rows m per pass
+        constexpr int kPitch = TM * 32 * kElt + 16;
+        uint8_t* stg = lds + wave * (32 * kPitch);
+#pragma unroll
+        for (int i = 0; i < TN; ++i) {
+#pragma unroll
+            for (int j = 0; j < TM; ++j) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        const int nl = 8 * q + 4 * fhalf + t;          // column inside this 32-column tile
+                        const float v = scaled(i, j, q, t);
+                        if (OUT == QA_OUT_I8) {
+                            *reinterpret_cast<int8_t*>(stg + nl * kPitch + j * 32 + frow) =
+                                static_cast<int8_t>(quant8(v, round_mode));
+                        } else {
+                            *reinterpret_cast<__half*>(stg + nl * kPitch + (j * 32 + frow) * 2) = __float2half(v);
+                        }
+                    }
+                }
+            }
+            wave_lds_sync();
+            constexpr int kPiecesPerRow = TM * 32 * kElt / 16;
+#pragma unroll
+            for (int piece = lane; piece < 32 * kPiecesPerRow; piece += 64) {
+                const int r = piece / kPiecesPerRow, cb = (piece % kPiecesPerRow) * 16;
+                const int nn = wave_n0 + i * 32 + r;
+                const int mm2 = wave_m0 + cb / kElt;
+                if (nn >= n || mm2 >= m) continue;
+                uint8_t* dst = static_cast<uint8_t*>(e.d) + (static_cast<int64_t>(nn) * e.ldd + mm2) * kElt;
+                const uint4 val = *reinterpret_cast<const uint4*>(stg + r * kPitch + cb);
+                if (vec_ok && mm2 + 16 / kElt <= m) {
+                    *reinterpret_cast<uint4*>(dst) = val;
+                } else {
+                    const uint8_t* src = reinterpret_cast<const uint8_t*>(&val);
+                    const int nbytes = min(16, (m - mm2) * kElt);
+                    for (int t = 0; t < nbytes; ++t) dst[t] = src[t];
+                }
+            }
+            wave_lds_sync();
+        }
+    }
+}
+
+// Largest epilogue staging footprint (fp16, either orientation) must fit in the operand stages.
+template <int TM, int TN, int WAVES>
+constexpr int epilogue_lds_bytes() {
+    return WAVES * 32 * ((TM > TN ? TM : TN) * 32 * 2 + 16);
+}
+
+}  // namespace gemm
+}  // namespace qa
