@@ -197,7 +197,7 @@ int qa_gemm_w8a8(const QaGemmW8A8Params* p, void* stream);
  * W4A8 GEMM (int4 weights, group-wise fp16 scales, int8 activations).
  * Replaces quant_linear_cuda.w4a8o8_gemm / w4a8o16_gemm
  *   (csrc/linear/marlin_qqq_gemm_kernel.cuh:1187-1314, marlin_qqq_gemm_kernel_o8.cuh).
- * Weights are held in this library's own packing (see qa_w4a8_pack_weights); arithmetic is the
+ * Weights are held in this library's own packing (below); k must be a multiple of 128; arithmetic is the
  * reference's: w8 = rne((q4-8) * s_group) as int8, int32 accumulation, out = (acc*s_ch[n])*s_tok[m|0].
  * ---------------------------------------------------------------------------------------- */
 typedef struct QaGemmW4A8Params {
@@ -209,7 +209,9 @@ typedef struct QaGemmW4A8Params {
     int32_t reserved0;
     int64_t lda, ldd;
     const int8_t* a;         /* (M,K) */
-    const uint8_t* w_packed; /* (N, K/2): two 4-bit codes per byte, low nibble = even k */
+    const uint8_t* w_packed; /* (N, K/2): per row, each aligned group of 8 codes is 4 bytes; byte i holds
+                                code[8w+i] in the low nibble and code[8w+4+i] in the high nibble.
+                                Grouped: code in [0,15] meaning code-8; per-channel: signed nibble. */
     const void* s_group;     /* fp16 (K/group_size, N) or null when per-channel */
     const float* s_channel;  /* fp32 (N) */
     const float* s_token;    /* fp32 (1) or (M) */

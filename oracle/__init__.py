@@ -164,3 +164,28 @@ def gemm_w8a8(a, w, s_a, s_b, round_half_away=False):
                        M, N, K, int(round_half_away), acc.ctypes.data_as(C.c_void_p),
                        f.ctypes.data_as(C.c_void_p), q.ctypes.data_as(C.c_void_p))
     return acc, f, q
+
+
+def gemm_w4a8(a, codes, s_group, s_channel, s_token, group_size=128):
+    """a int8 (M,K); codes uint8 (N,K) 4-bit codes; s_group fp16 (K/128,N) or None (per-channel);
+    s_channel fp32 (N); s_token fp32 (1|M).
+    Returns (w8 int8 (N,K) expanded weights, acc int32 (M,N), fp32 value before the cast, int8 cast)."""
+    a, ap = _req(a)
+    codes, cp = _req(codes, np.uint8)
+    M, K = a.shape
+    N = codes.shape[0]
+    if s_group is not None:
+        sg = np.ascontiguousarray(np.asarray(s_group, np.float16).astype(np.float32).reshape(-1, N))
+        sgp = sg.ctypes.data_as(C.c_void_p)
+    else:
+        sgp, group_size = None, -1
+    sc = np.ascontiguousarray(np.asarray(s_channel, np.float32).reshape(-1))
+    st = np.ascontiguousarray(np.asarray(s_token, np.float32).reshape(-1))
+    w8 = np.empty((N, K), np.int8)
+    acc = np.empty((M, N), np.int32)
+    f = np.empty((M, N), np.float32)
+    q = np.empty((M, N), np.int8)
+    lib().qo_gemm_w4a8(ap, cp, sgp, sc.ctypes.data_as(C.c_void_p), st.ctypes.data_as(C.c_void_p), st.size,
+                       M, N, K, group_size, w8.ctypes.data_as(C.c_void_p), acc.ctypes.data_as(C.c_void_p),
+                       f.ctypes.data_as(C.c_void_p), q.ctypes.data_as(C.c_void_p))
+    return w8, acc, f, q

@@ -261,3 +261,45 @@ void qo_gemm_w8a8(const int8_t* a, const int8_t* w, const float* s_a, int s_a_nu
         }
     }
 }
+
+/* ---------------------------------------------------------------------------------------------
+ * W4A8 GEMM, csrc/linear/marlin_qqq_gemm_kernel.cuh:
+ *   grouped (group 128):  w8 = low byte of ( rne_fp16( (code-8) * s_group + 1152 ) ) ^ 0x80  (:136-178)
+ *       = int8( rint( (code-8) * s_group ) ): the fp16 FMA rounds the exact product once, to an
+ *       integer because fp16 spacing is 1 in [1024,2048); values outside [-128,127] wrap.
+ *   per channel (group_size < 0): w8 = code << 4 as int8, i.e. 16 * signed nibble (:127-132).
+ *   acc = int32 sum_k a[m,k] * w8[k,n];  out = (float(acc) * s_channel[n]) * s_token[m|0]  (:744-749)
+ *   int8 output: round to nearest even, saturating (marlin_qqq_gemm_kernel_o8.cuh:107-116).
+ * codes: uint8 (N,K) one 4-bit code per byte; s_group: fp32 holding fp16 values, (K/128, N).
+ * ------------------------------------------------------------------------------------------- */
+void qo_gemm_w4a8(const int8_t* a, const uint8_t* codes, const float* s_group, const float* s_channel,
+                  const float* s_token, int s_token_numel, int m, int n, int k, int group_size,
+                  int8_t* w8_out, int32_t* acc_out, float* out_f32, int8_t* out_i8) {
+    for (int j = 0; j < n; ++j) {
+        for (int kk = 0; kk < k; ++kk) {
+            const int code = codes[(int64_t)j * k + kk] & 0xf;
+            int w;
+            if (group_size > 0) {
+                const float prod = (float)(code - 8) * s_group[(int64_t)(kk / group_size) * n + j];
+                w = (int)rintf(prod) & 0xff;
+            } else {
+                w = (code << 4) & 0xff;
+            }
+            w8_out[(int64_t)j * k + kk] = (int8_t)(uint8_t)w;
+        }
+    }
+#pragma omp parallel for schedule(static)
+    for (int i = 0; i < m; ++i) {
+        for (int j = 0; j < n; ++j) {
+            int32_t acc = 0;
+            const int8_t* ar = a + (int64_t)i * k;
+            const int8_t* wr = w8_out + (int64_t)j * k;
+            for (int kk = 0; kk < k; ++kk) acc += (int32_t)ar[kk] * (int32_t)wr[kk];
+            const float v = ((float)acc * s_channel[j]) * s_token[s_token_numel == 1 ? 0 : i];
+            const int64_t o = (int64_t)i * n + j;
+            if (acc_out) acc_out[o] = acc;
+            if (out_f32) out_f32[o] = v;
+            if (out_i8) out_i8[o] = sat8_rne(v);
+        }
+    }
+}

@@ -193,9 +193,14 @@ __device__ __forceinline__ void epilogue(const Epilogue& e, v16i (&acc)[TN][TM],
     }
     auto scaled = [&](int i, int j, int q, int t) -> float {
         const float accf = static_cast<float>(acc[i][j][q * 4 + t]);
-        if (use_alpha) return s_row[j] * accf;
+        float v;
+        if (use_alpha) v = s_row[j] * accf;
         // GEMV rule (round-half-away mode): the two scales are multiplied first
-        return away ? (s_col[i][q][t] * s_row[j]) * accf : s_row[j] * (s_col[i][q][t] * accf);
+        else v = away ? (s_col[i][q][t] * s_row[j]) * accf : s_row[j] * (s_col[i][q][t] * accf);
+        // keep the fp32 product a value of its own: folding the multiply into a mixed-precision
+        // convert would round once instead of twice and change the fp16 result in rare cases
+        asm volatile("" : "+v"(v));
+        return v;
     };
 
     if (!TRANS) {

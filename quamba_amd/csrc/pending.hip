@@ -1,5 +1,4 @@
 // Entry points whose kernels are not written yet report QA_ERR_UNSUPPORTED.
 #include "qa_common.hpp"
-extern "C" int qa_gemm_w4a8(const QaGemmW4A8Params*, void*) { return QA_ERR_UNSUPPORTED; }
 extern "C" int64_t qa_ssd_workspace_bytes(const QaSsdParams*) { return 0; }
 extern "C" int qa_ssd_chunk_scan_fwd(const QaSsdParams*, void*) { return QA_ERR_UNSUPPORTED; }

@@ -190,3 +190,114 @@ class W8A8B16O16Linear(_W8A8Base, _AlphaHooks):
 
     def __repr__(self):
         return f"W8A8B16O16Linear(in_features={self.in_features}, out_features={self.out_features})"
+
+
+# ------------------------------------------------------------------------------------------------
+# W4A8: int8 activations x 4-bit weights (group 128 fp16 scales over a per-channel int8 scale)
+# Drop-ins for quamba/qLinearLayer.py:139-536.  Buffer names are the reference's (workspace, weight,
+# input_scale, s_channel, s_group); ``weight`` holds this library's packing (uint8 (N, K/2), see
+# w4a8_utils.pack_w4a8) and the scales are in natural column order, so a reference checkpoint needs
+# re-packing before it can be loaded here.
+# ------------------------------------------------------------------------------------------------
+from .w4a8_utils import w4a8_quantize  # noqa: E402
+
+
+class _W4A8Base(nn.Module):
+    _out_dtype = torch.float16
+
+    def __init__(self, in_features, out_features, group_size=128, device=None, **kwargs):
+        super().__init__()
+        device = _default_device() if device is None else device
+        self.bias = None
+        self.in_features = in_features
+        self.out_features = out_features
+        self.size_n, self.size_k = out_features, in_features
+        self.pad_out = 0 if out_features % 64 == 0 else 64 - out_features % 64
+        self.size_n += self.pad_out
+        self.register_buffer("workspace", torch.zeros(1, dtype=torch.int32, device=device))
+        self.register_buffer("weight", torch.empty((self.size_n, self.size_k // 2), dtype=torch.uint8, device=device))
+        self.register_buffer("input_scale", torch.empty((), dtype=torch.float32, device=device))
+        self.register_buffer("s_channel", torch.empty((1, self.size_n), dtype=torch.float32, device=device))
+        n_groups = self.size_k // group_size if self.size_k > 128 else 0
+        self.register_buffer("s_group", torch.empty((n_groups, self.size_n), dtype=torch.float16, device=device))
+
+    @classmethod
+    def _from_fp16(cls, originalLayer, input_scale, out_scales):
+        assert input_scale.numel() == 1, "Only support per-tensor input scale"
+        assert originalLayer.bias is None, "Not support bias yet"
+        bits, group_scale = 4, None
+        group_size = 128 if originalLayer.in_features > 128 else -1
+        if getattr(originalLayer, "apply_gptq", False):
+            bits, group_size = originalLayer.bits, originalLayer.group_size
+            group_scale = originalLayer.group_scale.to(torch.float16).cpu()
+        assert bits == 4, "Only support 4-bit quantization"
+        if group_size not in (-1, 128):
+            raise ValueError("Only groupsize -1 and 128 are supported.")
+        device = originalLayer.weight.device
+        q = cls(originalLayer.in_features, originalLayer.out_features, group_size=128, device=device)
+        W = originalLayer.weight.detach()
+        channel_scale = (W.abs().amax(dim=1, keepdim=True) / 127.0).reshape(1, -1).float().cpu()
+        W_t = W.cpu().to(torch.float16).t().contiguous()
+        w_ref, packed, s_group, s_channel = w4a8_quantize(W_t, bits, group_size, group_scale, channel_scale,
+                                                          out_scales=out_scales, pad_out=q.pad_out)
+        q.size_k, q.size_n = w_ref.shape
+        q.weight = packed.to(device)
+        q.input_scale = input_scale.detach().reshape(()).float().to(device)
+        q.s_group = s_group.to(device)
+        q.s_channel = s_channel.to(device)
+        q.w_ref = w_ref          # dequantised (K, N) weights, kept for tests (not a buffer)
+        return q
+
+    def _gemm(self, x2d, transpose):
+        fn = ops.w4a8o8_gemm if self._out_dtype == torch.int8 else ops.w4a8o16_gemm
+        return fn(x2d, self.weight, self.input_scale.reshape(1), self.s_channel, self.s_group, self.workspace,
+                  x2d.shape[0], self.size_n, self.size_k, transpose)
+
+    @torch.no_grad()
+    def forward(self, x):
+        x_shape = x.shape
+        y = self._gemm(x.reshape(-1, x_shape[-1]).contiguous(), False)
+        if self.pad_out:
+            y = y[:, :-self.pad_out]
+        return y.view(*x_shape[:-1], -1)
+
+    @torch.no_grad()
+    def to_seqlen_last(self, x):
+        """(B, L, in) -> (B, out, L): a view with strides (L, B*L, 1) of an (out, B*L) buffer."""
+        B, L, D = x.shape
+        y = self._gemm(x.reshape(-1, D).contiguous(), True)
+        if self.pad_out:
+            y = y[:-self.pad_out]
+        return y.view(-1, B, L).transpose(0, 1)
+
+    def __repr__(self):
+        return f"{type(self).__name__}(in_features={self.in_features}, out_features={self.out_features})"
+
+
+class W4A8B16O16Linear(_W4A8Base):
+    _out_dtype = torch.float16
+
+    @classmethod
+    def from_fp16(cls, originalLayer: nn.Linear, input_scale: torch.Tensor):
+        return cls._from_fp16(originalLayer, input_scale, None)
+
+
+class W4A8B8O8Linear(_W4A8Base):
+    _out_dtype = torch.int8
+
+    @classmethod
+    def from_fp16(cls, originalLayer: nn.Linear, input_scale: torch.Tensor, output_scale: torch.Tensor):
+        assert output_scale.numel() == 1, "Only support per-tensor output scale"
+        return cls._from_fp16(originalLayer, input_scale, output_scale.reshape(1).cpu())
+
+
+class W4A8B8O8LinearParallel(_W4A8Base):
+    _out_dtype = torch.int8
+
+    @classmethod
+    def from_fp16(cls, originalLayer: nn.Linear, input_scale: torch.Tensor, output_scales, out_split_dims):
+        assert sum(out_split_dims) == originalLayer.out_features
+        assert len(out_split_dims) == len(output_scales)
+        per_channel = torch.cat([torch.as_tensor(s, dtype=torch.float32).reshape(1).repeat(d)
+                                 for d, s in zip(out_split_dims, output_scales)]).cpu()
+        return cls._from_fp16(originalLayer, input_scale, per_channel)

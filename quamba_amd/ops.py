@@ -343,3 +343,47 @@ def w8a8o8_gemv(y, w, x, b_scales, a_scale):
     The reference multiplies b_scales[n] * a_scale first (quant_linear_fwd_gemv_kernel.cuh:56-60); the two scale
     operands are therefore passed swapped so that the same product is formed."""
     return _gemm_w8a8(y, x, w, a_scale, b_scales, round_half_away=True)
+
+
+# ----------------------------------------------------------------------------------------------
+# W4A8 linear
+# ----------------------------------------------------------------------------------------------
+def _w4a8_gemm(a, b_q_weight, s_tok, s_ch, s_group, m, n, k, output_transpose, out_dtype):
+    _require(a.dtype == torch.int8 and a.is_cuda and a.dim() == 2 and a.is_contiguous(), "a must be a contiguous int8 GPU matrix")
+    _require(tuple(a.shape) == (m, k), "a must have shape (m, k)")
+    _require(b_q_weight.dtype == torch.uint8 and b_q_weight.is_cuda and tuple(b_q_weight.shape) == (n, k // 2)
+             and b_q_weight.is_contiguous(), "b_q_weight must be uint8 (n, k/2) in this library's packing")
+    _require(k % 128 == 0, "k must be a multiple of 128")
+    _require(s_ch.dtype == torch.float32 and s_ch.is_cuda and s_ch.numel() == n, "s_ch must be fp32 with n elements")
+    _require(s_tok.dtype == torch.float32 and s_tok.is_cuda and s_tok.numel() in (1, m),
+             "s_tok must be fp32 with 1 or m elements")
+    grouped = s_group is not None and s_group.numel() > 0
+    if grouped:
+        _require(s_group.dtype == torch.float16 and s_group.is_cuda and tuple(s_group.shape) == (k // 128, n)
+                 and s_group.is_contiguous(), "s_group must be contiguous fp16 (k/128, n)")
+    d = torch.empty((n, m) if output_transpose else (m, n), dtype=out_dtype, device=a.device)
+    p = _lib.QaGemmW4A8Params()
+    p.m, p.n, p.k = m, n, k
+    p.group_size = 128 if grouped else -1
+    p.out_type = _lib.QA_OUT_I8 if out_dtype == torch.int8 else _lib.QA_OUT_F16
+    p.tok_scale_numel = s_tok.numel()
+    p.output_transpose = int(bool(output_transpose))
+    p.lda, p.ldd = a.stride(0), d.stride(0)
+    s_ch_c, s_tok_c = s_ch.contiguous(), s_tok.contiguous()
+    p.a, p.w_packed, p.s_group = ptr(a), ptr(b_q_weight), ptr(s_group) if grouped else None
+    p.s_channel, p.s_token, p.d = ptr(s_ch_c), ptr(s_tok_c), ptr(d)
+    with torch.cuda.device(a.device):
+        st = _lib.lib().qa_gemm_w4a8(ct.byref(p), _lib.current_stream(a.device))
+    _lib.check(st, "gemm_w4a8")
+    return d
+
+
+def w4a8o16_gemm(a, b_q_weight, s_tok, s_ch, s_group, workspace, m, n, k, output_transpose=False):
+    """fp16 (m, n) [or (n, m)] = ((a @ dequant(b)^T) * s_ch[n]) * s_tok[m|0].  ``workspace`` is accepted for
+    interface compatibility and unused (no cross-workgroup reduction is needed)."""
+    return _w4a8_gemm(a, b_q_weight, s_tok, s_ch, s_group, m, n, k, output_transpose, torch.float16)
+
+
+def w4a8o8_gemm(a, b_q_weight, s_tok, s_ch, s_group, workspace, m, n, k, output_transpose=False):
+    """int8 variant: round-half-even, saturating."""
+    return _w4a8_gemm(a, b_q_weight, s_tok, s_ch, s_group, m, n, k, output_transpose, torch.int8)
