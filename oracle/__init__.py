@@ -189,3 +189,54 @@ def gemm_w4a8(a, codes, s_group, s_channel, s_token, group_size=128):
                        M, N, K, group_size, w8.ctypes.data_as(C.c_void_p), acc.ctypes.data_as(C.c_void_p),
                        f.ctypes.data_as(C.c_void_p), q.ctypes.data_as(C.c_void_p))
     return w8, acc, f, q
+
+
+class _QoSsdDims(C.Structure):
+    _fields_ = [(n, C.c_int) for n in ("batch", "seqlen", "nheads", "headdim", "dstate", "ngroups", "chunk",
+                                       "softplus", "dt_is_f32", "D_has_hdim", "nhead_groups", "ndim_groups")] + \
+               [("dt_min", C.c_float), ("dt_max", C.c_float)]
+
+
+def ssd_fwd(x, dt, A_log, B, C_, D=None, z=None, dt_bias=None, *, chunk_size, x_scale, s_dt=1.0, s_A, s_B, s_C,
+            s_D=0.0, s_z=0.0, state_scale=None, head_range=None, dim_range=None, softplus=True,
+            dt_limit=(0.0, float("inf")), stages=False):
+    """x int8 (B,L,H,P); dt int8 or float32 (B,L,H) (float32 = already processed); A_log int8 (H);
+    B, C int8 (B,L,G,N); D int8 (H) or (H,P); z int8 like x; dt_bias float (H) holding fp16 values.
+    x_scale / s_B / s_C / state_scale: scalars, or grouped arrays with head_range (G,hg) and
+    dim_range (G,hg,dg) int32 cumulative end indices.
+    Returns dict(y float32 (B,L,H,P) before the fp16 cast, final_f32, final_i8 [, dt, dA_cumsum, CB,
+    chunk_states, prev_states with stages=True])."""
+    x, xp = _req(x)
+    Bsz, L, H, P = x.shape
+    B, bp = _req(B)
+    C_, cp = _req(C_)
+    G, N = B.shape[2], B.shape[3]
+    A_log, ap = _req(A_log)
+    dt = np.ascontiguousarray(dt)
+    dt_is_f32 = dt.dtype == np.float32
+    assert dt_is_f32 or dt.dtype == np.int8
+    grouped = head_range is not None
+    dims = _QoSsdDims(Bsz, L, H, P, N, G, chunk_size, int(softplus), int(dt_is_f32),
+                      int(D is not None and np.asarray(D).ndim == 2),
+                      head_range.shape[1] if grouped else 0, dim_range.shape[2] if grouped else 0,
+                      float(dt_limit[0]), float(min(dt_limit[1], 3.0e38)))
+    f32 = lambda a: np.ascontiguousarray(np.asarray(a, np.float32).reshape(-1))
+    xs, sB, sC = f32(x_scale), f32(s_B), f32(s_C)
+    ss = f32(state_scale if state_scale is not None else 1.0)
+    dbias = None if dt_bias is None else f32(np.asarray(dt_bias, np.float16))
+    hr = None if not grouped else np.ascontiguousarray(head_range, np.int32)
+    dr = None if not grouped else np.ascontiguousarray(dim_range, np.int32)
+    nc = (L + chunk_size - 1) // chunk_size
+    out = dict(y=np.zeros((Bsz, L, H, P), np.float32), final_f32=np.empty((Bsz, H, P, N), np.float32),
+               final_i8=np.empty((Bsz, H, P, N), np.int8))
+    if stages:
+        out.update(dt=np.empty((Bsz, H, nc, chunk_size), np.float32), dA_cumsum=np.empty((Bsz, H, nc, chunk_size), np.float32),
+                   CB=np.zeros((Bsz, nc, G, chunk_size, chunk_size), np.float32),
+                   chunk_states=np.empty((Bsz, nc, H, P, N), np.float32), prev_states=np.empty((Bsz, nc, H, P, N), np.float32))
+    vp = lambda a: None if a is None else a.ctypes.data_as(C.c_void_p)
+    lib().qo_ssd_fwd(C.byref(dims), xp, vp(dt), ap, bp, cp, _opt(D), _opt(z), vp(dbias), vp(xs), vp(hr), vp(dr),
+                     _f(s_dt), _f(s_A), vp(sB), vp(sC), _f(s_D), _f(s_z), vp(ss),
+                     vp(out["y"]), vp(out["final_f32"]), vp(out["final_i8"]),
+                     vp(out.get("dt")), vp(out.get("dA_cumsum")), vp(out.get("CB")), vp(out.get("chunk_states")),
+                     vp(out.get("prev_states")))
+    return out

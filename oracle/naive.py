@@ -40,3 +40,31 @@ def selective_scan(u, delta, A, B, C, D=None, z=None, delta_bias=None, delta_sof
             yt = yt * silu(np.asarray(z, np.float64)[:, :, t])
         y[:, t] = yt
     return y, h
+
+
+def ssd_recurrence(x, dt, A, B, C, D=None, z=None):
+    """Textbook Mamba2 (scalar A per head) recurrence in float64 on real-valued inputs.
+
+    x: (batch, L, H, P); dt: (batch, L, H) already processed; A: (H) negative; B, C: (batch, L, G, N);
+    D: (H) or (H, P).  h_t = exp(dt_t A) h_{t-1} + dt_t x_t B_t^T;  y_t = h_t C_t + D x_t.
+    Returns (y (batch, L, H, P), final state (batch, H, P, N)).
+    """
+    x = np.asarray(x, np.float64)
+    batch, L, H, P = x.shape
+    G, N = B.shape[2], B.shape[3]
+    rep = H // G
+    h = np.zeros((batch, H, P, N))
+    y = np.zeros((batch, L, H, P))
+    for t in range(L):
+        dA = np.exp(dt[:, t] * A[None])                                   # (batch, H)
+        Bt = np.repeat(B[:, t], rep, axis=1)                              # (batch, H, N)
+        Ct = np.repeat(C[:, t], rep, axis=1)
+        h = dA[:, :, None, None] * h + (dt[:, t, :, None] * x[:, t])[..., None] * Bt[:, :, None, :]
+        yt = np.einsum("bhpn,bhn->bhp", h, Ct)
+        if D is not None:
+            Dv = np.asarray(D, np.float64)
+            yt = yt + x[:, t] * (Dv[None, :, None] if Dv.ndim == 1 else Dv[None])
+        if z is not None:
+            yt = yt * silu(np.asarray(z, np.float64)[:, t])
+        y[:, t] = yt
+    return y, h

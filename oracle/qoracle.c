@@ -11,6 +11,7 @@
  */
 #include <math.h>
 #include <stdint.h>
+#include <stdlib.h>
 #include <string.h>
 
 /* ---------------------------------------------------------------------------------------------
@@ -300,6 +301,202 @@ void qo_gemm_w4a8(const int8_t* a, const uint8_t* codes, const float* s_group, c
             if (acc_out) acc_out[o] = acc;
             if (out_f32) out_f32[o] = v;
             if (out_i8) out_i8[o] = sat8_rne(v);
+        }
+    }
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * Mamba2 quantized SSD chunk scan, quamba/triton/quant_ssd_combined.py:61-77 (per-tensor scales)
+ * and :146-162 (head/dim-grouped scales).  Stages, each as its Triton kernel computes it:
+ *   1 quant_chunk_cumsum.py:56-70      dt = clamp(softplus(s_dt q_dt + dt_bias)), 0 past seqlen;
+ *                                      dA_cs = cumsum within the chunk of dt * A, A = -exp(s_A q_A)
+ *   2 quant_chunk_state.py:76-89       S_c[p,n] = sum_k f16(x^[k,p]) * f16(B^[k,n] * exp(dA_last-dA_k) * dt_k)
+ *   3 quant_state_passing.py:60-83     P_0 = 0; P_{c+1} = exp(dA_last,c) P_c + S_c; P_c kept as fp16
+ *   4 quant_bmm_chunk.py:60-66         CB[m,k] = sum_n C^[m,n] B^[k,n]   (fp32)
+ *   5 quant_chunk_scan.py:96-171       y[m,p] = exp(dA_m) sum_n f16(C^[m,n]) f16(P_c[p,n])
+ *                                               + sum_{k<=m} f16(CB[m,k] exp(dA_m-dA_k) dt_k) f16(x^[k,p])
+ *                                               + x^[m,p] D;   y *= z sigmoid(z) when z is given
+ *   6 quant_ssm_states.py:43,119       final int8 = sat8(rint(f16(P_final)*K / (scale*K))), K = 1e2 (1e6 grouped)
+ * Products of fp16 operands are accumulated in fp32 (the order of accumulation is the kernels' own).
+ * x^ = s_x[g,hg,dg] q_x with the group looked up from cumulative end indices
+ * (quant_chunk_state.py:202-214): hg = #{j : h mod (H/G) >= head_range[g,j]}, dg = #{j : p >= dim_range[g,hg,j]}.
+ * ------------------------------------------------------------------------------------------- */
+static float f16_round(float v) {
+    /* round to nearest even fp16 and back (normal, subnormal, overflow to inf) */
+    uint32_t x;
+    memcpy(&x, &v, 4);
+    const uint32_t sign = x & 0x80000000u;
+    x &= 0x7fffffffu;
+    float a;
+    memcpy(&a, &x, 4);
+    if (x >= 0x7f800000u) return v;                       /* inf / nan */
+    if (a >= 65520.0f) { uint32_t inf = sign | 0x7f800000u; float r; memcpy(&r, &inf, 4); return r; }
+    float r;
+    if (a < 6.103515625e-05f) {                           /* subnormal half: multiples of 2^-24 */
+        r = rintf(a * 16777216.0f) / 16777216.0f;
+    } else {
+        const uint32_t lsb = (x >> 13) & 1u;
+        uint32_t y = x + 0xfffu + lsb;
+        y &= 0xffffe000u;
+        memcpy(&r, &y, 4);
+    }
+    uint32_t rb;
+    memcpy(&rb, &r, 4);
+    rb |= sign;
+    memcpy(&r, &rb, 4);
+    return r;
+}
+
+float qo_f16_round(float v) { return f16_round(v); }
+
+typedef struct {
+    int batch, seqlen, nheads, headdim, dstate, ngroups, chunk;
+    int softplus, dt_is_f32, D_has_hdim, nhead_groups, ndim_groups;
+    float dt_min, dt_max;
+} QoSsdDims;
+
+void qo_ssd_fwd(const QoSsdDims* d, const int8_t* x, const void* dt_in, const int8_t* A_log, const int8_t* Bm,
+                const int8_t* Cm, const int8_t* D, const int8_t* z, const float* dt_bias,
+                const float* x_scale, const int32_t* head_range, const int32_t* dim_range,
+                float s_dt, float s_A, const float* s_B, const float* s_C, float s_D, float s_z,
+                const float* state_scale,
+                float* y, float* final_f32, int8_t* final_i8,
+                float* dt_out, float* dA_out, float* cb_out, float* chunk_states_out, float* prev_states_out) {
+    const int Bsz = d->batch, L = d->seqlen, H = d->nheads, P = d->headdim, N = d->dstate, G = d->ngroups, Q = d->chunk;
+    const int nc = (L + Q - 1) / Q;
+    const int hpg = H / G;
+    const int grouped = d->nhead_groups > 0;
+#pragma omp parallel for collapse(2) schedule(dynamic)
+    for (int b = 0; b < Bsz; ++b) {
+        for (int h = 0; h < H; ++h) {
+            const int g = h / hpg;
+            int hg = 0;
+            if (grouped) {
+                for (int j = 0; j < d->nhead_groups; ++j) hg += (h % hpg) >= head_range[g * d->nhead_groups + j];
+            }
+            float xs_p[256];          /* x scale per p */
+            int dg_p[256];
+            for (int p = 0; p < P; ++p) {
+                int dg = 0;
+                if (grouped) {
+                    const int32_t* dr = dim_range + (g * d->nhead_groups + hg) * d->ndim_groups;
+                    for (int j = 0; j < d->ndim_groups; ++j) dg += p >= dr[j];
+                    xs_p[p] = x_scale[(g * d->nhead_groups + hg) * d->ndim_groups + dg];
+                } else {
+                    xs_p[p] = x_scale[0];
+                }
+                dg_p[p] = dg;
+            }
+            const float sB = grouped ? s_B[g] : s_B[0];
+            const float sC = grouped ? s_C[g] : s_C[0];
+            const float A = -expf(s_A * (float)A_log[h]);
+            float* Pst = (float*)calloc((size_t)P * N, sizeof(float));      /* running state, fp32 */
+            float* P16 = (float*)malloc((size_t)P * N * sizeof(float));     /* state entering the chunk, fp16 values */
+            float* S = (float*)malloc((size_t)P * N * sizeof(float));
+            float* dtc = (float*)malloc((size_t)Q * sizeof(float));
+            float* dAc = (float*)malloc((size_t)Q * sizeof(float));
+            float* cb = (float*)malloc((size_t)Q * Q * sizeof(float));
+            for (int c = 0; c < nc; ++c) {
+                const int t0 = c * Q;
+                const int lim = L - t0 < Q ? L - t0 : Q;
+                /* stage 1 */
+                float run = 0.0f;
+                for (int k = 0; k < Q; ++k) {
+                    float dtv = 0.0f;
+                    if (k < lim) {
+                        const int64_t di = ((int64_t)b * L + t0 + k) * H + h;
+                        if (d->dt_is_f32) {
+                            dtv = ((const float*)dt_in)[di];
+                        } else {
+                            dtv = s_dt * (float)((const int8_t*)dt_in)[di];
+                            if (dt_bias) dtv += dt_bias[h];
+                            if (d->softplus) dtv = softplus20(dtv);
+                            dtv = fminf(fmaxf(dtv, d->dt_min), d->dt_max);
+                        }
+                    }
+                    dtc[k] = dtv;
+                    run += dtv * A;
+                    dAc[k] = run;
+                    if (dt_out) dt_out[(((int64_t)b * H + h) * nc + c) * Q + k] = dtv;
+                    if (dA_out) dA_out[(((int64_t)b * H + h) * nc + c) * Q + k] = run;
+                }
+                const float dA_last = dAc[Q - 1];
+                /* stage 4: CB for this (b, c, g) (recomputed per head; identical for heads of a group) */
+                for (int m = 0; m < Q; ++m) {
+                    for (int k = 0; k < Q; ++k) {
+                        float acc = 0.0f;
+                        if (m < lim && k < lim) {
+                            const int8_t* cr = Cm + (((int64_t)b * L + t0 + m) * G + g) * N;
+                            const int8_t* br = Bm + (((int64_t)b * L + t0 + k) * G + g) * N;
+                            int32_t iacc = 0;
+                            for (int n = 0; n < N; ++n) iacc += (int32_t)cr[n] * (int32_t)br[n];
+                            /* sum_n (sC c)(sB b): every product is exact up to the two scale roundings;
+                               the integer sum times the scale product is the same value to fp32 accuracy */
+                            acc = (sC * sB) * (float)iacc;
+                        }
+                        cb[(int64_t)m * Q + k] = acc;
+                        if (cb_out && h % hpg == 0) cb_out[((((int64_t)b * nc + c) * G + g) * Q + m) * Q + k] = acc;
+                    }
+                }
+                /* stage 3 (entering state) */
+                for (int i = 0; i < P * N; ++i) P16[i] = f16_round(Pst[i]);
+                if (prev_states_out) memcpy(prev_states_out + ((((int64_t)b * nc + c) * H + h) * P) * N, P16, (size_t)P * N * 4);
+                /* stage 5 */
+                for (int m = 0; m < lim; ++m) {
+                    const int8_t* cr = Cm + (((int64_t)b * L + t0 + m) * G + g) * N;
+                    const float scale_m = expf(dAc[m]);
+                    for (int p = 0; p < P; ++p) {
+                        float acc = 0.0f;
+                        for (int n = 0; n < N; ++n) acc += f16_round(sC * (float)cr[n]) * P16[p * N + n];
+                        acc *= scale_m;
+                        for (int k = 0; k <= m; ++k) {
+                            const float w = f16_round(cb[(int64_t)m * Q + k] * expf(dAc[m] - dAc[k]) * dtc[k]);
+                            const float xv = f16_round(xs_p[p] * (float)x[(((int64_t)b * L + t0 + k) * H + h) * P + p]);
+                            acc += w * xv;
+                        }
+                        const int64_t oi = (((int64_t)b * L + t0 + m) * H + h) * P + p;
+                        if (D) {
+                            const float Dv = s_D * (float)D[d->D_has_hdim ? h * P + p : h];
+                            acc += (xs_p[p] * (float)x[oi]) * Dv;
+                        }
+                        if (z) {
+                            const float zv = s_z * (float)z[oi];
+                            acc *= zv * (1.0f / (1.0f + expf(-zv)));
+                        }
+                        y[oi] = acc;
+                    }
+                }
+                /* stage 2 */
+                for (int p = 0; p < P; ++p) {
+                    for (int n = 0; n < N; ++n) {
+                        float acc = 0.0f;
+                        for (int k = 0; k < lim; ++k) {
+                            const float xv = f16_round(xs_p[p] * (float)x[(((int64_t)b * L + t0 + k) * H + h) * P + p]);
+                            const float bv = sB * (float)Bm[(((int64_t)b * L + t0 + k) * G + g) * N + n];
+                            acc += xv * f16_round(bv * (expf(dA_last - dAc[k]) * dtc[k]));
+                        }
+                        S[p * N + n] = acc;
+                    }
+                }
+                if (chunk_states_out) memcpy(chunk_states_out + ((((int64_t)b * nc + c) * H + h) * P) * N, S, (size_t)P * N * 4);
+                /* stage 3 (update) */
+                const float decay = expf(dA_last);
+                for (int i = 0; i < P * N; ++i) Pst[i] = decay * Pst[i] + S[i];
+            }
+            for (int p = 0; p < P; ++p) {
+                for (int n = 0; n < N; ++n) {
+                    const int64_t si = (((int64_t)b * H + h) * P + p) * N + n;
+                    const float v = Pst[p * N + n];
+                    if (final_f32) final_f32[si] = v;
+                    if (final_i8) {
+                        const float K = grouped ? 1e6f : 1e2f;
+                        const float sc = grouped ? state_scale[((g * d->nhead_groups + hg) * d->ndim_groups + dg_p[p]) * N + n]
+                                                 : state_scale[0];
+                        final_i8[si] = sat8_rne((f16_round(v) * K) / (sc * K));
+                    }
+                }
+            }
+            free(Pst); free(P16); free(S); free(dtc); free(dAc); free(cb);
         }
     }
 }

@@ -115,3 +115,61 @@ def linear_weights(out_features, in_features, seed, name="w", per_channel=True):
         return q, s.astype(np.float32), w
     q, s = quantize_absmax(w)
     return q, np.array([s], np.float32), w
+
+
+def mamba2_ssd_inputs(batch, seqlen, nheads, headdim, dstate, ngroups, seed=1234, grouped=False,
+                      nhead_groups=4, ndim_groups=4, with_z=False):
+    """Quantised inputs of the Mamba2 SSD chunk scan.
+
+    x (batch, seqlen, nheads, headdim), dt (batch, seqlen, nheads), B, C (batch, seqlen, ngroups, dstate)
+    int8; A_log, D (nheads) int8; dt_bias (nheads) fp16.  With ``grouped`` the x scale is per
+    (ssd group, head group, dim group) with equal-sized groups and B/C scales per ssd group.
+    """
+    out = {}
+    x = activations((batch, seqlen, nheads, headdim), 2, seed, "x2")
+    g = rng_for(seed, "dt2")
+    dt_target = np.exp(g.uniform(np.log(1e-3), np.log(1e-1), (batch, seqlen, nheads))).astype(np.float32)
+    dt_init = np.exp(rng_for(seed, "dt_bias2").uniform(np.log(1e-3), np.log(1e-1), (nheads,))).astype(np.float32)
+    dt_bias = inv_softplus(dt_init.astype(np.float64)).astype(np.float16)
+    dt_raw = (inv_softplus(dt_target.astype(np.float64)) - dt_bias.astype(np.float64)[None, None, :]).astype(np.float32)
+    out["dt"], out["s_dt"] = quantize_absmax(dt_raw)
+    out["dt_bias"] = dt_bias
+    out["dt_f32"] = dt_target
+    A_log = rng_for(seed, "A2").uniform(0.0, np.log(16.0), (nheads,)).astype(np.float32)      # A = -exp(U[0, log 16])
+    out["A_log"], out["s_A"] = quantize_absmax(A_log)
+    out["D"], out["s_D"] = quantize_absmax(np.ones((nheads,), np.float32))
+    Bm = activations((batch, seqlen, ngroups, dstate), 3, seed, "B2", outliers=False)
+    Cm = activations((batch, seqlen, ngroups, dstate), 3, seed, "C2", outliers=False)
+    if not grouped:
+        out["x"], sx = quantize_absmax(x)
+        out["x_scale"] = np.array([sx], np.float32)
+        out["B"], sB = quantize_absmax(Bm)
+        out["C"], sC = quantize_absmax(Cm)
+        out["s_B"], out["s_C"] = np.array([sB], np.float32), np.array([sC], np.float32)
+        out["head_range"] = out["dim_range"] = None
+    else:
+        hpg = nheads // ngroups
+        assert hpg % nhead_groups == 0 and headdim % ndim_groups == 0
+        hs, ds = hpg // nhead_groups, headdim // ndim_groups
+        out["head_range"] = np.tile(np.arange(1, nhead_groups + 1, dtype=np.int32) * hs, (ngroups, 1))
+        out["dim_range"] = np.tile(np.arange(1, ndim_groups + 1, dtype=np.int32) * ds, (ngroups, nhead_groups, 1))
+        qx = np.empty(x.shape, np.int8)
+        xs = np.empty((ngroups, nhead_groups, ndim_groups), np.float32)
+        for gi in range(ngroups):
+            for hg in range(nhead_groups):
+                for dg in range(ndim_groups):
+                    sl = (slice(None), slice(None), slice(gi * hpg + hg * hs, gi * hpg + (hg + 1) * hs),
+                          slice(dg * ds, (dg + 1) * ds))
+                    qx[sl], xs[gi, hg, dg] = quantize_absmax(x[sl])
+        out["x"], out["x_scale"] = qx, xs
+        qB, qC = np.empty(Bm.shape, np.int8), np.empty(Cm.shape, np.int8)
+        sB, sC = np.empty(ngroups, np.float32), np.empty(ngroups, np.float32)
+        for gi in range(ngroups):
+            qB[:, :, gi], sB[gi] = quantize_absmax(Bm[:, :, gi])
+            qC[:, :, gi], sC[gi] = quantize_absmax(Cm[:, :, gi])
+        out["B"], out["C"], out["s_B"], out["s_C"] = qB, qC, sB, sC
+    if with_z:
+        out["z"], out["s_z"] = quantize_absmax(activations((batch, seqlen, nheads, headdim), 2, seed, "z2"))
+    else:
+        out["z"], out["s_z"] = None, np.float32(0.0)
+    return out
