@@ -1,0 +1,494 @@
+// Mamba2 quantized SSD chunk scan (prefill) for gfx950.
+//
+// Stages and arithmetic follow the reference's Triton pipeline (quamba/triton/quant_ssd_combined.py
+// :61-77, grouped :146-162); see each kernel for the file it restates.  fp16 operands, fp32
+// accumulation, as there; the one pure int8 contraction (C B^T) runs on the int8 matrix cores.
+//   cumsum      dt = clamp(softplus(s_dt q_dt + dt_bias)), dA_cs = within-chunk cumsum(dt * A)
+//   cb          CB[m,k] = (s_C s_B) * sum_n q_C[m,n] q_B[k,n]                       (int8 MFMA, lower tiles)
+//   chunk_state S_c[p,n] = sum_k f16(x^[k,p]) f16(B^[k,n] exp(dA_last - dA_k) dt_k)   (fp16 MFMA)
+//   passing     P_0 = 0, P_{c+1} = exp(dA_last,c) P_c + S_c; P_c kept in fp16; final state fp32 / int8
+//   chunk_scan  y[m,p] = exp(dA_m) sum_n f16(C^[m,n]) P_c[p,n] + sum_{k<=m} f16(CB[m,k] e^{dA_m-dA_k} dt_k) f16(x^[k,p])
+//               + D x^[m,p], optional z gate, fp16 out                               (fp16 MFMA)
+// Both fp16 contractions over the time index need x (and B) with time as the fastest-moving index,
+// while memory has channels fastest; the tiles are transposed once on the way into LDS (4x4 blocks:
+// four dword loads, four 8-byte LDS stores) and then read as 16-byte MFMA operands.
+#include "qa_common.hpp"
+
+namespace qa {
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int kP = 64;          // head dimension this build supports
+constexpr float kLog2e = 1.44269504088896341f;
+
+__device__ __forceinline__ float fexp(float x) { return __builtin_amdgcn_exp2f(x * kLog2e); }
+__device__ __forceinline__ int8_t byte_of(uint32_t w, int j) { return static_cast<int8_t>((w >> (8 * j)) & 0xffu); }
+
+struct Ws {            // workspace sections (byte offsets), see qa_ssd_workspace_bytes
+    int64_t dt, dA, cb, states, prev, final_f32, total;
+};
+
+__host__ __device__ inline int64_t align256(int64_t v) { return (v + 255) & ~int64_t(255); }
+
+__host__ __device__ inline Ws ws_layout(const QaSsdParams& p) {
+    const int64_t nc = (p.seqlen + p.chunk_size - 1) / p.chunk_size;
+    const int64_t B = p.batch, H = p.nheads, Q = p.chunk_size, G = p.ngroups, P = p.headdim, N = p.dstate;
+    Ws w;
+    int64_t off = 0;
+    w.dt = off; off = align256(off + B * H * nc * Q * 4);
+    w.dA = off; off = align256(off + B * H * nc * Q * 4);
+    w.cb = off; off = align256(off + B * nc * G * Q * Q * 4);
+    w.states = off; off = align256(off + B * nc * H * P * N * 4);
+    w.prev = off; off = align256(off + B * nc * H * P * N * 2);
+    w.final_f32 = off; off = align256(off + B * H * P * N * 4);
+    w.total = off;
+    return w;
+}
+
+// x scale of channel p of head h (per-tensor, or looked up from the cumulative group ranges,
+// quamba/triton/quant_chunk_state.py:202-214)
+__device__ __forceinline__ void group_of(const QaSsdParams& p, int h, int& g, int& hg) {
+    const int hpg = p.nheads / p.ngroups;
+    g = h / hpg;
+    hg = 0;
+    if (p.nhead_groups > 0) {
+        for (int j = 0; j < p.nhead_groups; ++j) hg += (h % hpg) >= p.x_head_group_range[g * p.nhead_groups + j] ? 1 : 0;
+        hg = min(hg, p.nhead_groups - 1);
+    }
+}
+__device__ __forceinline__ int dim_group_of(const QaSsdParams& p, int g, int hg, int ch) {
+    const int32_t* dr = p.x_dim_group_range + (g * p.nhead_groups + hg) * p.ndim_groups;
+    int dg = 0;
+    for (int j = 0; j < p.ndim_groups; ++j) dg += ch >= dr[j] ? 1 : 0;
+    return min(dg, p.ndim_groups - 1);
+}
+__device__ __forceinline__ float x_scale_of(const QaSsdParams& p, int g, int hg, int ch) {
+    if (p.nhead_groups == 0) return p.x_scale[0];
+    return p.x_scale[(g * p.nhead_groups + hg) * p.ndim_groups + dim_group_of(p, g, hg, ch)];
+}
+
+// ---------------------------------------------------------------------------------------------
+// Stage 1 (quamba/triton/quant_chunk_cumsum.py:56-70).  One thread per (batch, chunk, head), heads
+// fastest so the dt reads of a step are contiguous.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void ssd_cumsum_kernel(QaSsdParams p, float* dt_out, float* dA_out, int nc) {
+    const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (idx >= static_cast<int64_t>(p.batch) * nc * p.nheads) return;
+    const int h = static_cast<int>(idx % p.nheads);
+    const int c = static_cast<int>((idx / p.nheads) % nc);
+    const int b = static_cast<int>(idx / (static_cast<int64_t>(p.nheads) * nc));
+    const int Q = p.chunk_size;
+    const float A = -expf(*p.A_log_scale * static_cast<float>(p.A_log[h]));
+    const float s_dt = p.dt_is_fp32 ? 0.0f : *p.dt_scale;
+    const float bias = (!p.dt_is_fp32 && p.dt_bias) ? __half2float(static_cast<const __half*>(p.dt_bias)[h]) : 0.0f;
+    float* dt_row = dt_out + ((static_cast<int64_t>(b) * p.nheads + h) * nc + c) * Q;
+    float* dA_row = dA_out + ((static_cast<int64_t>(b) * p.nheads + h) * nc + c) * Q;
+    float run = 0.0f;
+    for (int k = 0; k < Q; ++k) {
+        const int t = c * Q + k;
+        float dtv = 0.0f;
+        if (t < p.seqlen) {
+            const int64_t di = (static_cast<int64_t>(b) * p.seqlen + t) * p.nheads + h;
+            if (p.dt_is_fp32) {
+                dtv = static_cast<const float*>(p.dt)[di];
+            } else {
+                dtv = s_dt * static_cast<float>(static_cast<const int8_t*>(p.dt)[di]) + bias;
+                if (p.dt_softplus) dtv = dtv <= 20.0f ? log1pf(expf(dtv)) : dtv;
+                dtv = fminf(fmaxf(dtv, p.dt_min), p.dt_max);
+            }
+        }
+        run += dtv * A;
+        dt_row[k] = dtv;
+        dA_row[k] = run;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Stage 4 (quamba/triton/quant_bmm_chunk.py:60-66): one wave per 64x64 tile of CB, lower tiles only.
+// Both operands are rows of dstate int8 values, i.e. already MFMA operands.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(64) void ssd_cb_kernel(QaSsdParams p, float* cb_out, int nc) {
+    const int Q = p.chunk_size, N = p.dstate, G = p.ngroups;
+    const int nt = Q / 64;
+    // blockIdx.x enumerates lower-triangular tile pairs (mt >= kt)
+    int mt = 0, rem = blockIdx.x;
+    while (rem > mt) { rem -= mt + 1; ++mt; }
+    const int kt = rem;
+    if (mt >= nt) return;
+    const int bcg = blockIdx.y;
+    const int g = bcg % G, c = (bcg / G) % nc, b = bcg / (G * nc);
+    const int lane = threadIdx.x, frow = lane & 31, fhalf = lane >> 5;
+    const int t0 = c * Q;
+    const int lim = min(Q, p.seqlen - t0);
+    const float scale = (p.nhead_groups > 0 ? p.C_scale[g] : p.C_scale[0]) * (p.nhead_groups > 0 ? p.B_scale[g] : p.B_scale[0]);
+
+    v16i acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+    for (int ks = 0; ks < N / 32; ++ks) {
+        v4i fc[2], fb[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int m = mt * 64 + i * 32 + frow, k = kt * 64 + i * 32 + frow;
+            fc[i] = m < lim ? *reinterpret_cast<const v4i*>(p.C + ((static_cast<int64_t>(b) * p.seqlen + t0 + m) * G + g) * N + ks * 32 + fhalf * 16)
+                            : v4i{0, 0, 0, 0};
+            fb[i] = k < lim ? *reinterpret_cast<const v4i*>(p.B + ((static_cast<int64_t>(b) * p.seqlen + t0 + k) * G + g) * N + ks * 32 + fhalf * 16)
+                            : v4i{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fc[i], fb[j], acc[i][j], 0, 0, 0);
+    }
+    // acc[i][j]: lane holds column k = kt*64 + j*32 + (lane & 31), register r row m = mt*64 + i*32 + 8*(r/4) + 4*(lane/32) + r%4
+    float* tile = cb_out + ((static_cast<int64_t>(b) * nc + c) * G + g) * Q * Q;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = mt * 64 + i * 32 + 8 * (r / 4) + 4 * fhalf + (r % 4);
+                const int k = kt * 64 + j * 32 + frow;
+                tile[static_cast<int64_t>(m) * Q + k] = scale * static_cast<float>(acc[i][j][r]);
+            }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Transposing stage: dst[col][k] (fp16, `pitch` halves per row) <- src rows k (int8, `row_stride`
+// bytes apart, NC columns), k in [0, KC).  value = f16((col_scale[col] * q) * k_scale[k]) when
+// K_SCALE, else f16(col_scale[col] * q).  Rows k >= k_valid read as zero.
+// ---------------------------------------------------------------------------------------------
+template <int NC, bool K_SCALE>
+__device__ __forceinline__ void stage_transposed(_Float16* dst, int pitch, const int8_t* src, int64_t row_stride,
+                                                 int KC, int k_valid, const float* col_scale, const float* k_scale,
+                                                 int tid, int nthreads) {
+    constexpr int CB = NC / 4;
+    for (int id = tid; id < (KC / 4) * CB; id += nthreads) {
+        const int kb = id / CB, cb = id % CB;
+        uint32_t w[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int k = kb * 4 + r;
+            w[r] = k < k_valid ? *reinterpret_cast<const uint32_t*>(src + k * row_stride + cb * 4) : 0u;
+        }
+#pragma unroll
+        for (int cc = 0; cc < 4; ++cc) {
+            const float cs = col_scale[cb * 4 + cc];
+            v4h o;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float v = cs * static_cast<float>(byte_of(w[r], cc));
+                if (K_SCALE) v *= k_scale[kb * 4 + r];
+                o[r] = static_cast<_Float16>(v);
+            }
+            *reinterpret_cast<v4h*>(dst + (cb * 4 + cc) * pitch + kb * 4) = o;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Stage 2 (quamba/triton/quant_chunk_state.py:76-89): one workgroup per (batch, chunk, head).
+// S[p,n] = sum_k XT[p][k] * BT[n][k]; 4 waves, wave w owns p-tile w&1 and n-tiles 2*(w>>1)..+1 (of 32).
+// The chunk is consumed in passes of 128 steps.
+// ---------------------------------------------------------------------------------------------
+template <int N>
+__global__ __launch_bounds__(256) void ssd_chunk_state_kernel(QaSsdParams p, const float* dt_ws, const float* dA_ws,
+                                                              float* states, int nc) {
+    constexpr int KC = 128, PITCH = KC + 8, NT = N / 64;      // NT n-tiles per wave
+    __shared__ __attribute__((aligned(16))) _Float16 s_xt[kP * PITCH];
+    __shared__ __attribute__((aligned(16))) _Float16 s_bt[N * PITCH];
+    __shared__ float s_w[KC];
+    __shared__ float s_xs[kP];
+    __shared__ float s_bs[N];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, frow = lane & 31, fhalf = lane >> 5;
+    const int h = blockIdx.x % p.nheads;
+    const int c = (blockIdx.x / p.nheads) % nc;
+    const int b = blockIdx.x / (p.nheads * nc);
+    const int Q = p.chunk_size, G = p.ngroups, H = p.nheads;
+    int g, hg;
+    group_of(p, h, g, hg);
+    const int t0 = c * Q;
+    const int lim = min(Q, p.seqlen - t0);
+    const float* dt_row = dt_ws + ((static_cast<int64_t>(b) * H + h) * nc + c) * Q;
+    const float* dA_row = dA_ws + ((static_cast<int64_t>(b) * H + h) * nc + c) * Q;
+    const float dA_last = dA_row[Q - 1];
+    if (tid < kP) s_xs[tid] = x_scale_of(p, g, hg, tid);
+    const float sB = p.nhead_groups > 0 ? p.B_scale[g] : p.B_scale[0];
+    for (int i = tid; i < N; i += 256) s_bs[i] = sB;
+
+    const int pt = wave & 1, nt0 = (wave >> 1) * NT;
+    v16f acc[NT];
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[j][r] = 0.0f;
+
+    for (int k0 = 0; k0 < Q; k0 += KC) {
+        const int kc = min(KC, Q - k0);
+        __syncthreads();                       // previous pass fully consumed (and scale tables written)
+        if (tid < KC) s_w[tid] = tid < kc ? fexp(dA_last - dA_row[k0 + tid]) * dt_row[k0 + tid] : 0.0f;
+        __syncthreads();
+        const int valid = max(0, min(kc, lim - k0));
+        stage_transposed<kP, false>(s_xt, PITCH, p.x + ((static_cast<int64_t>(b) * p.seqlen + t0 + k0) * H + h) * kP,
+                                    static_cast<int64_t>(H) * kP, KC, valid, s_xs, nullptr, tid, 256);
+        stage_transposed<N, true>(s_bt, PITCH, p.B + ((static_cast<int64_t>(b) * p.seqlen + t0 + k0) * G + g) * N,
+                                  static_cast<int64_t>(G) * N, KC, valid, s_bs, s_w, tid, 256);
+        __syncthreads();
+        for (int ks = 0; ks < KC / 16; ++ks) {
+            const v8h fx = *reinterpret_cast<const v8h*>(s_xt + (pt * 32 + frow) * PITCH + ks * 16 + fhalf * 8);
+#pragma unroll
+            for (int j = 0; j < NT; ++j) {
+                const v8h fb = *reinterpret_cast<const v8h*>(s_bt + ((nt0 + j) * 32 + frow) * PITCH + ks * 16 + fhalf * 8);
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fx, fb, acc[j], 0, 0, 0);
+            }
+        }
+    }
+    // acc[j]: lane holds column n = (nt0+j)*32 + (lane & 31); register r row p = pt*32 + 8*(r/4) + 4*(lane/32) + r%4
+    float* out = states + ((static_cast<int64_t>(b) * nc + c) * H + h) * kP * N;
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int pp = pt * 32 + 8 * (r / 4) + 4 * fhalf + (r % 4);
+            out[pp * N + (nt0 + j) * 32 + frow] = acc[j][r];
+        }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Stages 3 and 6 (quamba/triton/quant_state_passing.py:60-83, quant_ssm_states.py:43,119): one
+// thread per state element, sequential over chunks.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void ssd_state_passing_kernel(QaSsdParams p, const float* dA_ws, const float* states,
+                                                                __half* prev, float* final_ws, int nc) {
+    const int N = p.dstate, H = p.nheads, Q = p.chunk_size;
+    const int64_t per_head = static_cast<int64_t>(kP) * N;
+    const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (idx >= static_cast<int64_t>(p.batch) * H * per_head) return;
+    const int e = static_cast<int>(idx % per_head);
+    const int h = static_cast<int>((idx / per_head) % H);
+    const int b = static_cast<int>(idx / (per_head * H));
+    float s = 0.0f;
+    for (int c = 0; c < nc; ++c) {
+        const int64_t off = ((static_cast<int64_t>(b) * nc + c) * H + h) * per_head + e;
+        prev[off] = __float2half(s);
+        const float dA_last = dA_ws[((static_cast<int64_t>(b) * H + h) * nc + c) * Q + Q - 1];
+        s = expf(dA_last) * s + states[off];
+    }
+    const int64_t fo = (static_cast<int64_t>(b) * H + h) * per_head + e;
+    if (final_ws) final_ws[fo] = s;
+    if (p.final_states) {
+        if (p.final_state_is_fp32) {
+            static_cast<float*>(p.final_states)[fo] = s;
+        } else {
+            const int pp = e / N, n = e % N;
+            float sc, K;
+            if (p.nhead_groups > 0) {
+                int g, hg;
+                group_of(p, h, g, hg);
+                const int dg = dim_group_of(p, g, hg, pp);
+                sc = p.state_scale[((g * p.nhead_groups + hg) * p.ndim_groups + dg) * N + n];
+                K = 1e6f;
+            } else {
+                sc = p.state_scale[0];
+                K = 1e2f;
+            }
+            const float s16 = __half2float(__float2half(s));      // the reference hands fp16 states to the quantiser
+            static_cast<int8_t*>(p.final_states)[fo] = sat8_rne((s16 * K) / (sc * K));
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Stage 5 (quamba/triton/quant_chunk_scan.py:96-171): one workgroup per (batch, chunk, head);
+// each wave owns whole 32-row m-tiles (paired small/large so the causal work balances).
+// ---------------------------------------------------------------------------------------------
+template <int N>
+__global__ __launch_bounds__(256) void ssd_chunk_scan_kernel(QaSsdParams p, const float* dt_ws, const float* dA_ws,
+                                                             const float* cb_ws, const __half* prev, int nc) {
+    constexpr int QMAX = 256, PITCH = QMAX + 8;
+    __shared__ __attribute__((aligned(16))) _Float16 s_xt[kP * PITCH];
+    __shared__ __attribute__((aligned(16))) float s_dt[QMAX];
+    __shared__ __attribute__((aligned(16))) float s_dA[QMAX];
+    __shared__ float s_xs[kP];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, frow = lane & 31, fhalf = lane >> 5;
+    const int h = blockIdx.x % p.nheads;
+    const int c = (blockIdx.x / p.nheads) % nc;
+    const int b = blockIdx.x / (p.nheads * nc);
+    const int Q = p.chunk_size, G = p.ngroups, H = p.nheads;
+    int g, hg;
+    group_of(p, h, g, hg);
+    const int t0 = c * Q;
+    const int lim = min(Q, p.seqlen - t0);
+    const int64_t row_base = (static_cast<int64_t>(b) * H + h) * nc + c;
+    for (int i = tid; i < Q; i += 256) {
+        s_dt[i] = dt_ws[row_base * Q + i];
+        s_dA[i] = dA_ws[row_base * Q + i];
+    }
+    if (tid < kP) s_xs[tid] = x_scale_of(p, g, hg, tid);
+    __syncthreads();
+    stage_transposed<kP, false>(s_xt, PITCH, p.x + ((static_cast<int64_t>(b) * p.seqlen + t0) * H + h) * kP,
+                                static_cast<int64_t>(H) * kP, Q, lim, s_xs, nullptr, tid, 256);
+    __syncthreads();
+
+    const float sC = p.nhead_groups > 0 ? p.C_scale[g] : p.C_scale[0];
+    const float* cb = cb_ws + ((static_cast<int64_t>(b) * nc + c) * G + g) * Q * Q;
+    const __half* pst = prev + ((static_cast<int64_t>(b) * nc + c) * H + h) * kP * N;
+    const float D_scale = p.D ? *p.D_scale : 0.0f;
+    const float z_scale = p.z ? *p.z_scale : 0.0f;
+    const int nmt = Q / 32;
+    const int per_wave = max(1, nmt / 4);
+
+    for (int s = 0; s < per_wave; ++s) {
+        // tile order 0, nmt-1, 1, nmt-2, ...: wave w takes entries w*per_wave + s
+        const int entry = wave * per_wave + s;
+        if (entry >= nmt) break;
+        const int mt = (entry & 1) ? nmt - 1 - (entry >> 1) : (entry >> 1);
+        const int m_lane = mt * 32 + frow;                 // row of this lane's A operands
+        v16f acc[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[j][r] = 0.0f;
+
+        // term 1: C^ (rows m, dstate contiguous) x entering state (rows p, dstate contiguous)
+        const int8_t* c_row = p.C + ((static_cast<int64_t>(b) * p.seqlen + t0 + m_lane) * G + g) * N;
+        for (int ks = 0; ks < N / 16; ++ks) {
+            v8h fc;
+            uint2 raw = make_uint2(0u, 0u);
+            if (m_lane < lim) raw = *reinterpret_cast<const uint2*>(c_row + ks * 16 + fhalf * 8);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) fc[e] = static_cast<_Float16>(sC * static_cast<float>(byte_of(e < 4 ? raw.x : raw.y, e & 3)));
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const v8h fs = *reinterpret_cast<const v8h*>(pst + (j * 32 + frow) * N + ks * 16 + fhalf * 8);
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fc, fs, acc[j], 0, 0, 0);
+            }
+        }
+        // scale rows by exp(dA_m): register r holds row m = mt*32 + 8*(r/4) + 4*(lane/32) + r%4
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const float sm = fexp(s_dA[mt * 32 + 8 * (r / 4) + 4 * fhalf + (r % 4)]);
+            acc[0][r] *= sm;
+            acc[1][r] *= sm;
+        }
+        // term 2: decayed causal CB (rows m, k contiguous) x XT (rows p, k contiguous)
+        const float dA_m = s_dA[m_lane];
+        const float* cb_row = cb + static_cast<int64_t>(m_lane) * Q;
+        for (int ks = 0; ks < 2 * (mt + 1); ++ks) {
+            const int k0 = ks * 16 + fhalf * 8;
+            const float4 c0 = *reinterpret_cast<const float4*>(cb_row + k0);
+            const float4 c1 = *reinterpret_cast<const float4*>(cb_row + k0 + 4);
+            const float cbv[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+            v8h fl;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int k = k0 + e;
+                const float wv = (cbv[e] * fexp(dA_m - s_dA[k])) * s_dt[k];
+                fl[e] = static_cast<_Float16>(k <= m_lane ? wv : 0.0f);
+            }
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const v8h fx = *reinterpret_cast<const v8h*>(s_xt + (j * 32 + frow) * PITCH + k0);
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fl, fx, acc[j], 0, 0, 0);
+            }
+        }
+        // epilogue: lane holds column p = j*32 + (lane & 31)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int pp = j * 32 + frow;
+            const float Dv = p.D ? D_scale * static_cast<float>(p.D[p.D_has_hdim ? h * kP + pp : h]) : 0.0f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = mt * 32 + 8 * (r / 4) + 4 * fhalf + (r % 4);
+                if (m >= lim) continue;
+                const int64_t oi = ((static_cast<int64_t>(b) * p.seqlen + t0 + m) * H + h) * kP + pp;
+                float y = acc[j][r];
+                if (p.D) y += (s_xs[pp] * static_cast<float>(p.x[oi])) * Dv;
+                if (p.z) {
+                    const float zv = z_scale * static_cast<float>(p.z[oi]);
+                    y *= zv * (1.0f / (1.0f + fexp(-zv)));
+                }
+                static_cast<__half*>(p.out)[oi] = __float2half(y);
+            }
+        }
+    }
+}
+
+int validate(const QaSsdParams* p) {
+    if (!p || !p->x || !p->dt || !p->A_log || !p->B || !p->C || !p->out) return QA_ERR_NULL;
+    if (!p->x_scale || !p->A_log_scale || !p->B_scale || !p->C_scale) return QA_ERR_NULL;
+    if (!p->dt_is_fp32 && !p->dt_scale) return QA_ERR_NULL;
+    if ((p->D && !p->D_scale) || (p->z && !p->z_scale)) return QA_ERR_NULL;
+    if (p->final_states && !p->final_state_is_fp32 && !p->state_scale) return QA_ERR_NULL;
+    if (p->nhead_groups > 0 && (!p->x_head_group_range || !p->x_dim_group_range || p->ndim_groups < 1)) return QA_ERR_NULL;
+    if (p->batch < 0 || p->seqlen < 0 || p->nheads < 1 || p->ngroups < 1 || p->nheads % p->ngroups != 0) return QA_ERR_SHAPE;
+    if (p->headdim != kP) return QA_ERR_UNSUPPORTED;
+    if (p->dstate != 64 && p->dstate != 128) return QA_ERR_UNSUPPORTED;
+    if (p->chunk_size != 64 && p->chunk_size != 128 && p->chunk_size != 256) return QA_ERR_UNSUPPORTED;
+    if (!aligned16(p->x) || !aligned16(p->B) || !aligned16(p->C)) return QA_ERR_STRIDE;
+    return QA_OK;
+}
+
+}  // namespace
+}  // namespace qa
+
+extern "C" int64_t qa_ssd_workspace_bytes(const QaSsdParams* p) {
+    if (qa::validate(p) != QA_OK) return 0;
+    return qa::ws_layout(*p).total;
+}
+
+extern "C" int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream_) {
+    using namespace qa;
+    const int st = validate(p);
+    if (st != QA_OK) return st;
+    if (p->batch == 0 || p->seqlen == 0) return QA_OK;
+    const Ws ws = ws_layout(*p);
+    if (!p->workspace) return QA_ERR_NULL;
+    if (p->workspace_bytes < ws.total || (reinterpret_cast<uintptr_t>(p->workspace) & 255u)) return QA_ERR_STRIDE;
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    uint8_t* base = static_cast<uint8_t*>(p->workspace);
+    float* dt_ws = reinterpret_cast<float*>(base + ws.dt);
+    float* dA_ws = reinterpret_cast<float*>(base + ws.dA);
+    float* cb_ws = reinterpret_cast<float*>(base + ws.cb);
+    float* states = reinterpret_cast<float*>(base + ws.states);
+    __half* prev = reinterpret_cast<__half*>(base + ws.prev);
+    float* final_ws = reinterpret_cast<float*>(base + ws.final_f32);
+    const int nc = (p->seqlen + p->chunk_size - 1) / p->chunk_size;
+    const int64_t bch = static_cast<int64_t>(p->batch) * nc * p->nheads;
+    if (bch > 0x7fffffffLL || static_cast<int64_t>(p->batch) * nc * p->ngroups > 65535) return QA_ERR_SHAPE;
+
+    hipLaunchKernelGGL(ssd_cumsum_kernel, dim3(static_cast<unsigned>((bch + 255) / 256)), dim3(256), 0, stream, *p, dt_ws,
+                       dA_ws, nc);
+    const int nt = p->chunk_size / 64;
+    hipLaunchKernelGGL(ssd_cb_kernel, dim3(nt * (nt + 1) / 2, p->batch * nc * p->ngroups), dim3(64), 0, stream, *p, cb_ws, nc);
+    if (p->dstate == 128) {
+        hipLaunchKernelGGL(ssd_chunk_state_kernel<128>, dim3(static_cast<unsigned>(bch)), dim3(256), 0, stream, *p, dt_ws, dA_ws,
+                           states, nc);
+    } else {
+        hipLaunchKernelGGL(ssd_chunk_state_kernel<64>, dim3(static_cast<unsigned>(bch)), dim3(256), 0, stream, *p, dt_ws, dA_ws,
+                           states, nc);
+    }
+    const int64_t elems = static_cast<int64_t>(p->batch) * p->nheads * kP * p->dstate;
+    hipLaunchKernelGGL(ssd_state_passing_kernel, dim3(static_cast<unsigned>((elems + 255) / 256)), dim3(256), 0, stream, *p,
+                       dA_ws, states, prev, final_ws, nc);
+    if (p->dstate == 128) {
+        hipLaunchKernelGGL(ssd_chunk_scan_kernel<128>, dim3(static_cast<unsigned>(bch)), dim3(256), 0, stream, *p, dt_ws, dA_ws,
+                           cb_ws, prev, nc);
+    } else {
+        hipLaunchKernelGGL(ssd_chunk_scan_kernel<64>, dim3(static_cast<unsigned>(bch)), dim3(256), 0, stream, *p, dt_ws, dA_ws,
+                           cb_ws, prev, nc);
+    }
+    return check_launch();
+}

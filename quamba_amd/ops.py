@@ -387,3 +387,95 @@ def w4a8o16_gemm(a, b_q_weight, s_tok, s_ch, s_group, workspace, m, n, k, output
 def w4a8o8_gemm(a, b_q_weight, s_tok, s_ch, s_group, workspace, m, n, k, output_transpose=False):
     """int8 variant: round-half-even, saturating."""
     return _w4a8_gemm(a, b_q_weight, s_tok, s_ch, s_group, m, n, k, output_transpose, torch.int8)
+
+
+# ----------------------------------------------------------------------------------------------
+# Mamba2 SSD chunk scan
+# ----------------------------------------------------------------------------------------------
+def ssd_chunk_scan_combined_fwd(q_x, x_scale, q_dt, dt_scale, q_A_log, A_log_scale, q_B, B_scale, q_C, C_scale,
+                                ssm_state_scale, chunk_size, q_D=None, D_scale=None, q_z=None, z_scale=None,
+                                dt_bias=None, initial_states=None, seq_idx=None, cu_seqlens=None, dt_softplus=False,
+                                dt_limit=(0.0, float("inf")), x_head_group_range=None, x_dim_group_range=None,
+                                final_state_dtype=torch.int8, return_workspace=False):
+    """Quantized SSD forward; interface of _quant_mamba_chunk_scan_combined_fwd and, with the group
+    ranges, of _quamba2_mamba_chunk_scan_combined_fwd (quamba/triton/quant_ssd_combined.py:11-166).
+
+    q_x int8 (batch, seqlen, nheads, headdim); q_dt int8 (batch, seqlen, nheads), or fp32 holding the
+    already processed step sizes; q_A_log int8 (nheads); q_B, q_C int8 (batch, seqlen, ngroups,
+    dstate); q_D int8 (nheads) or (nheads, headdim); dt_bias fp16 (nheads).
+    Returns (out fp16 like q_x, final_states (batch, nheads, headdim, dstate) int8 or fp32).
+    """
+    if initial_states is not None:
+        raise NotImplementedError("initial_states is not supported")
+    if seq_idx is not None:
+        raise NotImplementedError("seq_idx is not supported")
+    if cu_seqlens is not None:
+        raise NotImplementedError("Only supports `cu_seqlens=None`")
+    _require(q_x.dtype == torch.int8 and q_x.is_cuda and q_x.dim() == 4, "q_x must be int8 (batch, seqlen, nheads, headdim) on the GPU")
+    batch, seqlen, nheads, headdim = q_x.shape
+    _require(q_B.dtype == torch.int8 and q_B.dim() == 4 and q_B.shape[:2] == (batch, seqlen), "q_B must be int8 (batch, seqlen, ngroups, dstate)")
+    ngroups, dstate = q_B.shape[2], q_B.shape[3]
+    _require(tuple(q_C.shape) == tuple(q_B.shape) and q_C.dtype == torch.int8, "q_C must match q_B")
+    _require(nheads % ngroups == 0, "nheads must be divisible by ngroups")
+    _require(tuple(q_dt.shape) == (batch, seqlen, nheads) and q_dt.dtype in (torch.int8, torch.float32),
+             "q_dt must be int8 or fp32 (batch, seqlen, nheads)")
+    _require(tuple(q_A_log.shape) == (nheads,) and q_A_log.dtype == torch.int8, "q_A_log must be int8 (nheads,)")
+    dev = q_x.device
+    keep = []
+
+    def f32(t):
+        t = torch.as_tensor(t, device=dev).to(torch.float32).contiguous()
+        keep.append(t)
+        return ptr(t)
+
+    q_x, q_B, q_C, q_dt = q_x.contiguous(), q_B.contiguous(), q_C.contiguous(), q_dt.contiguous()
+    p = _lib.QaSsdParams()
+    p.batch, p.seqlen, p.nheads, p.headdim, p.dstate, p.ngroups = batch, seqlen, nheads, headdim, dstate, ngroups
+    p.chunk_size = chunk_size
+    p.dt_softplus = int(bool(dt_softplus))
+    p.dt_is_fp32 = int(q_dt.dtype == torch.float32)
+    p.dt_min, p.dt_max = float(dt_limit[0]), float(min(dt_limit[1], 3.0e38))
+    p.x, p.dt, p.A_log, p.B, p.C = ptr(q_x), ptr(q_dt), ptr(q_A_log.contiguous()), ptr(q_B), ptr(q_C)
+    p.x_scale, p.A_log_scale, p.B_scale, p.C_scale = f32(x_scale), f32(A_log_scale), f32(B_scale), f32(C_scale)
+    if not p.dt_is_fp32:
+        p.dt_scale = f32(dt_scale)
+        if dt_bias is not None:
+            b16 = dt_bias.to(device=dev, dtype=torch.float16).contiguous()
+            keep.append(b16)
+            p.dt_bias = ptr(b16)
+    if x_head_group_range is not None:
+        _require(x_head_group_range.dtype == torch.int32 and x_dim_group_range.dtype == torch.int32, "group ranges must be int32")
+        hr, dr = x_head_group_range.contiguous(), x_dim_group_range.contiguous()
+        keep += [hr, dr]
+        p.nhead_groups, p.ndim_groups = hr.shape[1], dr.shape[2]
+        p.x_head_group_range, p.x_dim_group_range = ptr(hr), ptr(dr)
+        _require(keep[0].numel() == ngroups * p.nhead_groups * p.ndim_groups, "x_scale has the wrong number of groups")
+    if q_D is not None:
+        _require(tuple(q_D.shape) in ((nheads,), (nheads, headdim)) and q_D.dtype == torch.int8, "q_D must be int8 (nheads[, headdim])")
+        qd = q_D.contiguous()
+        keep.append(qd)
+        p.D, p.D_scale, p.D_has_hdim = ptr(qd), f32(D_scale), int(q_D.dim() == 2)
+    if q_z is not None:
+        _require(tuple(q_z.shape) == tuple(q_x.shape) and q_z.dtype == torch.int8, "q_z must be int8 shaped like q_x")
+        qz = q_z.contiguous()
+        keep.append(qz)
+        p.z, p.z_scale = ptr(qz), f32(z_scale)
+    out = torch.empty(q_x.shape, dtype=torch.float16, device=dev)
+    final = torch.empty((batch, nheads, headdim, dstate), dtype=final_state_dtype, device=dev)
+    p.out, p.final_states = ptr(out), ptr(final)
+    p.final_state_is_fp32 = int(final_state_dtype == torch.float32)
+    if not p.final_state_is_fp32:
+        _require(final_state_dtype == torch.int8, "final_state_dtype must be torch.int8 or torch.float32")
+        p.state_scale = f32(ssm_state_scale)
+    lib = _lib.lib()
+    nbytes = lib.qa_ssd_workspace_bytes(ct.byref(p))
+    if nbytes <= 0:
+        _lib.check(lib.qa_ssd_chunk_scan_fwd(ct.byref(p), None) or -4, "ssd_chunk_scan_fwd")
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    p.workspace, p.workspace_bytes = ptr(ws), nbytes
+    with torch.cuda.device(dev):
+        st = lib.qa_ssd_chunk_scan_fwd(ct.byref(p), _lib.current_stream(dev))
+    _lib.check(st, "ssd_chunk_scan_fwd")
+    if return_workspace:
+        return out, final, ws
+    return out, final
