@@ -44,6 +44,34 @@ __device__ __forceinline__ float silu_gate(float z) {
     return z * fast_rcp(1.0f + fast_exp2(-z * kLog2e));
 }
 
+// Value of `v` in the lane of this quad that holds slice SRC of the same channel (NSPLIT lanes per
+// channel, NSPLIT in {1,2,4}), as a DPP quad permutation that the compiler folds into the consumer.
+template <int NSPLIT, int SRC>
+__device__ __forceinline__ float quad_bcast(float v) {
+    if (NSPLIT == 1) return v;
+    constexpr int ctrl = NSPLIT == 4 ? (SRC | (SRC << 2) | (SRC << 4) | (SRC << 6))
+                                     : (SRC | (SRC << 2) | ((2 + SRC) << 4) | ((2 + SRC) << 6));
+    const int r = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xf, 0xf, false);
+    return __builtin_bit_cast(float, r);
+}
+// Same with a source slice that is a constant only after loop unrolling.
+template <int NSPLIT>
+__device__ __forceinline__ float quad_bcast_sel(float v, int src) {
+    switch (src) {
+        case 0: return quad_bcast<NSPLIT, 0>(v);
+        case 1: return quad_bcast<NSPLIT, 1>(v);
+        case 2: return quad_bcast<NSPLIT, (NSPLIT > 2 ? 2 : 0)>(v);
+        default: return quad_bcast<NSPLIT, (NSPLIT > 2 ? 3 : 1)>(v);
+    }
+}
+// Value of `v` in lane (lane ^ M) of the quad, M in {1,2}.
+template <int M>
+__device__ __forceinline__ float quad_xor(float v) {
+    constexpr int ctrl = M == 1 ? (1 | (0 << 2) | (3 << 4) | (2 << 6)) : (2 | (3 << 2) | (0 << 4) | (1 << 6));
+    const int r = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xf, 0xf, false);
+    return __builtin_bit_cast(float, r);
+}
+
 __device__ __forceinline__ float i8_of(uint32_t word, int j) {
     return static_cast<float>(static_cast<int8_t>((word >> (8 * j)) & 0xffu));
 }
@@ -190,40 +218,101 @@ __global__ __launch_bounds__(64 * WAVES) void sscan_fwd_kernel(QaSScanParams p, 
         const uint32_t* su = &s_in[0][c_local * kRow / 4];
         const uint32_t* sd = &s_in[1][c_local * kRow / 4];
         const uint32_t* sz = &s_in[2][c_local * kRow / 4];
-        for (int tq = 0; tq < T / 4; ++tq) {
-            if (tq * 4 >= nt) break;
+        const int n_quads = (nt + 3) / 4;
+        for (int tq = 0; tq < n_quads; ++tq) {
             const uint32_t u4 = su[tq], d4 = sd[tq];
             const uint32_t z4 = has_z ? sz[tq] : 0u;
+            if constexpr (NSPLIT <= 4) {
+                // The per-step work that does not depend on the state index (dequantise, softplus,
+                // gate) is shared out: of the 4 steps in this dword, the lane with slice s does
+                // steps o*NSPLIT + s and the others read its results through quad DPP.
+                constexpr int OWN = 4 / NSPLIT;
+                float own_u[OWN], own_dt[OWN], own_du[OWN];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int t = tq * 4 + j;
-                if (t >= nt) break;
-                const float u_val = s_u * i8_of(u4, j);
-                float dt = __builtin_fmaf(s_dt, i8_of(d4, j), db);
-                if (p.delta_softplus) dt = softplus20(dt);
-                const float du = dt * u_val;
-                const float4* bf = reinterpret_cast<const float4*>(&s_bc[t][0][slice * NPL]);
-                const float4* cf = reinterpret_cast<const float4*>(&s_bc[t][1][slice * NPL]);
-                float acc = 0.0f;
+                for (int o = 0; o < OWN; ++o) {
+                    const int j = o * NSPLIT + slice;
+                    own_u[o] = s_u * i8_of(u4, j);
+                    float dt = __builtin_fmaf(s_dt, i8_of(d4, j), db);
+                    if (p.delta_softplus) dt = softplus20(dt);
+                    // steps past the end of the sequence must leave the state alone: a = 1, b = 0
+                    dt = tq * 4 + j < nt ? dt : 0.0f;
+                    own_dt[o] = dt;
+                    own_du[o] = dt * own_u[o];
+                }
+                float acc[4];
 #pragma unroll
-                for (int q = 0; q < NPL / 4; ++q) {
-                    const float4 Bv = bf[q];
-                    const float4 Cv = cf[q];
-                    const float Bs[4] = {Bv.x, Bv.y, Bv.z, Bv.w};
-                    const float Cs[4] = {Cv.x, Cv.y, Cv.z, Cv.w};
+                for (int j = 0; j < 4; ++j) {
+                    const int t = tq * 4 + j;
+                    acc[j] = 0.0f;
+                    const float dt = quad_bcast_sel<NSPLIT>(own_dt[j / NSPLIT], j % NSPLIT);
+                    const float du = quad_bcast_sel<NSPLIT>(own_du[j / NSPLIT], j % NSPLIT);
+                    const float4* bf = reinterpret_cast<const float4*>(&s_bc[t][0][slice * NPL]);
+                    const float4* cf = reinterpret_cast<const float4*>(&s_bc[t][1][slice * NPL]);
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const int n = q * 4 + e;
-                        const float a = fast_exp2(dt * A2[n]);
-                        h[n] = __builtin_fmaf(a, h[n], Bs[e] * du);
-                        acc = __builtin_fmaf(h[n], Cs[e], acc);
+                    for (int q = 0; q < NPL / 4; ++q) {
+                        const float4 Bv = bf[q];
+                        const float4 Cv = cf[q];
+                        const float Bs[4] = {Bv.x, Bv.y, Bv.z, Bv.w};
+                        const float Cs[4] = {Cv.x, Cv.y, Cv.z, Cv.w};
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const int n = q * 4 + e;
+                            const float a = fast_exp2(dt * A2[n]);
+                            h[n] = __builtin_fmaf(a, h[n], Bs[e] * du);
+                            acc[j] = __builtin_fmaf(h[n], Cs[e], acc[j]);
+                        }
                     }
                 }
+                // all lanes of a channel get the full sums, then each finishes the steps it owns
 #pragma unroll
-                for (int m = 1; m < NSPLIT; m <<= 1) acc += __shfl_xor(acc, m);
-                float y = __builtin_fmaf(D_f, u_val, acc);
-                if (has_z) y *= silu_gate(s_z * i8_of(z4, j));
-                if (slice == 0) s_out[t][c_local] = __float2half(y);
+                for (int j = 0; j < 4; ++j) {
+                    if (NSPLIT >= 2) acc[j] += quad_xor<1>(acc[j]);
+                    if (NSPLIT >= 4) acc[j] += quad_xor<2>(acc[j]);
+                }
+#pragma unroll
+                for (int o = 0; o < OWN; ++o) {
+                    const int j = o * NSPLIT + slice;
+                    const int t = tq * 4 + j;
+                    float sum;
+                    if (NSPLIT == 1) sum = acc[o];
+                    else if (NSPLIT == 2) sum = slice ? acc[o * 2 + 1] : acc[o * 2];
+                    else sum = slice == 0 ? acc[0] : slice == 1 ? acc[1] : slice == 2 ? acc[2] : acc[3];
+                    float y = __builtin_fmaf(D_f, own_u[o], sum);
+                    if (has_z) y *= silu_gate(s_z * i8_of(z4, j));
+                    if (t < nt) s_out[t][c_local] = __float2half(y);
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int t = tq * 4 + j;
+                    if (t >= nt) break;
+                    const float u_val = s_u * i8_of(u4, j);
+                    float dt = __builtin_fmaf(s_dt, i8_of(d4, j), db);
+                    if (p.delta_softplus) dt = softplus20(dt);
+                    const float du = dt * u_val;
+                    const float4* bf = reinterpret_cast<const float4*>(&s_bc[t][0][slice * NPL]);
+                    const float4* cf = reinterpret_cast<const float4*>(&s_bc[t][1][slice * NPL]);
+                    float acc = 0.0f;
+#pragma unroll
+                    for (int q = 0; q < NPL / 4; ++q) {
+                        const float4 Bv = bf[q];
+                        const float4 Cv = cf[q];
+                        const float Bs[4] = {Bv.x, Bv.y, Bv.z, Bv.w};
+                        const float Cs[4] = {Cv.x, Cv.y, Cv.z, Cv.w};
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const int n = q * 4 + e;
+                            const float a = fast_exp2(dt * A2[n]);
+                            h[n] = __builtin_fmaf(a, h[n], Bs[e] * du);
+                            acc = __builtin_fmaf(h[n], Cs[e], acc);
+                        }
+                    }
+#pragma unroll
+                    for (int m = 1; m < NSPLIT; m <<= 1) acc += __shfl_xor(acc, m);
+                    float y = __builtin_fmaf(D_f, u_val, acc);
+                    if (has_z) y *= silu_gate(s_z * i8_of(z4, j));
+                    if (slice == 0) s_out[t][c_local] = __float2half(y);
+                }
             }
         }
         __syncthreads();   // s_out complete; everyone is done reading the staged tile
@@ -413,10 +502,11 @@ extern "C" int qa_sscan_fwd(const QaSScanParams* p, void* stream_) {
     if (N <= 16) {
         int nsplit = 0, waves = 0;
         if (!sscan_variant_from_env(&nsplit, &waves)) {
-            // enough waves to give every SIMD of the chip (1024) a few, else split the states
-            const int64_t rows = static_cast<int64_t>(p->batch) * p->dim;
-            nsplit = rows >= 4 * 65536 ? 1 : rows >= 2 * 65536 ? 2 : 4;
-            waves = 1;
+            // The kernel is bound by vector-ALU issue, so the mapping that wastes the fewest issue slots
+            // wins: four lanes per channel (the per-step work is shared out over the quad) and, when
+            // the channel count allows, four waves per workgroup sharing one staged B/C tile.
+            nsplit = 4;
+            waves = p->dim % 64 == 0 ? 4 : (p->dim % 32 == 0 ? 2 : 1);
         }
         if (nsplit == 1 && waves == 1) return launch_fwd<16, 1, 64, 1>(*p, stream, vec_in, vec_bc, vec_out);
         if (nsplit == 2 && waves == 1) return launch_fwd<8, 2, 64, 1>(*p, stream, vec_in, vec_bc, vec_out);
