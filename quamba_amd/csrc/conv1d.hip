@@ -23,6 +23,25 @@ __device__ __forceinline__ int8_t conv_epilogue(float v, float s_out, int silu) 
     return sat8_half_away(v / s_out);
 }
 
+// Requantised output by the cheap route (hardware exp2 / rcp, multiply by 1/s_out, round to nearest)
+// whenever that provably equals the exact route, else by the exact route.  The cheap value y differs
+// from the exactly-evaluated one by less than 2e-4 for |y| < 129 (a few ulp of relative error), so if
+// y is further than 2e-3 from every half-integer both round to the same integer; values beyond
+// +-129 saturate either way.  Only lanes inside that margin (about 0.4 %) take the exact route.
+__device__ __forceinline__ int conv_quant(float v, float s_out, float inv_s_out, int silu) {
+    float y = v;
+    if (silu) {
+        const float e = __builtin_amdgcn_exp2f(v * -1.44269504088896341f);
+        y = v * __builtin_amdgcn_rcpf(1.0f + e);
+    }
+    y *= inv_s_out;
+    const float yr = __builtin_rintf(y);
+    const float d = __builtin_fabsf(y - yr);
+    int q = static_cast<int>(__builtin_amdgcn_fmed3f(yr, -128.0f, 127.0f));
+    if (!(d <= 0.498f) && !(__builtin_fabsf(y) >= 129.0f)) q = conv_epilogue(v, s_out, silu);
+    return q;
+}
+
 // packed taps for sdot4: byte j of the window holds x[t-3+j]; tap for x[t-(k-1-w)] is W[w],
 // so byte j pairs with W[j-(4-k)] (zero for j < 4-k).
 __device__ __forceinline__ uint32_t pack_taps(const int8_t* w, int64_t wstride, int width) {
@@ -55,6 +74,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_fwd_rows_kernel(QaConvParam
     const uint32_t taps = pack_taps(p.weight + c * p.weight_c_stride, p.weight_width_stride, p.width);
     const float s_wx = p.scale_w * p.scale_x;
     const float bias_f = p.bias ? static_cast<float>(p.bias[c]) * p.scale_b : 0.0f;
+    const float inv_s_out = 1.0f / p.scale_out;
 
     const int t0 = seg * 16;
     const int remaining = p.seqlen - t0;
@@ -79,8 +99,8 @@ __global__ __launch_bounds__(kConvThreads) void conv_fwd_rows_kernel(QaConvParam
             const uint32_t win = j == 3 ? w[q + 1] : __builtin_amdgcn_alignbyte(w[q + 1], w[q], j + 1);
             const float acc = static_cast<float>(dot4(win, taps));
             const float v = __builtin_fmaf(s_wx, acc, bias_f);
-            const int8_t r = conv_epilogue(v, p.scale_out, p.silu_activation);
-            packed |= static_cast<uint32_t>(static_cast<uint8_t>(r)) << (8 * j);
+            const int r = conv_quant(v, p.scale_out, inv_s_out, p.silu_activation);
+            packed |= static_cast<uint32_t>(r & 0xff) << (8 * j);
         }
         o[q] = packed;
     }

@@ -73,38 +73,52 @@ __device__ __forceinline__ float x_scale_of(const QaSsdParams& p, int g, int hg,
 }
 
 // ---------------------------------------------------------------------------------------------
-// Stage 1 (quamba/triton/quant_chunk_cumsum.py:56-70).  One thread per (batch, chunk, head), heads
-// fastest so the dt reads of a step are contiguous.
+// Stage 1 (quamba/triton/quant_chunk_cumsum.py:56-70).  One wave per (batch, chunk, head): every
+// lane processes chunk_size/64 consecutive steps, then an inclusive scan across the lanes.
 // ---------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void ssd_cumsum_kernel(QaSsdParams p, float* dt_out, float* dA_out, int nc) {
-    const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    const int lane = threadIdx.x & 63;
+    const int64_t idx = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
     if (idx >= static_cast<int64_t>(p.batch) * nc * p.nheads) return;
     const int h = static_cast<int>(idx % p.nheads);
     const int c = static_cast<int>((idx / p.nheads) % nc);
     const int b = static_cast<int>(idx / (static_cast<int64_t>(p.nheads) * nc));
-    const int Q = p.chunk_size;
+    const int Q = p.chunk_size, E = Q / 64;            // Q in {64, 128, 256}
     const float A = -expf(*p.A_log_scale * static_cast<float>(p.A_log[h]));
     const float s_dt = p.dt_is_fp32 ? 0.0f : *p.dt_scale;
     const float bias = (!p.dt_is_fp32 && p.dt_bias) ? __half2float(static_cast<const __half*>(p.dt_bias)[h]) : 0.0f;
-    float* dt_row = dt_out + ((static_cast<int64_t>(b) * p.nheads + h) * nc + c) * Q;
-    float* dA_row = dA_out + ((static_cast<int64_t>(b) * p.nheads + h) * nc + c) * Q;
-    float run = 0.0f;
-    for (int k = 0; k < Q; ++k) {
-        const int t = c * Q + k;
-        float dtv = 0.0f;
+    float dtv[4], run[4];
+    float local = 0.0f;
+    for (int e = 0; e < E; ++e) {
+        const int t = c * Q + lane * E + e;
+        float v = 0.0f;
         if (t < p.seqlen) {
             const int64_t di = (static_cast<int64_t>(b) * p.seqlen + t) * p.nheads + h;
             if (p.dt_is_fp32) {
-                dtv = static_cast<const float*>(p.dt)[di];
+                v = static_cast<const float*>(p.dt)[di];
             } else {
-                dtv = s_dt * static_cast<float>(static_cast<const int8_t*>(p.dt)[di]) + bias;
-                if (p.dt_softplus) dtv = dtv <= 20.0f ? log1pf(expf(dtv)) : dtv;
-                dtv = fminf(fmaxf(dtv, p.dt_min), p.dt_max);
+                v = s_dt * static_cast<float>(static_cast<const int8_t*>(p.dt)[di]) + bias;
+                if (p.dt_softplus) v = v <= 20.0f ? log1pf(expf(v)) : v;
+                v = fminf(fmaxf(v, p.dt_min), p.dt_max);
             }
         }
-        run += dtv * A;
-        dt_row[k] = dtv;
-        dA_row[k] = run;
+        dtv[e] = v;
+        local += v * A;
+        run[e] = local;
+    }
+    // exclusive prefix of the lane totals
+    float incl = local;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const float up = __shfl_up(incl, off);
+        if (lane >= off) incl += up;
+    }
+    const float before = incl - local;
+    float* dt_row = dt_out + ((static_cast<int64_t>(b) * p.nheads + h) * nc + c) * Q + lane * E;
+    float* dA_row = dA_out + ((static_cast<int64_t>(b) * p.nheads + h) * nc + c) * Q + lane * E;
+    for (int e = 0; e < E; ++e) {
+        dt_row[e] = dtv[e];
+        dA_row[e] = before + run[e];
     }
 }
 
@@ -469,7 +483,7 @@ extern "C" int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream_) {
     const int64_t bch = static_cast<int64_t>(p->batch) * nc * p->nheads;
     if (bch > 0x7fffffffLL || static_cast<int64_t>(p->batch) * nc * p->ngroups > 65535) return QA_ERR_SHAPE;
 
-    hipLaunchKernelGGL(ssd_cumsum_kernel, dim3(static_cast<unsigned>((bch + 255) / 256)), dim3(256), 0, stream, *p, dt_ws,
+    hipLaunchKernelGGL(ssd_cumsum_kernel, dim3(static_cast<unsigned>((bch + 3) / 4)), dim3(256), 0, stream, *p, dt_ws,
                        dA_ws, nc);
     const int nt = p->chunk_size / 64;
     hipLaunchKernelGGL(ssd_cb_kernel, dim3(nt * (nt + 1) / 2, p->batch * nc * p->ngroups), dim3(64), 0, stream, *p, cb_ws, nc);
