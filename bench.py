@@ -165,6 +165,87 @@ def cpu_baseline(dev_mixer, seconds_budget=30.0):
                        "conv and scan: C oracle with OpenMP; GEMMs: fp32 torch.matmul on dequantised operands")
 
 
+def _time_fn(fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps
+
+
+def other_workloads(dev, steps, warmup):
+    """Secondary shapes of the same path (not the headline line): Mamba1-2.8b decode step, Mamba2-2.7b SSD
+    chunk scan, Mamba2-8b W4A8 layer.  Returns a list of dicts with per-launch time and roofline fraction."""
+    from quamba_amd import QSScan  # noqa: F401
+    out = []
+    ri = lambda *s: torch.randint(-128, 128, s, dtype=torch.int8, device=dev)
+    sc = lambda v: torch.tensor([v], dtype=torch.float32, device=dev)
+    # decode: batch 64, d_inner 5120, d_state 16, conv state width 3, fp32 recurrent state
+    B, D, N = 64, 5120, 16
+    conv = QCausalConv1D(D, D, 4, groups=D, device=dev)
+    conv.weight, conv.bias = ri(D, 4), ri(D)
+    conv.weight_scale, conv.bias_scale, conv.input_scale, conv.output_scale = 0.004, 0.004, 0.04, 0.03
+    conv_state, ssm_state = ri(B, D, 3), torch.randn(B, D, N, device=dev) * 0.1
+    ring = [(ri(B, D), ri(B, D), ri(B, N), ri(B, N), ri(B, D)) for _ in range(16)]
+    A, Dq, db = ri(D, N), ri(D), ri(D)
+    it = [0]
+    s_x, s_dt, s_A, s_B, s_C, s_D, s_z, s_db = (sc(v) for v in (0.03, 0.02, 0.02, 0.03, 0.03, 0.008, 0.04, 0.01))
+
+    def decode():
+        x, dt, Bv, Cv, z = ring[it[0] % 16]
+        it[0] += 1
+        xc = conv.update(x, conv_state)
+        ops.sscan_update(ssm_state, xc, s_x, dt, s_dt, A, s_A, None, Bv, s_B, Cv, s_C, Dq, s_D, z, s_z, db, s_db, True)
+    ms_eager = _time_fn(decode, 208, 16)
+    # the same 16 steps captured into one HIP graph (how decode loops are run in practice)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(16):
+            decode()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for _ in range(16):
+            decode()
+    ms = _time_fn(graph.replay, 64, 4) / 16
+    nbytes = 3 * B * D + 2 * B * D * 3 + 2 * B * D * N * 4 + 2 * B * D + D * N
+    out.append(dict(workload="Mamba1-2.8b decode step (conv update + state update), batch 64, fp32 state, HIP graph of 16 steps",
+                    us=ms * 1e3, us_eager_python=ms_eager * 1e3, tokens_per_s=B / ms * 1e3, bound="hbm",
+                    achieved_GBs=nbytes / ms / 1e6, frac=nbytes / ms / 1e6 / HBM_PEAK_GBS))
+    # SSD: batch 4, seqlen 4096, 80 heads of 64, d_state 128, 1 group, chunk 256
+    B, L, H, N, G, Q = 4, 4096, 80, 128, 1, 256
+    x, dt, Bm, Cm = ri(B, L, H, 64), ri(B, L, H), ri(B, L, G, N), ri(B, L, G, N)
+    A2, D2 = ri(H), ri(H)
+    bias = torch.zeros(H, dtype=torch.float16, device=dev)
+    ssd = lambda: ops.ssd_chunk_scan_combined_fwd(x, sc(0.03), dt, sc(0.02), A2, sc(0.02), Bm, sc(0.03), Cm, sc(0.03), None, Q,
+                                                  q_D=D2, D_scale=sc(0.008), dt_bias=bias, dt_softplus=True,
+                                                  final_state_dtype=torch.float32)
+    ms = _time_fn(ssd, steps, warmup)
+    nbytes = B * L * H * 64 + 2 * B * L * G * N + B * L * H + 2 * B * L * H * 64 + 4 * B * H * 64 * N
+    out.append(dict(workload="Mamba2-2.7b SSD chunk scan, batch 4 x 4096, 80 heads, d_state 128, chunk 256", us=ms * 1e3,
+                    tokens_per_s=B * L / ms * 1e3, bound="hbm", achieved_GBs=nbytes / ms / 1e6, frac=nbytes / ms / 1e6 / HBM_PEAK_GBS,
+                    dense_TFLOPs=86.9e9 / ms / 1e9))
+    del x, dt, Bm, Cm
+    # W4A8: in_proj 16384 x 4096 -> 18560 (int8 out), out_proj 16384 x 8192 -> 4096 (fp16 out)
+    for (M, Nn, K, o8, name) in ((16384, 18560, 4096, True, "in_proj"), (16384, 4096, 8192, False, "out_proj")):
+        a = ri(M, K)
+        w = torch.randint(0, 256, (Nn, K // 2), dtype=torch.uint8, device=dev)
+        sg = (torch.rand(K // 128, Nn, device=dev) * 10 + 2).half()
+        s_ch, s_tok = torch.full((1, Nn), 1e-4, device=dev), torch.ones(M, device=dev)
+        fn = ops.w4a8o8_gemm if o8 else ops.w4a8o16_gemm
+        ms = _time_fn(lambda: fn(a, w, s_tok, s_ch, sg, None, M, Nn, K, False), steps, warmup)
+        tops = 2.0 * M * Nn * K / ms / 1e9
+        out.append(dict(workload=f"Mamba2-8b W4A8 {name} {M}x{K}->{Nn}", us=ms * 1e3, tokens_per_s=M / ms * 1e3, bound="mfma",
+                        achieved_TOPs=tops, frac=tops / INT8_PEAK_TOPS))
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -173,6 +254,8 @@ def main():
     ap.add_argument("--batch", type=int, default=CFG["batch"])
     ap.add_argument("--seqlen", type=int, default=CFG["seqlen"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--other-workloads", action="store_true",
+                    help="also time the decode step, the Mamba2 SSD scan and the W4A8 GEMMs (extra key in the JSON line)")
     ap.add_argument("--traffic-json", default=os.path.join(ROOT, "profiles", "traffic.json"),
                     help="HBM bytes per launch measured with rocprofv3 --pmc (written by hand from profiles/)")
     args = ap.parse_args()
@@ -239,6 +322,11 @@ def main():
     }
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(mixer)
+    if args.other_workloads:
+        del mixer
+        torch.cuda.empty_cache()
+        line["other_workloads"] = [{k: (round(v, 4) if isinstance(v, float) else v) for k, v in w.items()}
+                                   for w in other_workloads(dev, min(args.steps, 20), args.warmup)]
     print(json.dumps(line))
 
 

@@ -242,9 +242,10 @@ def sscan_update(state, q_x, x_scale, q_dt, dt_scale, q_A_log, A_log_scale, ssm_
     keep = []
 
     def f32(t):
-        t = t.to(device=q_x.device, dtype=torch.float32).contiguous()
-        keep.append(t)
-        return ptr(t)
+        if not (t.dtype == torch.float32 and t.device == q_x.device and t.is_contiguous()):
+            t = t.to(device=q_x.device, dtype=torch.float32).contiguous()
+            keep.append(t)
+        return t.data_ptr()
 
     p.x_scale, p.dt_scale, p.A_log_scale = f32(x_scale), f32(dt_scale), f32(A_log_scale)
     p.B_scale, p.C_scale = f32(B_scale), f32(C_scale)
