@@ -363,27 +363,29 @@ int launch_fwd(const QaSScanParams& p, hipStream_t stream, int vec_in, int vec_b
 }
 
 // ---------------------------------------------------------------------------------------------
-// Single-token update.  LPR lanes share one (batch, head, channel) row, four states per lane, so
-// consecutive lanes touch consecutive 16-byte (fp32 state) or 4-byte (int8 state) pieces.
+// Single-token update.  LPR lanes share one (batch, head, channel) row, up to sixteen states per lane
+// in pieces of four, so consecutive lanes touch consecutive 16-byte (fp32 state) or 4-byte (int8
+// state) pieces.
 // Reference: quamba/triton/selective_state_update.py:83-126 and :303-362.
 // ---------------------------------------------------------------------------------------------
-template <int LPR>
+// VEC: the state axis has unit stride in state, A_log, B and C and every row piece of four states is
+// naturally aligned, so a lane moves its four states with one load and one store per operand.
+// A wave's life here is a chain of memory round trips, not arithmetic, so optional operands are read
+// through a stand-in address instead of behind a branch: every load of the row is in flight at once.
+template <int LPR, bool VEC, bool FP32>
 __global__ __launch_bounds__(256) void ssm_update_kernel(QaSsmUpdateParams p) {
-    const int64_t gid = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-    const int64_t row = gid / LPR;
-    const int sub = static_cast<int>(gid % LPR);
-    const int64_t nrows = static_cast<int64_t>(p.batch) * p.nheads * p.dim;
-    const bool row_ok = row < nrows;
-    const int64_t r = row_ok ? row : nrows - 1;
-    const int d = static_cast<int>(r % p.dim);
-    const int hd = static_cast<int>((r / p.dim) % p.nheads);
-    const int b = static_cast<int>(r / (static_cast<int64_t>(p.dim) * p.nheads));
+    // grid: x over the channels of one head, y = head, z = batch (no integer division on the way in)
+    const int gid = blockIdx.x * 256 + threadIdx.x;
+    const int sub = gid % LPR;
+    const bool row_ok = gid / LPR < p.dim;
+    const int d = row_ok ? gid / LPR : p.dim - 1;
+    const int hd = blockIdx.y;
+    const int64_t b = blockIdx.z;
     const int heads_per_group = p.nheads / p.ngroups;
     const int g = hd / heads_per_group;
 
     const bool grouped = p.nhead_groups > 0;
-    float x_scale, B_scale, C_scale;
-    const float* state_scale_row;      // grouped: [dstate] scales of this (g, hg, dg)
+    int sidx = 0;                       // grouped: index of this row's (g, head group, dim group)
     if (grouped) {
         int hg = 0, dg = 0;
         const int hrel = hd % heads_per_group;
@@ -392,62 +394,120 @@ __global__ __launch_bounds__(256) void ssm_update_kernel(QaSsmUpdateParams p) {
         const int32_t* dr = p.x_dim_group_range + (g * p.nhead_groups + hg) * p.ndim_groups;
         for (int j = 0; j < p.ndim_groups; ++j) dg += d >= dr[j] ? 1 : 0;
         dg = min(dg, p.ndim_groups - 1);
-        const int sidx = (g * p.nhead_groups + hg) * p.ndim_groups + dg;
-        x_scale = p.x_scale[sidx];
-        state_scale_row = p.state_is_fp32 ? nullptr : p.state_scale + static_cast<int64_t>(sidx) * p.dstate;
-        B_scale = p.B_scale[g];
-        C_scale = p.C_scale[g];
-    } else {
-        x_scale = *p.x_scale;
-        state_scale_row = nullptr;
-        B_scale = *p.B_scale;
-        C_scale = *p.C_scale;
+        sidx = (g * p.nhead_groups + hg) * p.ndim_groups + dg;
     }
-    const float s_state = (!grouped && !p.state_is_fp32) ? *p.state_scale : 1.0f;
+    const float* standin = p.x_scale;   // always readable, four bytes
+    const float* state_scale_row = (grouped && !FP32) ? p.state_scale + static_cast<int64_t>(sidx) * p.dstate : nullptr;
+    const bool bias_i8 = p.dt_bias && !p.dt_bias_is_fp16;
+    const bool bias_f16 = p.dt_bias && p.dt_bias_is_fp16;
+    const int64_t bias_i = hd * p.dt_bias_head_stride + d * p.dt_bias_dim_stride;
+    const int8_t* x_a = p.x + b * p.x_batch_stride + hd * p.x_head_stride + d * p.x_dim_stride;
+    const int8_t* dt_a = p.dt + b * p.dt_batch_stride + hd * p.dt_head_stride + d * p.dt_dim_stride;
+    const int8_t* z_a = p.z ? p.z + b * p.z_batch_stride + hd * p.z_head_stride + d * p.z_dim_stride : x_a;
+    const int8_t* D_a = p.D ? p.D + hd * p.D_head_stride + d * p.D_dim_stride : x_a;
+    const int8_t* b8_a = bias_i8 ? static_cast<const int8_t*>(p.dt_bias) + bias_i : x_a;
+    const __half* b16_a = bias_f16 ? static_cast<const __half*>(p.dt_bias) + bias_i : reinterpret_cast<const __half*>(standin);
+
+    const float x_scale = p.x_scale[sidx];
+    const float B_scale = p.B_scale[grouped ? g : 0];
+    const float C_scale = p.C_scale[grouped ? g : 0];
+    const float dt_scale = *p.dt_scale;
+    const float A_scale = *p.A_log_scale;
+    const float s_state = *((!grouped && !FP32) ? p.state_scale : standin);
+    const float D_scale = *(p.D ? p.D_scale : standin);
+    const float z_scale = *(p.z ? p.z_scale : standin);
+    const float bias_scale = *(bias_i8 ? p.dt_bias_scale : standin);
+    const float xq = static_cast<float>(*x_a), dtq = static_cast<float>(*dt_a);
+    const float zq = static_cast<float>(*z_a), Dq = static_cast<float>(*D_a);
+    const float b8 = static_cast<float>(*b8_a), b16 = __half2float(*b16_a);
     const float requant_k = grouped ? 1e6f : 1e2f;
 
-    const float xv = x_scale * static_cast<float>(p.x[b * p.x_batch_stride + hd * p.x_head_stride + d * p.x_dim_stride]);
-    float dt = *p.dt_scale * static_cast<float>(p.dt[b * p.dt_batch_stride + hd * p.dt_head_stride + d * p.dt_dim_stride]);
-    if (p.dt_bias) {
-        const int64_t bi = hd * p.dt_bias_head_stride + d * p.dt_bias_dim_stride;
-        dt += p.dt_bias_is_fp16 ? __half2float(static_cast<const __half*>(p.dt_bias)[bi])
-                                : *p.dt_bias_scale * static_cast<float>(static_cast<const int8_t*>(p.dt_bias)[bi]);
-    }
-    if (p.dt_softplus) dt = dt <= 20.0f ? log1pf(expf(dt)) : dt;
-    const float A_scale = *p.A_log_scale;
-
-    float acc = 0.0f;
     const int64_t st_base = b * p.state_batch_stride + hd * p.state_head_stride + d * p.state_dim_stride;
     const int8_t* Bp = p.B + b * p.B_batch_stride + g * p.B_group_stride;
     const int8_t* Cp = p.C + b * p.C_batch_stride + g * p.C_group_stride;
     const int8_t* Ap = p.A_log + hd * p.A_head_stride + d * p.A_dim_stride;
-    for (int n0 = sub * 4; n0 < p.dstate; n0 += LPR * 4) {
+    // A lane owns up to kPieces pieces of four states: piece k of lane `sub` starts at state
+    // (sub + k * LPR) * 4.  All loads first, then the arithmetic, then the stores.
+    constexpr int kPieces = 4;
+    float hv[kPieces][4], sc[kPieces][4];
+    int8_t a8[kPieces][4], b8v[kPieces][4], c8[kPieces][4], s8[kPieces][4];
+#pragma unroll
+    for (int k = 0; k < kPieces; ++k) {
+        const int n0 = (sub + k * LPR) * 4;
+        if (n0 >= p.dstate) continue;
+        if constexpr (VEC) {
+            // dstate is a multiple of four here, so the piece is whole
+            *reinterpret_cast<int32_t*>(a8[k]) = *reinterpret_cast<const int32_t*>(Ap + n0);
+            *reinterpret_cast<int32_t*>(b8v[k]) = *reinterpret_cast<const int32_t*>(Bp + n0);
+            *reinterpret_cast<int32_t*>(c8[k]) = *reinterpret_cast<const int32_t*>(Cp + n0);
+            if constexpr (FP32) {
+                const float4 v = *reinterpret_cast<const float4*>(static_cast<const float*>(p.state) + st_base + n0);
+                hv[k][0] = v.x; hv[k][1] = v.y; hv[k][2] = v.z; hv[k][3] = v.w;
+            } else {
+                *reinterpret_cast<int32_t*>(s8[k]) = *reinterpret_cast<const int32_t*>(static_cast<const int8_t*>(p.state) + st_base + n0);
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) sc[k][e] = state_scale_row ? state_scale_row[n0 + e] : s_state;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int n = min(n0 + e, p.dstate - 1);
+                const int64_t si = st_base + n * p.state_dstate_stride;
+                sc[k][e] = state_scale_row ? state_scale_row[n] : s_state;
+                if constexpr (FP32) hv[k][e] = static_cast<const float*>(p.state)[si];
+                else s8[k][e] = static_cast<const int8_t*>(p.state)[si];
+                a8[k][e] = Ap[n * p.A_dstate_stride];
+                b8v[k][e] = Bp[n * p.B_dstate_stride];
+                c8[k][e] = Cp[n * p.C_dstate_stride];
+            }
+        }
+    }
+    const float xv = x_scale * xq;
+    float dt = dt_scale * dtq;
+    dt += bias_i8 ? bias_scale * b8 : (bias_f16 ? b16 : 0.0f);
+    if (p.dt_softplus) dt = dt <= 20.0f ? log1pf(expf(dt)) : dt;
+    float acc = 0.0f;
+#pragma unroll
+    for (int k = 0; k < kPieces; ++k) {
+        const int n0 = (sub + k * LPR) * 4;
+        if (n0 >= p.dstate) continue;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            const int n = n0 + e;
-            if (n >= p.dstate) break;
-            const int64_t si = st_base + n * p.state_dstate_stride;
-            const float sc = state_scale_row ? state_scale_row[n] : s_state;
-            float hv = p.state_is_fp32 ? static_cast<const float*>(p.state)[si]
-                                       : sc * static_cast<float>(static_cast<const int8_t*>(p.state)[si]);
-            const float A = -expf(A_scale * static_cast<float>(Ap[n * p.A_dstate_stride]));
-            const float dA = expf(A * dt);
-            const float Bv = B_scale * static_cast<float>(Bp[n * p.B_dstate_stride]);
-            const float Cv = C_scale * static_cast<float>(Cp[n * p.C_dstate_stride]);
-            hv = hv * dA + (Bv * dt) * xv;
-            if (row_ok) {
-                if (p.state_is_fp32) static_cast<float*>(p.state)[si] = hv;
-                else static_cast<int8_t*>(p.state)[si] = sat8_rne((hv * requant_k) / (sc * requant_k));
+            if constexpr (!FP32) hv[k][e] = sc[k][e] * static_cast<float>(s8[k][e]);
+            const float A = -__expf(A_scale * static_cast<float>(a8[k][e]));
+            const float dA = __expf(A * dt);
+            const float Bv = B_scale * static_cast<float>(b8v[k][e]);
+            const float Cv = C_scale * static_cast<float>(c8[k][e]);
+            hv[k][e] = hv[k][e] * dA + (Bv * dt) * xv;
+            if (VEC || n0 + e < p.dstate) acc += hv[k][e] * Cv;
+        }
+        if (!row_ok) continue;
+        if constexpr (VEC) {
+            if constexpr (FP32) {
+                *reinterpret_cast<float4*>(static_cast<float*>(p.state) + st_base + n0) =
+                    make_float4(hv[k][0], hv[k][1], hv[k][2], hv[k][3]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) s8[k][e] = sat8_rne((hv[k][e] * requant_k) / (sc[k][e] * requant_k));
+                *reinterpret_cast<int32_t*>(static_cast<int8_t*>(p.state) + st_base + n0) = *reinterpret_cast<const int32_t*>(s8[k]);
             }
-            acc += hv * Cv;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int n = n0 + e;
+                if (n >= p.dstate) break;
+                const int64_t si = st_base + n * p.state_dstate_stride;
+                if constexpr (FP32) static_cast<float*>(p.state)[si] = hv[k][e];
+                else static_cast<int8_t*>(p.state)[si] = sat8_rne((hv[k][e] * requant_k) / (sc[k][e] * requant_k));
+            }
         }
     }
 #pragma unroll
     for (int m = 1; m < LPR; m <<= 1) acc += __shfl_xor(acc, m);
     if (row_ok && sub == 0) {
-        if (p.D) acc += xv * (*p.D_scale * static_cast<float>(p.D[hd * p.D_head_stride + d * p.D_dim_stride]));
+        if (p.D) acc += xv * (D_scale * Dq);
         if (p.z) {
-            const float zv = *p.z_scale * static_cast<float>(p.z[b * p.z_batch_stride + hd * p.z_head_stride + d * p.z_dim_stride]);
+            const float zv = z_scale * zq;
             acc *= zv * (1.0f / (1.0f + expf(-zv)));
         }
         static_cast<__half*>(p.out)[b * p.out_batch_stride + hd * p.out_head_stride + d * p.out_dim_stride] =
@@ -457,10 +517,23 @@ __global__ __launch_bounds__(256) void ssm_update_kernel(QaSsmUpdateParams p) {
 
 template <int LPR>
 int launch_update(const QaSsmUpdateParams& p, hipStream_t stream) {
-    const int64_t threads = static_cast<int64_t>(p.batch) * p.nheads * p.dim * LPR;
-    const int64_t blocks = (threads + 255) / 256;
-    if (blocks > 0x7fffffffLL) return QA_ERR_SHAPE;
-    hipLaunchKernelGGL(ssm_update_kernel<LPR>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, p);
+    const int64_t blocks = (static_cast<int64_t>(p.dim) * LPR + 255) / 256;
+    if (blocks > 0x7fffffffLL / 256 || p.nheads > 65535 || p.batch > 65535) return QA_ERR_SHAPE;
+    const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(p.nheads), static_cast<unsigned>(p.batch));
+    const int64_t st_align = p.state_is_fp32 ? 16 : 4;      // bytes of one lane's four states
+    const int64_t st_el = p.state_is_fp32 ? 4 : 1;
+    auto mult = [](int64_t v, int64_t m) { return v % m == 0; };
+    const bool vec = p.dstate % 4 == 0 && p.state_dstate_stride == 1 && p.A_dstate_stride == 1 &&
+                     p.B_dstate_stride == 1 && p.C_dstate_stride == 1 &&
+                     reinterpret_cast<uintptr_t>(p.state) % st_align == 0 &&
+                     mult(p.state_batch_stride * st_el, st_align) && mult(p.state_head_stride * st_el, st_align) &&
+                     mult(p.state_dim_stride * st_el, st_align) &&
+                     aligned4(p.A_log) && mult(p.A_head_stride, 4) && mult(p.A_dim_stride, 4) &&
+                     aligned4(p.B) && mult(p.B_batch_stride, 4) && mult(p.B_group_stride, 4) &&
+                     aligned4(p.C) && mult(p.C_batch_stride, 4) && mult(p.C_group_stride, 4);
+    auto go = [&](auto kernel) { hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, p); };
+    if (p.state_is_fp32) vec ? go(ssm_update_kernel<LPR, true, true>) : go(ssm_update_kernel<LPR, false, true>);
+    else vec ? go(ssm_update_kernel<LPR, true, false>) : go(ssm_update_kernel<LPR, false, false>);
     return check_launch();
 }
 
@@ -535,11 +608,10 @@ extern "C" int qa_ssm_state_update(const QaSsmUpdateParams* p, void* stream_) {
     if (p->batch == 0 || p->dim == 0) return QA_OK;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const int N = p->dstate;
-    if (N <= 4) return launch_update<1>(*p, stream);
-    if (N <= 8) return launch_update<2>(*p, stream);
-    if (N <= 16) return launch_update<4>(*p, stream);
-    if (N <= 32) return launch_update<8>(*p, stream);
-    if (N <= 64) return launch_update<16>(*p, stream);
-    if (N <= 128) return launch_update<32>(*p, stream);
-    return launch_update<64>(*p, stream);
+    // up to sixteen states per lane: the per-row work (addresses, softplus, gate) is paid once per lane
+    if (N <= 16) return launch_update<1>(*p, stream);
+    if (N <= 32) return launch_update<2>(*p, stream);
+    if (N <= 64) return launch_update<4>(*p, stream);
+    if (N <= 128) return launch_update<8>(*p, stream);
+    return launch_update<16>(*p, stream);
 }
