@@ -256,6 +256,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--other-workloads", action="store_true",
                     help="also time the decode step, the Mamba2 SSD scan and the W4A8 GEMMs (extra key in the JSON line)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run three plain 1 GiB device copies (reference points for hardware-counter runs)")
     ap.add_argument("--traffic-json", default=os.path.join(ROOT, "profiles", "traffic.json"),
                     help="HBM bytes per launch measured with rocprofv3 --pmc (written by hand from profiles/)")
     args = ap.parse_args()
@@ -320,6 +322,13 @@ def main():
         "roofline": roofline,
         "kernels": per_kernel,
     }
+    if args.copy_calibration:
+        src = torch.zeros(1 << 30, dtype=torch.int8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(mixer)
     if args.other_workloads:

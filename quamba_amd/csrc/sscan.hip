@@ -107,6 +107,7 @@ __global__ __launch_bounds__(64 * WAVES) void sscan_fwd_kernel(QaSScanParams p, 
     __shared__ __attribute__((aligned(16))) uint32_t s_in[3][kCh * kRow / 4];
     __shared__ __attribute__((aligned(16))) float s_bc[T][2][kNP];
     __shared__ __attribute__((aligned(16))) __half s_out[T][kOutPitch];
+    __shared__ float s_gate[256];      // SiLU gate per z code (indexed by the raw byte)
 
     const int tid = threadIdx.x;
     const int c_local = tid / NSPLIT;
@@ -207,6 +208,9 @@ __global__ __launch_bounds__(64 * WAVES) void sscan_fwd_kernel(QaSScanParams p, 
 
     const int n_tiles = (L + T - 1) / T;
     issue_loads(0);
+    if (has_z) {
+        for (int i = tid; i < 256; i += kThreads) s_gate[i] = silu_gate(s_z * static_cast<float>(static_cast<int8_t>(i)));
+    }
     stage();
     __syncthreads();
 
@@ -263,22 +267,29 @@ __global__ __launch_bounds__(64 * WAVES) void sscan_fwd_kernel(QaSScanParams p, 
                         }
                     }
                 }
-                // all lanes of a channel get the full sums, then each finishes the steps it owns
+                // each lane needs the full sum of the steps it owns only: a transposing reduction
+                // (keep one half, hand the other half to the neighbour) instead of four full ones
+                float own_sum[OWN];
+                if constexpr (NSPLIT == 4) {
+                    const bool odd = slice & 1, hi = slice & 2;
+                    const float w01 = (odd ? acc[1] : acc[0]) + quad_xor<1>(odd ? acc[0] : acc[1]);
+                    const float w23 = (odd ? acc[3] : acc[2]) + quad_xor<1>(odd ? acc[2] : acc[3]);
+                    own_sum[0] = (hi ? w23 : w01) + quad_xor<2>(hi ? w01 : w23);
+                } else if constexpr (NSPLIT == 2) {
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    if (NSPLIT >= 2) acc[j] += quad_xor<1>(acc[j]);
-                    if (NSPLIT >= 4) acc[j] += quad_xor<2>(acc[j]);
+                    for (int o = 0; o < OWN; ++o) {
+                        own_sum[o] = (slice ? acc[o * 2 + 1] : acc[o * 2]) + quad_xor<1>(slice ? acc[o * 2] : acc[o * 2 + 1]);
+                    }
+                } else {
+#pragma unroll
+                    for (int o = 0; o < OWN; ++o) own_sum[o] = acc[o];
                 }
 #pragma unroll
                 for (int o = 0; o < OWN; ++o) {
                     const int j = o * NSPLIT + slice;
                     const int t = tq * 4 + j;
-                    float sum;
-                    if (NSPLIT == 1) sum = acc[o];
-                    else if (NSPLIT == 2) sum = slice ? acc[o * 2 + 1] : acc[o * 2];
-                    else sum = slice == 0 ? acc[0] : slice == 1 ? acc[1] : slice == 2 ? acc[2] : acc[3];
-                    float y = __builtin_fmaf(D_f, own_u[o], sum);
-                    if (has_z) y *= silu_gate(s_z * i8_of(z4, j));
+                    float y = __builtin_fmaf(D_f, own_u[o], own_sum[o]);
+                    if (has_z) y *= s_gate[(z4 >> (8 * j)) & 0xffu];
                     if (t < nt) s_out[t][c_local] = __float2half(y);
                 }
             } else {
@@ -310,7 +321,7 @@ __global__ __launch_bounds__(64 * WAVES) void sscan_fwd_kernel(QaSScanParams p, 
 #pragma unroll
                     for (int m = 1; m < NSPLIT; m <<= 1) acc += __shfl_xor(acc, m);
                     float y = __builtin_fmaf(D_f, u_val, acc);
-                    if (has_z) y *= silu_gate(s_z * i8_of(z4, j));
+                    if (has_z) y *= s_gate[(z4 >> (8 * j)) & 0xffu];
                     if (slice == 0) s_out[t][c_local] = __float2half(y);
                 }
             }
