@@ -118,6 +118,21 @@ extern "C" int qa_gemm_w8a8(const QaGemmW8A8Params* p, void* stream_) {
     // the single-row rules (host alpha, round-half-away) only ever come with tiny M
     if (p->use_alpha || p->round_mode != QA_ROUND_RNE) return launch_gemm<2, 2, 2, 2, 2, true>(*p, stream);
     const int64_t big_tiles = static_cast<int64_t>((p->m + 255) / 256) * ((p->n + 255) / 256);
-    if (big_tiles >= 192) return launch_gemm<4, 2, 2, 4, 2, false>(*p, stream);     // 256x256 tile, 8 waves
+    if (big_tiles >= 192) {
+        // One workgroup per CU at a time: the launch runs in rounds of `cus` tiles, so a tile count
+        // just above a multiple of the CU count wastes most of a round.  A 256x320 tile (same 8 waves,
+        // 64x160 each) is taken when it needs fewer tile-rounds' worth of arithmetic.
+        int dev = 0, cus = 256;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) {
+            cus = 256;
+        }
+        auto cost = [&](int64_t bm, int64_t bn) {
+            const int64_t tiles = ((p->m + bm - 1) / bm) * ((p->n + bn - 1) / bn);
+            return ((tiles + cus - 1) / cus) * bm * bn;
+        };
+        if (cost(256, 320) < cost(256, 256)) return launch_gemm<2, 5, 4, 2, 2, false>(*p, stream);
+        return launch_gemm<4, 2, 2, 4, 2, false>(*p, stream);                        // 256x256 tile, 8 waves
+    }
     return launch_gemm<2, 2, 2, 2, 2, false>(*p, stream);                            // 128x128 tile, 4 waves
 }

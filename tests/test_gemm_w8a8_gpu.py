@@ -52,6 +52,29 @@ def test_fp16_output_bit_exact(dev, M, N, K):
     np.testing.assert_array_equal(c.cpu().numpy(), f.astype(np.float16))
 
 
+@pytest.mark.parametrize("out_dtype", [torch.int8, torch.float16])
+def test_wide_tile_path_matches_exact_fp32(dev, out_dtype):
+    """16384 x 2560 is the shape for which the 256x320 tile is chosen (two full rounds of workgroups).
+    K = 256 keeps every integer sum below 2^24, so an fp32 matmul is exact and torch applies the same
+    two IEEE multiplications; rounding to int8 is torch's round-half-even."""
+    M, N, K = 16384, 2560, 256
+    g = torch.Generator(device="cpu").manual_seed(5)
+    a = torch.randint(-128, 128, (M, K), dtype=torch.int8, generator=g).to(dev)
+    w = torch.randint(-128, 128, (N, K), dtype=torch.int8, generator=g).to(dev)
+    sa = (torch.rand(M, generator=g) * 0.02 + 0.01).to(dev)
+    sb = (torch.rand(N, generator=g) * 0.02 + 0.01).to(dev)
+    c = torch.empty((M, N), dtype=out_dtype, device=dev)
+    ops.scaled_mm_dq(c, a, w.t(), sa, sb)
+    acc = a.float() @ w.float().t()
+    want = sa[:, None] * (sb[None, :] * acc)
+    if out_dtype == torch.int8:
+        want = torch.clamp(torch.round(want), -128, 127).to(torch.int8)
+        assert want.abs().max().item() > 50
+    else:
+        want = want.half()
+    assert torch.equal(c, want)
+
+
 def test_output_with_row_padding(dev):
     M, N, K = 100, 72, 64
     a, w, sa, sb = _operands(M, N, K, seed=9)
