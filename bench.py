@@ -181,7 +181,7 @@ def _time_fn(fn, steps, warmup):
 def other_workloads(dev, steps, warmup):
     """Secondary shapes of the same path (not the headline line): Mamba1-2.8b decode step, Mamba2-2.7b SSD
     chunk scan, Mamba2-8b W4A8 layer.  Returns a list of dicts with per-launch time and roofline fraction."""
-    from quamba_amd import QSScan  # noqa: F401
+    from quamba_amd import Quamb2Conv1D
     out = []
     ri = lambda *s: torch.randint(-128, 128, s, dtype=torch.int8, device=dev)
     sc = lambda v: torch.tensor([v], dtype=torch.float32, device=dev)
@@ -232,6 +232,25 @@ def other_workloads(dev, steps, warmup):
                     tokens_per_s=B * L / ms * 1e3, bound="hbm", achieved_GBs=nbytes / ms / 1e6, frac=nbytes / ms / 1e6 / HBM_PEAK_GBS,
                     dense_TFLOPs=86.9e9 / ms / 1e9))
     del x, dt, Bm, Cm
+    # Mamba2-8b xBC conv: batch 16 x 1024, x 8192 channels (128 heads of 64), 8 groups of d_state 128, grouped scales
+    B, L, H, N, G = 16, 1024, 128, 128, 8
+    dim = H * 64 + 2 * G * N
+    conv2 = Quamb2Conv1D(H * 64, 64, N, G, 4, 4, dim, dim, 4, groups=dim, device=dev)
+    conv2.weight, conv2.bias = ri(dim, 4), ri(dim)
+    conv2.x_scale = conv2.B_scale = conv2.C_scale = 0.04
+    conv2.wx_scale = conv2.wB_scale = conv2.wC_scale = 0.004
+    conv2.bx_scale = conv2.bB_scale = conv2.bC_scale = 0.004
+    conv2.x_out_scales = torch.rand(G, 4, 4, device=dev) * 0.02 + 0.02
+    conv2.B_out_scales, conv2.C_out_scales = torch.rand(G, device=dev) * 0.02 + 0.02, torch.rand(G, device=dev) * 0.02 + 0.02
+    conv2.x_head_group_range = torch.tensor([[4, 8, 12, 16]] * G, dtype=torch.int32, device=dev)
+    conv2.x_dim_group_range = torch.tensor([[[16, 32, 48, 64]] * 4] * G, dtype=torch.int32, device=dev)
+    xBC = ri(B, L, dim).transpose(1, 2)
+    ms = _time_fn(lambda: conv2(xBC), steps, warmup)
+    nbytes = 2 * B * L * dim + 5 * dim
+    out.append(dict(workload="Mamba2-8b xBC conv, batch 16 x 1024, 10240 channels, grouped output scales", us=ms * 1e3,
+                    tokens_per_s=B * L / ms * 1e3, bound="hbm", achieved_GBs=nbytes / ms / 1e6,
+                    frac=nbytes / ms / 1e6 / HBM_PEAK_GBS))
+    del xBC
     # W4A8: in_proj 16384 x 4096 -> 18560 (int8 out), out_proj 16384 x 8192 -> 4096 (fp16 out)
     for (M, Nn, K, o8, name) in ((16384, 18560, 4096, True, "in_proj"), (16384, 4096, 8192, False, "out_proj")):
         a = ri(M, K)

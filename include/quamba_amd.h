@@ -66,6 +66,53 @@ int qa_causal_conv1d_fwd(const QaConvParams* p, void* stream);
 int qa_causal_conv1d_update(const QaConvParams* p, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Mamba2 xBC conv: one depthwise causal conv1d (+ SiLU) over the concatenated channels
+ * [x (x_dim) | B (n_groups*d_state) | C (n_groups*d_state)], each part with its own input, weight
+ * and bias scales, requantised into three int8 tensors: x with one output scale or one per
+ * (ssd group, head group, dim group) found through cumulative end-index tables, B and C with one
+ * output scale or one per ssd group.
+ * Replaces quamba2_conv1d_cuda.fwd / .update
+ *   (csrc/causal_conv1d/quamba2_conv1d.cpp:109-251, :254-379; kernels
+ *    quamba2_conv1d_fwd_kernel.cuh:57-347, quamba2_conv1d_update_kernel.cuh:28-147).
+ * Forward takes the channel-contiguous layout only, as the reference does: element (b, c, l) of
+ * xBC at b*xBC_batch_stride + l*xBC_l_stride + c; the outputs likewise (x_l_stride etc.).
+ * Update: xBC (batch, dim) with xBC_c_stride; outputs (batch, part) with *_c_stride; conv_state
+ * int8 (batch, dim, conv_state_len), conv_state_len == width or width-1, shifted in place.
+ * ---------------------------------------------------------------------------------------- */
+typedef struct QaConv2Params {
+    int32_t batch, dim, seqlen, width;   /* dim == x_dim + 2*n_groups*d_state, width in [2,4] */
+    int32_t silu_activation;
+    int32_t x_dim, x_headdim, d_state, n_groups;
+    int32_t nhead_groups, ndim_groups;   /* 0, 0: one output scale per part */
+    int32_t conv_state_len;
+    int64_t xBC_batch_stride, xBC_l_stride, xBC_c_stride;   /* fwd: c stride 1; update: l stride unused */
+    int64_t x_batch_stride, x_l_stride, x_c_stride;
+    int64_t B_batch_stride, B_l_stride, B_c_stride;
+    int64_t C_batch_stride, C_l_stride, C_c_stride;
+    int64_t weight_c_stride, weight_width_stride;           /* weight int8 (dim, width) */
+    int64_t conv_state_batch_stride, conv_state_c_stride, conv_state_l_stride;
+    const int8_t* xBC;
+    const int8_t* weight;
+    const int8_t* bias;                  /* int8 (dim) or null */
+    int8_t* x;
+    int8_t* B;
+    int8_t* C;
+    int8_t* conv_state;                  /* update only */
+    const float* x_out_scales;           /* [1] or [n_groups, nhead_groups, ndim_groups] */
+    const float* B_out_scales;           /* [1] or [n_groups] */
+    const float* C_out_scales;
+    const int32_t* x_head_group_range;   /* [n_groups, nhead_groups] cumulative end indices, or null */
+    const int32_t* x_dim_group_range;    /* [n_groups, nhead_groups, ndim_groups], or null */
+    float scale_x, scale_B, scale_C;     /* input scales of the three parts */
+    float scale_wx, scale_wB, scale_wC;  /* weight scales */
+    float scale_bx, scale_bB, scale_bC;  /* bias scales */
+    float reserved0;
+} QaConv2Params;
+
+int qa_quamba2_conv1d_fwd(const QaConv2Params* p, void* stream);
+int qa_quamba2_conv1d_update(const QaConv2Params* p, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Mamba1 int8 selective scan, forward over a sequence.
  * Replaces quant_sscan_cuda.fwd (csrc/selective_scan/quant_sscan.cpp:122-265; parameter block
  * csrc/selective_scan/quant_sscan.h:26-86).  Differences kept deliberate: the output is written

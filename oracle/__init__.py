@@ -96,6 +96,81 @@ def conv1d_update(x, state, weight, bias, s_x, s_w, s_b, s_out, silu=True):
     return out, state
 
 
+def quamba2_conv_channel_scales(x_dim, x_headdim, d_state, n_groups, scales_in, scales_w, scales_b,
+                                x_out_scales, B_out_scales, C_out_scales, x_head_group_range=None,
+                                x_dim_group_range=None):
+    """Per-channel (s_in, s_bias, s_out) of the concatenated [x | B | C] channels, resolved the way
+    quamba2_conv1d_fwd_kernel.cuh:147-212 does: an x channel belongs to ssd group c // (x_dim / n_groups),
+    head (c % group_size) // headdim, position c % headdim; the head group is the first whose
+    cumulative end index exceeds the head, the dim group likewise; B/C channel c belongs to ssd group
+    c // d_state.  scales_in / scales_w / scales_b are (x, B, C) triples of floats."""
+    bc = d_state * n_groups
+    dim = x_dim + 2 * bc
+    s_in = np.empty(dim, np.float32)
+    s_bias = np.empty(dim, np.float32)
+    s_out = np.zeros(dim, np.float32)
+    grouped = x_head_group_range is not None and x_dim_group_range is not None
+    xs = np.asarray(x_out_scales, np.float32)
+    Bs = np.asarray(B_out_scales, np.float32).reshape(-1)
+    Cs = np.asarray(C_out_scales, np.float32).reshape(-1)
+    for c in range(dim):
+        part = 0 if c < x_dim else (1 if c < x_dim + bc else 2)
+        s_in[c] = np.float32(scales_w[part]) * np.float32(scales_in[part])
+        s_bias[c] = np.float32(scales_b[part]) if scales_b[part] is not None else np.float32(0)
+        if part == 0:
+            if not grouped:
+                s_out[c] = xs.reshape(-1)[0]
+                continue
+            group_size = x_dim // n_groups
+            g, head, d = c // group_size, (c % group_size) // x_headdim, c % x_headdim
+            hr = np.asarray(x_head_group_range)[g]
+            dr = np.asarray(x_dim_group_range)[g]
+            h_start = 0
+            for hg in range(hr.shape[0]):
+                if h_start <= head < hr[hg]:
+                    d_start = 0
+                    for dg in range(dr.shape[1]):
+                        if d_start <= d < dr[hg, dg]:
+                            s_out[c] = xs.reshape(n_groups, hr.shape[0], dr.shape[1])[g, hg, dg]
+                            break
+                        d_start = dr[hg, dg]
+                    break
+                h_start = hr[hg]
+        else:
+            local = c - x_dim - (bc if part == 2 else 0)
+            src = Bs if part == 1 else Cs
+            s_out[c] = src[local // d_state] if grouped else src[0]
+    return s_in, s_bias, s_out
+
+
+def quamba2_conv1d_fwd(xBC, weight, bias, s_in, s_bias, s_out, x_dim, bc, silu=True):
+    """xBC int8 (B, dim, L) -> (x int8 (B, x_dim, L), B int8 (B, bc, L), C int8 (B, bc, L)) with the
+    per-channel scales of quamba2_conv_channel_scales."""
+    xBC, xp = _req(xBC)
+    weight, wp = _req(weight)
+    batch, dim, L = xBC.shape
+    out = np.empty_like(xBC)
+    s_in, s_bias, s_out = (np.ascontiguousarray(a, np.float32) for a in (s_in, s_bias, s_out))
+    fp = lambda a: a.ctypes.data_as(C.c_void_p)
+    lib().qo_conv1d_fwd_perchannel(xp, wp, _opt(bias), fp(out), batch, dim, L, weight.shape[1],
+                                   fp(s_in), fp(s_bias), fp(s_out), int(silu))
+    return out[:, :x_dim], out[:, x_dim:x_dim + bc], out[:, x_dim + bc:]
+
+
+def quamba2_conv1d_update(xBC, state, weight, bias, s_in, s_bias, s_out, x_dim, bc, silu=True):
+    """xBC int8 (B, dim); state int8 (B, dim, S), S in {k, k-1}.  Returns (x, B, C, new state)."""
+    xBC, xp = _req(xBC)
+    weight, wp = _req(weight)
+    state = np.array(state, dtype=np.int8, order="C", copy=True)
+    batch, dim = xBC.shape
+    out = np.empty_like(xBC)
+    s_in, s_bias, s_out = (np.ascontiguousarray(a, np.float32) for a in (s_in, s_bias, s_out))
+    fp = lambda a: a.ctypes.data_as(C.c_void_p)
+    lib().qo_conv1d_update_perchannel(xp, fp(state), wp, _opt(bias), fp(out), batch, dim, weight.shape[1],
+                                      state.shape[2], fp(s_in), fp(s_bias), fp(s_out), int(silu))
+    return out[:, :x_dim], out[:, x_dim:x_dim + bc], out[:, x_dim + bc:], state
+
+
 def sscan_fwd(u, delta, A_log, B, C_, D=None, delta_bias=None, z=None, *, s_u, s_delta, s_A, s_B, s_C,
               s_D=0.0, s_db=0.0, s_z=0.0, s_state=1.0, softplus=True):
     """u/delta/z int8 (B,D,L); A_log int8 (D,N); B,C int8 (B,G,N,L) or (B,N,L).

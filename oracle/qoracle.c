@@ -134,6 +134,60 @@ void qo_conv1d_update(const int8_t* x, int8_t* state, const int8_t* weight, cons
     }
 }
 
+/*
+ * Mamba2 xBC conv with per-channel scales, quamba2_conv1d_fwd_kernel.cuh:215-262 (forward) and
+ * quamba2_conv1d_update_kernel.cuh:134-143 (update).  The caller resolves, per channel of the
+ * concatenated [x | B | C] input, s_in = weight scale * input scale of its part, s_bias, and the output
+ * scale of its group (the range walk of fwd kernel :151-212 is restated in oracle/__init__.py).
+ * x int8 (batch, dim, seqlen) seqlen-major here (the layout is not part of the arithmetic).
+ *   forward: tmp = sum_w W[w]*x[t-(width-1-w)]; v = s_in*tmp + s_bias*bias (:233-237, contracted to one fma)
+ *   update:  v = s_bias*bias; v += s_in*W[i]*x[i] per tap (:134-136)
+ */
+void qo_conv1d_fwd_perchannel(const int8_t* x, const int8_t* weight, const int8_t* bias, int8_t* out,
+                              int batch, int dim, int seqlen, int width,
+                              const float* s_in, const float* s_bias, const float* s_out, int silu) {
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int b = 0; b < batch; ++b) {
+        for (int d = 0; d < dim; ++d) {
+            const int8_t* xr = x + ((int64_t)b * dim + d) * seqlen;
+            int8_t* orow = out + ((int64_t)b * dim + d) * seqlen;
+            const int8_t* w = weight + (int64_t)d * width;
+            const float bias_f = bias ? s_bias[d] * (float)bias[d] : 0.0f;
+            for (int t = 0; t < seqlen; ++t) {
+                float acc = 0.0f;
+                for (int k = 0; k < width; ++k) {
+                    const int ti = t - (width - 1 - k);
+                    const float xv = ti >= 0 ? (float)xr[ti] : 0.0f;
+                    acc += (float)w[k] * xv;                                /* exact in fp32 */
+                }
+                const float v = fmaf(s_in[d], acc, bias_f);
+                orow[t] = sat8_half_away(conv_finish(v, s_out[d], silu));   /* :238, :250-252 */
+            }
+        }
+    }
+}
+
+void qo_conv1d_update_perchannel(const int8_t* x, int8_t* state, const int8_t* weight, const int8_t* bias,
+                                 int8_t* out, int batch, int dim, int width, int state_len,
+                                 const float* s_in, const float* s_bias, const float* s_out, int silu) {
+    const int drop = state_len - (width - 1);
+    for (int b = 0; b < batch; ++b) {
+        for (int d = 0; d < dim; ++d) {
+            int8_t* st = state + ((int64_t)b * dim + d) * state_len;
+            const int8_t* w = weight + (int64_t)d * width;
+            int8_t xs[8];
+            for (int i = 0; i < width - 1; ++i) xs[i] = st[i + drop];       /* update kernel :50-55 */
+            xs[width - 1] = x[(int64_t)b * dim + d];
+            for (int i = 0; i < state_len; ++i) st[i] = xs[i + (width - state_len)];
+            float v = bias ? s_bias[d] * (float)bias[d] : 0.0f;             /* :134 */
+            for (int i = 0; i < width; ++i) {
+                v = fmaf(s_in[d] * (float)w[i], (float)xs[i], v);           /* :136 */
+            }
+            out[(int64_t)b * dim + d] = sat8_half_away(conv_finish(v, s_out[d], silu));   /* :137-141 */
+        }
+    }
+}
+
 /* ---------------------------------------------------------------------------------------------
  * Mamba1 selective scan forward, quant_sscan_fwd_kernel.cuh:110-293.
  * u, delta, z int8 (batch, dim, seqlen); A_log int8 (dim, dstate); B, C int8 (batch, groups,

@@ -30,6 +30,28 @@ class QaConvParams(C.Structure):
     ]
 
 
+class QaConv2Params(C.Structure):
+    _fields_ = [
+        ("batch", i32), ("dim", i32), ("seqlen", i32), ("width", i32),
+        ("silu_activation", i32),
+        ("x_dim", i32), ("x_headdim", i32), ("d_state", i32), ("n_groups", i32),
+        ("nhead_groups", i32), ("ndim_groups", i32), ("conv_state_len", i32),
+        ("xBC_batch_stride", i64), ("xBC_l_stride", i64), ("xBC_c_stride", i64),
+        ("x_batch_stride", i64), ("x_l_stride", i64), ("x_c_stride", i64),
+        ("B_batch_stride", i64), ("B_l_stride", i64), ("B_c_stride", i64),
+        ("C_batch_stride", i64), ("C_l_stride", i64), ("C_c_stride", i64),
+        ("weight_c_stride", i64), ("weight_width_stride", i64),
+        ("conv_state_batch_stride", i64), ("conv_state_c_stride", i64), ("conv_state_l_stride", i64),
+        ("xBC", vp), ("weight", vp), ("bias", vp), ("x", vp), ("B", vp), ("C", vp), ("conv_state", vp),
+        ("x_out_scales", vp), ("B_out_scales", vp), ("C_out_scales", vp),
+        ("x_head_group_range", vp), ("x_dim_group_range", vp),
+        ("scale_x", f32), ("scale_B", f32), ("scale_C", f32),
+        ("scale_wx", f32), ("scale_wB", f32), ("scale_wC", f32),
+        ("scale_bx", f32), ("scale_bB", f32), ("scale_bC", f32),
+        ("reserved0", f32),
+    ]
+
+
 class QaSScanParams(C.Structure):
     _fields_ = [
         ("batch", i32), ("dim", i32), ("seqlen", i32), ("dstate", i32),
@@ -116,6 +138,8 @@ SYMBOLS = {
     "qa_last_hip_error": (C.c_int, []),
     "qa_causal_conv1d_fwd": (C.c_int, [C.POINTER(QaConvParams), vp]),
     "qa_causal_conv1d_update": (C.c_int, [C.POINTER(QaConvParams), vp]),
+    "qa_quamba2_conv1d_fwd": (C.c_int, [C.POINTER(QaConv2Params), vp]),
+    "qa_quamba2_conv1d_update": (C.c_int, [C.POINTER(QaConv2Params), vp]),
     "qa_sscan_fwd": (C.c_int, [C.POINTER(QaSScanParams), vp]),
     "qa_ssm_state_update": (C.c_int, [C.POINTER(QaSsmUpdateParams), vp]),
     "qa_gemm_w8a8": (C.c_int, [C.POINTER(QaGemmW8A8Params), vp]),

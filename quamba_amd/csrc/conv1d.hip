@@ -11,52 +11,12 @@
 // The kernel is memory-shaped: one 16-byte load and one 16-byte store per 16 outputs, the 3-byte
 // causal halo comes from one extra aligned dword, and the four taps are one packed int8 dot
 // product (exact, so equal to the reference's fp32 accumulation of integer products).
-#include "qa_common.hpp"
+#include "conv_common.hpp"
 
 namespace qa {
 namespace {
 
 constexpr int kConvThreads = 256;
-
-__device__ __forceinline__ int8_t conv_epilogue(float v, float s_out, int silu) {
-    if (silu) v = v / (1.0f + exp_det(-v));
-    return sat8_half_away(v / s_out);
-}
-
-// Requantised output by the cheap route (hardware exp2 / rcp, multiply by 1/s_out, round to nearest)
-// whenever that provably equals the exact route, else by the exact route.  The cheap value y differs
-// from the exactly-evaluated one by less than 2e-4 for |y| < 129 (a few ulp of relative error), so if
-// y is further than 2e-3 from every half-integer both round to the same integer; values beyond
-// +-129 saturate either way.  Only lanes inside that margin (about 0.4 %) take the exact route.
-__device__ __forceinline__ int conv_quant(float v, float s_out, float inv_s_out, int silu) {
-    float y = v;
-    if (silu) {
-        const float e = __builtin_amdgcn_exp2f(v * -1.44269504088896341f);
-        y = v * __builtin_amdgcn_rcpf(1.0f + e);
-    }
-    y *= inv_s_out;
-    const float yr = __builtin_rintf(y);
-    const float d = __builtin_fabsf(y - yr);
-    int q = static_cast<int>(__builtin_amdgcn_fmed3f(yr, -128.0f, 127.0f));
-    if (!(d <= 0.498f) && !(__builtin_fabsf(y) >= 129.0f)) q = conv_epilogue(v, s_out, silu);
-    return q;
-}
-
-// packed taps for sdot4: byte j of the window holds x[t-3+j]; tap for x[t-(k-1-w)] is W[w],
-// so byte j pairs with W[j-(4-k)] (zero for j < 4-k).
-__device__ __forceinline__ uint32_t pack_taps(const int8_t* w, int64_t wstride, int width) {
-    uint32_t packed = 0;
-    for (int j = 0; j < 4; ++j) {
-        const int wi = j - (4 - width);
-        const uint32_t b = wi >= 0 ? static_cast<uint8_t>(w[wi * wstride]) : 0u;
-        packed |= b << (8 * j);
-    }
-    return packed;
-}
-
-__device__ __forceinline__ int dot4(uint32_t a, uint32_t b) {
-    return __builtin_amdgcn_sdot4(static_cast<int>(a), static_cast<int>(b), 0, false);
-}
 
 // One thread = 16 consecutive time steps of one (batch, channel) row.  Rows are 16-byte aligned
 // (checked on the host); a ragged tail (seqlen % 16) is handled bytewise by the row's last thread.

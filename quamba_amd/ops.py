@@ -111,6 +111,129 @@ def _scale1(t, name):
     return t
 
 
+def _conv2_params(xBC, x_dim, x_headdim, d_state, n_groups, x_head_group_range, x_dim_group_range, x_scales,
+                  scale_B_out, scale_C_out, weight, bias, dim):
+    """Argument checks shared by the Mamba2 xBC conv entry points (conditions of
+    csrc/causal_conv1d/quamba2_conv1d.cpp:125-186)."""
+    _require(xBC.dtype == torch.int8 and weight.dtype == torch.int8, "xBC and weight must be int8")
+    _require_gpu(xBC, "xBC")
+    _require_gpu(weight, "weight")
+    width = weight.shape[-1]
+    _require(tuple(weight.shape) == (dim, width), "weight must have shape (dim, width)")
+    if bias is not None:
+        _require(bias.dtype == torch.int8 and bias.is_cuda and tuple(bias.shape) == (dim,) and bias.stride(-1) == 1,
+                 "bias must be a contiguous int8 GPU tensor of shape (dim,)")
+    _require(x_dim <= dim, "x_dim must less or equal to input dim")
+    _require(x_dim % x_headdim == 0, "x_dim must be divided by x_headdim")
+    _require(x_dim + 2 * d_state * n_groups == dim, "x_dim + 2*d_state*n_groups must be equal to total dim")
+    p = _lib.QaConv2Params()
+    p.dim, p.width = dim, width
+    p.x_dim, p.x_headdim, p.d_state, p.n_groups = x_dim, x_headdim, d_state, n_groups
+    for t, n in ((x_scales, "x_scales"), (scale_B_out, "scale_B_out"), (scale_C_out, "scale_C_out")):
+        _require(t.dtype == torch.float32 and t.is_cuda and t.is_contiguous(), f"{n} must be a contiguous fp32 GPU tensor")
+    if x_head_group_range is not None and x_dim_group_range is not None:
+        for t in (x_head_group_range, x_dim_group_range):
+            _require(t.dtype == torch.int32 and t.is_cuda and t.is_contiguous(), "group ranges must be contiguous int32 GPU tensors")
+        _require(x_head_group_range.dim() == 2 and x_head_group_range.shape[0] == n_groups,
+                 "x_head_group_range.shape[0] must be equal to total number of groups")
+        _require(x_dim_group_range.dim() == 3 and x_dim_group_range.shape[0] == n_groups,
+                 "x_dim_group_range.shape[0] must be equal to total number of groups")
+        p.nhead_groups, p.ndim_groups = x_head_group_range.shape[1], x_dim_group_range.shape[2]
+        _require(x_dim_group_range.shape[1] == p.nhead_groups,
+                 "x_dim_group_range.shape[1] must be equal to total number of head groups")
+        _require(x_scales.numel() == n_groups * p.nhead_groups * p.ndim_groups,
+                 "number of x scales must be equal to total number of groups")
+        _require(scale_B_out.numel() == n_groups and scale_C_out.numel() == n_groups,
+                 "number of B / C scales must be equal to total number of SSD groups")
+        p.x_head_group_range, p.x_dim_group_range = ptr(x_head_group_range), ptr(x_dim_group_range)
+    else:
+        _require(x_head_group_range is None and x_dim_group_range is None,
+                 "x_head_group_range and x_dim_group_range must be both None or both not None")
+        _require(x_scales.numel() == 1 and scale_B_out.numel() == 1 and scale_C_out.numel() == 1,
+                 "number of x / B / C scales must be equal to 1")
+    p.x_out_scales, p.B_out_scales, p.C_out_scales = ptr(x_scales), ptr(scale_B_out), ptr(scale_C_out)
+    p.weight_c_stride, p.weight_width_stride = weight.stride()
+    p.weight, p.bias = ptr(weight), ptr(bias)
+    return p
+
+
+def quamba2_conv1d_fwd(xBC, scale_x, scale_B, scale_C, x_dim, x_headdim, d_state, n_groups, x_head_group_range,
+                       x_dim_group_range, x_scales, scale_B_out, scale_C_out, weight, scale_wx, scale_wB, scale_wC,
+                       bias=None, scale_bx=None, scale_bB=None, scale_bC=None, seq_idx=None, initial_states=None,
+                       final_states_out=None, silu_activation=True):
+    """Mamba2 xBC conv forward (quamba2_conv1d_cuda.fwd, csrc/causal_conv1d/quamba2_conv1d.cpp:109-251).
+    xBC int8 (batch, dim, seqlen) in channel-contiguous memory.  Returns x (batch, x_dim, seqlen), B and C
+    (batch, n_groups*d_state, seqlen), int8, each a transposed view of a (batch, seqlen, channels) buffer."""
+    _require(xBC.dim() == 3, "xBC must have shape (batch, dim, seqlen)")
+    batch, dim, seqlen = xBC.shape
+    _require(xBC.stride(1) == 1 and (xBC.stride(2) > 1 or dim == 1 or seqlen == 1), "only support channel_last")
+    if seq_idx is not None:
+        raise NotImplementedError("No implementation for seq_idx")
+    if initial_states is not None:
+        raise NotImplementedError("No implementation for initial_states")
+    if final_states_out is not None:
+        raise NotImplementedError("No implementation for final_states_out")
+    p = _conv2_params(xBC, x_dim, x_headdim, d_state, n_groups, x_head_group_range, x_dim_group_range, x_scales,
+                      scale_B_out, scale_C_out, weight, bias, dim)
+    _require(2 <= p.width <= 4, "causal_conv1d only supports width between 2 and 4")
+    bc = d_state * n_groups
+    x = torch.empty((batch, seqlen, x_dim), dtype=torch.int8, device=xBC.device).transpose(1, 2)
+    B = torch.empty((batch, seqlen, bc), dtype=torch.int8, device=xBC.device).transpose(1, 2)
+    C = torch.empty((batch, seqlen, bc), dtype=torch.int8, device=xBC.device).transpose(1, 2)
+    p.batch, p.seqlen = batch, seqlen
+    p.silu_activation = int(bool(silu_activation))
+    p.xBC_batch_stride, p.xBC_c_stride, p.xBC_l_stride = xBC.stride()
+    p.x_batch_stride, p.x_c_stride, p.x_l_stride = x.stride()
+    p.B_batch_stride, p.B_c_stride, p.B_l_stride = B.stride()
+    p.C_batch_stride, p.C_c_stride, p.C_l_stride = C.stride()
+    p.xBC, p.x, p.B, p.C = ptr(xBC), ptr(x), ptr(B), ptr(C)
+    p.scale_x, p.scale_B, p.scale_C = float(scale_x), float(scale_B), float(scale_C)
+    p.scale_wx, p.scale_wB, p.scale_wC = float(scale_wx), float(scale_wB), float(scale_wC)
+    p.scale_bx, p.scale_bB, p.scale_bC = (float(v) if v is not None else 0.0 for v in (scale_bx, scale_bB, scale_bC))
+    with torch.cuda.device(xBC.device):
+        st = _lib.lib().qa_quamba2_conv1d_fwd(ct.byref(p), _lib.current_stream(xBC.device))
+    _lib.check(st, "quamba2_conv1d_fwd")
+    return x, B, C
+
+
+def quamba2_conv1d_update(xBC, conv_state, scale_x, scale_B, scale_C, x_dim, x_headdim, d_state, n_groups,
+                          x_head_group_range, x_dim_group_range, x_scales, scale_B_out, scale_C_out, weight,
+                          scale_wx, scale_wB, scale_wC, bias=None, scale_bx=None, scale_bB=None, scale_bC=None,
+                          seq_idx=None, initial_states=None, final_states_out=None, silu_activation=True):
+    """One decode step of the Mamba2 xBC conv (quamba2_conv1d_cuda.update, quamba2_conv1d.cpp:254-379).
+    xBC int8 (batch, dim); conv_state int8 (batch, dim, width) (or width-1), shifted in place.
+    Returns x (batch, x_dim), B, C (batch, n_groups*d_state), int8."""
+    _require(xBC.dim() == 2, "xBC must have shape (batch, dim)")
+    batch, dim = xBC.shape
+    p = _conv2_params(xBC, x_dim, x_headdim, d_state, n_groups, x_head_group_range, x_dim_group_range, x_scales,
+                      scale_B_out, scale_C_out, weight, bias, dim)
+    _require(2 <= p.width <= 4, "causal_conv1d only supports width between 2 and 4")
+    _require(conv_state.dtype == torch.int8 and conv_state.is_cuda, "conv_state must be an int8 GPU tensor")
+    _require(conv_state.dim() == 3 and tuple(conv_state.shape[:2]) == (batch, dim)
+             and conv_state.shape[2] in (p.width, p.width - 1),
+             "conv_state must have shape (batch, dim, width) or (batch, dim, width-1)")
+    bc = d_state * n_groups
+    x = torch.empty((batch, x_dim), dtype=torch.int8, device=xBC.device)
+    B = torch.empty((batch, bc), dtype=torch.int8, device=xBC.device)
+    C = torch.empty((batch, bc), dtype=torch.int8, device=xBC.device)
+    p.batch, p.seqlen = batch, 1
+    p.silu_activation = int(bool(silu_activation))
+    p.xBC_batch_stride, p.xBC_c_stride = xBC.stride()
+    p.x_batch_stride, p.x_c_stride = x.stride()
+    p.B_batch_stride, p.B_c_stride = B.stride()
+    p.C_batch_stride, p.C_c_stride = C.stride()
+    p.conv_state_batch_stride, p.conv_state_c_stride, p.conv_state_l_stride = conv_state.stride()
+    p.conv_state_len = conv_state.shape[2]
+    p.xBC, p.x, p.B, p.C, p.conv_state = ptr(xBC), ptr(x), ptr(B), ptr(C), ptr(conv_state)
+    p.scale_x, p.scale_B, p.scale_C = float(scale_x), float(scale_B), float(scale_C)
+    p.scale_wx, p.scale_wB, p.scale_wC = float(scale_wx), float(scale_wB), float(scale_wC)
+    p.scale_bx, p.scale_bB, p.scale_bC = (float(v) if v is not None else 0.0 for v in (scale_bx, scale_bB, scale_bC))
+    with torch.cuda.device(xBC.device):
+        st = _lib.lib().qa_quamba2_conv1d_update(ct.byref(p), _lib.current_stream(xBC.device))
+    _lib.check(st, "quamba2_conv1d_update")
+    return x, B, C
+
+
 def sscan_fwd(u, scale_u, delta, scale_delta, A, scale_A, B, scale_B, C, scale_C, scale_ssm_state,
               D=None, scale_D=None, z=None, scale_z=None, delta_bias=None, scale_delta_bias=None,
               delta_softplus=False, state_dtype=torch.int8):

@@ -74,6 +74,99 @@ def conv_output_scale(qx, sx, qw, sw, qb, sb, silu=True):
     return np.float32(max(float(np.abs(acc).max()), 1e-5) / 127.0)
 
 
+def conv_float(qx, sx, qw, sw, qb, sb, silu=True):
+    """float64 evaluation of the dequantised depthwise causal conv (+SiLU): (B, D, L)."""
+    B, D, L = qx.shape
+    k = qw.shape[1]
+    x = qx.astype(np.float64) * float(sx)
+    w = qw.astype(np.float64) * float(sw)
+    acc = np.zeros((B, D, L))
+    for j in range(k):
+        shift = k - 1 - j
+        if shift < L:
+            acc[:, :, shift:] += w[None, :, j, None] * x[:, :, :L - shift]
+    if qb is not None:
+        acc += (qb.astype(np.float64) * float(sb))[None, :, None]
+    if silu:
+        acc = acc / (1.0 + np.exp(-acc))
+    return acc
+
+
+def mamba2_conv_inputs(batch, seqlen, nheads, headdim, dstate, ngroups, width=4, seed=1234, grouped=True,
+                       nhead_groups=4, ndim_groups=4, bias=True):
+    """Synthetic inputs of the Mamba2 xBC conv: int8 xBC (batch, dim, seqlen) with separate per-tensor
+    scales for the x, B and C parts, int8 taps and bias quantised per part, and output scales taken
+    from a float64 evaluation: per (ssd group, head group, dim group) for x when ``grouped`` (uneven
+    cumulative end-index tables), per ssd group for B and C, else one scale per part."""
+    x_dim, bc = nheads * headdim, ngroups * dstate
+    dim = x_dim + 2 * bc
+    parts = [(0, x_dim), (x_dim, x_dim + bc), (x_dim + bc, dim)]
+    act = activations((batch, dim, seqlen), 1, seed, "xBC")
+    qx = np.empty((batch, dim, seqlen), np.int8)
+    s_in = []
+    for lo, hi in parts:
+        q, s = quantize_absmax(act[:, lo:hi])
+        qx[:, lo:hi] = q
+        s_in.append(s)
+    w = rng_for(seed, "conv2_w").uniform(-0.5, 0.5, (dim, width)).astype(np.float32)
+    b = rng_for(seed, "conv2_b").uniform(-0.5, 0.5, (dim,)).astype(np.float32)
+    qw = np.empty((dim, width), np.int8)
+    qb = np.empty((dim,), np.int8) if bias else None
+    s_w, s_b = [], []
+    for lo, hi in parts:
+        q, s = quantize_absmax(w[lo:hi])
+        qw[lo:hi] = q
+        s_w.append(s)
+        if bias:
+            q, s = quantize_absmax(b[lo:hi])
+            qb[lo:hi] = q
+            s_b.append(s)
+        else:
+            s_b.append(None)
+    ref = np.empty((batch, dim, seqlen))
+    for i, (lo, hi) in enumerate(parts):
+        ref[:, lo:hi] = conv_float(qx[:, lo:hi], s_in[i], qw[lo:hi], s_w[i], qb[lo:hi] if bias else None,
+                                   s_b[i] if bias else 1.0)
+    amax = lambda a: np.float32(max(float(np.abs(a).max()), 1e-5) / 127.0)
+    out = dict(xBC=qx, weight=qw, bias=qb, scales_in=s_in, scales_w=s_w, scales_b=s_b, x_dim=x_dim, bc=bc, dim=dim,
+               ref=ref)
+    if not grouped:
+        out.update(x_out_scales=np.array([amax(ref[:, :x_dim])], np.float32),
+                   B_out_scales=np.array([amax(ref[:, x_dim:x_dim + bc])], np.float32),
+                   C_out_scales=np.array([amax(ref[:, x_dim + bc:])], np.float32),
+                   x_head_group_range=None, x_dim_group_range=None)
+        return out
+    heads_per_group = nheads // ngroups
+    g = rng_for(seed, "conv2_groups")
+
+    def cuts(total, n):
+        # n uneven pieces: cumulative end indices, last == total
+        if n == 1:
+            return np.array([total], np.int32)
+        inner = np.sort(g.choice(np.arange(1, total), size=n - 1, replace=False))
+        return np.concatenate([inner, [total]]).astype(np.int32)
+
+    nhg = min(nhead_groups, heads_per_group)
+    ndg = min(ndim_groups, headdim)
+    hr = np.stack([cuts(heads_per_group, nhg) for _ in range(ngroups)])
+    dr = np.stack([np.stack([cuts(headdim, ndg) for _ in range(nhg)]) for _ in range(ngroups)])
+    xs = np.empty((ngroups, nhg, ndg), np.float32)
+    rx = ref[:, :x_dim].reshape(batch, ngroups, heads_per_group, headdim, seqlen)
+    for gi in range(ngroups):
+        h0 = 0
+        for hg in range(nhg):
+            d0 = 0
+            for dg in range(ndg):
+                xs[gi, hg, dg] = amax(rx[:, gi, h0:hr[gi, hg], d0:dr[gi, hg, dg]])
+                d0 = dr[gi, hg, dg]
+            h0 = hr[gi, hg]
+    Bs = np.array([amax(ref[:, x_dim + gi * dstate:x_dim + (gi + 1) * dstate]) for gi in range(ngroups)], np.float32)
+    Cs = np.array([amax(ref[:, x_dim + bc + gi * dstate:x_dim + bc + (gi + 1) * dstate]) for gi in range(ngroups)],
+                  np.float32)
+    out.update(x_out_scales=xs, B_out_scales=Bs, C_out_scales=Cs, x_head_group_range=hr, x_dim_group_range=dr)
+    return out
+
+
 def mamba1_scan_inputs(batch, seqlen, dim, dstate, seed=1234, with_z=True):
     """Quantised inputs of the Mamba1 selective scan: dict of int8 arrays and float32 scales.
 
