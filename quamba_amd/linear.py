@@ -199,7 +199,7 @@ class W8A8B16O16Linear(_W8A8Base, _AlphaHooks):
 # w4a8_utils.pack_w4a8) and the scales are in natural column order, so a reference checkpoint needs
 # re-packing before it can be loaded here.
 # ------------------------------------------------------------------------------------------------
-from .w4a8_utils import w4a8_quantize  # noqa: E402
+from .w4a8_utils import marlin_qqq_to_native, w4a8_quantize  # noqa: E402
 
 
 class _W4A8Base(nn.Module):
@@ -247,6 +247,22 @@ class _W4A8Base(nn.Module):
         q.s_channel = s_channel.to(device)
         q.w_ref = w_ref          # dequantised (K, N) weights, kept for tests (not a buffer)
         return q
+
+    def _load_from_state_dict(self, state_dict, prefix, *args, **kwargs):
+        """Accepts a state dict written by the reference's module of the same name: an int32 ``weight`` is
+        Marlin-QQQ storage (quamba/qLinearLayer.py:160-162) and is re-packed, with its scales, on the way in;
+        the reference's lock ``workspace`` has no counterpart here."""
+        wkey = prefix + "weight"
+        if wkey in state_dict and state_dict[wkey].dtype == torch.int32:
+            w = state_dict[wkey]
+            size_k, size_n = w.shape[0] * 16, w.shape[1] // 2
+            packed, s_group, s_channel = marlin_qqq_to_native(w, state_dict[prefix + "s_group"],
+                                                              state_dict[prefix + "s_channel"], size_k, size_n)
+            state_dict[wkey] = packed
+            state_dict[prefix + "s_group"] = s_group
+            state_dict[prefix + "s_channel"] = s_channel
+            state_dict[prefix + "workspace"] = torch.zeros(1, dtype=torch.int32)
+        super()._load_from_state_dict(state_dict, prefix, *args, **kwargs)
 
     def _gemm(self, x2d, transpose):
         fn = ops.w4a8o8_gemm if self._out_dtype == torch.int8 else ops.w4a8o16_gemm

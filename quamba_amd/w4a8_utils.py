@@ -6,7 +6,13 @@ channel scale = max_k |w_ref| / 127, fused fp16 group scale = s_group / s_channe
 mode: code = clamp(round(w / (max|w| / 7)), -7, 7) as a signed nibble, s_channel /= 16.
 Only the storage differs: codes are packed for the gfx950 kernel (``pack_w4a8``) and the scales are
 kept in natural column order (the reference permutes both for its tensor-core tiles).
+
+The second half of the file reads and writes the reference's own storage (Marlin-QQQ, quamba/marlin_utils.py
+:33-133) so that checkpoints made by the reference load here: ``marlin_qqq_to_native`` turns the packed
+int32 weight and the permuted scales into this library's buffers, ``marlin_qqq_pack`` is the forward
+direction (used to check the inverse against vectors produced by the reference's own packer).
 """
+import numpy as np
 import torch
 
 
@@ -89,3 +95,100 @@ def w4a8_quantize(w, num_bits=4, group_size=-1, s_group=None, s_channel=None, ou
             s_group = pad(s_group, (0, pad_out), "constant", 0)
         s_channel = pad(s_channel, (0, pad_out), "constant", 1e-6)
     return [w_ref, pack_w4a8(q_w), s_group, s_channel]
+
+
+# ---------------------------------------------------------------------------------------------
+# Marlin-QQQ storage (the reference's checkpoints)
+# ---------------------------------------------------------------------------------------------
+def marlin_qqq_weight_perm(quant_type):
+    """The 1024-entry gather that orders four 16x16 tiles for the reference's tensor-core fragments
+    (quamba/marlin_utils.py:71-105).  Output position (i, j, e), i < 32 a fragment lane, j < 4 the tile,
+    e < 8 the nibble slot, reads flat tile element 256*j + 16*row + col with row = 4*(i % 4) + e % 4 and
+    col = i // 4 + 8*(e // 4); the eight slots of a word are then interleaved so that the kernel's
+    nibble extraction yields consecutive values (a different interleave for the per-channel scheme)."""
+    assert quant_type in ("per-channel", "per-group"), "not supported quantization type"
+    i = np.arange(32).reshape(32, 1, 1)
+    j = np.arange(4).reshape(1, 4, 1)
+    e = np.arange(8).reshape(1, 1, 8)
+    src = 256 * j + 16 * (4 * (i % 4) + e % 4) + i // 4 + 8 * (e // 4)
+    order = [4, 0, 5, 1, 6, 2, 7, 3] if quant_type == "per-channel" else [0, 2, 4, 6, 1, 3, 5, 7]
+    return torch.from_numpy(src[:, :, order].reshape(-1).astype(np.int64))
+
+
+def marlin_qqq_scale_perms():
+    """(group-scale permutation over 64 columns: an 8x8 transposition; channel-scale permutation over
+    32 columns) of quamba/marlin_utils.py:108-118."""
+    i = np.arange(8).reshape(8, 1)
+    scale_perm = (i + 8 * np.arange(8).reshape(1, 8)).reshape(-1)
+    offs = np.array([0, 1, 8, 9, 16, 17, 24, 25])
+    single = (2 * np.arange(4).reshape(4, 1) + offs.reshape(1, 8)).reshape(-1)
+    return torch.from_numpy(scale_perm.astype(np.int64)), torch.from_numpy(single.astype(np.int64))
+
+
+def _tile_rows(q_w, size_k, size_n):
+    """(K, N) -> (K/16, N*16): every 16x16 tile flattened row-major, tiles of a tile-row side by side."""
+    return q_w.reshape(size_k // 16, 16, size_n // 16, 16).permute(0, 2, 1, 3).reshape(size_k // 16, size_n * 16)
+
+
+def marlin_qqq_pack(q_w, size_k, size_n, group_size):
+    """Integer codes (K, N) -> int32 (K/16, N*16/8) in the reference's layout (marlin_utils.py:33-68)."""
+    assert tuple(q_w.shape) == (size_k, size_n) and size_k % 16 == 0 and size_n % 64 == 0
+    quant_type = "per-channel" if group_size in (-1, size_k) else "per-group"
+    perm = marlin_qqq_weight_perm(quant_type)
+    t = _tile_rows(q_w.to(torch.int64).cpu(), size_k, size_n)
+    t = t.reshape(-1, perm.numel())[:, perm].reshape(t.shape) & 0xF
+    shifts = (4 * torch.arange(8, dtype=torch.int64)).reshape(1, 1, 8)
+    words = (t.reshape(t.shape[0], -1, 8) << shifts).sum(dim=2)
+    return torch.from_numpy(words.numpy().astype(np.uint32).view(np.int32))
+
+
+def marlin_qqq_unpack(packed, size_k, size_n, group_size):
+    """Inverse of marlin_qqq_pack: int32 (K/16, N*2) -> int32 nibbles (K, N) in [0, 15]."""
+    assert tuple(packed.shape) == (size_k // 16, size_n * 2)
+    quant_type = "per-channel" if group_size in (-1, size_k) else "per-group"
+    perm = marlin_qqq_weight_perm(quant_type)
+    words = torch.from_numpy(packed.cpu().numpy().view(np.uint32).astype(np.int64))
+    shifts = (4 * torch.arange(8, dtype=torch.int64)).reshape(1, 1, 8)
+    t = ((words.unsqueeze(2) >> shifts) & 0xF).reshape(size_k // 16, size_n * 16)
+    chunks = t.reshape(-1, perm.numel())
+    out = torch.empty_like(chunks)
+    out[:, perm] = chunks
+    out = out.reshape(size_k // 16, size_n // 16, 16, 16).permute(0, 2, 1, 3).reshape(size_k, size_n)
+    return out.to(torch.int32)
+
+
+def marlin_qqq_permute_scales(s_group, s_channel, size_k, size_n, group_size):
+    """Natural column order -> the reference's (marlin_utils.py:121-133)."""
+    sp, sps = marlin_qqq_scale_perms()
+    if group_size not in (-1, size_k):
+        s_group = s_group.reshape(-1, sp.numel())[:, sp].reshape(-1, size_n).contiguous()
+    s_channel = s_channel.reshape(-1, sps.numel())[:, sps].reshape(-1, size_n).contiguous()
+    return s_group, s_channel
+
+
+def marlin_qqq_unpermute_scales(s_group, s_channel, size_k, size_n, group_size):
+    """The reference's column order -> natural."""
+    sp, sps = marlin_qqq_scale_perms()
+    if group_size not in (-1, size_k) and s_group.numel():
+        g = s_group.reshape(-1, sp.numel())
+        nat = torch.empty_like(g)
+        nat[:, sp] = g
+        s_group = nat.reshape(-1, size_n).contiguous()
+    c = s_channel.reshape(-1, sps.numel())
+    nat = torch.empty_like(c)
+    nat[:, sps] = c
+    return s_group, nat.reshape(-1, size_n).contiguous()
+
+
+def marlin_qqq_to_native(weight, s_group, s_channel, size_k, size_n, group_size=128):
+    """A reference W4A8 layer's buffers (``weight`` int32 (K/16, 2N), ``s_group`` fp16 (K/g, N) or empty,
+    ``s_channel`` fp32 (1, N)) -> this library's (``weight`` uint8 (N, K/2), s_group, s_channel in natural
+    column order).  The codes themselves are unchanged: offset-8 codes in the grouped scheme, two's
+    complement nibbles in the per-channel scheme."""
+    if s_group.numel() == 0:
+        group_size = -1
+    codes = marlin_qqq_unpack(weight, size_k, size_n, group_size)
+    s_group, s_channel = marlin_qqq_unpermute_scales(s_group.cpu(), s_channel.cpu(), size_k, size_n, group_size)
+    if s_group.numel() == 0:
+        s_group = s_group.reshape(0, size_n)
+    return pack_w4a8(codes), s_group, s_channel

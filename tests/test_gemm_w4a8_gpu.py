@@ -132,3 +132,26 @@ def test_errors(dev):
     one = torch.ones(1, device=dev)
     with pytest.raises(RuntimeError, match="multiple of 128"):
         ops.w4a8o16_gemm(a, w, one, torch.ones(16, device=dev), None, None, 8, 16, 64)
+
+
+def test_reference_checkpoint_loads_and_computes_the_same(dev):
+    """A state dict in the reference module's own format (Marlin-QQQ int32 weight, permuted scales, lock
+    workspace; vectors from the reference's packer in tests/golden) loads into the module here and gives
+    the same output as the layer quantised natively from the same fp16 weight."""
+    import os
+    fix = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "marlin_qqq_w4a8.npz"))
+    K, N = 256, 128
+    ref_sd = {"workspace": torch.zeros((N // 64) * 16, dtype=torch.int32),
+              "weight": torch.from_numpy(fix["g_marlin_q_w"]),
+              "input_scale": torch.tensor(0.02),
+              "s_channel": torch.from_numpy(fix["g_marlin_s_channel"]),
+              "s_group": torch.from_numpy(fix["g_marlin_s_group"])}
+    m = W4A8B16O16Linear(K, N, device=dev)
+    m.load_state_dict(ref_sd)
+    lin = torch.nn.Linear(K, N, bias=False, dtype=torch.float16)
+    lin.weight.data = torch.from_numpy(fix["g_w"]).t().contiguous()
+    native = W4A8B16O16Linear.from_fp16(lin.to(dev), torch.tensor(0.02))
+    assert torch.equal(m.weight, native.weight) and torch.equal(m.s_group, native.s_group)
+    x = torch.randint(-128, 128, (3, 50, K), dtype=torch.int8, device=dev)
+    assert torch.equal(m(x), native(x))
+    assert m(x).float().abs().max() > 0.1
