@@ -113,6 +113,28 @@ int qa_quamba2_conv1d_fwd(const QaConv2Params* p, void* stream);
 int qa_quamba2_conv1d_update(const QaConv2Params* p, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Hadamard transform of every row of a (rows, dim) matrix + int8 quantisation:
+ *   out[r, :] = sat8(round_half_away(H x[r, :] * scale)),  dim = S * 2^k with S in {1, 12, 40},
+ *   H = H_S (x) W_{2^k} (natural-order Walsh-Hadamard on the low index, the fixed 12- or 40-point
+ *   matrix on the high index); the caller folds 1/sqrt(dim) and 1/output scale into `scale`.
+ * Replaces quant_hadamard.fast_hadamard_transform / _12N / _40N
+ *   (csrc/hadamard/quant_hadamard.cpp, kernel csrc/hadamard/quant_hadamard_fwd.cu:153-229).
+ * Values beyond the int8 range saturate (the reference's cast is undefined there).
+ * ---------------------------------------------------------------------------------------- */
+enum { QA_IN_F16 = 0, QA_IN_F32 = 1 };
+
+typedef struct QaHadamardParams {
+    int32_t rows, dim;       /* dim <= 32768 */
+    int32_t in_type;         /* QA_IN_F16 / QA_IN_F32 */
+    float scale;
+    int64_t x_row_stride, out_row_stride;   /* elements; columns are contiguous */
+    const void* x;
+    int8_t* out;
+} QaHadamardParams;
+
+int qa_hadamard_quant(const QaHadamardParams* p, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Mamba1 int8 selective scan, forward over a sequence.
  * Replaces quant_sscan_cuda.fwd (csrc/selective_scan/quant_sscan.cpp:122-265; parameter block
  * csrc/selective_scan/quant_sscan.h:26-86).  Differences kept deliberate: the output is written

@@ -315,3 +315,60 @@ def ssd_fwd(x, dt, A_log, B, C_, D=None, z=None, dt_bias=None, *, chunk_size, x_
                      vp(out.get("dt")), vp(out.get("dA_cumsum")), vp(out.get("CB")), vp(out.get("chunk_states")),
                      vp(out.get("prev_states")))
     return out
+
+
+def _legendre(a, q):
+    a %= q
+    if a == 0:
+        return 0
+    return 1 if any((x * x) % q == a for x in range(1, q)) else -1
+
+
+def hadamard_special(S):
+    """The fixed S x S Hadamard matrix (+1/-1, int8) of the reference's 12N / 40N transforms
+    (csrc/hadamard/code_gen.py: ``had_12_paley``, ``had_40_tpal``), built from the definitions:
+    12: Paley's second construction for q = 5; 40: [[P, P], [P, -P]] with P the 20 x 20 Paley matrix for
+    q = 19 (first row + - ... -, first column +, core delta - chi(k - i))."""
+    if S == 12:
+        C6 = np.zeros((6, 6), int)
+        C6[0, 1:] = 1
+        C6[1:, 0] = 1
+        for i in range(1, 6):
+            for k in range(1, 6):
+                C6[i, k] = _legendre(k - i, 5)
+        blk = {0: [[1, -1], [-1, -1]], 1: [[1, 1], [1, -1]], -1: [[-1, -1], [-1, 1]]}
+        H = np.zeros((12, 12), int)
+        for i in range(6):
+            for k in range(6):
+                H[2 * i:2 * i + 2, 2 * k:2 * k + 2] = blk[int(C6[i, k])]
+        return H.astype(np.int8)
+    if S == 40:
+        P = np.ones((20, 20), int)
+        P[0, 1:] = -1
+        for i in range(1, 20):
+            for k in range(1, 20):
+                P[i, k] = 1 if i == k else -_legendre(k - i, 19)
+        return np.block([[P, P], [P, -P]]).astype(np.int8)
+    raise ValueError("S must be 12 or 40")
+
+
+def hadamard_split(dim):
+    """(S, M) with dim == S * M, the way quamba/hadamard_utils.py:33-47 picks the transform."""
+    S = 12 if dim % 12 == 0 else (40 if dim % 40 == 0 else 1)
+    M = dim // S
+    assert M & (M - 1) == 0 and M > 0, "dim must be S * 2^k"
+    return S, M
+
+
+def hadamard_quant(x, scale):
+    """x float16/float32 (..., dim) -> int8 of round(H x * scale)."""
+    x = np.asarray(x)
+    dim = x.shape[-1]
+    S, _ = hadamard_split(dim)
+    x2 = np.ascontiguousarray(x.reshape(-1, dim).astype(np.float32))
+    out = np.empty(x2.shape, np.int8)
+    signs = hadamard_special(S) if S > 1 else np.ones((1, 1), np.int8)
+    signs = np.ascontiguousarray(signs)
+    fp = lambda a: a.ctypes.data_as(C.c_void_p)
+    lib().qo_hadamard_quant(fp(x2), fp(out), x2.shape[0], dim, S, fp(signs), _f(scale))
+    return out.reshape(x.shape)

@@ -554,3 +554,46 @@ void qo_ssd_fwd(const QoSsdDims* d, const int8_t* x, const void* dt_in, const in
         }
     }
 }
+
+/* ---------------------------------------------------------------------------------------------
+ * Hadamard transform + int8 quantisation of each row, csrc/hadamard/quant_hadamard_fwd.cu:153-229.
+ * x fp32 (rows, dim) holds the input values already widened (the kernel widens on load,
+ * fast_hadamard_transform_common.h:128-143); dim = S * M, M a power of two.  The kernel applies
+ * butterflies (a+b, a-b) to the index bits of m from the lowest (registers, :84-104) through the lane
+ * bits (:107-123: sign*x + other) to the warp bits, then the S-point matrix to the chunk index c
+ * (element c*M + m, quant_hadamard_fwd.cu:203-224) as one left-to-right signed sum per output
+ * (fast_hadamard_transform_special.h).  signs is that S x S matrix as +1/-1 (S == 1: unused).
+ * Output: roundf(y * scale) (:147-154), saturated to int8 here.
+ * ------------------------------------------------------------------------------------------- */
+void qo_hadamard_quant(const float* x, int8_t* out, int rows, int dim, int S, const int8_t* signs, float scale) {
+    const int M = dim / S;
+#pragma omp parallel for schedule(static)
+    for (int r = 0; r < rows; ++r) {
+        float* v = (float*)malloc(sizeof(float) * (size_t)dim);
+        float tmp[64];
+        for (int e = 0; e < dim; ++e) v[e] = x[(int64_t)r * dim + e];
+        for (int stride = 1; stride < M; stride <<= 1) {
+            for (int e = 0; e < dim; ++e) {
+                if ((e & stride) == 0) {
+                    const float a = v[e], b = v[e + stride];
+                    v[e] = a + b;
+                    v[e + stride] = a - b;
+                }
+            }
+        }
+        if (S > 1) {
+            for (int m = 0; m < M; ++m) {
+                for (int i = 0; i < S; ++i) {
+                    float acc = signs[i * S] > 0 ? v[m] : -v[m];
+                    for (int j = 1; j < S; ++j) {
+                        acc = signs[i * S + j] > 0 ? acc + v[j * M + m] : acc - v[j * M + m];
+                    }
+                    tmp[i] = acc;
+                }
+                for (int i = 0; i < S; ++i) v[i * M + m] = tmp[i];
+            }
+        }
+        for (int e = 0; e < dim; ++e) out[(int64_t)r * dim + e] = sat8_half_away(v[e] * scale);
+        free(v);
+    }
+}

@@ -12,6 +12,7 @@ LIB_PATH = os.path.join(_HERE, "libquamba_amd.so")
 QA_OK = 0
 QA_OUT_I8, QA_OUT_F16 = 0, 1
 QA_ROUND_RNE, QA_ROUND_HALF_AWAY = 0, 1
+QA_IN_F16, QA_IN_F32 = 0, 1
 
 i32, i64, f32, vp = C.c_int32, C.c_int64, C.c_float, C.c_void_p
 
@@ -49,6 +50,14 @@ class QaConv2Params(C.Structure):
         ("scale_wx", f32), ("scale_wB", f32), ("scale_wC", f32),
         ("scale_bx", f32), ("scale_bB", f32), ("scale_bC", f32),
         ("reserved0", f32),
+    ]
+
+
+class QaHadamardParams(C.Structure):
+    _fields_ = [
+        ("rows", i32), ("dim", i32), ("in_type", i32), ("scale", f32),
+        ("x_row_stride", i64), ("out_row_stride", i64),
+        ("x", vp), ("out", vp),
     ]
 
 
@@ -140,6 +149,7 @@ SYMBOLS = {
     "qa_causal_conv1d_update": (C.c_int, [C.POINTER(QaConvParams), vp]),
     "qa_quamba2_conv1d_fwd": (C.c_int, [C.POINTER(QaConv2Params), vp]),
     "qa_quamba2_conv1d_update": (C.c_int, [C.POINTER(QaConv2Params), vp]),
+    "qa_hadamard_quant": (C.c_int, [C.POINTER(QaHadamardParams), vp]),
     "qa_sscan_fwd": (C.c_int, [C.POINTER(QaSScanParams), vp]),
     "qa_ssm_state_update": (C.c_int, [C.POINTER(QaSsmUpdateParams), vp]),
     "qa_gemm_w8a8": (C.c_int, [C.POINTER(QaGemmW8A8Params), vp]),

@@ -234,6 +234,29 @@ def quamba2_conv1d_update(xBC, conv_state, scale_x, scale_B, scale_C, x_dim, x_h
     return x, B, C
 
 
+def hadamard_quant(x, scale):
+    """int8 of round(H x * scale) along the last dimension (quant_hadamard.fast_hadamard_transform[_12N|_40N],
+    csrc/hadamard/quant_hadamard.cpp).  x fp16 or fp32 (..., dim), dim = S * 2^k with S in {1, 12, 40}."""
+    _require(x.dtype in (torch.float16, torch.float32), "x must be fp16 or fp32")
+    _require_gpu(x, "x")
+    shape = x.shape
+    dim = shape[-1]
+    x2 = x.reshape(-1, dim)
+    if x2.stride(-1) != 1:
+        x2 = x2.contiguous()
+    out = torch.empty(x2.shape, dtype=torch.int8, device=x.device)
+    p = _lib.QaHadamardParams()
+    p.rows, p.dim = x2.shape
+    p.in_type = _lib.QA_IN_F16 if x.dtype == torch.float16 else _lib.QA_IN_F32
+    p.scale = float(scale)
+    p.x_row_stride, p.out_row_stride = x2.stride(0) if x2.shape[0] > 1 else dim, dim
+    p.x, p.out = ptr(x2), ptr(out)
+    with torch.cuda.device(x.device):
+        st = _lib.lib().qa_hadamard_quant(ct.byref(p), _lib.current_stream(x.device))
+    _lib.check(st, "hadamard_quant")
+    return out.reshape(shape)
+
+
 def sscan_fwd(u, scale_u, delta, scale_delta, A, scale_A, B, scale_B, C, scale_C, scale_ssm_state,
               D=None, scale_D=None, z=None, scale_z=None, delta_bias=None, scale_delta_bias=None,
               delta_softplus=False, state_dtype=torch.int8):

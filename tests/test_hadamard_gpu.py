@@ -1,0 +1,84 @@
+"""GPU parity of the Hadamard + int8 quantisation kernel against the CPU oracle: bit-exact (both sides
+evaluate the same fp32 butterflies and left-to-right sums)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from quamba_amd import QHadamard, ops
+
+pytestmark = pytest.mark.gpu
+
+
+def _rows(rows, dim, seed, outliers=True):
+    g = np.random.default_rng(seed)
+    x = g.standard_normal((rows, dim)).astype(np.float32) * 2.0
+    if outliers:
+        cols = g.choice(dim, size=max(1, dim // 100), replace=False)
+        x[:, cols] *= 20.0
+    return x.astype(np.float16)
+
+
+# model widths: 130m (12 * 128), 2.8b (40 * 128), Mamba2-8b (2^13), plus small and extreme forms
+DIMS = [1536, 5120, 8192, 8, 16, 12, 40, 96, 640, 256, 4096, 32768, 12288]
+
+
+@pytest.mark.parametrize("dim", DIMS)
+def test_fp16_rows_bit_exact(dev, dim):
+    x = _rows(7, dim, seed=dim)
+    scale = np.float32(1.0 / math.sqrt(dim) / 0.06)
+    want = oracle.hadamard_quant(x, scale)
+    got = ops.hadamard_quant(torch.from_numpy(x).to(dev), float(scale))
+    assert got.dtype == torch.int8 and got.shape == x.shape
+    np.testing.assert_array_equal(got.cpu().numpy(), want)
+    assert np.abs(want).max() > 60
+
+
+def test_fp32_input_and_leading_dims(dev):
+    x = _rows(24, 5120, seed=3).astype(np.float32).reshape(2, 12, 5120)
+    scale = np.float32(1.0 / math.sqrt(5120) / 0.05)
+    want = oracle.hadamard_quant(x, scale)
+    got = ops.hadamard_quant(torch.from_numpy(x).to(dev), float(scale))
+    np.testing.assert_array_equal(got.cpu().numpy(), want)
+
+
+def test_strided_rows(dev):
+    x = _rows(9, 1536, seed=5)
+    buf = torch.zeros((9, 2048), dtype=torch.float16, device=dev)
+    buf[:, :1536] = torch.from_numpy(x).to(dev)
+    want = oracle.hadamard_quant(x, 0.4)
+    got = ops.hadamard_quant(buf[:, :1536], 0.4)
+    np.testing.assert_array_equal(got.cpu().numpy(), want)
+
+
+def test_module_folds_scales_and_keeps_state(dev):
+    dim = 5120
+    m = QHadamard(dim, x_H_scale=0.043)
+    assert m.N == 40 and abs(m.had_scale - 1 / math.sqrt(dim)) < 1e-12
+    x = _rows(5, dim, seed=8)
+    want = oracle.hadamard_quant(x, np.float32(m.had_scale / 0.043))
+    np.testing.assert_array_equal(m(torch.from_numpy(x).to(dev)).cpu().numpy(), want)
+    m2 = QHadamard(dim)
+    m2.load_state_dict(m.state_dict())
+    assert m2.x_H_scale == pytest.approx(0.043)
+    assert QHadamard(1536).N == 12 and QHadamard(8192).N == 2
+
+
+def test_rotation_preserves_the_linear_layer(dev):
+    # (H x / sqrt(d)) . (H w / sqrt(d)) == x . w : what makes the rotated out_proj equivalent
+    dim = 1536
+    g = np.random.default_rng(0)
+    x = g.standard_normal((3, dim)).astype(np.float16)
+    w = g.standard_normal((3, dim)).astype(np.float16)
+    s = 24.0 / math.sqrt(dim)       # int8 grid of 1/24 over +-5.3: no saturation for unit-variance rows
+    hx = ops.hadamard_quant(torch.from_numpy(x).to(dev), s).float() / 24.0
+    hw = ops.hadamard_quant(torch.from_numpy(w).to(dev), s).float() / 24.0
+    want = (torch.from_numpy(x).float() * torch.from_numpy(w).float()).sum(-1)
+    assert torch.allclose((hx * hw).sum(-1).cpu(), want, atol=3.0)      # rounding noise ~ sqrt(dim) * 0.017
+
+
+def test_unsupported_width(dev):
+    with pytest.raises(NotImplementedError):
+        ops.hadamard_quant(torch.zeros((2, 24 * 5), dtype=torch.float16, device=dev), 1.0)
