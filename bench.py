@@ -251,6 +251,14 @@ def other_workloads(dev, steps, warmup):
                     tokens_per_s=B * L / ms * 1e3, bound="hbm", achieved_GBs=nbytes / ms / 1e6,
                     frac=nbytes / ms / 1e6 / HBM_PEAK_GBS))
     del xBC
+    # Hadamard + quantisation of the scan output in front of out_proj: 16384 rows of 5120 (40 x 128) and of 8192
+    for dim in (5120, 8192):
+        xh = torch.randn(16384, dim, device=dev, dtype=torch.float16)
+        ms = _time_fn(lambda: ops.hadamard_quant(xh, 0.2), steps, warmup)
+        nbytes = 3 * 16384 * dim
+        out.append(dict(workload=f"Hadamard + int8 quantisation, 16384 rows x {dim}", us=ms * 1e3, tokens_per_s=16384 / ms * 1e3,
+                        bound="hbm", achieved_GBs=nbytes / ms / 1e6, frac=nbytes / ms / 1e6 / HBM_PEAK_GBS))
+        del xh
     # W4A8: in_proj 16384 x 4096 -> 18560 (int8 out), out_proj 16384 x 8192 -> 4096 (fp16 out)
     for (M, Nn, K, o8, name) in ((16384, 18560, 4096, True, "in_proj"), (16384, 4096, 8192, False, "out_proj")):
         a = ri(M, K)
