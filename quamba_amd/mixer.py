@@ -1,0 +1,131 @@
+"""W8A8QMamba: the quantized Mamba1 mixer assembled from this package's operators.
+
+The call order, tensor layouts and state handling of quamba/qMambaLayer.py:757-1010 (``W8A8QMamba``):
+in_proj (seqlen-last int8) -> x | z halves -> causal conv -> x_proj -> dt | B | C -> dt_proj (seqlen-last)
+-> selective scan with z gate -> Hadamard + quantisation -> out_proj (fp16).  ``step`` is the one-token
+form with the rolling conv state and the recurrent state updated in place.  This is the caller the
+operators are built for; it owns no arithmetic of its own.
+
+Two things the reference does with a copy are done in place here because the kernels take strides:
+the conv and the scan read the x and z halves of in_proj's buffer directly, and B / C are passed to the
+scan as transposed views only when that is free (they are tiny; a contiguous copy is made otherwise).
+"""
+import copy
+import math
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .conv import QCausalConv1D
+from .hadamard import QHadamard
+from .linear import W8A8B8O8Linear, W8A8B16O16Linear
+from .sscan import QSScan
+
+
+class W8A8QMamba(nn.Module):
+
+    def __init__(self, d_model, d_state=16, d_conv=4, expand=2, dt_rank="auto", conv_bias=True, bias=False,
+                 use_had_transform=True, layer_idx=None, device=None, state_dtype=torch.int8, **kwargs):
+        super().__init__()
+        assert bias is False, "Only support bias=False for now"
+        assert use_had_transform, "the mixer is built with the Hadamard + quantisation op in front of out_proj"
+        device = torch.device("cuda") if device is None else device
+        self.d_model = d_model
+        self.d_state = d_state
+        self.d_conv = d_conv
+        self.expand = expand
+        self.d_inner = int(expand * d_model)
+        self.dt_rank = math.ceil(d_model / 16) if dt_rank == "auto" else dt_rank
+        self.layer_idx = layer_idx
+        self.state_dtype = state_dtype        # int8 (the reference) or fp32 recurrent state
+        self.in_proj = W8A8B8O8Linear(d_model, self.d_inner * 2, device=device)
+        self.conv1d = QCausalConv1D(self.d_inner, self.d_inner, d_conv, groups=self.d_inner, padding=d_conv - 1,
+                                    bias=conv_bias, device=device)
+        self.x_proj = W8A8B8O8Linear(self.d_inner, self.dt_rank + 2 * d_state, device=device)
+        self.dt_proj = W8A8B8O8Linear(self.dt_rank, self.d_inner, device=device)
+        self.selective_scan = QSScan(d_state, self.d_inner, delta_softplus=True, device=device)
+        self.had = QHadamard(self.d_inner, x_H_scale=1.0)
+        self.out_proj = W8A8B16O16Linear(self.d_inner, d_model, device=device)
+
+    @classmethod
+    def from_fp16(cls, originalLayer, act_scales, use_had_transform=True):
+        """originalLayer: an fp16 Mamba mixer exposing in_proj, conv1d, x_proj, dt_proj (nn modules),
+        dt_proj_bias, A_log, D and the size attributes; act_scales: the calibration dict of
+        quamba/qMambaLayer.py:814-889 (same keys).  out_proj's weight must already carry the rotation."""
+        dev = originalLayer.in_proj.weight.device
+        q = cls(originalLayer.d_model, originalLayer.d_state, originalLayer.d_conv, originalLayer.expand,
+                originalLayer.dt_rank, use_had_transform=use_had_transform, layer_idx=getattr(originalLayer, "layer_idx", None),
+                device=dev)
+        s = lambda k: float(torch.as_tensor(act_scales[k]).item())
+        q.in_proj = W8A8B8O8Linear.from_fp16(copy.deepcopy(originalLayer.in_proj), s("in_proj:input"), s("in_proj:output"))
+        q.conv1d = QCausalConv1D.from_fp16(copy.deepcopy(originalLayer.conv1d), s("in_proj:output"), s("x_proj:input"))
+        q.x_proj = W8A8B8O8Linear.from_fp16(copy.deepcopy(originalLayer.x_proj), s("x_proj:input"), s("x_proj:output"))
+        q.dt_proj = W8A8B8O8Linear.from_fp16(copy.deepcopy(originalLayer.dt_proj), s("x_proj:output"), s("dt_proj:output"))
+        q.selective_scan = QSScan.from_fp16(
+            originalLayer.d_state, originalLayer.d_inner, originalLayer.A_log.clone(), D=originalLayer.D.clone(),
+            dt_bias=originalLayer.dt_proj_bias.clone(), delta_softplus=True,
+            ssm_state_scale=act_scales["ssm_state_act:input"], u_scale=act_scales["x_proj:input"],
+            dt_scale=act_scales["dt_proj:output"], B_scale=act_scales["x_proj:output"],
+            C_scale=act_scales["x_proj:output"], z_scale=act_scales["in_proj:output"])
+        q.had.x_H_scale = s("out_proj:input")
+        q.out_proj = W8A8B16O16Linear.from_fp16(copy.deepcopy(originalLayer.out_proj), s("out_proj:input"))
+        return q
+
+    @torch.no_grad()
+    def forward(self, hidden_states, inference_params=None, conv_state=None, ssm_state=None):
+        """hidden_states int8 (B, L, d_model) -> fp16 (B, L, d_model).  With conv_state / ssm_state (or an
+        inference_params cache) the states after the last token are stored into them."""
+        batch, seqlen, _ = hidden_states.shape
+        if inference_params is not None:
+            conv_state, ssm_state = self._get_states_from_cache(inference_params, batch)
+            if inference_params.seqlen_offset > 0:
+                out, _, _ = self.step(hidden_states, conv_state, ssm_state)
+                return out
+        xz = self.in_proj.to_seqlen_last(hidden_states)                 # (B, 2D, L), strides (L, B*L, 1)
+        x, z = xz.chunk(2, dim=1)                                       # views
+        if conv_state is not None:
+            conv_state.copy_(F.pad(x, (conv_state.shape[-1] - x.shape[-1], 0)))
+        x = self.conv1d(x)                                              # same strides as its input
+        x_dbl = self.x_proj(x.transpose(1, 2).contiguous())             # (B, L, dt_rank + 2N)
+        dt, B, C = torch.split(x_dbl, [self.dt_rank, self.d_state, self.d_state], dim=-1)
+        dt = self.dt_proj.to_seqlen_last(dt.contiguous())               # (B, D, L)
+        B = B.transpose(1, 2).contiguous()                              # (B, N, L)
+        C = C.transpose(1, 2).contiguous()
+        want_state = ssm_state is not None
+        y = self.selective_scan(x, dt, B, C, z=z, return_last_state=want_state,
+                                state_dtype=ssm_state.dtype if want_state else torch.int8)
+        if want_state:
+            y, last_state = y
+            ssm_state.copy_(last_state)
+        return self.out_proj(self.had(y))                               # (B, L, d_model) fp16
+
+    @torch.no_grad()
+    def step(self, hidden_states, conv_state, ssm_state):
+        assert hidden_states.shape[1] == 1, "Only support decoding with 1 token at a time for now"
+        xz = self.in_proj(hidden_states.squeeze(1))                     # (B, 2D)
+        x, z = xz.chunk(2, dim=-1)
+        x = self.conv1d.update(x, conv_state)
+        x_db = self.x_proj(x)
+        dt, B, C = torch.split(x_db, [self.dt_rank, self.d_state, self.d_state], dim=-1)
+        dt = self.dt_proj(dt.contiguous())
+        y, ssm_state = self.selective_scan.update(ssm_state, x, dt, B, C, z=z)
+        out = self.out_proj(self.had(y))
+        return out.unsqueeze(1), conv_state, ssm_state
+
+    def allocate_inference_cache(self, batch_size, max_seqlen=None, dtype=None, **kwargs):
+        device = self.out_proj.weight.device
+        conv_state = torch.zeros(batch_size, self.d_inner, self.d_conv, device=device, dtype=torch.int8)
+        ssm_state = torch.zeros(batch_size, self.d_inner, self.d_state, device=device, dtype=self.state_dtype)
+        return conv_state, ssm_state
+
+    def _get_states_from_cache(self, inference_params, batch_size, initialize_states=False):
+        assert self.layer_idx is not None
+        cache = inference_params.key_value_memory_dict
+        if self.layer_idx not in cache:
+            cache[self.layer_idx] = self.allocate_inference_cache(batch_size)
+        conv_state, ssm_state = cache[self.layer_idx]
+        if initialize_states:
+            conv_state.zero_()
+            ssm_state.zero_()
+        return conv_state, ssm_state
