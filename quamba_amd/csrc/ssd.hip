@@ -27,6 +27,12 @@ constexpr int kP = 64;          // head dimension this build supports
 constexpr float kLog2e = 1.44269504088896341f;
 
 __device__ __forceinline__ float fexp(float x) { return __builtin_amdgcn_exp2f(x * kLog2e); }
+// orders a wave's own LDS writes before its later LDS reads (wave-private scratch needs no workgroup barrier)
+__device__ __forceinline__ void wave_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
 __device__ __forceinline__ int8_t byte_of(uint32_t w, int j) { return static_cast<int8_t>((w >> (8 * j)) & 0xffu); }
 
 struct Ws {            // workspace sections (byte offsets), see qa_ssd_workspace_bytes
@@ -327,13 +333,15 @@ __global__ __launch_bounds__(256) void ssd_state_passing_kernel(QaSsdParams p, c
 // Stage 5 (quamba/triton/quant_chunk_scan.py:96-171): one workgroup per (batch, chunk, head);
 // each wave owns whole 32-row m-tiles (paired small/large so the causal work balances).
 // ---------------------------------------------------------------------------------------------
-template <int N>
-__global__ __launch_bounds__(256) void ssd_chunk_scan_kernel(QaSsdParams p, const float* dt_ws, const float* dA_ws,
+template <int N, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 4 : 1) void ssd_chunk_scan_kernel(QaSsdParams p, const float* dt_ws, const float* dA_ws,
                                                              const float* cb_ws, const __half* prev, int nc) {
-    constexpr int QMAX = 256, PITCH = QMAX + 8;
+    constexpr int QMAX = 256, PITCH = QMAX + 8, PPITCH = N + 8, kThreads = 64 * WAVES;
     __shared__ __attribute__((aligned(16))) _Float16 s_xt[kP * PITCH];
+    __shared__ __attribute__((aligned(16))) _Float16 s_prev[kP * PPITCH];     // entering state, rows p
     __shared__ __attribute__((aligned(16))) float s_dt[QMAX];
     __shared__ __attribute__((aligned(16))) float s_dA[QMAX];
+    __shared__ __attribute__((aligned(16))) float s_g[WAVES * QMAX];              // per wave: decay * dt of earlier steps
     __shared__ float s_xs[kP];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, frow = lane & 31, fhalf = lane >> 5;
@@ -346,23 +354,29 @@ __global__ __launch_bounds__(256) void ssd_chunk_scan_kernel(QaSsdParams p, cons
     const int t0 = c * Q;
     const int lim = min(Q, p.seqlen - t0);
     const int64_t row_base = (static_cast<int64_t>(b) * H + h) * nc + c;
-    for (int i = tid; i < Q; i += 256) {
+    for (int i = tid; i < Q; i += kThreads) {
         s_dt[i] = dt_ws[row_base * Q + i];
         s_dA[i] = dA_ws[row_base * Q + i];
     }
     if (tid < kP) s_xs[tid] = x_scale_of(p, g, hg, tid);
+    {
+        const __half* pst = prev + ((static_cast<int64_t>(b) * nc + c) * H + h) * kP * N;
+        for (int piece = tid; piece < kP * N / 8; piece += kThreads) {
+            const int pr = piece / (N / 8), col = (piece % (N / 8)) * 8;
+            *reinterpret_cast<uint4*>(s_prev + pr * PPITCH + col) = *reinterpret_cast<const uint4*>(pst + pr * N + col);
+        }
+    }
     __syncthreads();
     stage_transposed<kP, false>(s_xt, PITCH, p.x + ((static_cast<int64_t>(b) * p.seqlen + t0) * H + h) * kP,
-                                static_cast<int64_t>(H) * kP, Q, lim, s_xs, nullptr, tid, 256);
+                                static_cast<int64_t>(H) * kP, Q, lim, s_xs, nullptr, tid, kThreads);
     __syncthreads();
 
     const float sC = p.nhead_groups > 0 ? p.C_scale[g] : p.C_scale[0];
     const float* cb = cb_ws + ((static_cast<int64_t>(b) * nc + c) * G + g) * Q * Q;
-    const __half* pst = prev + ((static_cast<int64_t>(b) * nc + c) * H + h) * kP * N;
     const float D_scale = p.D ? *p.D_scale : 0.0f;
     const float z_scale = p.z ? *p.z_scale : 0.0f;
     const int nmt = Q / 32;
-    const int per_wave = max(1, nmt / 4);
+    const int per_wave = max(1, nmt / WAVES);
 
     for (int s = 0; s < per_wave; ++s) {
         // tile order 0, nmt-1, 1, nmt-2, ...: wave w takes entries w*per_wave + s
@@ -376,65 +390,158 @@ __global__ __launch_bounds__(256) void ssd_chunk_scan_kernel(QaSsdParams p, cons
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[j][r] = 0.0f;
 
-        // term 1: C^ (rows m, dstate contiguous) x entering state (rows p, dstate contiguous)
+        // Loads of this tile that do not depend on each other go out first: the lane's pieces of its
+        // C row (term 1) and the first two k-steps of its CB row (term 2).
         const int8_t* c_row = p.C + ((static_cast<int64_t>(b) * p.seqlen + t0 + m_lane) * G + g) * N;
+        uint2 c_raw[N / 16];
+#pragma unroll
+        for (int ks = 0; ks < N / 16; ++ks) {
+            c_raw[ks] = m_lane < lim ? *reinterpret_cast<const uint2*>(c_row + ks * 16 + fhalf * 8) : make_uint2(0u, 0u);
+        }
+        const float* cb_row = cb + static_cast<int64_t>(m_lane) * Q + fhalf * 8;
+        const int nks = 2 * (mt + 1);
+        constexpr int kAhead = 2;
+        float4 pre[kAhead][2];
+#pragma unroll
+        for (int a = 0; a < kAhead; ++a) {
+            if (a < nks) {
+                pre[a][0] = *reinterpret_cast<const float4*>(cb_row + a * 16);
+                pre[a][1] = *reinterpret_cast<const float4*>(cb_row + a * 16 + 4);
+            }
+        }
+
+        // term 1: C^ (rows m, dstate contiguous) x entering state (rows p, dstate contiguous, staged in LDS)
+#pragma unroll
         for (int ks = 0; ks < N / 16; ++ks) {
             v8h fc;
-            uint2 raw = make_uint2(0u, 0u);
-            if (m_lane < lim) raw = *reinterpret_cast<const uint2*>(c_row + ks * 16 + fhalf * 8);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) fc[e] = static_cast<_Float16>(sC * static_cast<float>(byte_of(e < 4 ? raw.x : raw.y, e & 3)));
+            for (int e = 0; e < 8; ++e) {
+                fc[e] = static_cast<_Float16>(sC * static_cast<float>(byte_of(e < 4 ? c_raw[ks].x : c_raw[ks].y, e & 3)));
+            }
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                const v8h fs = *reinterpret_cast<const v8h*>(pst + (j * 32 + frow) * N + ks * 16 + fhalf * 8);
+                const v8h fs = *reinterpret_cast<const v8h*>(s_prev + (j * 32 + frow) * PPITCH + ks * 16 + fhalf * 8);
                 acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fc, fs, acc[j], 0, 0, 0);
             }
         }
-        // scale rows by exp(dA_m): register r holds row m = mt*32 + 8*(r/4) + 4*(lane/32) + r%4
+        // Decay factors.  The cumulative dA decreases along the chunk, so with ref = dA at the first row
+        // of this m-tile, exp(dA_m - dA_k) = exp(dA_m - ref) * exp(ref - dA_k) for every k before the
+        // tile, both factors <= 1.  The k factor (times dt_k) is tabulated once per tile by the wave; the
+        // row factor is applied to the accumulator after the off-diagonal k-steps, together with term 1
+        // (whose decay exp(dA_m) = exp(ref) * exp(dA_m - ref)).  Only the two diagonal k-steps evaluate
+        // the decay per element.  acc = E_m * (exp(ref) * T1 + sum_{k < m0} (CB * G_k) x_k) + diagonal.
+        const int m0 = mt * 32;
+        const float ref = s_dA[m0];
+        float* g_tab = s_g + wave * QMAX;
+        for (int k = lane; k < m0; k += 64) g_tab[k] = fexp(ref - s_dA[k]) * s_dt[k];
+        wave_sync();
+        const float e_ref = fexp(ref);
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const float sm = fexp(s_dA[mt * 32 + 8 * (r / 4) + 4 * fhalf + (r % 4)]);
-            acc[0][r] *= sm;
-            acc[1][r] *= sm;
+            acc[0][r] *= e_ref;
+            acc[1][r] *= e_ref;
         }
-        // term 2: decayed causal CB (rows m, k contiguous) x XT (rows p, k contiguous)
-        const float dA_m = s_dA[m_lane];
-        const float* cb_row = cb + static_cast<int64_t>(m_lane) * Q;
-        for (int ks = 0; ks < 2 * (mt + 1); ++ks) {
-            const int k0 = ks * 16 + fhalf * 8;
-            const float4 c0 = *reinterpret_cast<const float4*>(cb_row + k0);
-            const float4 c1 = *reinterpret_cast<const float4*>(cb_row + k0 + 4);
-            const float cbv[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
-            v8h fl;
+        const int n_off = 2 * mt;                       // k-steps entirely before the tile
+        for (int ks = 0; ks < nks; ks += kAhead) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const int k = k0 + e;
-                const float wv = (cbv[e] * fexp(dA_m - s_dA[k])) * s_dt[k];
-                fl[e] = static_cast<_Float16>(k <= m_lane ? wv : 0.0f);
-            }
+            for (int a = 0; a < kAhead; ++a) {
+                const int kk = ks + a;
+                if (kk >= nks) break;                   // nks is even, kept for safety
+                const float4 c0 = pre[a][0], c1 = pre[a][1];
+                if (kk + kAhead < nks) {
+                    pre[a][0] = *reinterpret_cast<const float4*>(cb_row + (kk + kAhead) * 16);
+                    pre[a][1] = *reinterpret_cast<const float4*>(cb_row + (kk + kAhead) * 16 + 4);
+                }
+                const int k0 = kk * 16 + fhalf * 8;
+                const float cbv[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+                v8h fl;
+                if (kk < n_off) {
+                    const float4 g0 = *reinterpret_cast<const float4*>(g_tab + k0), g1 = *reinterpret_cast<const float4*>(g_tab + k0 + 4);
+                    const float gk[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const v8h fx = *reinterpret_cast<const v8h*>(s_xt + (j * 32 + frow) * PITCH + k0);
-                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fl, fx, acc[j], 0, 0, 0);
+                    for (int e = 0; e < 8; ++e) fl[e] = static_cast<_Float16>(cbv[e] * gk[e]);
+                } else {
+                    if (kk == n_off) {
+                        // leaving the off-diagonal part: apply the row factors once
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) {
+                            const float em = fexp(s_dA[m0 + 8 * (r / 4) + 4 * fhalf + (r % 4)] - ref);
+                            acc[0][r] *= em;
+                            acc[1][r] *= em;
+                        }
+                    }
+                    const float dA_m = s_dA[m_lane];
+                    const float4 dA0 = *reinterpret_cast<const float4*>(s_dA + k0), dA1 = *reinterpret_cast<const float4*>(s_dA + k0 + 4);
+                    const float4 dt0 = *reinterpret_cast<const float4*>(s_dt + k0), dt1 = *reinterpret_cast<const float4*>(s_dt + k0 + 4);
+                    const float dAk[8] = {dA0.x, dA0.y, dA0.z, dA0.w, dA1.x, dA1.y, dA1.z, dA1.w};
+                    const float dtk[8] = {dt0.x, dt0.y, dt0.z, dt0.w, dt1.x, dt1.y, dt1.z, dt1.w};
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const int k = k0 + e;
+                        const float wv = (cbv[e] * fexp(dA_m - dAk[e])) * dtk[e];
+                        fl[e] = static_cast<_Float16>(k <= m_lane ? wv : 0.0f);
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const v8h fx = *reinterpret_cast<const v8h*>(s_xt + (j * 32 + frow) * PITCH + k0);
+                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fl, fx, acc[j], 0, 0, 0);
+                }
             }
         }
-        // epilogue: lane holds column p = j*32 + (lane & 31)
+        wave_sync();                                    // g_tab is rewritten by the next tile
+        // epilogue: lane holds column p = j*32 + (lane & 31) and 16 rows per accumulator.  The int8 x
+        // (skip term) and z (gate) values of all 16 rows are fetched before any arithmetic; rows past
+        // the end of the sequence read the last valid row and are not stored.
+        const int64_t row_stride = static_cast<int64_t>(H) * kP;
+        const bool whole = mt * 32 + 32 <= lim;
+        // register r holds row lane_row0 + 8*(r/4) + r%4: offsets from the lane's first row are wave-uniform
+        const int lane_row0 = mt * 32 + 4 * fhalf;
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const int pp = j * 32 + frow;
+            const int64_t base = (static_cast<int64_t>(b) * p.seqlen + t0) * row_stride + static_cast<int64_t>(h) * kP + pp;
+            const int64_t lane_base = base + lane_row0 * row_stride;
+            int8_t xq[16], zq[16];
+            if (whole) {
+                if (p.D) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) xq[r] = p.x[lane_base + (8 * (r / 4) + (r % 4)) * row_stride];
+                }
+                if (p.z) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) zq[r] = p.z[lane_base + (8 * (r / 4) + (r % 4)) * row_stride];
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int m = min(lane_row0 + 8 * (r / 4) + (r % 4), lim - 1);
+                    xq[r] = p.D ? p.x[base + m * row_stride] : int8_t(0);
+                    zq[r] = p.z ? p.z[base + m * row_stride] : int8_t(0);
+                }
+            }
             const float Dv = p.D ? D_scale * static_cast<float>(p.D[p.D_has_hdim ? h * kP + pp : h]) : 0.0f;
+            const float xs_p = s_xs[pp];
+            float y[16];
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int m = mt * 32 + 8 * (r / 4) + 4 * fhalf + (r % 4);
-                if (m >= lim) continue;
-                const int64_t oi = ((static_cast<int64_t>(b) * p.seqlen + t0 + m) * H + h) * kP + pp;
-                float y = acc[j][r];
-                if (p.D) y += (s_xs[pp] * static_cast<float>(p.x[oi])) * Dv;
+                y[r] = acc[j][r];
+                if (p.D) y[r] += (xs_p * static_cast<float>(xq[r])) * Dv;
                 if (p.z) {
-                    const float zv = z_scale * static_cast<float>(p.z[oi]);
-                    y *= zv * (1.0f / (1.0f + fexp(-zv)));
+                    const float zv = z_scale * static_cast<float>(zq[r]);
+                    y[r] *= zv * __builtin_amdgcn_rcpf(1.0f + fexp(-zv));
                 }
-                static_cast<__half*>(p.out)[oi] = __float2half(y);
+            }
+            __half* out = static_cast<__half*>(p.out);
+            if (whole) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) out[lane_base + (8 * (r / 4) + (r % 4)) * row_stride] = __float2half(y[r]);
+            } else {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int m = lane_row0 + 8 * (r / 4) + (r % 4);
+                    if (m < lim) out[base + m * row_stride] = __float2half(y[r]);
+                }
             }
         }
     }
@@ -497,12 +604,9 @@ extern "C" int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream_) {
     const int64_t elems = static_cast<int64_t>(p->batch) * p->nheads * kP * p->dstate;
     hipLaunchKernelGGL(ssd_state_passing_kernel, dim3(static_cast<unsigned>((elems + 255) / 256)), dim3(256), 0, stream, *p,
                        dA_ws, states, prev, final_ws, nc);
-    if (p->dstate == 128) {
-        hipLaunchKernelGGL(ssd_chunk_scan_kernel<128>, dim3(static_cast<unsigned>(bch)), dim3(256), 0, stream, *p, dt_ws, dA_ws,
-                           cb_ws, prev, nc);
-    } else {
-        hipLaunchKernelGGL(ssd_chunk_scan_kernel<64>, dim3(static_cast<unsigned>(bch)), dim3(256), 0, stream, *p, dt_ws, dA_ws,
-                           cb_ws, prev, nc);
-    }
+    // four waves per workgroup, m-tiles paired small/large per wave (eight waves with one tile each measured slower)
+    const dim3 sgrid(static_cast<unsigned>(bch));
+    if (p->dstate == 128) hipLaunchKernelGGL((ssd_chunk_scan_kernel<128, 4>), sgrid, dim3(256), 0, stream, *p, dt_ws, dA_ws, cb_ws, prev, nc);
+    else hipLaunchKernelGGL((ssd_chunk_scan_kernel<64, 4>), sgrid, dim3(256), 0, stream, *p, dt_ws, dA_ws, cb_ws, prev, nc);
     return check_launch();
 }
