@@ -299,11 +299,26 @@ __global__ __launch_bounds__(256) void ssd_state_passing_kernel(QaSsdParams p, c
     const int h = static_cast<int>((idx / per_head) % H);
     const int b = static_cast<int>(idx / (per_head * H));
     float s = 0.0f;
-    for (int c = 0; c < nc; ++c) {
-        const int64_t off = ((static_cast<int64_t>(b) * nc + c) * H + h) * per_head + e;
-        prev[off] = __float2half(s);
-        const float dA_last = dA_ws[((static_cast<int64_t>(b) * H + h) * nc + c) * Q + Q - 1];
-        s = expf(dA_last) * s + states[off];
+    // the chunk states do not depend on the running state: fetch eight chunks at a time, then recur
+    constexpr int kBlock = 8;
+    const int64_t c_stride = static_cast<int64_t>(H) * per_head;
+    const int64_t off0 = (static_cast<int64_t>(b) * nc * H + h) * per_head + e;
+    const float* dA_last_p = dA_ws + (static_cast<int64_t>(b) * H + h) * nc * Q + Q - 1;
+    for (int c0 = 0; c0 < nc; c0 += kBlock) {
+        float st[kBlock], da[kBlock];
+#pragma unroll
+        for (int i = 0; i < kBlock; ++i) {
+            const int c = min(c0 + i, nc - 1);
+            st[i] = states[off0 + c * c_stride];
+            da[i] = dA_last_p[static_cast<int64_t>(c) * Q];
+        }
+#pragma unroll
+        for (int i = 0; i < kBlock; ++i) {
+            if (c0 + i < nc) {
+                prev[off0 + (c0 + i) * c_stride] = __float2half(s);
+                s = expf(da[i]) * s + st[i];
+            }
+        }
     }
     const int64_t fo = (static_cast<int64_t>(b) * H + h) * per_head + e;
     if (final_ws) final_ws[fo] = s;
