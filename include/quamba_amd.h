@@ -113,6 +113,34 @@ int qa_quamba2_conv1d_fwd(const QaConv2Params* p, void* stream);
 int qa_quamba2_conv1d_update(const QaConv2Params* p, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Gated RMS norm of fp16 rows with int8 gate input and int8 or fp16 output (Mamba2, between the SSD
+ * scan and out_proj).  Per (row, group of group_size columns):
+ *   x' = x * silu(z_scale*qz)            (gate first: norm_before_gate == 0)
+ *   y  = x' / sqrt(mean(x'^2) + eps) * w
+ *   y *= silu(z_scale*qz)                (norm_before_gate == 1)
+ *   out = fp16(y) | sat8(rint(y / out_scale)) | sat8(rint(y / (max(y)/127))) with that scale stored at
+ *         dyn_scale[group*rows + row]    (out_mode 0 | 1 | 2; max(y), not max|y|, as the reference)
+ * Replaces _qlayer_normgated_fwd (quamba/triton/quant_normgated.py:11-134) as used by QRMSNormGated
+ * (quamba/qNorm.py:93-177).  RMS norm without bias only.
+ * ---------------------------------------------------------------------------------------- */
+enum { QA_NORM_OUT_F16 = 0, QA_NORM_OUT_I8_STATIC = 1, QA_NORM_OUT_I8_DYNAMIC = 2 };
+
+typedef struct QaNormGatedParams {
+    int32_t rows, dim, group_size;   /* dim % group_size == 0, group_size % 8 == 0, group_size <= 8192 */
+    int32_t norm_before_gate;
+    int32_t out_mode;
+    float eps, z_scale, out_scale;
+    int64_t x_row_stride, z_row_stride, out_row_stride;   /* elements */
+    const void* x;        /* fp16 (rows, dim) */
+    const void* weight;   /* fp16 (dim) */
+    const int8_t* qz;     /* int8 (rows, dim) or null (no gate) */
+    void* out;            /* fp16 or int8 (rows, dim) */
+    float* dyn_scale;     /* [dim/group_size * rows], out_mode 2 only */
+} QaNormGatedParams;
+
+int qa_rmsnorm_gated(const QaNormGatedParams* p, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Hadamard transform of every row of a (rows, dim) matrix + int8 quantisation:
  *   out[r, :] = sat8(round_half_away(H x[r, :] * scale)),  dim = S * 2^k with S in {1, 12, 40},
  *   H = H_S (x) W_{2^k} (natural-order Walsh-Hadamard on the low index, the fixed 12- or 40-point

@@ -372,3 +372,37 @@ def hadamard_quant(x, scale):
     fp = lambda a: a.ctypes.data_as(C.c_void_p)
     lib().qo_hadamard_quant(fp(x2), fp(out), x2.shape[0], dim, S, fp(signs), _f(scale))
     return out.reshape(x.shape)
+
+
+def rmsnorm_gated(x, weight, qz=None, *, eps, z_scale=0.0, group_size=None, norm_before_gate=True, out_mode="f16",
+                  out_scale=None):
+    """Gated RMS norm of quamba/triton/quant_normgated.py:34-82, evaluated in float64 (the kernel's fp32
+    tree sums have no fixed order, so this restatement keeps the formula exact and leaves the last bit of
+    the row statistic to the tolerance of the comparison).
+    x float16 (M, N); weight float16 (N); qz int8 (M, N) or None.  Returns (y float64 (M, N) before the
+    output cast, q, scales): q is float16 (out_mode "f16"), int8 with ``out_scale`` ("static") or int8 with
+    the per-(row, group) scale max(y)/127 ("dynamic", scales float32 (groups, M))."""
+    x = np.asarray(x, np.float16).astype(np.float64)
+    M, N = x.shape
+    g = N if group_size is None else group_size
+    w = np.asarray(weight, np.float16).astype(np.float64)
+    gate = None
+    if qz is not None:
+        z = np.float64(np.float32(z_scale)) * np.asarray(qz, np.int8).astype(np.float64)
+        gate = z / (1.0 + np.exp(-z))
+        if not norm_before_gate:
+            x = x * gate                                                       # :48-50
+    xg = x.reshape(M, N // g, g)
+    var = (xg * xg).sum(axis=2, keepdims=True) / g                             # :55-56
+    rstd = 1.0 / np.sqrt(var + np.float64(np.float32(eps)))                    # :58
+    y = (xg * rstd).reshape(M, N) * w[None, :]                                 # :65-66
+    if gate is not None and norm_before_gate:
+        y = y * gate                                                           # :67-69
+    if out_mode == "f16":
+        return y, y.astype(np.float16), None
+    if out_mode == "static":
+        s = np.float64(np.float32(out_scale))
+        return y, np.clip(np.rint(y / s), -128, 127).astype(np.int8), None     # :74-75
+    s = y.reshape(M, N // g, g).max(axis=2) / 127.0                            # :77 (max, not max |.|)
+    q = np.clip(np.rint(y.reshape(M, N // g, g) / s[:, :, None]), -128, 127).astype(np.int8).reshape(M, N)
+    return y, q, np.ascontiguousarray(s.T).astype(np.float32)                  # scale index = group * M + row

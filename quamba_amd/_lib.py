@@ -61,6 +61,15 @@ class QaHadamardParams(C.Structure):
     ]
 
 
+class QaNormGatedParams(C.Structure):
+    _fields_ = [
+        ("rows", i32), ("dim", i32), ("group_size", i32), ("norm_before_gate", i32), ("out_mode", i32),
+        ("eps", f32), ("z_scale", f32), ("out_scale", f32),
+        ("x_row_stride", i64), ("z_row_stride", i64), ("out_row_stride", i64),
+        ("x", vp), ("weight", vp), ("qz", vp), ("out", vp), ("dyn_scale", vp),
+    ]
+
+
 class QaSScanParams(C.Structure):
     _fields_ = [
         ("batch", i32), ("dim", i32), ("seqlen", i32), ("dstate", i32),
@@ -150,6 +159,7 @@ SYMBOLS = {
     "qa_quamba2_conv1d_fwd": (C.c_int, [C.POINTER(QaConv2Params), vp]),
     "qa_quamba2_conv1d_update": (C.c_int, [C.POINTER(QaConv2Params), vp]),
     "qa_hadamard_quant": (C.c_int, [C.POINTER(QaHadamardParams), vp]),
+    "qa_rmsnorm_gated": (C.c_int, [C.POINTER(QaNormGatedParams), vp]),
     "qa_sscan_fwd": (C.c_int, [C.POINTER(QaSScanParams), vp]),
     "qa_ssm_state_update": (C.c_int, [C.POINTER(QaSsmUpdateParams), vp]),
     "qa_gemm_w8a8": (C.c_int, [C.POINTER(QaGemmW8A8Params), vp]),

@@ -257,6 +257,43 @@ def hadamard_quant(x, scale):
     return out.reshape(shape)
 
 
+def qlayer_normgated_fwd(x, weight, bias, eps, q_z=None, z_scale=None, static_out_scale=None,
+                         use_float16_output=False, group_size=None, norm_before_gate=True, is_rms_norm=True):
+    """Gated RMS norm of fp16 rows (``_qlayer_normgated_fwd``, quamba/triton/quant_normgated.py:85-134).
+    x fp16 (M, N); q_z int8 (M, N) or None.  Returns (out, per_token_scale): out fp16, or int8 with the
+    static scale, or int8 with one dynamic scale per (row, group) in per_token_scale[(group, row)]."""
+    _require(x.dtype == torch.float16 and x.dim() == 2, "x must be fp16 (M, N)")
+    _require_gpu(x, "x")
+    if bias is not None or not is_rms_norm:
+        raise NotImplementedError("only the bias-free RMS norm is implemented")
+    M, N = x.shape
+    group_size = N if group_size is None else group_size
+    _require(N % group_size == 0, "N must be divisible by group_size")
+    _require(x.stride(-1) == 1, "x must be contiguous along the last dimension")
+    _require(weight.dtype == torch.float16 and tuple(weight.shape) == (N,) and weight.stride(-1) == 1 and weight.is_cuda,
+             "weight must be a contiguous fp16 GPU tensor of shape (N,)")
+    if q_z is not None:
+        _require(q_z.dtype == torch.int8 and tuple(q_z.shape) == (M, N) and q_z.stride(-1) == 1 and q_z.is_cuda,
+                 "q_z must be an int8 GPU tensor of shape (M, N), contiguous along the last dimension")
+    ngroups = N // group_size
+    out = torch.empty((M, N), dtype=torch.float16 if use_float16_output else torch.int8, device=x.device)
+    per_token_scale = torch.empty((ngroups * M,), dtype=torch.float32, device=x.device)
+    p = _lib.QaNormGatedParams()
+    p.rows, p.dim, p.group_size = M, N, group_size
+    p.norm_before_gate = int(bool(norm_before_gate))
+    p.out_mode = 0 if use_float16_output else (1 if static_out_scale is not None else 2)
+    p.eps = float(eps)
+    p.z_scale = float(z_scale) if z_scale is not None else 0.0
+    p.out_scale = float(static_out_scale) if static_out_scale is not None else 0.0
+    p.x_row_stride, p.out_row_stride = x.stride(0) if M > 1 else N, N
+    p.z_row_stride = (q_z.stride(0) if M > 1 else N) if q_z is not None else 0
+    p.x, p.weight, p.qz, p.out, p.dyn_scale = ptr(x), ptr(weight), ptr(q_z), ptr(out), ptr(per_token_scale)
+    with torch.cuda.device(x.device):
+        st = _lib.lib().qa_rmsnorm_gated(ct.byref(p), _lib.current_stream(x.device))
+    _lib.check(st, "rmsnorm_gated")
+    return out, per_token_scale
+
+
 def sscan_fwd(u, scale_u, delta, scale_delta, A, scale_A, B, scale_B, C, scale_C, scale_ssm_state,
               D=None, scale_D=None, z=None, scale_z=None, delta_bias=None, scale_delta_bias=None,
               delta_softplus=False, state_dtype=torch.int8):
