@@ -129,3 +129,88 @@ class W8A8QMamba(nn.Module):
             conv_state.zero_()
             ssm_state.zero_()
         return conv_state, ssm_state
+
+
+class W4A8QMamba2(nn.Module):
+    """The quantized Mamba2 mixer of quamba/qMamba2.py:735-1068 (``W4A8QMamba2``) on this package's
+    operators: in_proj (W4A8, int8 out with one output scale per z | x | B | C | dt segment) -> xBC conv
+    (three int8 outputs) -> SSD chunk scan -> gated RMS norm (fp16) -> Hadamard + quantisation -> out_proj
+    (W4A8, fp16).  ``step`` is the one-token form.  ``from_fp16`` is not provided: it needs the grouping
+    tables produced by the reference's calibration pipeline; the sub-modules' own ``from_fp16`` exist."""
+
+    def __init__(self, d_model, d_state=128, d_conv=4, expand=2, headdim=64, d_ssm=None, ngroups=1, D_has_hdim=False,
+                 rmsnorm=True, norm_before_gate=False, dt_limit=(0.0, float("inf")), bias=False, conv_bias=True,
+                 chunk_size=256, use_had_transform=True, layer_idx=None, device=None, state_dtype=torch.int8,
+                 x_nhead_group=4, x_ndim_group=4, **kwargs):
+        super().__init__()
+        from .chunk_scan import Quamba2ChunkScan
+        from .conv import Quamb2Conv1D
+        from .linear import W4A8B8O8LinearParallel, W4A8B16O16Linear
+        from .norm import QRMSNormGated
+        assert bias is False, "Only support bias=False for now"
+        assert rmsnorm, "Only support Mamba2 block with rmsnorm"
+        assert use_had_transform, "the mixer is built with the Hadamard + quantisation op in front of out_proj"
+        device = torch.device("cuda") if device is None else device
+        self.d_model, self.d_state, self.d_conv, self.expand = d_model, d_state, d_conv, expand
+        self.d_inner = expand * d_model
+        self.headdim = headdim
+        self.d_ssm = self.d_inner if d_ssm is None else d_ssm
+        assert self.d_ssm == self.d_inner, "the gated-MLP split (d_ssm < d_inner) is not part of this mixer"
+        self.ngroups = ngroups
+        self.nheads = self.d_ssm // headdim
+        self.chunk_size = chunk_size
+        self.layer_idx = layer_idx
+        self.state_dtype = state_dtype
+        d_in_proj = 2 * self.d_inner + 2 * ngroups * d_state + self.nheads      # order: z, x, B, C, dt
+        self.in_proj = W4A8B8O8LinearParallel(d_model, d_in_proj, group_size=128, device=device)
+        conv_dim = self.d_ssm + 2 * ngroups * d_state
+        self.conv1d = Quamb2Conv1D(self.d_ssm, headdim, d_state, ngroups, x_nhead_group, x_ndim_group, conv_dim, conv_dim,
+                                   d_conv, groups=conv_dim, padding=d_conv - 1, bias=conv_bias, device=device)
+        self.qchunk_scan = Quamba2ChunkScan(self.d_ssm, headdim, d_state, ngroups, D_has_hdim, chunk_size, x_nhead_group,
+                                            x_ndim_group, delta_softplus=True, dt_limit=dt_limit, device=device)
+        self.norm = QRMSNormGated(self.d_ssm, eps=1e-5, norm_before_gate=norm_before_gate, group_size=self.d_ssm // ngroups,
+                                  use_float16_output=True, device=device)
+        self.had = QHadamard(self.d_inner, x_H_scale=1.0)
+        self.out_proj = W4A8B16O16Linear(self.d_inner, d_model, group_size=128, device=device)
+
+    def _split(self, zxbcdt):
+        return torch.split(zxbcdt, [self.d_ssm, self.d_ssm + 2 * self.ngroups * self.d_state, self.nheads], dim=-1)
+
+    @torch.no_grad()
+    def forward(self, u, conv_state=None, ssm_state=None):
+        """u int8 (B, L, d_model) -> fp16 (B, L, d_model); conv_state / ssm_state receive the states after
+        the last token when given."""
+        batch, seqlen, _ = u.shape
+        z, xBC, dt = self._split(self.in_proj(u))                   # views of (B, L, d_in_proj)
+        if conv_state is not None:
+            xBC_t = xBC.transpose(1, 2)
+            conv_state.copy_(F.pad(xBC_t, (self.d_conv - xBC_t.shape[-1], 0)))
+        x, B, C = self.conv1d(xBC.transpose(1, 2))                  # (B, ch, L) views of (B, L, ch) buffers
+        x = x.transpose(1, 2).reshape(batch, seqlen, self.nheads, self.headdim)
+        B = B.transpose(1, 2).reshape(batch, seqlen, self.ngroups, self.d_state)
+        C = C.transpose(1, 2).reshape(batch, seqlen, self.ngroups, self.d_state)
+        want_state = ssm_state is not None
+        y = self.qchunk_scan(x, dt, B, C, z=None, return_final_states=want_state,
+                             **({"state_dtype": ssm_state.dtype} if want_state else {}))
+        if want_state:
+            y, last_state = y
+            ssm_state.copy_(last_state)
+        y = self.norm(y.reshape(batch, seqlen, self.d_ssm), z)
+        return self.out_proj(self.had(y))
+
+    @torch.no_grad()
+    def step(self, hidden_states, conv_state, ssm_state):
+        assert hidden_states.shape[1] == 1, "Only support decoding with 1 token at a time for now"
+        z, xBC, dt = self._split(self.in_proj(hidden_states.squeeze(1)))
+        x, B, C = self.conv1d.update(xBC, conv_state)
+        y = self.qchunk_scan.update(ssm_state, x, dt, B, C, z=None)
+        y = self.norm(y.reshape(y.shape[0], self.d_ssm), z)
+        out = self.out_proj(self.had(y))
+        return out.unsqueeze(1), conv_state, ssm_state
+
+    def allocate_inference_cache(self, batch_size, max_seqlen=None, dtype=None, **kwargs):
+        device = self.out_proj.weight.device
+        conv_dim = self.conv1d.weight.shape[0]
+        conv_state = torch.zeros(batch_size, self.d_conv, conv_dim, device=device, dtype=torch.int8).transpose(1, 2)
+        ssm_state = torch.zeros(batch_size, self.nheads, self.headdim, self.d_state, device=device, dtype=self.state_dtype)
+        return conv_state, ssm_state
