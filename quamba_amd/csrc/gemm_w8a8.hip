@@ -97,6 +97,194 @@ int launch_gemm(const QaGemmW8A8Params& p, hipStream_t stream) {
                                    : launch_one<TM, TN, WGM, WGN, STAGES, QA_OUT_F16, FLEX>(p, stream);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Few activation rows (M <= 64, the decode step): the product is a stream over the weight matrix
+// and HBM-bound, so the shape of the launch is chosen for memory parallelism rather than reuse.
+// A workgroup owns 32 output columns and all rows; its WAVES waves split K between them in
+// interleaved 128-byte tiles.  A wave fetches its tiles with eight lanes per 128-byte row piece
+// (whole cache lines; fetching MFMA fragments directly would touch 64 lines per instruction),
+// DEPTH tiles in flight in registers, and turns a tile into fragments through a staging area in
+// LDS that is private to the wave, so the main loop has no workgroup barrier.  The small
+// activation matrix takes the same route and is served by the caches.  The partial sums of the
+// waves are added in LDS (integers: the order does not matter), then every thread scales and
+// writes four consecutive columns of one row.
+// ---------------------------------------------------------------------------------------------
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+
+template <int TM, int WAVES>
+constexpr int skinny_lds_bytes() { return WAVES * (1 + TM) * 32 * kBK + TM * 16 * 64 * 4; }
+
+template <int TM, int WAVES, int DEPTH, int OUT, bool FLEX>
+__global__ __launch_bounds__(64 * WAVES) void gemm_w8a8_skinny_kernel(QaGemmW8A8Params p) {
+    constexpr int kThreads = 64 * WAVES;
+    constexpr int kOob = 0x7ffffff0;                       // beyond any buffer: the load returns zeros
+    constexpr int kTile = 32 * kBK;                        // one staged 32-row tile
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    int* red = reinterpret_cast<int*>(lds + WAVES * (1 + TM) * kTile);   // [row block][acc register][lane]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int frow = lane & 31, fhalf = lane >> 5;
+    const int n0 = blockIdx.x * 32;
+    for (int i = tid; i < TM * 16 * 64; i += kThreads) red[i] = 0;
+
+    const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<int8_t*>(p.w), 0, static_cast<int>((static_cast<int64_t>(p.n) - 1) * p.ldw + p.k), kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<int8_t*>(p.a), 0, static_cast<int>((static_cast<int64_t>(p.m) - 1) * p.lda + p.k), kRsrcFlags);
+    // fetch mapping: instruction i, lane l -> tile row 8i + l/8, 16-byte chunk l%8
+    const int lrow = lane >> 3, lchunk = lane & 7;
+    int w_off[4], a_off[TM][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int row = n0 + 8 * i + lrow;
+        w_off[i] = row < p.n ? static_cast<int>(row * p.ldw) + lchunk * 16 : -1;
+#pragma unroll
+        for (int j = 0; j < TM; ++j) {
+            const int arow = j * 32 + 8 * i + lrow;
+            a_off[j][i] = arow < p.m ? static_cast<int>(arow * p.lda) + lchunk * 16 : -1;
+        }
+    }
+
+    const int k_tiles = (p.k + kBK - 1) / kBK;
+    const int my_tiles = (k_tiles - wave + WAVES - 1) / WAVES;      // tiles wave, wave + WAVES, ...
+    v4u fw[DEPTH][4], fa[DEPTH][TM][4];
+    auto load = [&](int i_tile, auto buf_c) {
+        constexpr int buf = decltype(buf_c)::value;
+        const int k0 = (wave + i_tile * WAVES) * kBK;
+        const bool k_ok = k0 + lchunk * 16 < p.k;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            fw[buf][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, (k_ok && w_off[i] >= 0) ? w_off[i] + k0 : kOob, 0, 0);
+#pragma unroll
+            for (int j = 0; j < TM; ++j) {
+                fa[buf][j][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, (k_ok && a_off[j][i] >= 0) ? a_off[j][i] + k0 : kOob, 0, 0);
+            }
+        }
+    };
+
+    v16i acc[TM];
+#pragma unroll
+    for (int j = 0; j < TM; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[j][r] = 0;
+
+    uint8_t* stage = lds + wave * ((1 + TM) * kTile);
+    static_for<0, DEPTH - 1>([&](auto s) { load(decltype(s)::value, s); });
+    for (int base = 0; base < my_tiles; base += DEPTH) {
+        static_for<0, DEPTH>([&](auto s_c) {
+            constexpr int s = decltype(s_c)::value;
+            // tiles past this wave's share are outside K: their loads touch no memory
+            load(base + s + DEPTH - 1, std::integral_constant<int, (s + DEPTH - 1) % DEPTH>{});
+            if (base + s < my_tiles) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int row = 8 * i + lrow;
+                    *reinterpret_cast<v4u*>(stage + row * kBK + swz(row, lchunk) * 16) = fw[s][i];
+#pragma unroll
+                    for (int j = 0; j < TM; ++j)
+                        *reinterpret_cast<v4u*>(stage + (1 + j) * kTile + row * kBK + swz(row, lchunk) * 16) = fa[s][j][i];
+                }
+                wave_lds_sync();
+#pragma unroll
+                for (int kk = 0; kk < 4; ++kk) {
+                    const int off = frow * kBK + swz(frow, kk * 2 + fhalf) * 16;
+                    const v4i bw = *reinterpret_cast<const v4i*>(stage + off);
+#pragma unroll
+                    for (int j = 0; j < TM; ++j) {
+                        const v4i ba = *reinterpret_cast<const v4i*>(stage + (1 + j) * kTile + off);
+                        acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bw, ba, acc[j], 0, 0, 0);
+                    }
+                }
+                wave_lds_sync();
+            }
+        });
+    }
+
+    __syncthreads();                                       // red is zero
+#pragma unroll
+    for (int j = 0; j < TM; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+            __hip_atomic_fetch_add(&red[(j * 16 + r) * 64 + lane], acc[j][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    __syncthreads();
+
+    // lane l of the accumulator layout holds row (l & 31) and, in registers 4q..4q+3, the columns
+    // 8q + 4*(l >> 5) + (0..3): one unit = (row block, q, lane)
+    constexpr int kElt = OUT == QA_OUT_I8 ? 1 : 2;
+    const bool use_alpha = FLEX && p.use_alpha;
+    const bool away = FLEX && p.round_mode == QA_ROUND_HALF_AWAY;
+    const int round_mode = FLEX ? p.round_mode : QA_ROUND_RNE;
+    const bool vec_ok = (p.ldd * kElt) % (4 * kElt) == 0 && (reinterpret_cast<uintptr_t>(p.d) & (4 * kElt - 1)) == 0;
+    for (int u = tid; u < TM * 4 * 64; u += kThreads) {
+        const int ul = u & 63, j = u >> 8, q = (u >> 6) & 3;
+        const int mm = j * 32 + (ul & 31);
+        const int nn = n0 + 8 * q + 4 * (ul >> 5);
+        if (mm >= p.m || nn >= p.n) continue;
+        const float s_row = use_alpha ? p.alpha : p.a_scale[p.a_scale_numel == 1 ? 0 : mm];
+        float v[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const float accf = static_cast<float>(red[(j * 16 + q * 4 + t) * 64 + ul]);
+            const float s_col = use_alpha ? 1.0f : p.w_scale[p.w_scale_numel == 1 ? 0 : min(nn + t, p.n - 1)];
+            if (use_alpha) v[t] = s_row * accf;
+            else v[t] = away ? (s_col * s_row) * accf : s_row * (s_col * accf);
+            asm volatile("" : "+v"(v[t]));                 // the fp32 product is rounded on its own
+        }
+        const int cols = min(4, p.n - nn);
+        if (OUT == QA_OUT_I8) {
+            int8_t* dst = static_cast<int8_t*>(p.d) + static_cast<int64_t>(mm) * p.ldd + nn;
+            if (vec_ok && cols == 4) {
+                const uint32_t b0 = quant8(v[0], round_mode) & 0xff, b1 = quant8(v[1], round_mode) & 0xff;
+                const uint32_t b2 = quant8(v[2], round_mode) & 0xff, b3 = quant8(v[3], round_mode);
+                *reinterpret_cast<uint32_t*>(dst) = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+            } else {
+                for (int t = 0; t < cols; ++t) dst[t] = static_cast<int8_t>(quant8(v[t], round_mode));
+            }
+        } else {
+            __half* dst = static_cast<__half*>(p.d) + static_cast<int64_t>(mm) * p.ldd + nn;
+            if (vec_ok && cols == 4) {
+                const __half2 lo = __floats2half2_rn(v[0], v[1]), hi = __floats2half2_rn(v[2], v[3]);
+                uint2 pk;
+                pk.x = *reinterpret_cast<const uint32_t*>(&lo);
+                pk.y = *reinterpret_cast<const uint32_t*>(&hi);
+                *reinterpret_cast<uint2*>(dst) = pk;
+            } else {
+                for (int t = 0; t < cols; ++t) dst[t] = __float2half(v[t]);
+            }
+        }
+    }
+}
+
+template <int TM, int WAVES, int OUT, bool FLEX>
+int launch_skinny_one(const QaGemmW8A8Params& p, hipStream_t stream) {
+    constexpr int kLds = skinny_lds_bytes<TM, WAVES>();
+    auto kernel = gemm_w8a8_skinny_kernel<TM, WAVES, 3, OUT, FLEX>;
+    if (kLds > 65536) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                kLds) != hipSuccess) {
+            return check_launch();
+        }
+    }
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>((p.n + 31) / 32)), dim3(64 * WAVES), kLds, stream, p);
+    return check_launch();
+}
+
+template <int TM, int WAVES, bool FLEX>
+int launch_skinny(const QaGemmW8A8Params& p, hipStream_t stream) {
+    return p.out_type == QA_OUT_I8 ? launch_skinny_one<TM, WAVES, QA_OUT_I8, FLEX>(p, stream)
+                                   : launch_skinny_one<TM, WAVES, QA_OUT_F16, FLEX>(p, stream);
+}
+
+template <bool FLEX>
+int dispatch_skinny(const QaGemmW8A8Params& p, hipStream_t stream) {
+    // eight waves per workgroup when four would leave the chip short of waves and K is long enough to split
+    const bool wide = (p.n + 31) / 32 < 512 && p.k >= 16 * kBK;
+    if (p.m <= 32) return wide ? launch_skinny<1, 8, FLEX>(p, stream) : launch_skinny<1, 4, FLEX>(p, stream);
+    return wide ? launch_skinny<2, 8, FLEX>(p, stream) : launch_skinny<2, 4, FLEX>(p, stream);
+}
+
 }  // namespace
 }  // namespace qa
 
@@ -115,8 +303,10 @@ extern "C" int qa_gemm_w8a8(const QaGemmW8A8Params* p, void* stream_) {
     // operands are addressed with 32-bit byte offsets inside a buffer descriptor
     if (static_cast<int64_t>(p->m) * p->lda >= 0x70000000LL || static_cast<int64_t>(p->n) * p->ldw >= 0x70000000LL) return QA_ERR_SHAPE;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const bool flex = p->use_alpha || p->round_mode != QA_ROUND_RNE;
+    if (p->m <= 64) return flex ? dispatch_skinny<true>(*p, stream) : dispatch_skinny<false>(*p, stream);
     // the single-row rules (host alpha, round-half-away) only ever come with tiny M
-    if (p->use_alpha || p->round_mode != QA_ROUND_RNE) return launch_gemm<2, 2, 2, 2, 2, true>(*p, stream);
+    if (flex) return launch_gemm<2, 2, 2, 2, 2, true>(*p, stream);
     const int64_t big_tiles = static_cast<int64_t>((p->m + 255) / 256) * ((p->n + 255) / 256);
     if (big_tiles >= 192) {
         // One workgroup per CU at a time: the launch runs in rounds of `cus` tiles, so a tile count

@@ -5,6 +5,8 @@
 #include <hip/hip_fp16.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "../../include/quamba_amd.h"
 
 namespace qa {
@@ -19,6 +21,15 @@ inline int check_launch() {
         return QA_ERR_LAUNCH;
     }
     return QA_OK;
+}
+
+// f(integral_constant<int, I>) for I = FIRST .. LAST-1: a loop whose index is a compile-time constant
+template <int FIRST, int LAST, typename F>
+__host__ __device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (FIRST < LAST) {
+        f(std::integral_constant<int, FIRST>{});
+        static_for<FIRST + 1, LAST>(f);
+    }
 }
 
 __host__ __device__ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

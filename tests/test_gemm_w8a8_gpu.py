@@ -26,7 +26,10 @@ def _operands(M, N, K, seed):
 
 # (M, N, K): tile-aligned, ragged in every dimension, tiny, single row, big-tile path
 SHAPES = [(256, 256, 128), (128, 128, 64), (300, 200, 208), (1, 48, 64), (17, 33, 16), (70, 1000, 1536),
-          (2048, 4096, 256), (4096, 4112, 320), (64, 16, 2560)]
+          (2048, 4096, 256), (4096, 4112, 320), (64, 16, 2560),
+          # few rows (the decode step's kernel): one and two row blocks, K split over four and eight waves,
+          # a K that ends inside a 32-byte step, fewer K tiles than waves
+          (33, 100, 5120), (5, 200, 2064), (64, 5120, 160), (1, 2560, 5120), (32, 10240, 2560), (65, 96, 4096)]
 
 
 @pytest.mark.parametrize("M,N,K", SHAPES)
@@ -43,7 +46,8 @@ def test_int8_output_bit_exact(dev, M, N, K, per_row, per_col):
     assert np.abs(want).max() > 20
 
 
-@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (300, 200, 208), (33, 24, 48), (2048, 2560, 512)])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (300, 200, 208), (33, 24, 48), (2048, 2560, 512),
+                                   (64, 2560, 5120), (7, 50, 4112)])
 def test_fp16_output_bit_exact(dev, M, N, K):
     a, w, sa, sb = _operands(M, N, K, seed=3 * M + K)
     _, f, _ = oracle.gemm_w8a8(a, w, sa[:1], sb)
