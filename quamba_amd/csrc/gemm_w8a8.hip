@@ -279,8 +279,10 @@ int launch_skinny(const QaGemmW8A8Params& p, hipStream_t stream) {
 
 template <bool FLEX>
 int dispatch_skinny(const QaGemmW8A8Params& p, hipStream_t stream) {
-    // eight waves per workgroup when four would leave the chip short of waves and K is long enough to split
-    const bool wide = (p.n + 31) / 32 < 512 && p.k >= 16 * kBK;
+    // Four waves per workgroup once there is at least one workgroup per CU (measured: more, smaller
+    // shares only add per-workgroup overhead); eight when the columns alone give too few workgroups
+    // and K is long enough to split further.
+    const bool wide = (p.n + 31) / 32 < 256 && p.k >= 16 * kBK;
     if (p.m <= 32) return wide ? launch_skinny<1, 8, FLEX>(p, stream) : launch_skinny<1, 4, FLEX>(p, stream);
     return wide ? launch_skinny<2, 8, FLEX>(p, stream) : launch_skinny<2, 4, FLEX>(p, stream);
 }

@@ -108,7 +108,10 @@ class W8A8QMamba(nn.Module):
         x = self.conv1d.update(x, conv_state)
         x_db = self.x_proj(x)
         dt, B, C = torch.split(x_db, [self.dt_rank, self.d_state, self.d_state], dim=-1)
-        dt = self.dt_proj(dt.contiguous())
+        # the GEMM reads a row-strided operand in place when rows and base are 16-byte aligned
+        if dt.stride(0) % 16 or dt.data_ptr() % 16:
+            dt = dt.contiguous()
+        dt = self.dt_proj(dt)
         y, ssm_state = self.selective_scan.update(ssm_state, x, dt, B, C, z=z)
         out = self.out_proj(self.had(y))
         return out.unsqueeze(1), conv_state, ssm_state

@@ -36,6 +36,20 @@ def test_fp16_rows_bit_exact(dev, dim):
     assert np.abs(want).max() > 60
 
 
+@pytest.mark.parametrize("dim", [1536, 5120, 8192, 2560, 12288])
+def test_many_rows_take_the_one_lane_per_column_path(dev, dim):
+    """More than 128 rows: 128 lanes per row, a lane produces all outputs of its column (few rows use
+    four lanes per column).  The oracle is only run on a sample of the rows to keep the test short."""
+    rows = 200
+    x = _rows(rows, dim, seed=dim + 1)
+    scale = np.float32(1.0 / math.sqrt(dim) / 0.06)
+    got = ops.hadamard_quant(torch.from_numpy(x).to(dev), float(scale)).cpu().numpy()
+    pick = np.array([0, 1, 63, 128, 199])
+    np.testing.assert_array_equal(got[pick], oracle.hadamard_quant(x[pick], scale))
+    few = ops.hadamard_quant(torch.from_numpy(x[:100]).to(dev), float(scale)).cpu().numpy()
+    np.testing.assert_array_equal(got[:100], few)
+
+
 def test_fp32_input_and_leading_dims(dev):
     x = _rows(24, 5120, seed=3).astype(np.float32).reshape(2, 12, 5120)
     scale = np.float32(1.0 / math.sqrt(5120) / 0.05)
