@@ -22,6 +22,7 @@ namespace gemm {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
 constexpr int kBK = 128;                 // k-bytes per tile row
@@ -298,6 +299,76 @@ __device__ __forceinline__ void epilogue(const Epilogue& e, v16i (&acc)[TN][TM],
 template <int TM, int TN, int WAVES>
 constexpr int epilogue_lds_bytes() {
     return WAVES * 32 * ((TM > TN ? TM : TN) * 32 * 2 + 16);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Pieces shared by the kernels for few activation rows (one 32-column block per workgroup, K split
+// over the waves, a wave-private staging area of one weight tile and TM activation tiles).
+// ---------------------------------------------------------------------------------------------
+template <int TM, int WAVES>
+constexpr int skinny_lds_bytes() { return WAVES * (1 + TM) * 32 * kBK + TM * 16 * 64 * 4; }
+
+// Adds the waves' partial accumulators in `red` (TM*16*64 ints, zeroed by the caller before any
+// barrier it has passed), then every thread scales and writes four consecutive columns of one row.
+// Lane l of the accumulator layout holds row (l & 31) and, in registers 4q..4q+3, the columns
+// 8q + 4*(l >> 5) + (0..3): one unit = (row block, q, lane).
+template <int TM, int OUT, bool FLEX, bool TRANS>
+__device__ __forceinline__ void skinny_reduce_store(const Epilogue& e, v16i (&acc)[TM], int* red, int m, int n,
+                                                    int n0, int tid, int threads) {
+    const int lane = tid & 63;
+    __syncthreads();                                       // red is zero
+#pragma unroll
+    for (int j = 0; j < TM; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+            __hip_atomic_fetch_add(&red[(j * 16 + r) * 64 + lane], acc[j][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    __syncthreads();
+
+    constexpr int kElt = OUT == QA_OUT_I8 ? 1 : 2;
+    const bool use_alpha = FLEX && e.use_alpha;
+    const bool away = FLEX && e.round_mode == QA_ROUND_HALF_AWAY;
+    const int round_mode = FLEX ? e.round_mode : QA_ROUND_RNE;
+    const bool vec_ok = !TRANS && e.ldd % 4 == 0 && (reinterpret_cast<uintptr_t>(e.d) & (4 * kElt - 1)) == 0;
+    for (int u = tid; u < TM * 4 * 64; u += threads) {
+        const int ul = u & 63, j = u >> 8, q = (u >> 6) & 3;
+        const int mm = j * 32 + (ul & 31);
+        const int nn = n0 + 8 * q + 4 * (ul >> 5);
+        if (mm >= m || nn >= n) continue;
+        const float s_row = use_alpha ? e.alpha : e.row_scale[e.row_numel == 1 ? 0 : mm];
+        float v[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const float accf = static_cast<float>(red[(j * 16 + q * 4 + t) * 64 + ul]);
+            const float s_col = use_alpha ? 1.0f : e.col_scale[e.col_numel == 1 ? 0 : min(nn + t, n - 1)];
+            if (use_alpha) v[t] = s_row * accf;
+            else v[t] = away ? (s_col * s_row) * accf : s_row * (s_col * accf);
+            asm volatile("" : "+v"(v[t]));                 // the fp32 product is rounded on its own
+        }
+        const int cols = min(4, n - nn);
+        const int64_t step = TRANS ? e.ldd : 1;            // distance between consecutive columns
+        const int64_t at = TRANS ? static_cast<int64_t>(nn) * e.ldd + mm : static_cast<int64_t>(mm) * e.ldd + nn;
+        if (OUT == QA_OUT_I8) {
+            int8_t* dst = static_cast<int8_t*>(e.d) + at;
+            if (vec_ok && cols == 4) {
+                const uint32_t b0 = quant8(v[0], round_mode) & 0xff, b1 = quant8(v[1], round_mode) & 0xff;
+                const uint32_t b2 = quant8(v[2], round_mode) & 0xff, b3 = quant8(v[3], round_mode);
+                *reinterpret_cast<uint32_t*>(dst) = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+            } else {
+                for (int t = 0; t < cols; ++t) dst[t * step] = static_cast<int8_t>(quant8(v[t], round_mode));
+            }
+        } else {
+            __half* dst = static_cast<__half*>(e.d) + at;
+            if (vec_ok && cols == 4) {
+                const __half2 lo = __floats2half2_rn(v[0], v[1]), hi = __floats2half2_rn(v[2], v[3]);
+                uint2 pk;
+                pk.x = *reinterpret_cast<const uint32_t*>(&lo);
+                pk.y = *reinterpret_cast<const uint32_t*>(&hi);
+                *reinterpret_cast<uint2*>(dst) = pk;
+            } else {
+                for (int t = 0; t < cols; ++t) dst[t * step] = __float2half(v[t]);
+            }
+        }
+    }
 }
 
 }  // namespace gemm

@@ -179,6 +179,188 @@ int launch_gemm(const QaGemmW4A8Params& p, hipStream_t stream) {
                               : launch_one<TM, TN, WGM, WGN, QA_OUT_F16, false>(p, stream);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Few activation rows (M <= 64, the decode step): a stream over the packed weights.  A workgroup
+// owns 32 output columns and all rows; its WAVES waves split K between them in interleaved pieces
+// of 256 codes, i.e. one full 128-byte line of packed weights per row.  A wave fetches a piece with
+// eight lanes per row (DEPTH pieces in flight in registers), expands its 32 codes per lane to int8
+// and passes them through a staging area in LDS that is private to the wave; the activation tiles
+// take the same route, one 128-byte half at a time.  Partial sums meet in LDS at the end.
+// ---------------------------------------------------------------------------------------------
+template <int TM, int AI, int WAVES, int DEPTH, int OUT, bool TRANS>
+__global__ __launch_bounds__(64 * WAVES) void gemm_w4a8_skinny_kernel(QaGemmW4A8Params p) {
+    constexpr int kThreads = 64 * WAVES;
+    constexpr int kOob = 0x7ffffff0;                       // beyond any buffer: the load returns zeros
+    constexpr int kTile = 32 * kBK;
+    constexpr int kPiece = 2 * kBK;                        // codes per row and piece
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    int* red = reinterpret_cast<int*>(lds + WAVES * (2 + TM) * kTile);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int frow = lane & 31, fhalf = lane >> 5;
+    const int n0 = blockIdx.x * 32;
+    const bool grouped = p.group_size > 0;
+    for (int i = tid; i < TM * 16 * 64; i += kThreads) red[i] = 0;
+    uint8_t* stage = lds + wave * ((2 + TM) * kTile);          // two weight halves, TM activation tiles
+    if (AI < 4) {
+        // only the first 8*AI rows of an activation tile are ever fetched (M <= 8*AI): the rest stays zero
+        for (int i = lane; i < TM * kTile / 16; i += 64) reinterpret_cast<v4u*>(stage + 2 * kTile)[i] = v4u{0u, 0u, 0u, 0u};
+    }
+
+    const int ldw = p.k / 2;
+    const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t*>(p.w_packed), 0, static_cast<int>(static_cast<int64_t>(p.n) * ldw), kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<int8_t*>(p.a), 0, static_cast<int>((static_cast<int64_t>(p.m) - 1) * p.lda + p.k), kRsrcFlags);
+    // fetch mapping: instruction i, lane l -> tile row 8i + l/8, 16-byte chunk l%8.  A packed chunk is
+    // 32 codes: chunks 0..3 expand into the first 128-code half of the piece, 4..7 into the second.
+    const int lrow = lane >> 3, lchunk = lane & 7;
+    const int my_half = lchunk >> 2, my_c0 = (lchunk & 3) * 2;
+    int w_off[4], a_off[TM][AI], s_col[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int row = n0 + 8 * i + lrow;
+        w_off[i] = row < p.n ? row * ldw + lchunk * 16 : -1;
+        s_col[i] = min(row, p.n - 1);
+        if (i < AI) {
+#pragma unroll
+            for (int j = 0; j < TM; ++j) {
+                const int arow = j * 32 + 8 * i + lrow;
+                a_off[j][i] = arow < p.m ? static_cast<int>(arow * p.lda) + lchunk * 16 : -1;
+            }
+        }
+    }
+    const __half* sg = static_cast<const __half*>(p.s_group);
+    const int n_groups = p.k / kBK;
+
+    const int pieces = (p.k + kPiece - 1) / kPiece;
+    const int my_pieces = (pieces - wave + WAVES - 1) / WAVES;
+    v4u fw[DEPTH][4], fa[DEPTH][2][TM][AI];
+    __half fs[DEPTH][4];
+    auto load = [&](int i_piece, auto buf_c) {
+        constexpr int buf = decltype(buf_c)::value;
+        const int k0 = (wave + i_piece * WAVES) * kPiece;
+        const bool w_ok = k0 + lchunk * 32 < p.k;
+        const int group = min(k0 / kBK + my_half, n_groups - 1);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            fw[buf][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, (w_ok && w_off[i] >= 0) ? w_off[i] + k0 / 2 : kOob, 0, 0);
+            if (grouped) fs[buf][i] = sg[static_cast<int64_t>(group) * p.n + s_col[i]];
+            if (i < AI) {
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const bool a_k_ok = k0 + h * kBK + lchunk * 16 < p.k;
+#pragma unroll
+                    for (int j = 0; j < TM; ++j) {
+                        fa[buf][h][j][i] = __builtin_amdgcn_raw_buffer_load_b128(
+                            rsrc_a, (a_k_ok && a_off[j][i] >= 0) ? a_off[j][i] + k0 + h * kBK : kOob, 0, 0);
+                    }
+                }
+            }
+        }
+    };
+
+    v16i acc[TM];
+#pragma unroll
+    for (int j = 0; j < TM; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[j][r] = 0;
+
+    static_for<0, DEPTH - 1>([&](auto s) {
+        if (decltype(s)::value < my_pieces) load(decltype(s)::value, s);
+    });
+    for (int base = 0; base < my_pieces; base += DEPTH) {
+        static_for<0, DEPTH>([&](auto s_c) {
+            constexpr int s = decltype(s_c)::value;
+            if (base + s + DEPTH - 1 < my_pieces) load(base + s + DEPTH - 1, std::integral_constant<int, (s + DEPTH - 1) % DEPTH>{});
+            if (base + s < my_pieces) {
+                // expand this lane's 32 codes per fetched row into its half of the staged weights
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const uint32_t w[4] = {fw[s][i].x, fw[s][i].y, fw[s][i].z, fw[s][i].w};
+                    uint2 e[4];
+                    if (grouped) {
+                        const __half2 s2 = __half2half2(fs[s][i]);
+#pragma unroll
+                        for (int t = 0; t < 4; ++t) e[t] = expand_grouped(w[t], s2);
+                    } else {
+#pragma unroll
+                        for (int t = 0; t < 4; ++t) e[t] = expand_per_channel(w[t]);
+                    }
+                    const int row = 8 * i + lrow;
+                    uint8_t* dst = stage + my_half * kTile + row * kBK;
+                    *reinterpret_cast<v4u*>(dst + swz(row, my_c0) * 16) = v4u{e[0].x, e[0].y, e[1].x, e[1].y};
+                    *reinterpret_cast<v4u*>(dst + swz(row, my_c0 + 1) * 16) = v4u{e[2].x, e[2].y, e[3].x, e[3].y};
+                }
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+#pragma unroll
+                    for (int i = 0; i < AI; ++i) {
+                        const int row = 8 * i + lrow;
+#pragma unroll
+                        for (int j = 0; j < TM; ++j)
+                            *reinterpret_cast<v4u*>(stage + (2 + j) * kTile + row * kBK + swz(row, lchunk) * 16) = fa[s][h][j][i];
+                    }
+                    wave_lds_sync();
+#pragma unroll
+                    for (int kk = 0; kk < 4; ++kk) {
+                        const int off = frow * kBK + swz(frow, kk * 2 + fhalf) * 16;
+                        const v4i bw = *reinterpret_cast<const v4i*>(stage + h * kTile + off);
+#pragma unroll
+                        for (int j = 0; j < TM; ++j) {
+                            const v4i ba = *reinterpret_cast<const v4i*>(stage + (2 + j) * kTile + off);
+                            acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bw, ba, acc[j], 0, 0, 0);
+                        }
+                    }
+                    wave_lds_sync();
+                }
+            }
+        });
+    }
+
+    Epilogue e;
+    e.row_scale = p.s_token; e.col_scale = p.s_channel;
+    e.row_numel = p.tok_scale_numel; e.col_numel = p.n;
+    e.use_alpha = 0; e.alpha = 0.0f; e.round_mode = QA_ROUND_RNE;
+    e.ldd = p.ldd; e.d = p.d;
+    skinny_reduce_store<TM, OUT, false, TRANS>(e, acc, red, p.m, p.n, n0, tid, kThreads);
+}
+
+template <int TM, int AI, int WAVES, int DEPTH, int OUT, bool TRANS>
+int launch_skinny_one(const QaGemmW4A8Params& p, hipStream_t stream) {
+    constexpr int kLds = skinny_lds_bytes<TM + 1, WAVES>() - 16 * 64 * 4;   // (2 + TM) tiles per wave, TM reduction blocks
+    auto kernel = gemm_w4a8_skinny_kernel<TM, AI, WAVES, DEPTH, OUT, TRANS>;
+    if (kLds > 65536) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                kLds) != hipSuccess) {
+            return check_launch();
+        }
+    }
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>((p.n + 31) / 32)), dim3(64 * WAVES), kLds, stream, p);
+    return check_launch();
+}
+
+template <int TM, int AI, int WAVES, int DEPTH>
+int launch_skinny(const QaGemmW4A8Params& p, hipStream_t stream) {
+    if (p.out_type == QA_OUT_I8) {
+        return p.output_transpose ? launch_skinny_one<TM, AI, WAVES, DEPTH, QA_OUT_I8, true>(p, stream)
+                                  : launch_skinny_one<TM, AI, WAVES, DEPTH, QA_OUT_I8, false>(p, stream);
+    }
+    return p.output_transpose ? launch_skinny_one<TM, AI, WAVES, DEPTH, QA_OUT_F16, true>(p, stream)
+                              : launch_skinny_one<TM, AI, WAVES, DEPTH, QA_OUT_F16, false>(p, stream);
+}
+
+int dispatch_skinny(const QaGemmW4A8Params& p, hipStream_t stream) {
+    // four waves per workgroup once the columns give a workgroup per CU, else eight when K is long enough
+    const bool wide = (p.n + 31) / 32 < 256 && p.k >= 16 * 2 * kBK;
+    // activation rows are fetched eight at a time: up to 8 rows need one fetch per tile, up to 32 four
+    if (p.m <= 8) return wide ? launch_skinny<1, 1, 8, 3>(p, stream) : launch_skinny<1, 1, 4, 3>(p, stream);
+    if (p.m <= 32) return wide ? launch_skinny<1, 4, 8, 2>(p, stream) : launch_skinny<1, 4, 4, 2>(p, stream);
+    return wide ? launch_skinny<2, 4, 8, 2>(p, stream) : launch_skinny<2, 4, 4, 2>(p, stream);
+}
+
 }  // namespace
 }  // namespace qa
 
@@ -196,6 +378,7 @@ extern "C" int qa_gemm_w4a8(const QaGemmW4A8Params* p, void* stream_) {
     if (p->m == 0 || p->n == 0) return QA_OK;
     if (static_cast<int64_t>(p->m) * p->lda >= 0x70000000LL) return QA_ERR_SHAPE;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (p->m <= 64 && static_cast<int64_t>(p->n) * (p->k / 2) < 0x70000000LL) return dispatch_skinny(*p, stream);
     const int64_t big_tiles = static_cast<int64_t>((p->m + 255) / 256) * ((p->n + 255) / 256);
     if (big_tiles >= 192) return launch_gemm<4, 2, 2, 4>(*p, stream);
     return launch_gemm<2, 2, 2, 2>(*p, stream);

@@ -109,11 +109,6 @@ int launch_gemm(const QaGemmW8A8Params& p, hipStream_t stream) {
 // waves are added in LDS (integers: the order does not matter), then every thread scales and
 // writes four consecutive columns of one row.
 // ---------------------------------------------------------------------------------------------
-typedef unsigned int v4u __attribute__((ext_vector_type(4)));
-
-template <int TM, int WAVES>
-constexpr int skinny_lds_bytes() { return WAVES * (1 + TM) * 32 * kBK + TM * 16 * 64 * 4; }
-
 template <int TM, int WAVES, int DEPTH, int OUT, bool FLEX>
 __global__ __launch_bounds__(64 * WAVES) void gemm_w8a8_skinny_kernel(QaGemmW8A8Params p) {
     constexpr int kThreads = 64 * WAVES;
@@ -202,59 +197,12 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_w8a8_skinny_kernel(QaGemmW8A8
         });
     }
 
-    __syncthreads();                                       // red is zero
-#pragma unroll
-    for (int j = 0; j < TM; ++j)
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-            __hip_atomic_fetch_add(&red[(j * 16 + r) * 64 + lane], acc[j][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    __syncthreads();
-
-    // lane l of the accumulator layout holds row (l & 31) and, in registers 4q..4q+3, the columns
-    // 8q + 4*(l >> 5) + (0..3): one unit = (row block, q, lane)
-    constexpr int kElt = OUT == QA_OUT_I8 ? 1 : 2;
-    const bool use_alpha = FLEX && p.use_alpha;
-    const bool away = FLEX && p.round_mode == QA_ROUND_HALF_AWAY;
-    const int round_mode = FLEX ? p.round_mode : QA_ROUND_RNE;
-    const bool vec_ok = (p.ldd * kElt) % (4 * kElt) == 0 && (reinterpret_cast<uintptr_t>(p.d) & (4 * kElt - 1)) == 0;
-    for (int u = tid; u < TM * 4 * 64; u += kThreads) {
-        const int ul = u & 63, j = u >> 8, q = (u >> 6) & 3;
-        const int mm = j * 32 + (ul & 31);
-        const int nn = n0 + 8 * q + 4 * (ul >> 5);
-        if (mm >= p.m || nn >= p.n) continue;
-        const float s_row = use_alpha ? p.alpha : p.a_scale[p.a_scale_numel == 1 ? 0 : mm];
-        float v[4];
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            const float accf = static_cast<float>(red[(j * 16 + q * 4 + t) * 64 + ul]);
-            const float s_col = use_alpha ? 1.0f : p.w_scale[p.w_scale_numel == 1 ? 0 : min(nn + t, p.n - 1)];
-            if (use_alpha) v[t] = s_row * accf;
-            else v[t] = away ? (s_col * s_row) * accf : s_row * (s_col * accf);
-            asm volatile("" : "+v"(v[t]));                 // the fp32 product is rounded on its own
-        }
-        const int cols = min(4, p.n - nn);
-        if (OUT == QA_OUT_I8) {
-            int8_t* dst = static_cast<int8_t*>(p.d) + static_cast<int64_t>(mm) * p.ldd + nn;
-            if (vec_ok && cols == 4) {
-                const uint32_t b0 = quant8(v[0], round_mode) & 0xff, b1 = quant8(v[1], round_mode) & 0xff;
-                const uint32_t b2 = quant8(v[2], round_mode) & 0xff, b3 = quant8(v[3], round_mode);
-                *reinterpret_cast<uint32_t*>(dst) = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
-            } else {
-                for (int t = 0; t < cols; ++t) dst[t] = static_cast<int8_t>(quant8(v[t], round_mode));
-            }
-        } else {
-            __half* dst = static_cast<__half*>(p.d) + static_cast<int64_t>(mm) * p.ldd + nn;
-            if (vec_ok && cols == 4) {
-                const __half2 lo = __floats2half2_rn(v[0], v[1]), hi = __floats2half2_rn(v[2], v[3]);
-                uint2 pk;
-                pk.x = *reinterpret_cast<const uint32_t*>(&lo);
-                pk.y = *reinterpret_cast<const uint32_t*>(&hi);
-                *reinterpret_cast<uint2*>(dst) = pk;
-            } else {
-                for (int t = 0; t < cols; ++t) dst[t] = __float2half(v[t]);
-            }
-        }
-    }
+    Epilogue e;
+    e.row_scale = p.a_scale; e.col_scale = p.w_scale;
+    e.row_numel = p.a_scale_numel; e.col_numel = p.w_scale_numel;
+    e.use_alpha = p.use_alpha; e.alpha = p.alpha; e.round_mode = p.round_mode;
+    e.ldd = p.ldd; e.d = p.d;
+    skinny_reduce_store<TM, OUT, FLEX, false>(e, acc, red, p.m, p.n, n0, tid, kThreads);
 }
 
 template <int TM, int WAVES, int OUT, bool FLEX>

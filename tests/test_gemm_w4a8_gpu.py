@@ -38,7 +38,10 @@ def _run(dev, a, codes, sg, sc, st, out8, transpose=False, per_token=True):
               None, M, N, K, transpose)
 
 
-SHAPES = [(256, 256, 128), (300, 200, 384), (17, 70, 256), (1, 64, 128), (2048, 1024, 512), (4096, 4160, 1024)]
+SHAPES = [(256, 256, 128), (300, 200, 384), (17, 70, 256), (1, 64, 128), (2048, 1024, 512), (4096, 4160, 1024),
+          # few rows (the decode step's kernel): one and two row blocks, K split over four and eight waves,
+          # a K that ends in the middle of a 256-code piece, fewer pieces than waves
+          (1, 4096, 8192), (33, 100, 4224), (64, 9000, 1280), (5, 200, 384), (65, 96, 4096)]
 
 
 @pytest.mark.parametrize("M,N,K", SHAPES)
@@ -52,7 +55,7 @@ def test_int8_output_bit_exact(dev, M, N, K, grouped):
     assert np.abs(want).max() > 20
 
 
-@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (300, 200, 384), (2048, 1024, 512)])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (300, 200, 384), (2048, 1024, 512), (64, 520, 4352), (3, 70, 640)])
 def test_fp16_and_transposed_outputs_bit_exact(dev, M, N, K):
     a, codes, sg, sc, st = _case(M, N, K, 7 * M + K)
     _, _, f, q = oracle.gemm_w4a8(a, codes, sg, sc, st[:1])
