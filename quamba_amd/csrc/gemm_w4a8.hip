@@ -12,9 +12,9 @@
 // nibble, so that the fp16 exponent trick below yields the int8 bytes in k order.
 // The expansion to int8 runs in registers on the way from global memory to LDS (once per
 // workgroup, not once per wave): (word & 0x000f000f) | 0x6400_6400 is the half2 (1024+c0, 1024+c2);
-// subtracting 1032 gives c-8 exactly; one packed FMA with the group scale and the constant 1152
-// leaves rne((c-8)*s) + 128 in the low byte of each half; v_perm gathers four bytes and an XOR with
-// 0x80 turns them into int8.  Everything else is the shared core in gemm_core.hpp.
+// subtracting 1032 gives c-8 exactly; one packed FMA with the group scale and the constant 1280
+// leaves rne((c-8)*s) as a two's-complement byte in the low byte of each half; v_perm gathers four
+// of them.  Everything else is the shared core in gemm_core.hpp.
 #include "gemm_core.hpp"
 
 namespace qa {
@@ -25,22 +25,32 @@ using namespace gemm;
 __device__ __forceinline__ uint32_t h2_bits(__half2 v) { return *reinterpret_cast<uint32_t*>(&v); }
 __device__ __forceinline__ __half2 bits_h2(uint32_t v) { return *reinterpret_cast<__half2*>(&v); }
 
-// 8 codes (one word) -> 8 int8 in k order (two words), grouped mode.
+// (x & mask) | bits in one instruction; `bits` is held in a vector register because the encoding
+// takes a single scalar or literal operand.
+__device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t bits) {
+    uint32_t r;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "s"(mask), "v"(bits));
+    return r;
+}
+
+// 8 codes (one word) -> 8 int8 in k order (two words), grouped mode.  The rounding constant 1280
+// (ulp 1, a multiple of 256) leaves the two's-complement byte of rne((c-8)*s) in the low byte.
 __device__ __forceinline__ uint2 expand_grouped(uint32_t p, __half2 s2) {
     const __half2 k1032 = bits_h2(0x64086408u);      // 1032, 1032
     const __half2 k16th = bits_h2(0x2c002c00u);      // 1/16
     const __half2 km72 = bits_h2(0xd480d480u);       // -72
-    const __half2 k1152 = bits_h2(0x64806480u);      // 1152
+    const __half2 k1280 = bits_h2(0x65006500u);      // 1280
+    const uint32_t kOne = 0x64006400u;               // 1024, 1024
     const uint32_t q = p >> 8;
-    const __half2 a = __hsub2(bits_h2((p & 0x000f000fu) | 0x64006400u), k1032);            // c0-8, c2-8
-    const __half2 b = __hfma2(bits_h2((p & 0x00f000f0u) | 0x64006400u), k16th, km72);      // c4-8, c6-8
-    const __half2 c = __hsub2(bits_h2((q & 0x000f000fu) | 0x64006400u), k1032);            // c1-8, c3-8
-    const __half2 d = __hfma2(bits_h2((q & 0x00f000f0u) | 0x64006400u), k16th, km72);      // c5-8, c7-8
-    const uint32_t ra = h2_bits(__hfma2(a, s2, k1152)), rb = h2_bits(__hfma2(b, s2, k1152));
-    const uint32_t rc = h2_bits(__hfma2(c, s2, k1152)), rd = h2_bits(__hfma2(d, s2, k1152));
+    const __half2 a = __hsub2(bits_h2(and_or(p, 0x000f000fu, kOne)), k1032);            // c0-8, c2-8
+    const __half2 b = __hfma2(bits_h2(and_or(p, 0x00f000f0u, kOne)), k16th, km72);      // c4-8, c6-8
+    const __half2 c = __hsub2(bits_h2(and_or(q, 0x000f000fu, kOne)), k1032);            // c1-8, c3-8
+    const __half2 d = __hfma2(bits_h2(and_or(q, 0x00f000f0u, kOne)), k16th, km72);      // c5-8, c7-8
+    const uint32_t ra = h2_bits(__hfma2(a, s2, k1280)), rb = h2_bits(__hfma2(b, s2, k1280));
+    const uint32_t rc = h2_bits(__hfma2(c, s2, k1280)), rd = h2_bits(__hfma2(d, s2, k1280));
     uint2 out;
-    out.x = __builtin_amdgcn_perm(rc, ra, 0x06020400u) ^ 0x80808080u;    // k0 k1 k2 k3
-    out.y = __builtin_amdgcn_perm(rd, rb, 0x06020400u) ^ 0x80808080u;    // k4 k5 k6 k7
+    out.x = __builtin_amdgcn_perm(rc, ra, 0x06020400u);    // k0 k1 k2 k3
+    out.y = __builtin_amdgcn_perm(rd, rb, 0x06020400u);    // k4 k5 k6 k7
     return out;
 }
 
