@@ -218,6 +218,43 @@ def other_workloads(dev, steps, warmup):
     out.append(dict(workload="Mamba1-2.8b decode step (conv update + state update), batch 64, fp32 state, HIP graph of 16 steps",
                     us=ms * 1e3, us_eager_python=ms_eager * 1e3, tokens_per_s=B / ms * 1e3, bound="hbm",
                     achieved_GBs=nbytes / ms / 1e6, frac=nbytes / ms / 1e6 / HBM_PEAK_GBS))
+    # the whole Mamba1-2.8b mixer for one token (in_proj, conv update, x_proj, dt_proj, state update, Hadamard,
+    # out_proj): eight layers with their own weights (330 MB, more than the last-level cache holds) in one graph
+    from quamba_amd import W8A8QMamba
+    layers = []
+    for _ in range(8):
+        m = W8A8QMamba(2560, 16, 4, device=dev, state_dtype=torch.float32)
+        for name in ("in_proj", "x_proj", "dt_proj", "out_proj"):
+            lin = getattr(m, name)
+            lin._set_weight(ri(lin.out_features, lin.in_features))
+            lin.a, lin.b, lin.alpha = sc(0.5).view(1, 1), sc(1e-3).view(1, 1), 5e-4
+        m.conv1d.weight, m.conv1d.bias = ri(D, 4), ri(D)
+        m.conv1d.input_scale = m.conv1d.weight_scale = m.conv1d.bias_scale = 0.01
+        m.conv1d.output_scale = 0.02
+        m.selective_scan.A_log, m.selective_scan.D, m.selective_scan.dt_bias = ri(D, N), ri(D), ri(D)
+        m.had.x_H_scale = 0.05
+        layers.append(m)
+    w_bytes = sum(getattr(layers[0], n).weight.numel() for n in ("in_proj", "x_proj", "dt_proj", "out_proj"))
+    for B in (1, 64):
+        states = [m.allocate_inference_cache(B) for m in layers]
+        h = ri(B, 1, 2560)
+
+        def token():
+            for m, (cs, ss) in zip(layers, states):
+                m.step(h, cs, ss)
+        for _ in range(3):
+            token()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            token()
+        ms = _time_fn(graph.replay, 64, 4) / len(layers)
+        nbytes = w_bytes + B * (2 * D * N * 4 + 2 * D * 3 + 2560 + 2 * 2560)
+        out.append(dict(workload=f"Mamba1-2.8b W8A8 mixer, one token (all seven kernels), batch {B}, HIP graph over 8 layers",
+                        us=ms * 1e3, tokens_per_s=B / ms * 1e3, bound="hbm", achieved_GBs=nbytes / ms / 1e6,
+                        frac=nbytes / ms / 1e6 / HBM_PEAK_GBS))
+        del graph, states
+    del layers
     # SSD: batch 4, seqlen 4096, 80 heads of 64, d_state 128, 1 group, chunk 256
     B, L, H, N, G, Q = 4, 4096, 80, 128, 1, 256
     x, dt, Bm, Cm = ri(B, L, H, 64), ri(B, L, H), ri(B, L, G, N), ri(B, L, G, N)
@@ -270,6 +307,31 @@ def other_workloads(dev, steps, warmup):
         tops = 2.0 * M * Nn * K / ms / 1e9
         out.append(dict(workload=f"Mamba2-8b W4A8 {name} {M}x{K}->{Nn}", us=ms * 1e3, tokens_per_s=M / ms * 1e3, bound="mfma",
                         achieved_TOPs=tops, frac=tops / INT8_PEAK_TOPS))
+        # the same layer for one token: a stream over the packed weights (eight copies in turn: 300 MB)
+        del a, w
+        ws = [torch.randint(0, 256, (Nn, K // 2), dtype=torch.uint8, device=dev) for _ in range(8)]
+        a1, s_tok1 = ri(1, K), torch.ones(1, device=dev)
+        for w in ws:
+            fn(a1, w, s_tok1, s_ch, sg, None, 1, Nn, K, False)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for w in ws:
+                fn(a1, w, s_tok1, s_ch, sg, None, 1, Nn, K, False)
+        ms = _time_fn(graph.replay, 64, 4) / len(ws)
+        nbytes = Nn * K // 2 + Nn * (K // 128) * 2
+        out.append(dict(workload=f"Mamba2-8b W4A8 {name} for one token, 1x{K}->{Nn}, HIP graph", us=ms * 1e3,
+                        tokens_per_s=1 / ms * 1e3, bound="hbm", achieved_GBs=nbytes / ms / 1e6,
+                        frac=nbytes / ms / 1e6 / HBM_PEAK_GBS))
+        del graph, ws
+    # gated RMS norm of the Mamba2-8b mixer: 16384 rows x 8192, fp16 in, int8 gate, fp16 out
+    xn = torch.randn(16384, 8192, device=dev, dtype=torch.float16)
+    zn, wn = ri(16384, 8192), torch.ones(8192, device=dev, dtype=torch.float16)
+    ms = _time_fn(lambda: ops.qlayer_normgated_fwd(xn, wn, None, 1e-5, q_z=zn, z_scale=0.02, use_float16_output=True, group_size=8192, norm_before_gate=False), steps, warmup)
+    nbytes = 16384 * 8192 * (2 + 1 + 2)
+    out.append(dict(workload="gated RMS norm, 16384 rows x 8192 (fp16 in, int8 gate, fp16 out)", us=ms * 1e3,
+                    tokens_per_s=16384 / ms * 1e3, bound="hbm", achieved_GBs=nbytes / ms / 1e6,
+                    frac=nbytes / ms / 1e6 / HBM_PEAK_GBS))
     return out
 
 

@@ -368,7 +368,9 @@ int dispatch_skinny(const QaGemmW4A8Params& p, hipStream_t stream) {
     // activation rows are fetched eight at a time: up to 8 rows need one fetch per tile, up to 32 four
     if (p.m <= 8) return wide ? launch_skinny<1, 1, 8, 3>(p, stream) : launch_skinny<1, 1, 4, 3>(p, stream);
     if (p.m <= 32) return wide ? launch_skinny<1, 4, 8, 2>(p, stream) : launch_skinny<1, 4, 4, 2>(p, stream);
-    return wide ? launch_skinny<2, 4, 8, 2>(p, stream) : launch_skinny<2, 4, 4, 2>(p, stream);
+    // two row blocks: a wave's registers allow one workgroup of eight waves or two of four per CU, and
+    // eight waves measured faster whenever K has at least two pieces per wave
+    return (wide || p.k >= 16 * 2 * kBK) ? launch_skinny<2, 4, 8, 2>(p, stream) : launch_skinny<2, 4, 4, 2>(p, stream);
 }
 
 }  // namespace

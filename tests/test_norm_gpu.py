@@ -37,7 +37,9 @@ def _int8_close(got, y, scale):
 
 
 # (rows, dim, group_size): Mamba2-8b (8192 in groups of 1024), 2.7b (5120, one group), small, ragged pieces
-SHAPES = [(33, 8192, 1024), (17, 5120, None), (8, 256, 64), (5, 1536, 1536), (3, 8192, None), (4, 2560, 40 * 8)]
+SHAPES = [(33, 8192, 1024), (17, 5120, None), (8, 256, 64), (5, 1536, 1536), (3, 8192, None), (4, 2560, 40 * 8),
+          # groups wider than 2048 columns are shared by four waves: ragged last piece, widest form
+          (3, 2560, None), (2, 16384, None), (5, 4096, 2048)]
 
 
 @pytest.mark.parametrize("M,N,group_size", SHAPES)
