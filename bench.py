@@ -260,8 +260,10 @@ def other_workloads(dev, steps, warmup):
     x, dt, Bm, Cm = ri(B, L, H, 64), ri(B, L, H), ri(B, L, G, N), ri(B, L, G, N)
     A2, D2 = ri(H), ri(H)
     bias = torch.zeros(H, dtype=torch.float16, device=dev)
-    ssd = lambda: ops.ssd_chunk_scan_combined_fwd(x, sc(0.03), dt, sc(0.02), A2, sc(0.02), Bm, sc(0.03), Cm, sc(0.03), None, Q,
-                                                  q_D=D2, D_scale=sc(0.008), dt_bias=bias, dt_softplus=True,
+    # scales live on the device before the timed region (creating one is a blocking host-to-device copy)
+    k_x, k_dt, k_A, k_B, k_C, k_D = (sc(v) for v in (0.03, 0.02, 0.02, 0.03, 0.03, 0.008))
+    ssd = lambda: ops.ssd_chunk_scan_combined_fwd(x, k_x, dt, k_dt, A2, k_A, Bm, k_B, Cm, k_C, None, Q,
+                                                  q_D=D2, D_scale=k_D, dt_bias=bias, dt_softplus=True,
                                                   final_state_dtype=torch.float32)
     ms = _time_fn(ssd, steps, warmup)
     nbytes = B * L * H * 64 + 2 * B * L * G * N + B * L * H + 2 * B * L * H * 64 + 4 * B * H * 64 * N
