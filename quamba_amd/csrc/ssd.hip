@@ -36,7 +36,7 @@ __device__ __forceinline__ void wave_sync() {
 __device__ __forceinline__ int8_t byte_of(uint32_t w, int j) { return static_cast<int8_t>((w >> (8 * j)) & 0xffu); }
 
 struct Ws {            // workspace sections (byte offsets), see qa_ssd_workspace_bytes
-    int64_t dt, dA, cb, states, prev, final_f32, total;
+    int64_t dt, dA, cb, states, prev, final_f32, c16, total;
 };
 
 __host__ __device__ inline int64_t align256(int64_t v) { return (v + 255) & ~int64_t(255); }
@@ -52,6 +52,7 @@ __host__ __device__ inline Ws ws_layout(const QaSsdParams& p) {
     w.states = off; off = align256(off + B * nc * H * P * N * 4);
     w.prev = off; off = align256(off + B * nc * H * P * N * 2);
     w.final_f32 = off; off = align256(off + B * H * P * N * 4);
+    w.c16 = off; off = align256(off + B * static_cast<int64_t>(p.seqlen) * G * N * 2);
     w.total = off;
     return w;
 }
@@ -130,9 +131,11 @@ __global__ __launch_bounds__(256) void ssd_cumsum_kernel(QaSsdParams p, float* d
 
 // ---------------------------------------------------------------------------------------------
 // Stage 4 (quamba/triton/quant_bmm_chunk.py:60-66): one wave per 64x64 tile of CB, lower tiles only.
-// Both operands are rows of dstate int8 values, i.e. already MFMA operands.
+// Both operands are rows of dstate int8 values, i.e. already MFMA operands.  The diagonal tiles also
+// write their C rows dequantised to fp16 (f16(s_C * q_C)): every head of the group multiplies those
+// rows with its entering state in the chunk scan, which then reads them ready-made.
 // ---------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(64) void ssd_cb_kernel(QaSsdParams p, float* cb_out, int nc) {
+__global__ __launch_bounds__(64) void ssd_cb_kernel(QaSsdParams p, float* cb_out, __half* c16_out, int nc) {
     const int Q = p.chunk_size, N = p.dstate, G = p.ngroups;
     const int nt = Q / 64;
     // blockIdx.x enumerates lower-triangular tile pairs (mt >= kt)
@@ -145,7 +148,8 @@ __global__ __launch_bounds__(64) void ssd_cb_kernel(QaSsdParams p, float* cb_out
     const int lane = threadIdx.x, frow = lane & 31, fhalf = lane >> 5;
     const int t0 = c * Q;
     const int lim = min(Q, p.seqlen - t0);
-    const float scale = (p.nhead_groups > 0 ? p.C_scale[g] : p.C_scale[0]) * (p.nhead_groups > 0 ? p.B_scale[g] : p.B_scale[0]);
+    const float sC = p.nhead_groups > 0 ? p.C_scale[g] : p.C_scale[0];
+    const float scale = sC * (p.nhead_groups > 0 ? p.B_scale[g] : p.B_scale[0]);
 
     v16i acc[2][2];
 #pragma unroll
@@ -163,6 +167,17 @@ __global__ __launch_bounds__(64) void ssd_cb_kernel(QaSsdParams p, float* cb_out
                             : v4i{0, 0, 0, 0};
             fb[i] = k < lim ? *reinterpret_cast<const v4i*>(p.B + ((static_cast<int64_t>(b) * p.seqlen + t0 + k) * G + g) * N + ks * 32 + fhalf * 16)
                             : v4i{0, 0, 0, 0};
+            if (mt == kt && m < lim) {
+                v8h lo, hi;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    lo[e] = static_cast<_Float16>(sC * static_cast<float>(byte_of(static_cast<uint32_t>(fc[i][e >> 2]), e & 3)));
+                    hi[e] = static_cast<_Float16>(sC * static_cast<float>(byte_of(static_cast<uint32_t>(fc[i][2 + (e >> 2)]), e & 3)));
+                }
+                __half* dst = c16_out + ((static_cast<int64_t>(b) * p.seqlen + t0 + m) * G + g) * N + ks * 32 + fhalf * 16;
+                *reinterpret_cast<v8h*>(dst) = lo;
+                *reinterpret_cast<v8h*>(dst + 8) = hi;
+            }
         }
 #pragma unroll
         for (int i = 0; i < 2; ++i)
@@ -350,13 +365,14 @@ __global__ __launch_bounds__(256) void ssd_state_passing_kernel(QaSsdParams p, c
 // ---------------------------------------------------------------------------------------------
 template <int N, int WAVES>
 __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 4 : 1) void ssd_chunk_scan_kernel(QaSsdParams p, const float* dt_ws, const float* dA_ws,
-                                                             const float* cb_ws, const __half* prev, int nc) {
+                                                             const float* cb_ws, const __half* prev, const __half* c16, int nc) {
     constexpr int QMAX = 256, PITCH = QMAX + 8, PPITCH = N + 8, kThreads = 64 * WAVES;
+    constexpr int kScratch = 512;      // floats per wave: the decay table (QMAX) or an 8 x 64 piece of the output tile
     __shared__ __attribute__((aligned(16))) _Float16 s_xt[kP * PITCH];
     __shared__ __attribute__((aligned(16))) _Float16 s_prev[kP * PPITCH];     // entering state, rows p
     __shared__ __attribute__((aligned(16))) float s_dt[QMAX];
     __shared__ __attribute__((aligned(16))) float s_dA[QMAX];
-    __shared__ __attribute__((aligned(16))) float s_g[WAVES * QMAX];              // per wave: decay * dt of earlier steps
+    __shared__ __attribute__((aligned(16))) float s_g[WAVES * kScratch];          // per wave: decay * dt of earlier steps
     __shared__ float s_xs[kP];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, frow = lane & 31, fhalf = lane >> 5;
@@ -386,12 +402,17 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 4 : 1) void ssd_chunk_scan
                                 static_cast<int64_t>(H) * kP, Q, lim, s_xs, nullptr, tid, kThreads);
     __syncthreads();
 
-    const float sC = p.nhead_groups > 0 ? p.C_scale[g] : p.C_scale[0];
     const float* cb = cb_ws + ((static_cast<int64_t>(b) * nc + c) * G + g) * Q * Q;
     const float D_scale = p.D ? *p.D_scale : 0.0f;
     const float z_scale = p.z ? *p.z_scale : 0.0f;
     const int nmt = Q / 32;
     const int per_wave = max(1, nmt / WAVES);
+    float e_Dv[8];                                           // D of the eight columns this lane writes
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const int pp = (lane & 7) * 8 + e;
+        e_Dv[e] = p.D ? D_scale * static_cast<float>(p.D[p.D_has_hdim ? h * kP + pp : h]) : 0.0f;
+    }
 
     for (int s = 0; s < per_wave; ++s) {
         // tile order 0, nmt-1, 1, nmt-2, ...: wave w takes entries w*per_wave + s
@@ -407,11 +428,13 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 4 : 1) void ssd_chunk_scan
 
         // Loads of this tile that do not depend on each other go out first: the lane's pieces of its
         // C row (term 1) and the first two k-steps of its CB row (term 2).
-        const int8_t* c_row = p.C + ((static_cast<int64_t>(b) * p.seqlen + t0 + m_lane) * G + g) * N;
-        uint2 c_raw[N / 16];
+        const __half* c_row = c16 + ((static_cast<int64_t>(b) * p.seqlen + t0 + m_lane) * G + g) * N;
+        v8h c_frag[N / 16];
 #pragma unroll
         for (int ks = 0; ks < N / 16; ++ks) {
-            c_raw[ks] = m_lane < lim ? *reinterpret_cast<const uint2*>(c_row + ks * 16 + fhalf * 8) : make_uint2(0u, 0u);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) c_frag[ks][e] = static_cast<_Float16>(0.0f);
+            if (m_lane < lim) c_frag[ks] = *reinterpret_cast<const v8h*>(c_row + ks * 16 + fhalf * 8);
         }
         const float* cb_row = cb + static_cast<int64_t>(m_lane) * Q + fhalf * 8;
         const int nks = 2 * (mt + 1);
@@ -428,11 +451,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 4 : 1) void ssd_chunk_scan
         // term 1: C^ (rows m, dstate contiguous) x entering state (rows p, dstate contiguous, staged in LDS)
 #pragma unroll
         for (int ks = 0; ks < N / 16; ++ks) {
-            v8h fc;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                fc[e] = static_cast<_Float16>(sC * static_cast<float>(byte_of(e < 4 ? c_raw[ks].x : c_raw[ks].y, e & 3)));
-            }
+            const v8h fc = c_frag[ks];
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
                 const v8h fs = *reinterpret_cast<const v8h*>(s_prev + (j * 32 + frow) * PPITCH + ks * 16 + fhalf * 8);
@@ -447,7 +466,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 4 : 1) void ssd_chunk_scan
         // the decay per element.  acc = E_m * (exp(ref) * T1 + sum_{k < m0} (CB * G_k) x_k) + diagonal.
         const int m0 = mt * 32;
         const float ref = s_dA[m0];
-        float* g_tab = s_g + wave * QMAX;
+        float* g_tab = s_g + wave * kScratch;
         for (int k = lane; k < m0; k += 64) g_tab[k] = fexp(ref - s_dA[k]) * s_dt[k];
         wave_sync();
         const float e_ref = fexp(ref);
@@ -504,59 +523,50 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 4 : 1) void ssd_chunk_scan
                 }
             }
         }
-        wave_sync();                                    // g_tab is rewritten by the next tile
-        // epilogue: lane holds column p = j*32 + (lane & 31) and 16 rows per accumulator.  The int8 x
-        // (skip term) and z (gate) values of all 16 rows are fetched before any arithmetic; rows past
-        // the end of the sequence read the last valid row and are not stored.
+        wave_sync();                                    // the table is done with: its space now carries the output tile
+        // Epilogue.  In the accumulators a lane holds one column p and 16 rows; memory wants rows of 64
+        // contiguous columns.  The tile passes through the wave's scratch eight rows at a time (registers
+        // 4q..4q+3 of both accumulators are rows 8q + 4*(lane/32) + 0..3), after which lane l holds row
+        // l/8 and the eight columns 8*(l%8)..+7: skip term and gate read 8 bytes, the output is one
+        // 16-byte store.
         const int64_t row_stride = static_cast<int64_t>(H) * kP;
-        const bool whole = mt * 32 + 32 <= lim;
-        // register r holds row lane_row0 + 8*(r/4) + r%4: offsets from the lane's first row are wave-uniform
-        const int lane_row0 = mt * 32 + 4 * fhalf;
+        const int erow = lane >> 3, ecol = (lane & 7) * 8;
+        const int64_t tile_base = (static_cast<int64_t>(b) * p.seqlen + t0) * row_stride + static_cast<int64_t>(h) * kP + ecol;
+        __half* out = static_cast<__half*>(p.out);
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int pp = j * 32 + frow;
-            const int64_t base = (static_cast<int64_t>(b) * p.seqlen + t0) * row_stride + static_cast<int64_t>(h) * kP + pp;
-            const int64_t lane_base = base + lane_row0 * row_stride;
-            int8_t xq[16], zq[16];
-            if (whole) {
+        for (int q = 0; q < 4; ++q) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int t = 0; t < 4; ++t) g_tab[(4 * fhalf + t) * 64 + j * 32 + frow] = acc[j][4 * q + t];
+            wave_sync();
+            const int m = mt * 32 + 8 * q + erow;
+            const float4 y0 = *reinterpret_cast<const float4*>(g_tab + erow * 64 + ecol);
+            const float4 y1 = *reinterpret_cast<const float4*>(g_tab + erow * 64 + ecol + 4);
+            wave_sync();                                // the next piece overwrites the scratch
+            if (m < lim) {
+                float y[8] = {y0.x, y0.y, y0.z, y0.w, y1.x, y1.y, y1.z, y1.w};
+                const int64_t at = tile_base + m * row_stride;
                 if (p.D) {
+                    const uint2 xr = *reinterpret_cast<const uint2*>(p.x + at);
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) xq[r] = p.x[lane_base + (8 * (r / 4) + (r % 4)) * row_stride];
+                    for (int e = 0; e < 8; ++e) {
+                        const float xv = static_cast<float>(byte_of(e < 4 ? xr.x : xr.y, e & 3));
+                        y[e] += (s_xs[ecol + e] * xv) * e_Dv[e];
+                    }
                 }
                 if (p.z) {
+                    const uint2 zr = *reinterpret_cast<const uint2*>(p.z + at);
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) zq[r] = p.z[lane_base + (8 * (r / 4) + (r % 4)) * row_stride];
+                    for (int e = 0; e < 8; ++e) {
+                        const float zv = z_scale * static_cast<float>(byte_of(e < 4 ? zr.x : zr.y, e & 3));
+                        y[e] *= zv * __builtin_amdgcn_rcpf(1.0f + fexp(-zv));
+                    }
                 }
-            } else {
+                v8h o;
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int m = min(lane_row0 + 8 * (r / 4) + (r % 4), lim - 1);
-                    xq[r] = p.D ? p.x[base + m * row_stride] : int8_t(0);
-                    zq[r] = p.z ? p.z[base + m * row_stride] : int8_t(0);
-                }
-            }
-            const float Dv = p.D ? D_scale * static_cast<float>(p.D[p.D_has_hdim ? h * kP + pp : h]) : 0.0f;
-            const float xs_p = s_xs[pp];
-            float y[16];
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                y[r] = acc[j][r];
-                if (p.D) y[r] += (xs_p * static_cast<float>(xq[r])) * Dv;
-                if (p.z) {
-                    const float zv = z_scale * static_cast<float>(zq[r]);
-                    y[r] *= zv * __builtin_amdgcn_rcpf(1.0f + fexp(-zv));
-                }
-            }
-            __half* out = static_cast<__half*>(p.out);
-            if (whole) {
-#pragma unroll
-                for (int r = 0; r < 16; ++r) out[lane_base + (8 * (r / 4) + (r % 4)) * row_stride] = __float2half(y[r]);
-            } else {
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int m = lane_row0 + 8 * (r / 4) + (r % 4);
-                    if (m < lim) out[base + m * row_stride] = __float2half(y[r]);
-                }
+                for (int e = 0; e < 8; ++e) o[e] = static_cast<_Float16>(y[e]);
+                *reinterpret_cast<v8h*>(out + at) = o;
             }
         }
     }
@@ -573,7 +583,8 @@ int validate(const QaSsdParams* p) {
     if (p->headdim != kP) return QA_ERR_UNSUPPORTED;
     if (p->dstate != 64 && p->dstate != 128) return QA_ERR_UNSUPPORTED;
     if (p->chunk_size != 64 && p->chunk_size != 128 && p->chunk_size != 256) return QA_ERR_UNSUPPORTED;
-    if (!aligned16(p->x) || !aligned16(p->B) || !aligned16(p->C)) return QA_ERR_STRIDE;
+    if (!aligned16(p->x) || !aligned16(p->B) || !aligned16(p->C) || !aligned16(p->out)) return QA_ERR_STRIDE;
+    if (p->z && (reinterpret_cast<uintptr_t>(p->z) & 7u)) return QA_ERR_STRIDE;      // the gate is read 8 bytes at a time
     return QA_OK;
 }
 
@@ -601,6 +612,7 @@ extern "C" int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream_) {
     float* states = reinterpret_cast<float*>(base + ws.states);
     __half* prev = reinterpret_cast<__half*>(base + ws.prev);
     float* final_ws = reinterpret_cast<float*>(base + ws.final_f32);
+    __half* c16_ws = reinterpret_cast<__half*>(base + ws.c16);
     const int nc = (p->seqlen + p->chunk_size - 1) / p->chunk_size;
     const int64_t bch = static_cast<int64_t>(p->batch) * nc * p->nheads;
     if (bch > 0x7fffffffLL || static_cast<int64_t>(p->batch) * nc * p->ngroups > 65535) return QA_ERR_SHAPE;
@@ -608,7 +620,7 @@ extern "C" int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream_) {
     hipLaunchKernelGGL(ssd_cumsum_kernel, dim3(static_cast<unsigned>((bch + 3) / 4)), dim3(256), 0, stream, *p, dt_ws,
                        dA_ws, nc);
     const int nt = p->chunk_size / 64;
-    hipLaunchKernelGGL(ssd_cb_kernel, dim3(nt * (nt + 1) / 2, p->batch * nc * p->ngroups), dim3(64), 0, stream, *p, cb_ws, nc);
+    hipLaunchKernelGGL(ssd_cb_kernel, dim3(nt * (nt + 1) / 2, p->batch * nc * p->ngroups), dim3(64), 0, stream, *p, cb_ws, c16_ws, nc);
     if (p->dstate == 128) {
         hipLaunchKernelGGL(ssd_chunk_state_kernel<128>, dim3(static_cast<unsigned>(bch)), dim3(256), 0, stream, *p, dt_ws, dA_ws,
                            states, nc);
@@ -621,7 +633,7 @@ extern "C" int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream_) {
                        dA_ws, states, prev, final_ws, nc);
     // four waves per workgroup, m-tiles paired small/large per wave (eight waves with one tile each measured slower)
     const dim3 sgrid(static_cast<unsigned>(bch));
-    if (p->dstate == 128) hipLaunchKernelGGL((ssd_chunk_scan_kernel<128, 4>), sgrid, dim3(256), 0, stream, *p, dt_ws, dA_ws, cb_ws, prev, nc);
-    else hipLaunchKernelGGL((ssd_chunk_scan_kernel<64, 4>), sgrid, dim3(256), 0, stream, *p, dt_ws, dA_ws, cb_ws, prev, nc);
+    if (p->dstate == 128) hipLaunchKernelGGL((ssd_chunk_scan_kernel<128, 4>), sgrid, dim3(256), 0, stream, *p, dt_ws, dA_ws, cb_ws, prev, c16_ws, nc);
+    else hipLaunchKernelGGL((ssd_chunk_scan_kernel<64, 4>), sgrid, dim3(256), 0, stream, *p, dt_ws, dA_ws, cb_ws, prev, c16_ws, nc);
     return check_launch();
 }
