@@ -114,6 +114,11 @@ struct TileLoader {
         }
     }
     template <int WAVES>
+    __device__ __forceinline__ void issue_one(int j, v4i rsrc, int k0, int k_end, uint32_t dst, int wave) const {
+        const int off = (k0 + kc[j] < k_end) ? voff[j] + k0 : 0x7ffffff0;
+        buffer_load_lds_b128(rsrc, dst + (j * WAVES + wave) * 1024, off);
+    }
+    template <int WAVES>
     __device__ __forceinline__ void issue(v4i rsrc, int k0, int k_end, uint32_t dst, int wave) const {
 #pragma unroll
         for (int j = 0; j < INSTR; ++j) {
@@ -150,6 +155,47 @@ __device__ __forceinline__ void mma_tile(const uint8_t* sa, const uint8_t* sw, i
 #pragma unroll
             for (int j = 0; j < TM; ++j)
                 acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fw[kk & 1][i], fa[kk & 1][j], acc[i][j], 0, 0, 0);
+    }
+}
+
+// The same accumulation with the instruction order pinned.  The fragments of step kk+1 are requested
+// before the multiplications of step kk are issued, and `hook(slot)` runs after every second
+// multiplication (slot = 0 .. 4*TM*TN/2 - 1): the caller places its global -> LDS requests for the
+// next tile there, one at a time, so that the wave never waits on a full memory queue with
+// multiplications behind it in program order.  sched_barrier keeps the compiler from regrouping.
+template <int TM, int TN, class Hook>
+__device__ __forceinline__ void mma_tile_paced(const uint8_t* sa, const uint8_t* sw, int frow, int fhalf,
+                                               v16i (&acc)[TN][TM], Hook&& hook) {
+    v4i fa[2][TM], fw[2][TN];
+    auto fetch = [&](int kk, int buf) {
+#pragma unroll
+        for (int i = 0; i < TN; ++i) {
+            const int row = i * 32 + frow;
+            fw[buf][i] = *reinterpret_cast<const v4i*>(sw + row * kBK + swz(row, kk * 2 + fhalf) * 16);
+        }
+#pragma unroll
+        for (int j = 0; j < TM; ++j) {
+            const int row = j * 32 + frow;
+            fa[buf][j] = *reinterpret_cast<const v4i*>(sa + row * kBK + swz(row, kk * 2 + fhalf) * 16);
+        }
+    };
+    fetch(0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int kk = 0; kk < kBK / 32; ++kk) {
+        if (kk + 1 < kBK / 32) fetch(kk + 1, (kk + 1) & 1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+#pragma unroll
+            for (int j = 0; j < TM; ++j) {
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fw[kk & 1][i], fa[kk & 1][j], acc[i][j], 0, 0, 0);
+                if ((i * TM + j) % 2 == 1) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    hook(kk * (TM * TN / 2) + (i * TM + j) / 2);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
     }
 }
 

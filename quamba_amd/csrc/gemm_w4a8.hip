@@ -146,10 +146,15 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_w4a8_kernel(QaGemmW4A8Par
         __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
         __syncthreads();
         const bool more = kt + 1 < k_tiles;
-        load_a.template issue<WAVES>(rsrc_a, (kt + 1) * kBK, p.k, lds_base + ((kt + 1) & 1) * C::kStageBytes, wave);
         if (more) load_w(kt + 1);
         const uint8_t* stage = lds + (kt & 1) * C::kStageBytes;
-        mma_tile<TM, TN>(stage + (wm * TM * 32) * kBK, stage + BM * kBK + (wn * TN * 32) * kBK, frow, fhalf, acc);
+        // the activation requests for the next tile go out one at a time between the multiplications
+        const uint32_t nbase = lds_base + ((kt + 1) & 1) * C::kStageBytes;
+        static_assert(C::kAInstr <= 4 * TM * TN / 2, "more requests than slots");
+        mma_tile_paced<TM, TN>(stage + (wm * TM * 32) * kBK, stage + BM * kBK + (wn * TN * 32) * kBK, frow, fhalf, acc,
+                               [&](int slot) {
+                                   if (slot < C::kAInstr) load_a.template issue_one<WAVES>(slot, rsrc_a, (kt + 1) * kBK, p.k, nbase, wave);
+                               });
         if (more) store_w((kt + 1) & 1);
     }
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));

@@ -47,6 +47,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_w8a8_kernel(QaGemmW8A8Par
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
     const int k_tiles = (p.k + kBK - 1) / kBK;
+    const int frow = lane & 31, fhalf = lane >> 5;
     auto issue = [&](int tile) {
         const uint32_t base = lds_base + (tile % STAGES) * C::kStageBytes;
         load_a.template issue<WAVES>(rsrc_a, tile * kBK, p.k, base, wave);
@@ -55,13 +56,21 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_w8a8_kernel(QaGemmW8A8Par
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s) issue(s);
 
-    const int frow = lane & 31, fhalf = lane >> 5;
     for (int kt = 0; kt < k_tiles; ++kt) {
         __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 2) * (C::kAInstr + C::kWInstr)));
         __syncthreads();
-        issue(kt + STAGES - 1);          // past the end: every lane is out of range and stores zeros
         const uint8_t* stage = lds + (kt % STAGES) * C::kStageBytes;
-        mma_tile<TM, TN>(stage + (wm * TM * 32) * kBK, stage + BM * kBK + (wn * TN * 32) * kBK, frow, fhalf, acc);
+        // the requests for the next tile go out one at a time between the multiplications of this one
+        // (past the end of K every lane is out of range and stores zeros)
+        const int nt = kt + STAGES - 1;
+        const uint32_t nbase = lds_base + (nt % STAGES) * C::kStageBytes;
+        static_assert(C::kAInstr + C::kWInstr <= 4 * TM * TN / 2, "more requests than slots");
+        mma_tile_paced<TM, TN>(stage + (wm * TM * 32) * kBK, stage + BM * kBK + (wn * TN * 32) * kBK, frow, fhalf, acc,
+                               [&](int slot) {
+                                   if (slot < C::kAInstr) load_a.template issue_one<WAVES>(slot, rsrc_a, nt * kBK, p.k, nbase, wave);
+                                   else if (slot < C::kAInstr + C::kWInstr)
+                                       load_w.template issue_one<WAVES>(slot - C::kAInstr, rsrc_w, nt * kBK, p.k, nbase + BM * kBK, wave);
+                               });
     }
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
     __syncthreads();
