@@ -337,6 +337,31 @@ def other_workloads(dev, steps, warmup):
     return out
 
 
+def mfma_calibration(dev):
+    """Sustained v_mfma_i32_32x32x32_i8 rate of a register-only loop (two waves per SIMD on every CU) for
+    constant and for pseudo-random operand bytes, six launches of about 5 ms each; the last one is reported.
+    The clock is the ratio of the shader-clock and 100 MHz counters over the loop."""
+    from quamba_amd import _lib
+    lib = _lib.lib()
+    wgs, iters = 512, 20000
+    sink = torch.empty(wgs * 256, dtype=torch.int32, device=dev)
+    ticks = torch.zeros(2, dtype=torch.int64, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    out = {}
+    for name, rnd in (("constant_operands", 0), ("random_operands", 1)):
+        for _ in range(6):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            _lib.check(lib.qa_diag_mfma_i8(sink.data_ptr(), sink.numel(), ticks.data_ptr(), wgs, iters, rnd, stream), "diag")
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1)
+        t = ticks.tolist()
+        out[name] = {"TOPs": round(8 * 65536.0 * iters * wgs * 4 / ms / 1e9, 1), "ms": round(ms, 3),
+                     "clock_MHz": round(100.0 * t[0] / max(t[1], 1), 1)}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -349,6 +374,9 @@ def main():
                     help="also time the decode step, the Mamba2 SSD scan and the W4A8 GEMMs (extra key in the JSON line)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain 1 GiB device copies (reference points for hardware-counter runs)")
+    ap.add_argument("--mfma-calibration", action="store_true",
+                    help="also measure the int8 matrix rate the part sustains in a register-only loop, with constant and "
+                         "with random operand bytes (extra key in the JSON line)")
     ap.add_argument("--traffic-json", default=os.path.join(ROOT, "profiles", "traffic.json"),
                     help="HBM bytes per launch measured with rocprofv3 --pmc (written by hand from profiles/)")
     args = ap.parse_args()
@@ -420,6 +448,8 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+    if args.mfma_calibration:
+        line["mfma_calibration"] = mfma_calibration(dev)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(mixer)
     if args.other_workloads:
