@@ -42,6 +42,20 @@ __device__ __forceinline__ int quant8(float v, int round_mode) {
     return static_cast<int>(__builtin_amdgcn_fmed3f(r, -128.0f, 127.0f));
 }
 
+// Four values -> four int8 bytes (round half to even, saturating) in one word.  Clamping to the
+// integers -128 and 127 first does not change the rounded result; adding 1.5 * 2^23 then rounds to
+// nearest-even in the addition itself and leaves the two's-complement byte in the low 8 bits.
+__device__ __forceinline__ uint32_t pack4_rne_sat8(float v0, float v1, float v2, float v3) {
+    constexpr float kMagic = 12582912.0f;
+    const uint32_t y0 = __float_as_uint(__builtin_amdgcn_fmed3f(v0, -128.0f, 127.0f) + kMagic);
+    const uint32_t y1 = __float_as_uint(__builtin_amdgcn_fmed3f(v1, -128.0f, 127.0f) + kMagic);
+    const uint32_t y2 = __float_as_uint(__builtin_amdgcn_fmed3f(v2, -128.0f, 127.0f) + kMagic);
+    const uint32_t y3 = __float_as_uint(__builtin_amdgcn_fmed3f(v3, -128.0f, 127.0f) + kMagic);
+    const uint32_t lo = __builtin_amdgcn_perm(y1, y0, 0x0c0c0400u);      // bytes: y0.0, y1.0, 0, 0
+    const uint32_t hi = __builtin_amdgcn_perm(y3, y2, 0x0c0c0400u);
+    return __builtin_amdgcn_perm(hi, lo, 0x05040100u);                   // lo.0, lo.1, hi.0, hi.1
+}
+
 struct Epilogue {
     const float* row_scale;   // s_row, numel 1 or M (unused with use_alpha)
     const float* col_scale;   // s_col, numel 1 or N
@@ -263,9 +277,15 @@ __device__ __forceinline__ void epilogue(const Epilogue& e, v16i (&acc)[TN][TM],
                     const float v0 = scaled(i, j, q, 0), v1 = scaled(i, j, q, 1);
                     const float v2 = scaled(i, j, q, 2), v3 = scaled(i, j, q, 3);
                     if (OUT == QA_OUT_I8) {
-                        const uint32_t b0 = quant8(v0, round_mode) & 0xff, b1 = quant8(v1, round_mode) & 0xff;
-                        const uint32_t b2 = quant8(v2, round_mode) & 0xff, b3 = quant8(v3, round_mode);
-                        *reinterpret_cast<uint32_t*>(stg + frow * kPitch + nl) = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+                        uint32_t word;
+                        if (!away) {
+                            word = pack4_rne_sat8(v0, v1, v2, v3);
+                        } else {
+                            const uint32_t b0 = quant8(v0, round_mode) & 0xff, b1 = quant8(v1, round_mode) & 0xff;
+                            const uint32_t b2 = quant8(v2, round_mode) & 0xff, b3 = quant8(v3, round_mode);
+                            word = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+                        }
+                        *reinterpret_cast<uint32_t*>(stg + frow * kPitch + nl) = word;
                     } else {
                         __half2 lo = __floats2half2_rn(v0, v1), hi = __floats2half2_rn(v2, v3);
                         uint2 pk;
