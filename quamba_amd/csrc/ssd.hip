@@ -36,7 +36,7 @@ __device__ __forceinline__ void wave_sync() {
 __device__ __forceinline__ int8_t byte_of(uint32_t w, int j) { return static_cast<int8_t>((w >> (8 * j)) & 0xffu); }
 
 struct Ws {            // workspace sections (byte offsets), see qa_ssd_workspace_bytes
-    int64_t dt, dA, cb, states, prev, final_f32, c16, total;
+    int64_t dt, dA, cb, prev, final_f32, c16, bt16, total;
 };
 
 __host__ __device__ inline int64_t align256(int64_t v) { return (v + 255) & ~int64_t(255); }
@@ -49,10 +49,10 @@ __host__ __device__ inline Ws ws_layout(const QaSsdParams& p) {
     w.dt = off; off = align256(off + B * H * nc * Q * 4);
     w.dA = off; off = align256(off + B * H * nc * Q * 4);
     w.cb = off; off = align256(off + B * nc * G * Q * Q * 4);
-    w.states = off; off = align256(off + B * nc * H * P * N * 4);
     w.prev = off; off = align256(off + B * nc * H * P * N * 2);
     w.final_f32 = off; off = align256(off + B * H * P * N * 4);
     w.c16 = off; off = align256(off + B * static_cast<int64_t>(p.seqlen) * G * N * 2);
+    w.bt16 = off; off = align256(off + B * nc * G * N * Q * 2);
     w.total = off;
     return w;
 }
@@ -232,131 +232,224 @@ __device__ __forceinline__ void stage_transposed(_Float16* dst, int pitch, const
 }
 
 // ---------------------------------------------------------------------------------------------
-// Stage 2 (quamba/triton/quant_chunk_state.py:76-89): one workgroup per (batch, chunk, head).
-// S[p,n] = sum_k XT[p][k] * BT[n][k]; 4 waves, wave w owns p-tile w&1 and n-tiles 2*(w>>1)..+1 (of 32).
-// The chunk is consumed in passes of 128 steps.
+// B operand of the chunk-state product, packed once per (batch, chunk, ssd group) for every head of
+// the group: f16(s_B q_B[k, n]) stored fragment-major, so that a wave's 16-byte-per-lane operand of
+// n-tile nt and k-step ks is one contiguous kilobyte:
+//   element (n, k) -> (((n/32) * (Q/16) + k/16) * 64 + ((k%16)/8) * 32 + n%32) * 8 + k%8
+// One workgroup per (batch, chunk, group, n-tile); the 32 columns of the tile pass through LDS.
 // ---------------------------------------------------------------------------------------------
-template <int N>
-__global__ __launch_bounds__(256) void ssd_chunk_state_kernel(QaSsdParams p, const float* dt_ws, const float* dA_ws,
-                                                              float* states, int nc) {
-    constexpr int KC = 128, PITCH = KC + 8, NT = N / 64;      // NT n-tiles per wave
-    __shared__ __attribute__((aligned(16))) _Float16 s_xt[kP * PITCH];
-    __shared__ __attribute__((aligned(16))) _Float16 s_bt[N * PITCH];
-    __shared__ float s_w[KC];
-    __shared__ float s_xs[kP];
-    __shared__ float s_bs[N];
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, frow = lane & 31, fhalf = lane >> 5;
-    const int h = blockIdx.x % p.nheads;
-    const int c = (blockIdx.x / p.nheads) % nc;
-    const int b = blockIdx.x / (p.nheads * nc);
-    const int Q = p.chunk_size, G = p.ngroups, H = p.nheads;
-    int g, hg;
-    group_of(p, h, g, hg);
+__global__ __launch_bounds__(256) void ssd_bpack_kernel(QaSsdParams p, __half* bt16, int nc) {
+    constexpr int QMAX = 256, PITCH = 36;
+    __shared__ __attribute__((aligned(16))) int8_t s_b[QMAX * PITCH];
+    const int Q = p.chunk_size, N = p.dstate, G = p.ngroups, NT = N / 32;
+    const int nt = blockIdx.x % NT;
+    const int bcg = blockIdx.x / NT;
+    const int g = bcg % G, c = (bcg / G) % nc, b = bcg / (G * nc);
+    const int tid = threadIdx.x;
     const int t0 = c * Q;
     const int lim = min(Q, p.seqlen - t0);
-    const float* dt_row = dt_ws + ((static_cast<int64_t>(b) * H + h) * nc + c) * Q;
-    const float* dA_row = dA_ws + ((static_cast<int64_t>(b) * H + h) * nc + c) * Q;
-    const float dA_last = dA_row[Q - 1];
-    if (tid < kP) s_xs[tid] = x_scale_of(p, g, hg, tid);
     const float sB = p.nhead_groups > 0 ? p.B_scale[g] : p.B_scale[0];
-    for (int i = tid; i < N; i += 256) s_bs[i] = sB;
-
-    const int pt = wave & 1, nt0 = (wave >> 1) * NT;
-    v16f acc[NT];
-#pragma unroll
-    for (int j = 0; j < NT; ++j)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[j][r] = 0.0f;
-
-    for (int k0 = 0; k0 < Q; k0 += KC) {
-        const int kc = min(KC, Q - k0);
-        __syncthreads();                       // previous pass fully consumed (and scale tables written)
-        if (tid < KC) s_w[tid] = tid < kc ? fexp(dA_last - dA_row[k0 + tid]) * dt_row[k0 + tid] : 0.0f;
-        __syncthreads();
-        const int valid = max(0, min(kc, lim - k0));
-        stage_transposed<kP, false>(s_xt, PITCH, p.x + ((static_cast<int64_t>(b) * p.seqlen + t0 + k0) * H + h) * kP,
-                                    static_cast<int64_t>(H) * kP, KC, valid, s_xs, nullptr, tid, 256);
-        stage_transposed<N, true>(s_bt, PITCH, p.B + ((static_cast<int64_t>(b) * p.seqlen + t0 + k0) * G + g) * N,
-                                  static_cast<int64_t>(G) * N, KC, valid, s_bs, s_w, tid, 256);
-        __syncthreads();
-        for (int ks = 0; ks < KC / 16; ++ks) {
-            const v8h fx = *reinterpret_cast<const v8h*>(s_xt + (pt * 32 + frow) * PITCH + ks * 16 + fhalf * 8);
-#pragma unroll
-            for (int j = 0; j < NT; ++j) {
-                const v8h fb = *reinterpret_cast<const v8h*>(s_bt + ((nt0 + j) * 32 + frow) * PITCH + ks * 16 + fhalf * 8);
-                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fx, fb, acc[j], 0, 0, 0);
-            }
-        }
+    // rows k of the tile: 32 bytes each, two 16-byte pieces
+    for (int piece = tid; piece < Q * 2; piece += 256) {
+        const int k = piece >> 1, half = piece & 1;
+        uint4 v = make_uint4(0u, 0u, 0u, 0u);
+        if (k < lim) v = *reinterpret_cast<const uint4*>(p.B + ((static_cast<int64_t>(b) * p.seqlen + t0 + k) * G + g) * N + nt * 32 + half * 16);
+        uint32_t* dst = reinterpret_cast<uint32_t*>(s_b + k * PITCH + half * 16);
+        dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;
     }
-    // acc[j]: lane holds column n = (nt0+j)*32 + (lane & 31); register r row p = pt*32 + 8*(r/4) + 4*(lane/32) + r%4
-    float* out = states + ((static_cast<int64_t>(b) * nc + c) * H + h) * kP * N;
+    __syncthreads();
+    __half* out = bt16 + (static_cast<int64_t>(bcg) * NT + nt) * (Q / 16) * 64 * 8;
+    for (int piece = tid; piece < (Q / 16) * 64; piece += 256) {
+        const int ks = piece >> 6, lane = piece & 63, frow = lane & 31, fhalf = lane >> 5;
+        v8h o;
 #pragma unroll
-    for (int j = 0; j < NT; ++j)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int pp = pt * 32 + 8 * (r / 4) + 4 * fhalf + (r % 4);
-            out[pp * N + (nt0 + j) * 32 + frow] = acc[j][r];
-        }
+        for (int e = 0; e < 8; ++e) o[e] = static_cast<_Float16>(sB * static_cast<float>(s_b[(ks * 16 + fhalf * 8 + e) * PITCH + frow]));
+        *reinterpret_cast<v8h*>(out + static_cast<int64_t>(piece) * 8) = o;
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
-// Stages 3 and 6 (quamba/triton/quant_state_passing.py:60-83, quant_ssm_states.py:43,119): one
-// thread per state element, sequential over chunks.
+// Stages 2, 3 and 6 in one pass (quamba/triton/quant_chunk_state.py:76-89, quant_state_passing.py
+// :60-83, quant_ssm_states.py:43,119): one workgroup per (batch, head) walks the chunks in order and
+// keeps the running state P (headdim x dstate, fp32) in registers, in the layout of the MFMA
+// accumulators:
+//   S_c[p,n] = sum_k f16(x^[k,p] w_k) f16(B^[k,n]),  w_k = exp(dA_last - dA_k) dt_k
+//   store f16(P) as the state entering chunk c;  P = exp(dA_last) P + S_c
+// The per-head weight w_k is applied to x (64 columns) rather than to B (dstate columns), so the B
+// operand is the same for every head of a group and comes ready-made from ssd_bpack_kernel; the
+// fp32 chunk states never travel through memory.  The x tile of chunk c+1 is fetched into registers
+// before the products of chunk c are issued.
+// Wave w owns n-tile w and both p-tiles (dstate 128) or n-tile w&1 and p-tile w>>1 (dstate 64).
 // ---------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void ssd_state_passing_kernel(QaSsdParams p, const float* dA_ws, const float* states,
-                                                                __half* prev, float* final_ws, int nc) {
-    const int N = p.dstate, H = p.nheads, Q = p.chunk_size;
-    const int64_t per_head = static_cast<int64_t>(kP) * N;
-    const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-    if (idx >= static_cast<int64_t>(p.batch) * H * per_head) return;
-    const int e = static_cast<int>(idx % per_head);
-    const int h = static_cast<int>((idx / per_head) % H);
-    const int b = static_cast<int>(idx / (per_head * H));
-    float s = 0.0f;
-    // the chunk states do not depend on the running state: fetch eight chunks at a time, then recur
-    constexpr int kBlock = 8;
-    const int64_t c_stride = static_cast<int64_t>(H) * per_head;
-    const int64_t off0 = (static_cast<int64_t>(b) * nc * H + h) * per_head + e;
-    const float* dA_last_p = dA_ws + (static_cast<int64_t>(b) * H + h) * nc * Q + Q - 1;
-    for (int c0 = 0; c0 < nc; c0 += kBlock) {
-        float st[kBlock], da[kBlock];
+template <int N, int Q>
+__global__ __launch_bounds__(256, 2) void ssd_state_kernel(QaSsdParams p, const float* dt_ws, const float* dA_ws,
+                                                        const __half* bt16, __half* prev, float* final_ws, int nc) {
+    constexpr int PITCH = Q + 8, NT = N / 32, PTW = NT == 4 ? 2 : 1, nks = Q / 16;
+    constexpr int XB = (Q / 4) * (kP / 4) / 256;               // 4x4 blocks of the x tile per thread
+    __shared__ __attribute__((aligned(16))) _Float16 s_xt[kP * PITCH];
+    __shared__ __attribute__((aligned(16))) float s_w[2][Q];
+    __shared__ float s_xs[kP];
+    constexpr int kPatchPitch = 40;                            // halves; rows stay 16-byte aligned
+    __shared__ __attribute__((aligned(16))) _Float16 s_patch[4 * 32 * kPatchPitch];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, frow = lane & 31, fhalf = lane >> 5;
+    const int h = blockIdx.x % p.nheads;
+    const int b = blockIdx.x / p.nheads;
+    const int G = p.ngroups, H = p.nheads;
+    int g, hg;
+    group_of(p, h, g, hg);
+    if (tid < kP) s_xs[tid] = x_scale_of(p, g, hg, tid);
+    const int ntile = NT == 4 ? wave : (wave & 1);
+    const int pt0 = NT == 4 ? 0 : (wave >> 1);
+    const int64_t row_stride = static_cast<int64_t>(H) * kP;
+    const int64_t rows0 = (static_cast<int64_t>(b) * H + h) * nc;
+
+    uint32_t xr[XB][4];
+    auto load_x = [&](int c) {
+        const int t0 = c * Q;
+        const int valid = min(Q, p.seqlen - t0);
+        const int8_t* src = p.x + ((static_cast<int64_t>(b) * p.seqlen + t0) * H + h) * kP;
 #pragma unroll
-        for (int i = 0; i < kBlock; ++i) {
-            const int c = min(c0 + i, nc - 1);
-            st[i] = states[off0 + c * c_stride];
-            da[i] = dA_last_p[static_cast<int64_t>(c) * Q];
-        }
+        for (int i = 0; i < XB; ++i) {
+            const int id = tid + i * 256, kb = id / (kP / 4), cb = id % (kP / 4);
 #pragma unroll
-        for (int i = 0; i < kBlock; ++i) {
-            if (c0 + i < nc) {
-                prev[off0 + (c0 + i) * c_stride] = __float2half(s);
-                s = expf(da[i]) * s + st[i];
+            for (int r = 0; r < 4; ++r) {
+                const int k = kb * 4 + r;
+                // rows past the end of the sequence read the last valid row and are zeroed (no branch)
+                const uint32_t v = *reinterpret_cast<const uint32_t*>(src + min(k, valid - 1) * row_stride + cb * 4);
+                xr[i][r] = k < valid ? v : 0u;
             }
         }
-    }
-    const int64_t fo = (static_cast<int64_t>(b) * H + h) * per_head + e;
-    if (final_ws) final_ws[fo] = s;
-    if (p.final_states) {
-        if (p.final_state_is_fp32) {
-            static_cast<float*>(p.final_states)[fo] = s;
-        } else {
-            const int pp = e / N, n = e % N;
-            float sc, K;
-            if (p.nhead_groups > 0) {
-                int g, hg;
-                group_of(p, h, g, hg);
-                const int dg = dim_group_of(p, g, hg, pp);
-                sc = p.state_scale[((g * p.nhead_groups + hg) * p.ndim_groups + dg) * N + n];
-                K = 1e6f;
-            } else {
-                sc = p.state_scale[0];
-                K = 1e2f;
-            }
-            const float s16 = __half2float(__float2half(s));      // the reference hands fp16 states to the quantiser
-            static_cast<int8_t*>(p.final_states)[fo] = sat8_rne((s16 * K) / (sc * K));
+    };
+    // s_w[c & 1][k] = exp(dA_last - dA_k) dt_k, in two halves so that the loads are issued an MFMA
+    // phase before their values are needed
+    float w_dt = 0.0f, w_dA = 0.0f, w_last = 0.0f;
+    auto weights_load = [&](int c) {
+        const float* dt_row = dt_ws + (rows0 + c) * Q;
+        const float* dA_row = dA_ws + (rows0 + c) * Q;
+        w_last = dA_row[Q - 1];
+        if (Q == 256 || tid < Q) {
+            w_dt = dt_row[tid];
+            w_dA = dA_row[tid];
         }
+    };
+    auto weights_store = [&](int c) {
+        if (Q == 256 || tid < Q) s_w[c & 1][tid] = fexp(w_last - w_dA) * w_dt;
+    };
+    auto store_x = [&](int c) {
+        const float* w = s_w[c & 1];
+#pragma unroll
+        for (int i = 0; i < XB; ++i) {
+            const int id = tid + i * 256, kb = id / (kP / 4), cb = id % (kP / 4);
+            const float4 wk = *reinterpret_cast<const float4*>(w + kb * 4);
+            const float wr[4] = {wk.x, wk.y, wk.z, wk.w};
+#pragma unroll
+            for (int cc = 0; cc < 4; ++cc) {
+                const float cs = s_xs[cb * 4 + cc];
+                v4h o;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) o[r] = static_cast<_Float16>((cs * static_cast<float>(byte_of(xr[i][r], cc))) * wr[r]);
+                *reinterpret_cast<v4h*>(s_xt + (cb * 4 + cc) * PITCH + kb * 4) = o;
+            }
+        }
+    };
+    v8h fb[nks];
+    auto load_b = [&](int c) {
+        const __half* src = bt16 + (((static_cast<int64_t>(b) * nc + c) * G + g) * NT + ntile) * nks * 512 + lane * 8;
+#pragma unroll
+        for (int ks = 0; ks < nks; ++ks) fb[ks] = *reinterpret_cast<const v8h*>(src + ks * 512);
+    };
+
+    v16f run[PTW], acc[PTW];
+#pragma unroll
+    for (int j = 0; j < PTW; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { run[j][r] = 0.0f; acc[j][r] = 0.0f; }
+
+    load_x(0);
+    weights_load(0);
+    load_b(0);
+    weights_store(0);
+    float dA_last = w_last;                                    // of the chunk being multiplied
+    __syncthreads();                                           // s_xs, s_w[0]
+    store_x(0);
+    __syncthreads();
+
+    for (int c = 0; c < nc; ++c) {
+        const bool more = c + 1 < nc;
+        if (more) {
+            load_x(c + 1);
+            weights_load(c + 1);
+        }
+#pragma unroll
+        for (int ks = 0; ks < nks; ++ks) {
+#pragma unroll
+            for (int j = 0; j < PTW; ++j) {
+                const v8h fx = *reinterpret_cast<const v8h*>(s_xt + ((pt0 + j) * 32 + frow) * PITCH + ks * 16 + fhalf * 8);
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fx, fb[ks], acc[j], 0, 0, 0);
+            }
+        }
+        if (more) load_b(c + 1);                               // in flight during the update and the staging below
+        // the state entering chunk c, then the recurrence.  Lane holds column n = ntile*32 + lane%32 and,
+        // in register r, row p = pt*32 + 8*(r/4) + 4*(lane/32) + r%4.
+        // The 32 x 32 tile passes through a wave-private LDS patch so that it leaves as 16-byte pieces.
+        const float decay = fexp(dA_last);
+        __half* pst = prev + ((static_cast<int64_t>(b) * nc + c) * H + h) * kP * N + ntile * 32;
+        _Float16* patch = s_patch + wave * (32 * kPatchPitch);
+#pragma unroll
+        for (int j = 0; j < PTW; ++j) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                patch[(8 * (r / 4) + 4 * fhalf + (r % 4)) * kPatchPitch + frow] = static_cast<_Float16>(run[j][r]);
+                run[j][r] = decay * run[j][r] + acc[j][r];
+                acc[j][r] = 0.0f;
+            }
+            wave_sync();
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                const int row = q * 16 + (lane >> 2), piece = lane & 3;
+                const uint4 v = *reinterpret_cast<const uint4*>(patch + row * kPatchPitch + piece * 8);
+                *reinterpret_cast<uint4*>(pst + ((pt0 + j) * 32 + row) * N + piece * 8) = v;
+            }
+            wave_sync();
+        }
+        if (more) {
+            weights_store(c + 1);
+            dA_last = w_last;
+        }
+        __syncthreads();                                       // every wave is done with this chunk's x tile; s_w written
+        if (more) store_x(c + 1);
+        __syncthreads();
     }
+
+    // final state: fp32 copy for the caller's workspace, and the requested output form
+#pragma unroll
+    for (int j = 0; j < PTW; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int pp = (pt0 + j) * 32 + 8 * (r / 4) + 4 * fhalf + (r % 4);
+            const int n = ntile * 32 + frow;
+            const int64_t fo = ((static_cast<int64_t>(b) * H + h) * kP + pp) * N + n;
+            const float sv = run[j][r];
+            if (final_ws) final_ws[fo] = sv;
+            if (p.final_states) {
+                if (p.final_state_is_fp32) {
+                    static_cast<float*>(p.final_states)[fo] = sv;
+                } else {
+                    float sc, K;
+                    if (p.nhead_groups > 0) {
+                        const int dg = dim_group_of(p, g, hg, pp);
+                        sc = p.state_scale[((g * p.nhead_groups + hg) * p.ndim_groups + dg) * N + n];
+                        K = 1e6f;
+                    } else {
+                        sc = p.state_scale[0];
+                        K = 1e2f;
+                    }
+                    const float s16 = __half2float(__float2half(sv));      // the reference hands fp16 states to the quantiser
+                    static_cast<int8_t*>(p.final_states)[fo] = sat8_rne((s16 * K) / (sc * K));
+                }
+            }
+        }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -609,7 +702,6 @@ extern "C" int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream_) {
     float* dt_ws = reinterpret_cast<float*>(base + ws.dt);
     float* dA_ws = reinterpret_cast<float*>(base + ws.dA);
     float* cb_ws = reinterpret_cast<float*>(base + ws.cb);
-    float* states = reinterpret_cast<float*>(base + ws.states);
     __half* prev = reinterpret_cast<__half*>(base + ws.prev);
     float* final_ws = reinterpret_cast<float*>(base + ws.final_f32);
     __half* c16_ws = reinterpret_cast<__half*>(base + ws.c16);
@@ -621,16 +713,21 @@ extern "C" int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream_) {
                        dA_ws, nc);
     const int nt = p->chunk_size / 64;
     hipLaunchKernelGGL(ssd_cb_kernel, dim3(nt * (nt + 1) / 2, p->batch * nc * p->ngroups), dim3(64), 0, stream, *p, cb_ws, c16_ws, nc);
+    __half* bt16_ws = reinterpret_cast<__half*>(base + ws.bt16);
+    const int64_t bcg_tiles = static_cast<int64_t>(p->batch) * nc * p->ngroups * (p->dstate / 32);
+    if (bcg_tiles > 0x7fffffffLL) return QA_ERR_SHAPE;
+    hipLaunchKernelGGL(ssd_bpack_kernel, dim3(static_cast<unsigned>(bcg_tiles)), dim3(256), 0, stream, *p, bt16_ws, nc);
+    const dim3 hgrid(static_cast<unsigned>(p->batch * p->nheads));
+    auto launch_state = [&](auto kernel) { hipLaunchKernelGGL(kernel, hgrid, dim3(256), 0, stream, *p, dt_ws, dA_ws, bt16_ws, prev, final_ws, nc); };
     if (p->dstate == 128) {
-        hipLaunchKernelGGL(ssd_chunk_state_kernel<128>, dim3(static_cast<unsigned>(bch)), dim3(256), 0, stream, *p, dt_ws, dA_ws,
-                           states, nc);
+        if (p->chunk_size == 256) launch_state(ssd_state_kernel<128, 256>);
+        else if (p->chunk_size == 128) launch_state(ssd_state_kernel<128, 128>);
+        else launch_state(ssd_state_kernel<128, 64>);
     } else {
-        hipLaunchKernelGGL(ssd_chunk_state_kernel<64>, dim3(static_cast<unsigned>(bch)), dim3(256), 0, stream, *p, dt_ws, dA_ws,
-                           states, nc);
+        if (p->chunk_size == 256) launch_state(ssd_state_kernel<64, 256>);
+        else if (p->chunk_size == 128) launch_state(ssd_state_kernel<64, 128>);
+        else launch_state(ssd_state_kernel<64, 64>);
     }
-    const int64_t elems = static_cast<int64_t>(p->batch) * p->nheads * kP * p->dstate;
-    hipLaunchKernelGGL(ssd_state_passing_kernel, dim3(static_cast<unsigned>((elems + 255) / 256)), dim3(256), 0, stream, *p,
-                       dA_ws, states, prev, final_ws, nc);
     // four waves per workgroup, m-tiles paired small/large per wave (eight waves with one tile each measured slower)
     const dim3 sgrid(static_cast<unsigned>(bch));
     if (p->dstate == 128) hipLaunchKernelGGL((ssd_chunk_scan_kernel<128, 4>), sgrid, dim3(256), 0, stream, *p, dt_ws, dA_ws, cb_ws, prev, c16_ws, nc);
