@@ -25,6 +25,9 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 
 constexpr int kP = 64;          // head dimension this build supports
 constexpr float kLog2e = 1.44269504088896341f;
+// C B^T is kept in fp16 divided by 16 (exact), so that products of full-range int8 rows stay inside
+// the fp16 range; the factor returns with the decay table.
+constexpr float kCbShift = 0.0625f, kCbUnshift = 16.0f;
 
 __device__ __forceinline__ float fexp(float x) { return __builtin_amdgcn_exp2f(x * kLog2e); }
 // orders a wave's own LDS writes before its later LDS reads (wave-private scratch needs no workgroup barrier)
@@ -48,7 +51,7 @@ __host__ __device__ inline Ws ws_layout(const QaSsdParams& p) {
     int64_t off = 0;
     w.dt = off; off = align256(off + B * H * nc * Q * 4);
     w.dA = off; off = align256(off + B * H * nc * Q * 4);
-    w.cb = off; off = align256(off + B * nc * G * Q * Q * 4);
+    w.cb = off; off = align256(off + B * nc * G * Q * Q * 2);
     w.prev = off; off = align256(off + B * nc * H * P * N * 2);
     w.final_f32 = off; off = align256(off + B * H * P * N * 4);
     w.c16 = off; off = align256(off + B * static_cast<int64_t>(p.seqlen) * G * N * 2);
@@ -135,7 +138,7 @@ __global__ __launch_bounds__(256) void ssd_cumsum_kernel(QaSsdParams p, float* d
 // write their C rows dequantised to fp16 (f16(s_C * q_C)): every head of the group multiplies those
 // rows with its entering state in the chunk scan, which then reads them ready-made.
 // ---------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(64) void ssd_cb_kernel(QaSsdParams p, float* cb_out, __half* c16_out, int nc) {
+__global__ __launch_bounds__(64) void ssd_cb_kernel(QaSsdParams p, __half* cb_out, __half* c16_out, int nc) {
     const int Q = p.chunk_size, N = p.dstate, G = p.ngroups;
     const int nt = Q / 64;
     // blockIdx.x enumerates lower-triangular tile pairs (mt >= kt)
@@ -185,7 +188,7 @@ __global__ __launch_bounds__(64) void ssd_cb_kernel(QaSsdParams p, float* cb_out
             for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fc[i], fb[j], acc[i][j], 0, 0, 0);
     }
     // acc[i][j]: lane holds column k = kt*64 + j*32 + (lane & 31), register r row m = mt*64 + i*32 + 8*(r/4) + 4*(lane/32) + r%4
-    float* tile = cb_out + ((static_cast<int64_t>(b) * nc + c) * G + g) * Q * Q;
+    __half* tile = cb_out + ((static_cast<int64_t>(b) * nc + c) * G + g) * Q * Q;
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -194,7 +197,7 @@ __global__ __launch_bounds__(64) void ssd_cb_kernel(QaSsdParams p, float* cb_out
             for (int r = 0; r < 16; ++r) {
                 const int m = mt * 64 + i * 32 + 8 * (r / 4) + 4 * fhalf + (r % 4);
                 const int k = kt * 64 + j * 32 + frow;
-                tile[static_cast<int64_t>(m) * Q + k] = scale * static_cast<float>(acc[i][j][r]);
+                tile[static_cast<int64_t>(m) * Q + k] = __float2half((scale * static_cast<float>(acc[i][j][r])) * kCbShift);
             }
 }
 
@@ -453,26 +456,30 @@ __global__ __launch_bounds__(256, 2) void ssd_state_kernel(QaSsdParams p, const 
 }
 
 // ---------------------------------------------------------------------------------------------
-// Stage 5 (quamba/triton/quant_chunk_scan.py:96-171): one workgroup per (batch, chunk, head);
-// each wave owns whole 32-row m-tiles (paired small/large so the causal work balances).
+// Stage 5 (quamba/triton/quant_chunk_scan.py:96-171): one workgroup per (batch, chunk, head), four
+// waves; each wave owns whole 32-row m-tiles (paired small/large so the causal work balances).
+// Everything a tile reads from global memory - its C rows, its rows of C B^T (fp16, all k-steps of the
+// causal range) and the x / z bytes of the epilogue - is requested at the top of the tile, so the
+// memory latency is paid once per tile instead of once per k-step.
 // ---------------------------------------------------------------------------------------------
-template <int N, int WAVES>
-__global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 4 : 1) void ssd_chunk_scan_kernel(QaSsdParams p, const float* dt_ws, const float* dA_ws,
-                                                             const float* cb_ws, const __half* prev, const __half* c16, int nc) {
-    constexpr int QMAX = 256, PITCH = QMAX + 8, PPITCH = N + 8, kThreads = 64 * WAVES;
-    constexpr int kScratch = 512;      // floats per wave: the decay table (QMAX) or an 8 x 64 piece of the output tile
+template <int N, int Q>
+__global__ __launch_bounds__(256, 2) void ssd_chunk_scan_kernel(QaSsdParams p, const float* dt_ws, const float* dA_ws,
+                                                                const __half* cb_ws, const __half* prev, const __half* c16, int nc) {
+    constexpr int WAVES = 4, PITCH = Q + 8, PPITCH = N + 8, kThreads = 64 * WAVES;
+    constexpr int kScratch = 512;      // floats per wave: the decay table (Q halves) or an 8 x 64 piece of the output tile
+    constexpr int NMT = Q / 32, PER_WAVE = NMT / WAVES > 0 ? NMT / WAVES : 1, KSMAX = Q / 16;
     __shared__ __attribute__((aligned(16))) _Float16 s_xt[kP * PITCH];
     __shared__ __attribute__((aligned(16))) _Float16 s_prev[kP * PPITCH];     // entering state, rows p
-    __shared__ __attribute__((aligned(16))) float s_dt[QMAX];
-    __shared__ __attribute__((aligned(16))) float s_dA[QMAX];
-    __shared__ __attribute__((aligned(16))) float s_g[WAVES * kScratch];          // per wave: decay * dt of earlier steps
+    __shared__ __attribute__((aligned(16))) float s_dt[Q];
+    __shared__ __attribute__((aligned(16))) float s_dA[Q];
+    __shared__ __attribute__((aligned(16))) float s_g[WAVES * kScratch];
     __shared__ float s_xs[kP];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, frow = lane & 31, fhalf = lane >> 5;
     const int h = blockIdx.x % p.nheads;
     const int c = (blockIdx.x / p.nheads) % nc;
     const int b = blockIdx.x / (p.nheads * nc);
-    const int Q = p.chunk_size, G = p.ngroups, H = p.nheads;
+    const int G = p.ngroups, H = p.nheads;
     int g, hg;
     group_of(p, h, g, hg);
     const int t0 = c * Q;
@@ -495,100 +502,98 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 4 : 1) void ssd_chunk_scan
                                 static_cast<int64_t>(H) * kP, Q, lim, s_xs, nullptr, tid, kThreads);
     __syncthreads();
 
-    const float* cb = cb_ws + ((static_cast<int64_t>(b) * nc + c) * G + g) * Q * Q;
+    const __half* cb = cb_ws + ((static_cast<int64_t>(b) * nc + c) * G + g) * Q * Q;
     const float D_scale = p.D ? *p.D_scale : 0.0f;
     const float z_scale = p.z ? *p.z_scale : 0.0f;
-    const int nmt = Q / 32;
-    const int per_wave = max(1, nmt / WAVES);
+    const int64_t row_stride = static_cast<int64_t>(H) * kP;
+    const int erow = lane >> 3, ecol = (lane & 7) * 8;       // epilogue: row within a piece of 8, first of 8 columns
+    const int64_t tile_base = (static_cast<int64_t>(b) * p.seqlen + t0) * row_stride + static_cast<int64_t>(h) * kP + ecol;
+    __half* out = static_cast<__half*>(p.out);
     float e_Dv[8];                                           // D of the eight columns this lane writes
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-        const int pp = (lane & 7) * 8 + e;
+        const int pp = ecol + e;
         e_Dv[e] = p.D ? D_scale * static_cast<float>(p.D[p.D_has_hdim ? h * kP + pp : h]) : 0.0f;
     }
 
-    for (int s = 0; s < per_wave; ++s) {
-        // tile order 0, nmt-1, 1, nmt-2, ...: wave w takes entries w*per_wave + s
-        const int entry = wave * per_wave + s;
-        if (entry >= nmt) break;
-        const int mt = (entry & 1) ? nmt - 1 - (entry >> 1) : (entry >> 1);
+#pragma unroll
+    for (int s = 0; s < PER_WAVE; ++s) {
+        // tile order 0, NMT-1, 1, NMT-2, ...: wave w takes entries w*PER_WAVE + s
+        const int entry = wave * PER_WAVE + s;
+        if (entry >= NMT) break;
+        const int mt = (entry & 1) ? NMT - 1 - (entry >> 1) : (entry >> 1);
         const int m_lane = mt * 32 + frow;                 // row of this lane's A operands
+        const int nks = 2 * (mt + 1);                      // k-steps of the causal range
+        const int n_off = 2 * mt;                          // of which entirely before the tile
         v16f acc[2];
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[j][r] = 0.0f;
 
-        // Loads of this tile that do not depend on each other go out first: the lane's pieces of its
-        // C row (term 1) and the first two k-steps of its CB row (term 2).
-        const __half* c_row = c16 + ((static_cast<int64_t>(b) * p.seqlen + t0 + m_lane) * G + g) * N;
+        // all global reads of the tile
+        const __half* c_row = c16 + ((static_cast<int64_t>(b) * p.seqlen + t0 + min(m_lane, lim - 1)) * G + g) * N;
         v8h c_frag[N / 16];
 #pragma unroll
-        for (int ks = 0; ks < N / 16; ++ks) {
+        for (int ks = 0; ks < N / 16; ++ks) c_frag[ks] = *reinterpret_cast<const v8h*>(c_row + ks * 16 + fhalf * 8);
+        const __half* cb_row = cb + static_cast<int64_t>(m_lane) * Q + fhalf * 8;
+        v8h cbf[KSMAX];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) c_frag[ks][e] = static_cast<_Float16>(0.0f);
-            if (m_lane < lim) c_frag[ks] = *reinterpret_cast<const v8h*>(c_row + ks * 16 + fhalf * 8);
-        }
-        const float* cb_row = cb + static_cast<int64_t>(m_lane) * Q + fhalf * 8;
-        const int nks = 2 * (mt + 1);
-        constexpr int kAhead = 2;
-        float4 pre[kAhead][2];
+        for (int ks = 0; ks < KSMAX; ++ks)
+            if (ks < nks) cbf[ks] = *reinterpret_cast<const v8h*>(cb_row + ks * 16);
+        uint2 xq[4], zq[4];
 #pragma unroll
-        for (int a = 0; a < kAhead; ++a) {
-            if (a < nks) {
-                pre[a][0] = *reinterpret_cast<const float4*>(cb_row + a * 16);
-                pre[a][1] = *reinterpret_cast<const float4*>(cb_row + a * 16 + 4);
-            }
+        for (int q = 0; q < 4; ++q) {
+            const int64_t at = tile_base + min(mt * 32 + 8 * q + erow, lim - 1) * row_stride;
+            xq[q] = p.D ? *reinterpret_cast<const uint2*>(p.x + at) : make_uint2(0u, 0u);
+            zq[q] = p.z ? *reinterpret_cast<const uint2*>(p.z + at) : make_uint2(0u, 0u);
         }
 
+        // Decay factors.  The cumulative dA decreases along the chunk, so with ref = dA at the first row
+        // of this m-tile, exp(dA_m - dA_k) = exp(dA_m - ref) * exp(ref - dA_k) for every k before the
+        // tile, both factors <= 1.  The k factor (times dt_k, times the power of two that C B^T was
+        // stored without) is tabulated once per tile by the wave, in fp16; the row factor is applied to
+        // the accumulator after the off-diagonal k-steps, together with term 1 (whose decay exp(dA_m) =
+        // exp(ref) * exp(dA_m - ref)).  Only the two diagonal k-steps evaluate the decay per element.
+        // acc = E_m * (exp(ref) * T1 + sum_{k < m0} (CB * G_k) x_k) + diagonal.
+        const int m0 = mt * 32;
+        const float ref = s_dA[m0];
+        _Float16* g_tab = reinterpret_cast<_Float16*>(s_g + wave * kScratch);
+        for (int k = lane; k < m0; k += 64) g_tab[k] = static_cast<_Float16>((fexp(ref - s_dA[k]) * s_dt[k]) * kCbUnshift);
+        wave_sync();
+
         // term 1: C^ (rows m, dstate contiguous) x entering state (rows p, dstate contiguous, staged in LDS)
+        const bool row_ok = m_lane < lim;
 #pragma unroll
         for (int ks = 0; ks < N / 16; ++ks) {
-            const v8h fc = c_frag[ks];
+            v8h fc = c_frag[ks];
+            if (!row_ok) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) fc[e] = static_cast<_Float16>(0.0f);
+            }
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
                 const v8h fs = *reinterpret_cast<const v8h*>(s_prev + (j * 32 + frow) * PPITCH + ks * 16 + fhalf * 8);
                 acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fc, fs, acc[j], 0, 0, 0);
             }
         }
-        // Decay factors.  The cumulative dA decreases along the chunk, so with ref = dA at the first row
-        // of this m-tile, exp(dA_m - dA_k) = exp(dA_m - ref) * exp(ref - dA_k) for every k before the
-        // tile, both factors <= 1.  The k factor (times dt_k) is tabulated once per tile by the wave; the
-        // row factor is applied to the accumulator after the off-diagonal k-steps, together with term 1
-        // (whose decay exp(dA_m) = exp(ref) * exp(dA_m - ref)).  Only the two diagonal k-steps evaluate
-        // the decay per element.  acc = E_m * (exp(ref) * T1 + sum_{k < m0} (CB * G_k) x_k) + diagonal.
-        const int m0 = mt * 32;
-        const float ref = s_dA[m0];
-        float* g_tab = s_g + wave * kScratch;
-        for (int k = lane; k < m0; k += 64) g_tab[k] = fexp(ref - s_dA[k]) * s_dt[k];
-        wave_sync();
         const float e_ref = fexp(ref);
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             acc[0][r] *= e_ref;
             acc[1][r] *= e_ref;
         }
-        const int n_off = 2 * mt;                       // k-steps entirely before the tile
-        for (int ks = 0; ks < nks; ks += kAhead) {
+        // term 2
 #pragma unroll
-            for (int a = 0; a < kAhead; ++a) {
-                const int kk = ks + a;
-                if (kk >= nks) break;                   // nks is even, kept for safety
-                const float4 c0 = pre[a][0], c1 = pre[a][1];
-                if (kk + kAhead < nks) {
-                    pre[a][0] = *reinterpret_cast<const float4*>(cb_row + (kk + kAhead) * 16);
-                    pre[a][1] = *reinterpret_cast<const float4*>(cb_row + (kk + kAhead) * 16 + 4);
-                }
-                const int k0 = kk * 16 + fhalf * 8;
-                const float cbv[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+        for (int ks = 0; ks < KSMAX; ++ks) {
+            if (ks < nks) {
+                const int k0 = ks * 16 + fhalf * 8;
                 v8h fl;
-                if (kk < n_off) {
-                    const float4 g0 = *reinterpret_cast<const float4*>(g_tab + k0), g1 = *reinterpret_cast<const float4*>(g_tab + k0 + 4);
-                    const float gk[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) fl[e] = static_cast<_Float16>(cbv[e] * gk[e]);
+                if (ks < n_off) {
+                    const v8h gh = *reinterpret_cast<const v8h*>(g_tab + k0);
+                    fl = cbf[ks] * gh;
                 } else {
-                    if (kk == n_off) {
+                    if (ks == n_off) {
                         // leaving the off-diagonal part: apply the row factors once
 #pragma unroll
                         for (int r = 0; r < 16; ++r) {
@@ -605,7 +610,8 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 4 : 1) void ssd_chunk_scan
 #pragma unroll
                     for (int e = 0; e < 8; ++e) {
                         const int k = k0 + e;
-                        const float wv = (cbv[e] * fexp(dA_m - dAk[e])) * dtk[e];
+                        const float cbv = static_cast<float>(cbf[ks][e]) * kCbUnshift;
+                        const float wv = (cbv * fexp(dA_m - dAk[e])) * dtk[e];
                         fl[e] = static_cast<_Float16>(k <= m_lane ? wv : 0.0f);
                     }
                 }
@@ -620,39 +626,34 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 4 : 1) void ssd_chunk_scan
         // Epilogue.  In the accumulators a lane holds one column p and 16 rows; memory wants rows of 64
         // contiguous columns.  The tile passes through the wave's scratch eight rows at a time (registers
         // 4q..4q+3 of both accumulators are rows 8q + 4*(lane/32) + 0..3), after which lane l holds row
-        // l/8 and the eight columns 8*(l%8)..+7: skip term and gate read 8 bytes, the output is one
-        // 16-byte store.
-        const int64_t row_stride = static_cast<int64_t>(H) * kP;
-        const int erow = lane >> 3, ecol = (lane & 7) * 8;
-        const int64_t tile_base = (static_cast<int64_t>(b) * p.seqlen + t0) * row_stride + static_cast<int64_t>(h) * kP + ecol;
-        __half* out = static_cast<__half*>(p.out);
+        // l/8 and the eight columns 8*(l%8)..+7: the skip term and the gate use the 8 bytes fetched at
+        // the top of the tile, the output is one 16-byte store.
+        float* o_tab = s_g + wave * kScratch;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
 #pragma unroll
             for (int j = 0; j < 2; ++j)
 #pragma unroll
-                for (int t = 0; t < 4; ++t) g_tab[(4 * fhalf + t) * 64 + j * 32 + frow] = acc[j][4 * q + t];
+                for (int t = 0; t < 4; ++t) o_tab[(4 * fhalf + t) * 64 + j * 32 + frow] = acc[j][4 * q + t];
             wave_sync();
             const int m = mt * 32 + 8 * q + erow;
-            const float4 y0 = *reinterpret_cast<const float4*>(g_tab + erow * 64 + ecol);
-            const float4 y1 = *reinterpret_cast<const float4*>(g_tab + erow * 64 + ecol + 4);
+            const float4 y0 = *reinterpret_cast<const float4*>(o_tab + erow * 64 + ecol);
+            const float4 y1 = *reinterpret_cast<const float4*>(o_tab + erow * 64 + ecol + 4);
             wave_sync();                                // the next piece overwrites the scratch
             if (m < lim) {
                 float y[8] = {y0.x, y0.y, y0.z, y0.w, y1.x, y1.y, y1.z, y1.w};
                 const int64_t at = tile_base + m * row_stride;
                 if (p.D) {
-                    const uint2 xr = *reinterpret_cast<const uint2*>(p.x + at);
 #pragma unroll
                     for (int e = 0; e < 8; ++e) {
-                        const float xv = static_cast<float>(byte_of(e < 4 ? xr.x : xr.y, e & 3));
+                        const float xv = static_cast<float>(byte_of(e < 4 ? xq[q].x : xq[q].y, e & 3));
                         y[e] += (s_xs[ecol + e] * xv) * e_Dv[e];
                     }
                 }
                 if (p.z) {
-                    const uint2 zr = *reinterpret_cast<const uint2*>(p.z + at);
 #pragma unroll
                     for (int e = 0; e < 8; ++e) {
-                        const float zv = z_scale * static_cast<float>(byte_of(e < 4 ? zr.x : zr.y, e & 3));
+                        const float zv = z_scale * static_cast<float>(byte_of(e < 4 ? zq[q].x : zq[q].y, e & 3));
                         y[e] *= zv * __builtin_amdgcn_rcpf(1.0f + fexp(-zv));
                     }
                 }
@@ -701,7 +702,7 @@ extern "C" int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream_) {
     uint8_t* base = static_cast<uint8_t*>(p->workspace);
     float* dt_ws = reinterpret_cast<float*>(base + ws.dt);
     float* dA_ws = reinterpret_cast<float*>(base + ws.dA);
-    float* cb_ws = reinterpret_cast<float*>(base + ws.cb);
+    __half* cb_ws = reinterpret_cast<__half*>(base + ws.cb);
     __half* prev = reinterpret_cast<__half*>(base + ws.prev);
     float* final_ws = reinterpret_cast<float*>(base + ws.final_f32);
     __half* c16_ws = reinterpret_cast<__half*>(base + ws.c16);
@@ -728,9 +729,16 @@ extern "C" int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream_) {
         else if (p->chunk_size == 128) launch_state(ssd_state_kernel<64, 128>);
         else launch_state(ssd_state_kernel<64, 64>);
     }
-    // four waves per workgroup, m-tiles paired small/large per wave (eight waves with one tile each measured slower)
     const dim3 sgrid(static_cast<unsigned>(bch));
-    if (p->dstate == 128) hipLaunchKernelGGL((ssd_chunk_scan_kernel<128, 4>), sgrid, dim3(256), 0, stream, *p, dt_ws, dA_ws, cb_ws, prev, c16_ws, nc);
-    else hipLaunchKernelGGL((ssd_chunk_scan_kernel<64, 4>), sgrid, dim3(256), 0, stream, *p, dt_ws, dA_ws, cb_ws, prev, c16_ws, nc);
+    auto launch_scan = [&](auto kernel) { hipLaunchKernelGGL(kernel, sgrid, dim3(256), 0, stream, *p, dt_ws, dA_ws, cb_ws, prev, c16_ws, nc); };
+    if (p->dstate == 128) {
+        if (p->chunk_size == 256) launch_scan(ssd_chunk_scan_kernel<128, 256>);
+        else if (p->chunk_size == 128) launch_scan(ssd_chunk_scan_kernel<128, 128>);
+        else launch_scan(ssd_chunk_scan_kernel<128, 64>);
+    } else {
+        if (p->chunk_size == 256) launch_scan(ssd_chunk_scan_kernel<64, 256>);
+        else if (p->chunk_size == 128) launch_scan(ssd_chunk_scan_kernel<64, 128>);
+        else launch_scan(ssd_chunk_scan_kernel<64, 64>);
+    }
     return check_launch();
 }

@@ -62,13 +62,14 @@ def test_every_stage_matches_the_oracle(dev):
     a256 = lambda v: (v + 255) & ~255
     off, parts = 0, {}
     for name, shape, dt in [("dt", (B, H, nc, Q), torch.float32), ("dA_cumsum", (B, H, nc, Q), torch.float32),
-                            ("CB", (B, nc, G, Q, Q), torch.float32), ("prev_states", (B, nc, H, 64, N), torch.float16)]:
+                            ("CB", (B, nc, G, Q, Q), torch.float16), ("prev_states", (B, nc, H, 64, N), torch.float16)]:
         n = int(np.prod(shape)) * (4 if dt == torch.float32 else 2)
         parts[name] = ws[off:off + n].view(dt).view(shape).float().cpu().numpy()
         off = a256(off + n)
     np.testing.assert_allclose(parts["dt"], ref["dt"], rtol=1e-5, atol=1e-9)
     np.testing.assert_allclose(parts["dA_cumsum"], ref["dA_cumsum"], rtol=1e-5, atol=1e-8)
-    np.testing.assert_allclose(parts["CB"], ref["CB"], rtol=1e-5)                 # Q == 64: one tile, all of it written
+    # C B^T is kept in fp16, divided by 16; Q == 64: one tile, all of it written
+    np.testing.assert_allclose(parts["CB"] * 16.0, ref["CB"], rtol=1e-3, atol=1e-3 * np.abs(ref["CB"]).max())
     # the fp32 chunk states stay in registers; the states entering each chunk (their running sum) are checked
     assert np.abs(parts["prev_states"] - ref["prev_states"]).max() <= 1e-3 * np.abs(ref["prev_states"]).max()
 
