@@ -5,13 +5,16 @@
 // accumulation, as there; the one pure int8 contraction (C B^T) runs on the int8 matrix cores.
 //   cumsum      dt = clamp(softplus(s_dt q_dt + dt_bias)), dA_cs = within-chunk cumsum(dt * A)
 //   cb          CB[m,k] = (s_C s_B) * sum_n q_C[m,n] q_B[k,n]                       (int8 MFMA, lower tiles)
-//   chunk_state S_c[p,n] = sum_k f16(x^[k,p]) f16(B^[k,n] exp(dA_last - dA_k) dt_k)   (fp16 MFMA)
-//   passing     P_0 = 0, P_{c+1} = exp(dA_last,c) P_c + S_c; P_c kept in fp16; final state fp32 / int8
+//   state       S_c[p,n] = sum_k f16(x^[k,p] exp(dA_last - dA_k) dt_k) f16(B^[k,n])   (fp16 MFMA; the reference
+//               rounds B^ times the weight instead, the difference is inside the fp16 tolerance)
+//               P_0 = 0, P_{c+1} = exp(dA_last,c) P_c + S_c in registers; P_c stored in fp16; final state fp32 / int8
 //   chunk_scan  y[m,p] = exp(dA_m) sum_n f16(C^[m,n]) P_c[p,n] + sum_{k<=m} f16(CB[m,k] e^{dA_m-dA_k} dt_k) f16(x^[k,p])
-//               + D x^[m,p], optional z gate, fp16 out                               (fp16 MFMA)
+//               + D x^[m,p], optional z gate, fp16 out                               (fp16 MFMA; C B^T is held
+//               in fp16 and meets its decay factor in a packed fp16 multiply)
 // Both fp16 contractions over the time index need x (and B) with time as the fastest-moving index,
-// while memory has channels fastest; the tiles are transposed once on the way into LDS (4x4 blocks:
-// four dword loads, four 8-byte LDS stores) and then read as 16-byte MFMA operands.
+// while memory has channels fastest; x tiles are transposed once on the way into LDS (4x4 blocks:
+// four dword loads, four 8-byte LDS stores) and then read as 16-byte MFMA operands, B is packed in
+// operand order once per ssd group.
 #include "qa_common.hpp"
 
 namespace qa {
@@ -199,39 +202,6 @@ __global__ __launch_bounds__(64) void ssd_cb_kernel(QaSsdParams p, __half* cb_ou
                 const int k = kt * 64 + j * 32 + frow;
                 tile[static_cast<int64_t>(m) * Q + k] = __float2half((scale * static_cast<float>(acc[i][j][r])) * kCbShift);
             }
-}
-
-// ---------------------------------------------------------------------------------------------
-// Transposing stage: dst[col][k] (fp16, `pitch` halves per row) <- src rows k (int8, `row_stride`
-// bytes apart, NC columns), k in [0, KC).  value = f16((col_scale[col] * q) * k_scale[k]) when
-// K_SCALE, else f16(col_scale[col] * q).  Rows k >= k_valid read as zero.
-// ---------------------------------------------------------------------------------------------
-template <int NC, bool K_SCALE>
-__device__ __forceinline__ void stage_transposed(_Float16* dst, int pitch, const int8_t* src, int64_t row_stride,
-                                                 int KC, int k_valid, const float* col_scale, const float* k_scale,
-                                                 int tid, int nthreads) {
-    constexpr int CB = NC / 4;
-    for (int id = tid; id < (KC / 4) * CB; id += nthreads) {
-        const int kb = id / CB, cb = id % CB;
-        uint32_t w[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int k = kb * 4 + r;
-            w[r] = k < k_valid ? *reinterpret_cast<const uint32_t*>(src + k * row_stride + cb * 4) : 0u;
-        }
-#pragma unroll
-        for (int cc = 0; cc < 4; ++cc) {
-            const float cs = col_scale[cb * 4 + cc];
-            v4h o;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                float v = cs * static_cast<float>(byte_of(w[r], cc));
-                if (K_SCALE) v *= k_scale[kb * 4 + r];
-                o[r] = static_cast<_Float16>(v);
-            }
-            *reinterpret_cast<v4h*>(dst + (cb * 4 + cc) * pitch + kb * 4) = o;
-        }
-    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -485,29 +455,102 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_kernel(QaSsdParams p, c
     const int t0 = c * Q;
     const int lim = min(Q, p.seqlen - t0);
     const int64_t row_base = (static_cast<int64_t>(b) * H + h) * nc + c;
-    for (int i = tid; i < Q; i += kThreads) {
-        s_dt[i] = dt_ws[row_base * Q + i];
-        s_dA[i] = dA_ws[row_base * Q + i];
-    }
-    if (tid < kP) s_xs[tid] = x_scale_of(p, g, hg, tid);
-    {
-        const __half* pst = prev + ((static_cast<int64_t>(b) * nc + c) * H + h) * kP * N;
-        for (int piece = tid; piece < kP * N / 8; piece += kThreads) {
-            const int pr = piece / (N / 8), col = (piece % (N / 8)) * 8;
-            *reinterpret_cast<uint4*>(s_prev + pr * PPITCH + col) = *reinterpret_cast<const uint4*>(pst + pr * N + col);
-        }
-    }
-    __syncthreads();
-    stage_transposed<kP, false>(s_xt, PITCH, p.x + ((static_cast<int64_t>(b) * p.seqlen + t0) * H + h) * kP,
-                                static_cast<int64_t>(H) * kP, Q, lim, s_xs, nullptr, tid, kThreads);
-    __syncthreads();
-
     const __half* cb = cb_ws + ((static_cast<int64_t>(b) * nc + c) * G + g) * Q * Q;
-    const float D_scale = p.D ? *p.D_scale : 0.0f;
-    const float z_scale = p.z ? *p.z_scale : 0.0f;
     const int64_t row_stride = static_cast<int64_t>(H) * kP;
     const int erow = lane >> 3, ecol = (lane & 7) * 8;       // epilogue: row within a piece of 8, first of 8 columns
     const int64_t tile_base = (static_cast<int64_t>(b) * p.seqlen + t0) * row_stride + static_cast<int64_t>(h) * kP + ecol;
+
+    // Per-tile operands that come from global memory: this lane's pieces of its C row (term 1), of its
+    // row of C B^T (term 2, every k-step of the causal range) and the x / z bytes of the epilogue.  They
+    // are requested one tile ahead: the first tile's together with the prologue's reads, the next
+    // tile's piece by piece as the current tile lets go of the registers.
+    // tile order 0, NMT-1, 1, NMT-2, ...: wave w takes entries w*PER_WAVE + s
+    auto tile_of = [&](int s) {
+        const int entry = wave * PER_WAVE + s;
+        return (entry & 1) ? NMT - 1 - (entry >> 1) : (entry >> 1);
+    };
+    v8h c_frag[N / 16], cbf[KSMAX];
+    uint2 xq[4], zq[4];
+    auto c_ptr = [&](int mt, int ks) {
+        return c16 + ((static_cast<int64_t>(b) * p.seqlen + t0 + min(mt * 32 + frow, lim - 1)) * G + g) * N + ks * 16 + fhalf * 8;
+    };
+    auto cb_ptr = [&](int mt, int ks) { return cb + static_cast<int64_t>(mt * 32 + frow) * Q + fhalf * 8 + ks * 16; };
+    auto load_xz = [&](int mt, int q) {
+        const int64_t at = tile_base + min(mt * 32 + 8 * q + erow, lim - 1) * row_stride;
+        xq[q] = p.D ? *reinterpret_cast<const uint2*>(p.x + at) : make_uint2(0u, 0u);
+        zq[q] = p.z ? *reinterpret_cast<const uint2*>(p.z + at) : make_uint2(0u, 0u);
+    };
+    if (wave * PER_WAVE < NMT) {
+        const int mt = tile_of(0);
+#pragma unroll
+        for (int ks = 0; ks < N / 16; ++ks) c_frag[ks] = *reinterpret_cast<const v8h*>(c_ptr(mt, ks));
+#pragma unroll
+        for (int ks = 0; ks < KSMAX; ++ks)
+            if (ks < 2 * (mt + 1)) cbf[ks] = *reinterpret_cast<const v8h*>(cb_ptr(mt, ks));
+#pragma unroll
+        for (int q = 0; q < 4; ++q) load_xz(mt, q);
+    }
+    {
+        // Prologue: every global read is issued before the first LDS write, so that the workgroup waits
+        // for memory once.  x is transposed on the way (4x4 blocks: four dword loads, four 8-byte stores).
+        static_assert(Q <= kThreads, "one step per thread");
+        constexpr int XB = (Q / 4) * (kP / 4) / kThreads, PB = kP * N / 8 / kThreads;
+        float r_dt = 0.0f, r_dA = 0.0f;
+        if (Q == kThreads || tid < Q) {
+            r_dt = dt_ws[row_base * Q + tid];
+            r_dA = dA_ws[row_base * Q + tid];
+        }
+        const __half* pst = prev + ((static_cast<int64_t>(b) * nc + c) * H + h) * kP * N;
+        uint4 r_prev[PB];
+#pragma unroll
+        for (int i = 0; i < PB; ++i) {
+            const int piece = tid + i * kThreads, pr = piece / (N / 8), col = (piece % (N / 8)) * 8;
+            r_prev[i] = *reinterpret_cast<const uint4*>(pst + pr * N + col);
+        }
+        const int8_t* xsrc = p.x + ((static_cast<int64_t>(b) * p.seqlen + t0) * H + h) * kP;
+        const int64_t xstride = static_cast<int64_t>(H) * kP;
+        const int cb4 = tid % (kP / 4);                      // the same four columns in every block of this thread
+        uint32_t xr[XB][4];
+#pragma unroll
+        for (int i = 0; i < XB; ++i) {
+            const int kb = (tid + i * kThreads) / (kP / 4);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int k = kb * 4 + r;
+                const uint32_t v = *reinterpret_cast<const uint32_t*>(xsrc + min(k, lim - 1) * xstride + cb4 * 4);
+                xr[i][r] = k < lim ? v : 0u;
+            }
+        }
+        float cs[4];
+#pragma unroll
+        for (int cc = 0; cc < 4; ++cc) cs[cc] = x_scale_of(p, g, hg, cb4 * 4 + cc);
+        if (tid < kP) s_xs[tid] = x_scale_of(p, g, hg, tid);
+
+        if (Q == kThreads || tid < Q) {
+            s_dt[tid] = r_dt;
+            s_dA[tid] = r_dA;
+        }
+#pragma unroll
+        for (int i = 0; i < PB; ++i) {
+            const int piece = tid + i * kThreads, pr = piece / (N / 8), col = (piece % (N / 8)) * 8;
+            *reinterpret_cast<uint4*>(s_prev + pr * PPITCH + col) = r_prev[i];
+        }
+#pragma unroll
+        for (int i = 0; i < XB; ++i) {
+            const int kb = (tid + i * kThreads) / (kP / 4);
+#pragma unroll
+            for (int cc = 0; cc < 4; ++cc) {
+                v4h o;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) o[r] = static_cast<_Float16>(cs[cc] * static_cast<float>(byte_of(xr[i][r], cc)));
+                *reinterpret_cast<v4h*>(s_xt + (cb4 * 4 + cc) * PITCH + kb * 4) = o;
+            }
+        }
+    }
+    __syncthreads();
+
+    const float D_scale = p.D ? *p.D_scale : 0.0f;
+    const float z_scale = p.z ? *p.z_scale : 0.0f;
     __half* out = static_cast<__half*>(p.out);
     float e_Dv[8];                                           // D of the eight columns this lane writes
 #pragma unroll
@@ -518,10 +561,11 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_kernel(QaSsdParams p, c
 
 #pragma unroll
     for (int s = 0; s < PER_WAVE; ++s) {
-        // tile order 0, NMT-1, 1, NMT-2, ...: wave w takes entries w*PER_WAVE + s
-        const int entry = wave * PER_WAVE + s;
-        if (entry >= NMT) break;
-        const int mt = (entry & 1) ? NMT - 1 - (entry >> 1) : (entry >> 1);
+        if (wave * PER_WAVE + s >= NMT) break;
+        const int mt = tile_of(s);
+        const bool has_next = s + 1 < PER_WAVE;
+        const int mt_next = has_next ? tile_of(s + 1) : 0;
+        const int nks_next = has_next ? 2 * (mt_next + 1) : 0;
         const int m_lane = mt * 32 + frow;                 // row of this lane's A operands
         const int nks = 2 * (mt + 1);                      // k-steps of the causal range
         const int n_off = 2 * mt;                          // of which entirely before the tile
@@ -530,24 +574,6 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_kernel(QaSsdParams p, c
         for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[j][r] = 0.0f;
-
-        // all global reads of the tile
-        const __half* c_row = c16 + ((static_cast<int64_t>(b) * p.seqlen + t0 + min(m_lane, lim - 1)) * G + g) * N;
-        v8h c_frag[N / 16];
-#pragma unroll
-        for (int ks = 0; ks < N / 16; ++ks) c_frag[ks] = *reinterpret_cast<const v8h*>(c_row + ks * 16 + fhalf * 8);
-        const __half* cb_row = cb + static_cast<int64_t>(m_lane) * Q + fhalf * 8;
-        v8h cbf[KSMAX];
-#pragma unroll
-        for (int ks = 0; ks < KSMAX; ++ks)
-            if (ks < nks) cbf[ks] = *reinterpret_cast<const v8h*>(cb_row + ks * 16);
-        uint2 xq[4], zq[4];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int64_t at = tile_base + min(mt * 32 + 8 * q + erow, lim - 1) * row_stride;
-            xq[q] = p.D ? *reinterpret_cast<const uint2*>(p.x + at) : make_uint2(0u, 0u);
-            zq[q] = p.z ? *reinterpret_cast<const uint2*>(p.z + at) : make_uint2(0u, 0u);
-        }
 
         // Decay factors.  The cumulative dA decreases along the chunk, so with ref = dA at the first row
         // of this m-tile, exp(dA_m - dA_k) = exp(dA_m - ref) * exp(ref - dA_k) for every k before the
@@ -567,6 +593,7 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_kernel(QaSsdParams p, c
 #pragma unroll
         for (int ks = 0; ks < N / 16; ++ks) {
             v8h fc = c_frag[ks];
+            if (has_next) c_frag[ks] = *reinterpret_cast<const v8h*>(c_ptr(mt_next, ks));
             if (!row_ok) {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) fc[e] = static_cast<_Float16>(0.0f);
@@ -621,6 +648,7 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_kernel(QaSsdParams p, c
                     acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fl, fx, acc[j], 0, 0, 0);
                 }
             }
+            if (ks < nks_next) cbf[ks] = *reinterpret_cast<const v8h*>(cb_ptr(mt_next, ks));
         }
         wave_sync();                                    // the table is done with: its space now carries the output tile
         // Epilogue.  In the accumulators a lane holds one column p and 16 rows; memory wants rows of 64
@@ -640,20 +668,22 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_kernel(QaSsdParams p, c
             const float4 y0 = *reinterpret_cast<const float4*>(o_tab + erow * 64 + ecol);
             const float4 y1 = *reinterpret_cast<const float4*>(o_tab + erow * 64 + ecol + 4);
             wave_sync();                                // the next piece overwrites the scratch
+            const uint2 xb = xq[q], zb = zq[q];
+            if (has_next) load_xz(mt_next, q);
             if (m < lim) {
                 float y[8] = {y0.x, y0.y, y0.z, y0.w, y1.x, y1.y, y1.z, y1.w};
                 const int64_t at = tile_base + m * row_stride;
                 if (p.D) {
 #pragma unroll
                     for (int e = 0; e < 8; ++e) {
-                        const float xv = static_cast<float>(byte_of(e < 4 ? xq[q].x : xq[q].y, e & 3));
+                        const float xv = static_cast<float>(byte_of(e < 4 ? xb.x : xb.y, e & 3));
                         y[e] += (s_xs[ecol + e] * xv) * e_Dv[e];
                     }
                 }
                 if (p.z) {
 #pragma unroll
                     for (int e = 0; e < 8; ++e) {
-                        const float zv = z_scale * static_cast<float>(byte_of(e < 4 ? zq[q].x : zq[q].y, e & 3));
+                        const float zv = z_scale * static_cast<float>(byte_of(e < 4 ? zb.x : zb.y, e & 3));
                         y[e] *= zv * __builtin_amdgcn_rcpf(1.0f + fexp(-zv));
                     }
                 }
