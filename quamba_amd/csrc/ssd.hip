@@ -351,8 +351,8 @@ __global__ __launch_bounds__(256, 2) void ssd_state_kernel(QaSsdParams p, const 
     for (int c = 0; c < nc; ++c) {
         const bool more = c + 1 < nc;
         if (more) {
+            weights_load(c + 1);                               // requests return in order: the one needed first goes first
             load_x(c + 1);
-            weights_load(c + 1);
         }
 #pragma unroll
         for (int ks = 0; ks < nks; ++ks) {
