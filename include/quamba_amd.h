@@ -60,6 +60,12 @@ typedef struct QaConvParams {
     int8_t* out;
     int8_t* conv_state;        /* update only, modified in place */
     float scale_x, scale_w, scale_b, scale_out;
+    /* fwd only, optional: a second copy of the output with channels contiguous, int8 (batch, seqlen, dim),
+     * element (b, t, c) at out_t + b*out_t_batch_stride + t*out_t_l_stride + c.  It replaces the separate
+     * transposition the reference's caller runs before x_proj (quamba/qMambaLayer.py:923).  Needs the
+     * seqlen-contiguous input layout; null to skip. */
+    int8_t* out_t;
+    int64_t out_t_batch_stride, out_t_l_stride;
 } QaConvParams;
 
 int qa_causal_conv1d_fwd(const QaConvParams* p, void* stream);

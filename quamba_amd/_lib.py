@@ -28,6 +28,7 @@ class QaConvParams(C.Structure):
         ("conv_state_len", i32), ("reserved1", i32),
         ("x", vp), ("weight", vp), ("bias", vp), ("out", vp), ("conv_state", vp),
         ("scale_x", f32), ("scale_w", f32), ("scale_b", f32), ("scale_out", f32),
+        ("out_t", vp), ("out_t_batch_stride", i64), ("out_t_l_stride", i64),
     ]
 
 

@@ -73,9 +73,12 @@ class QCausalConv1D(nn.Module):
             setattr(self, k, float(state_dict.pop(prefix + k)))
 
     @torch.no_grad()
-    def forward(self, x):
+    def forward(self, x, also_channel_last=False):
+        """int8 (batch, dim, seqlen) -> int8, same strides.  ``also_channel_last=True`` returns the pair
+        (out, out as a contiguous (batch, seqlen, dim) tensor), both written by the one kernel."""
         return ops.causal_conv1d_fwd(x, self.input_scale, self.weight, self.weight_scale, self.output_scale,
-                                     self.bias_scale, self.bias, None, None, None, True)
+                                     self.bias_scale, self.bias, None, None, None, True,
+                                     also_channel_last=also_channel_last)
 
     @torch.no_grad()
     def update(self, x, conv_state):

@@ -73,6 +73,76 @@ __global__ __launch_bounds__(kConvThreads) void conv_fwd_rows_kernel(QaConvParam
     }
 }
 
+// The same arithmetic for a tile of 64 channels x 64 time steps per workgroup, writing the output twice:
+// in the input's layout (16 bytes per thread, as above) and with channels contiguous, (batch, seqlen, dim).
+// Thread (channel tid/4, segment tid%4) computes 16 steps of one channel; the 64 x 64 byte tile then
+// passes through LDS and thread (step tid/4, piece tid%4) gathers 16 channels of one step.
+__global__ __launch_bounds__(kConvThreads) void conv_fwd_rows_dual_kernel(QaConvParams p, int tiles_l, int tiles_c) {
+    constexpr int kPitch = 80;                       // bytes per staged channel row (16-byte aligned, 64 used)
+    __shared__ __attribute__((aligned(16))) uint8_t s_tile[64 * kPitch];
+    const int tid = threadIdx.x;
+    const int tl = blockIdx.x % tiles_l;
+    const int tc = (blockIdx.x / tiles_l) % tiles_c;
+    const int b = blockIdx.x / (tiles_l * tiles_c);
+    const int c_local = tid >> 2, seg = tid & 3;
+    const int c = tc * 64 + c_local;
+    const int t0 = tl * 64 + seg * 16;
+    const int remaining = p.seqlen - t0;
+    uint32_t o[4] = {0u, 0u, 0u, 0u};
+    if (c < p.dim && remaining > 0) {
+        const int8_t* x = p.x + b * p.x_batch_stride + c * p.x_c_stride;
+        int8_t* out = p.out + b * p.out_batch_stride + c * p.out_c_stride;
+        const uint32_t taps = pack_taps(p.weight + c * p.weight_c_stride, p.weight_width_stride, p.width);
+        const float s_wx = p.scale_w * p.scale_x;
+        const float bias_f = p.bias ? static_cast<float>(p.bias[c]) * p.scale_b : 0.0f;
+        const float inv_s_out = 1.0f / p.scale_out;
+        uint32_t w[5];   // w[0] = x[t0-4 .. t0-1], w[1..4] = x[t0 .. t0+15]
+        w[0] = t0 > 0 ? *reinterpret_cast<const uint32_t*>(x + t0 - 4) : 0u;
+        if (remaining >= 16) {
+            const uint4 v = *reinterpret_cast<const uint4*>(x + t0);
+            w[1] = v.x; w[2] = v.y; w[3] = v.z; w[4] = v.w;
+        } else {
+            w[1] = w[2] = w[3] = w[4] = 0u;
+            for (int i = 0; i < remaining; ++i) {
+                w[1 + (i >> 2)] |= static_cast<uint32_t>(static_cast<uint8_t>(x[t0 + i])) << (8 * (i & 3));
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            uint32_t packed = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t win = j == 3 ? w[q + 1] : __builtin_amdgcn_alignbyte(w[q + 1], w[q], j + 1);
+                const float acc = static_cast<float>(dot4(win, taps));
+                const float v = __builtin_fmaf(s_wx, acc, bias_f);
+                const int r = conv_quant(v, p.scale_out, inv_s_out, p.silu_activation);
+                packed |= static_cast<uint32_t>(r & 0xff) << (8 * j);
+            }
+            o[q] = packed;
+        }
+        if (remaining >= 16) {
+            *reinterpret_cast<uint4*>(out + t0) = make_uint4(o[0], o[1], o[2], o[3]);
+        } else {
+            for (int i = 0; i < remaining; ++i) out[t0 + i] = static_cast<int8_t>((o[i >> 2] >> (8 * (i & 3))) & 0xff);
+        }
+    }
+    *reinterpret_cast<uint4*>(s_tile + c_local * kPitch + seg * 16) = make_uint4(o[0], o[1], o[2], o[3]);
+    __syncthreads();
+    const int t_local = tid >> 2, piece = tid & 3;
+    const int t = tl * 64 + t_local;
+    const int cc0 = tc * 64 + piece * 16;
+    if (t >= p.seqlen || cc0 >= p.dim) return;
+    uint32_t g[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int i = 0; i < 16; ++i) g[i >> 2] |= static_cast<uint32_t>(s_tile[(piece * 16 + i) * kPitch + t_local]) << (8 * (i & 3));
+    int8_t* dst = p.out_t + b * p.out_t_batch_stride + t * p.out_t_l_stride + cc0;
+    if (cc0 + 16 <= p.dim && (reinterpret_cast<uintptr_t>(dst) & 15u) == 0) {
+        *reinterpret_cast<uint4*>(dst) = make_uint4(g[0], g[1], g[2], g[3]);
+    } else {
+        for (int i = 0; i < 16 && cc0 + i < p.dim; ++i) dst[i] = static_cast<int8_t>((g[i >> 2] >> (8 * (i & 3))) & 0xff);
+    }
+}
+
 // Any strides, one thread per output element.  kTapWise selects the channel-contiguous op order.
 // Lanes run along the contiguous dimension chosen by the host (lanes_along_l).
 template <bool kTapWise>
@@ -165,6 +235,15 @@ extern "C" int qa_causal_conv1d_fwd(const QaConvParams* p, void* stream_) {
         const bool rows_ok = p->out_l_stride == 1 && aligned16(p->x) && aligned16(p->out) &&
                              p->x_batch_stride % 16 == 0 && p->x_c_stride % 16 == 0 &&
                              p->out_batch_stride % 16 == 0 && p->out_c_stride % 16 == 0;
+        if (p->out_t && !rows_ok) return QA_ERR_STRIDE;
+        if (rows_ok && p->out_t) {
+            const int tiles_l = (p->seqlen + 63) / 64, tiles_c = (p->dim + 63) / 64;
+            const int64_t blocks = static_cast<int64_t>(p->batch) * tiles_l * tiles_c;
+            if (blocks > 0x7fffffffLL) return QA_ERR_SHAPE;
+            hipLaunchKernelGGL(conv_fwd_rows_dual_kernel, dim3(static_cast<unsigned>(blocks)), dim3(kConvThreads), 0,
+                               stream, *p, tiles_l, tiles_c);
+            return check_launch();
+        }
         if (rows_ok) {
             const int segs = (p->seqlen + 15) / 16;
             const int64_t threads = static_cast<int64_t>(p->batch) * p->dim * segs;
@@ -175,6 +254,7 @@ extern "C" int qa_causal_conv1d_fwd(const QaConvParams* p, void* stream_) {
             return check_launch();
         }
     }
+    if (p->out_t) return QA_ERR_STRIDE;               // the second output exists for the seqlen-contiguous layout only
     const int64_t blocks = (total + kConvThreads - 1) / kConvThreads;
     if (blocks > 0x7fffffffLL) return QA_ERR_SHAPE;
     if (channel_last) {

@@ -86,8 +86,14 @@ class W8A8QMamba(nn.Module):
         x, z = xz.chunk(2, dim=1)                                       # views
         if conv_state is not None:
             conv_state.copy_(F.pad(x, (conv_state.shape[-1] - x.shape[-1], 0)))
-        x = self.conv1d(x)                                              # same strides as its input
-        x_dbl = self.x_proj(x.transpose(1, 2).contiguous())             # (B, L, dt_rank + 2N)
+        # the conv writes its output in both layouts: (B, D, L) for the scan, (B, L, D) for x_proj
+        fused = x.stride(2) == 1 and x.stride(1) % 16 == 0 and x.stride(0) % 16 == 0 and x.data_ptr() % 16 == 0
+        if fused:
+            x, x_rows = self.conv1d(x, also_channel_last=True)
+        else:
+            x = self.conv1d(x)                                          # same strides as its input
+            x_rows = x.transpose(1, 2).contiguous()
+        x_dbl = self.x_proj(x_rows)                                     # (B, L, dt_rank + 2N)
         dt, B, C = torch.split(x_dbl, [self.dt_rank, self.d_state, self.d_state], dim=-1)
         dt = self.dt_proj.to_seqlen_last(dt.contiguous())               # (B, D, L)
         B = B.transpose(1, 2).contiguous()                              # (B, N, L)

@@ -29,8 +29,10 @@ def _require_gpu(t, name):
 # causal conv1d
 # ----------------------------------------------------------------------------------------------
 def causal_conv1d_fwd(x, scale_x, weight, scale_w, scale_out, scale_b, bias=None, seq_idx=None,
-                      initial_states=None, final_states_out=None, silu_activation=True):
-    """int8 (batch, dim, seqlen) -> int8 of the same shape and strides."""
+                      initial_states=None, final_states_out=None, silu_activation=True, also_channel_last=False):
+    """int8 (batch, dim, seqlen) -> int8 of the same shape and strides.  With ``also_channel_last`` the kernel
+    writes the result a second time as a contiguous (batch, seqlen, dim) tensor (what x_proj reads; the
+    reference's caller makes that copy in a separate pass, quamba/qMambaLayer.py:923) and both are returned."""
     _require(x.dtype == torch.int8 and weight.dtype == torch.int8, "x and weight must be int8")
     _require_gpu(x, "x")
     _require_gpu(weight, "weight")
@@ -60,10 +62,17 @@ def causal_conv1d_fwd(x, scale_x, weight, scale_w, scale_out, scale_b, bias=None
     p.weight_c_stride, p.weight_width_stride = weight.stride()
     p.x, p.weight, p.bias, p.out = ptr(x), ptr(weight), ptr(bias), ptr(out)
     p.scale_x, p.scale_w, p.scale_b, p.scale_out = float(scale_x), float(scale_w), float(scale_b), float(scale_out)
+    out_t = None
+    if also_channel_last:
+        _require(x.stride(2) == 1 and x.stride(1) % 16 == 0 and x.stride(0) % 16 == 0 and x.data_ptr() % 16 == 0,
+                 "also_channel_last needs a seqlen-contiguous input with 16-byte aligned rows")
+        out_t = torch.empty((batch, seqlen, dim), dtype=torch.int8, device=x.device)
+        p.out_t = ptr(out_t)
+        p.out_t_batch_stride, p.out_t_l_stride = out_t.stride(0), out_t.stride(1)
     with torch.cuda.device(x.device):
         st = _lib.lib().qa_causal_conv1d_fwd(ct.byref(p), _lib.current_stream(x.device))
     _lib.check(st, "causal_conv1d_fwd")
-    return out
+    return (out, out_t) if also_channel_last else out
 
 
 def causal_conv1d_update(x, conv_state, scale_x, weight, scale_w, scale_out, scale_b, bias=None,

@@ -121,3 +121,19 @@ def test_errors(dev):
         ops.causal_conv1d_fwd(x, 1.0, w, 1.0, 1.0, 1.0, None, torch.zeros(1, device=dev))
     with pytest.raises(RuntimeError, match="GPU"):
         ops.causal_conv1d_fwd(x.cpu(), 1.0, w, 1.0, 1.0, 1.0)
+
+
+@pytest.mark.parametrize("B,D,L", [(2, 64, 64), (1, 96, 100), (3, 200, 333), (2, 5120, 256), (1, 48, 17)])
+def test_second_output_with_channels_contiguous(dev, B, D, L):
+    """The optional (batch, seqlen, dim) copy written by the same kernel equals the transposed first output, and
+    the first output equals the oracle bit for bit (ragged tiles in both directions included)."""
+    qx, sx = synth.quantize_absmax(synth.activations((B, D, L + (-L) % 16), 1, 7 + D, "x"))
+    qw, sw, qb, sb = synth.conv_weights(D, 4, 11)
+    so = synth.conv_output_scale(qx, sx, qw, sw, qb, sb)
+    x = torch.from_numpy(qx).to(dev)[:, :, :L]               # rows stay 16-byte aligned, seqlen may be ragged
+    out, out_t = ops.causal_conv1d_fwd(x, sx, torch.from_numpy(qw).to(dev), sw, so, sb, torch.from_numpy(qb).to(dev),
+                                       also_channel_last=True)
+    want = oracle.conv1d_fwd(np.ascontiguousarray(qx[:, :, :L]), qw, qb, sx, sw, sb, so)
+    assert out_t.shape == (B, L, D) and out_t.is_contiguous()
+    np.testing.assert_array_equal(out.cpu().numpy(), want)
+    np.testing.assert_array_equal(out_t.cpu().numpy(), want.transpose(0, 2, 1))
