@@ -254,7 +254,17 @@ def other_workloads(dev, steps, warmup):
                         us=ms * 1e3, tokens_per_s=B / ms * 1e3, bound="hbm", achieved_GBs=nbytes / ms / 1e6,
                         frac=nbytes / ms / 1e6 / HBM_PEAK_GBS))
         del graph, states
-    del layers
+    # the same mixer module over a whole prompt: W8A8QMamba.forward, batch 8 x 2048 (in_proj, conv writing both
+    # layouts, x_proj, dt_proj, selective scan, Hadamard, out_proj, and the small layout copies between them)
+    m = layers[0]
+    Bp, Lp = 8, 2048
+    hp = ri(Bp, Lp, 2560)
+    ms = _time_fn(lambda: m.forward(hp), min(steps, 10), 3)
+    out.append(dict(workload="Mamba1-2.8b W8A8 mixer forward over a prompt (all seven kernels), batch 8 x 2048",
+                    us=ms * 1e3, tokens_per_s=Bp * Lp / ms * 1e3, bound="mfma",
+                    achieved_TOPs=2.0 * Bp * Lp * (2560 * 10240 + 5120 * 192 + 160 * 5120 + 5120 * 2560) / ms / 1e9,
+                    frac=2.0 * Bp * Lp * (2560 * 10240 + 5120 * 192 + 160 * 5120 + 5120 * 2560) / ms / 1e9 / INT8_PEAK_TOPS))
+    del layers, m, hp
     # SSD: batch 4, seqlen 4096, 80 heads of 64, d_state 128, 1 group, chunk 256
     B, L, H, N, G, Q = 4, 4096, 80, 128, 1, 256
     x, dt, Bm, Cm = ri(B, L, H, 64), ri(B, L, H), ri(B, L, G, N), ri(B, L, G, N)
