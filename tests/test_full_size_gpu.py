@@ -1,0 +1,235 @@
+"""Parity at the full sizes of the benchmark configurations.
+
+The CPU oracle cannot cover 16384 tokens x 5120 channels in seconds, so every kernel runs once at the full
+shape on random int8 operands generated on the GPU and is checked two ways:
+  * the oracle on a sample of rows / channels / heads cut from the same operands (bit-exact for int8 and
+    GEMM outputs, rtol 1e-2 / atol 1e-2 for fp16 scan outputs, 1e-3 relative for fp32 states);
+  * a property that does not depend on the size: a prefix of the sequence gives a prefix of the result,
+    the second output of the conv is the transposed first, the SSD result does not depend on the chunk
+    size, a row of a GEMM does not depend on the other rows.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from quamba_amd import QCausalConv1D, ops
+from quamba_amd import w4a8_utils as wu
+
+pytestmark = pytest.mark.gpu
+
+
+def _ri(dev, *shape, seed=0, lo=-128, hi=128):
+    g = torch.Generator(device=dev).manual_seed(seed)
+    return torch.randint(lo, hi, shape, dtype=torch.int8, device=dev, generator=g)
+
+
+def _s(v, dev):
+    return torch.tensor([float(v)], dtype=torch.float32, device=dev)
+
+
+def _np(t):
+    return np.ascontiguousarray(t.cpu().numpy())
+
+
+# ---------------------------------------------------------------- Mamba1-2.8b prefill: batch 8 x 2048, d_inner 5120
+B1, L1, D1, N1 = 8, 2048, 5120, 16
+
+
+def test_conv_full_size(dev):
+    xz = _ri(dev, 2 * D1, B1, L1, seed=1).permute(1, 0, 2)           # what in_proj.to_seqlen_last leaves
+    x = xz[:, :D1]
+    w, b = _ri(dev, D1, 4, seed=2), _ri(dev, D1, seed=3)
+    sx, sw, sb, so = 0.04, 0.004, 0.004, 0.03
+    out, out_rows = ops.causal_conv1d_fwd(x, sx, w, sw, so, sb, b, also_channel_last=True)
+    single = ops.causal_conv1d_fwd(x, sx, w, sw, so, sb, b)
+    assert torch.equal(out, single) and out.stride() == x.stride()
+    assert torch.equal(out_rows, out.transpose(1, 2))
+    # oracle on sampled (batch, channel) rows
+    g = np.random.default_rng(0)
+    for bi in (0, 5, 7):
+        ch = np.sort(g.choice(D1, 24, replace=False))
+        cht = torch.from_numpy(ch).to(dev)
+        want = oracle.conv1d_fwd(_np(x[bi:bi + 1, cht]), _np(w[cht]), _np(b[cht]), sx, sw, sb, so)
+        np.testing.assert_array_equal(_np(out[bi:bi + 1, cht]), want)
+    # a prefix of the sequence gives a prefix of the result (ragged length: the bytewise tail)
+    part = ops.causal_conv1d_fwd(x[:, :, :1003], sx, w, sw, so, sb, b)
+    assert torch.equal(part, out[:, :, :1003])
+
+
+def test_selective_scan_full_size(dev):
+    u, dt, z = (_ri(dev, B1, D1, L1, seed=s) for s in (4, 5, 6))
+    Bm, Cm = _ri(dev, B1, 1, N1, L1, seed=7), _ri(dev, B1, 1, N1, L1, seed=8)
+    A, Dq, db = _ri(dev, D1, N1, seed=9), _ri(dev, D1, seed=10), _ri(dev, D1, seed=11)
+    sc = dict(s_u=0.03, s_delta=0.02, s_A=0.02, s_B=0.03, s_C=0.03, s_D=0.008, s_z=0.03, s_db=0.01)
+    run = lambda sl: ops.sscan_fwd(u[..., sl], _s(sc["s_u"], dev), dt[..., sl], _s(sc["s_delta"], dev), A, _s(sc["s_A"], dev),
+                                   Bm[..., sl], _s(sc["s_B"], dev), Cm[..., sl], _s(sc["s_C"], dev), _s(1.0, dev), Dq,
+                                   _s(sc["s_D"], dev), z[..., sl], _s(sc["s_z"], dev), db, _s(sc["s_db"], dev), True,
+                                   state_dtype=torch.float32)
+    y, state = run(slice(None))
+    assert y.shape == (B1, L1, D1) and state.shape == (B1, D1, 1, N1)
+    # oracle on sampled channels of sampled batch entries
+    for bi, c0 in ((0, 0), (3, 2555), (7, D1 - 8)):
+        ch = slice(c0, c0 + 8)
+        y_ref, _, st_ref = oracle.sscan_fwd(_np(u[bi:bi + 1, ch]), _np(dt[bi:bi + 1, ch]), _np(A[ch]), _np(Bm[bi:bi + 1, 0]),
+                                            _np(Cm[bi:bi + 1, 0]), _np(Dq[ch]), _np(db[ch]), _np(z[bi:bi + 1, ch]), **sc)
+        got = y[bi:bi + 1, :, ch].float().cpu().numpy()
+        np.testing.assert_allclose(got, y_ref.astype(np.float16).astype(np.float32), rtol=1e-2, atol=1e-2)
+        got_st = state[bi:bi + 1, ch, 0].cpu().numpy()
+        assert np.abs(got_st - st_ref).max() <= 1e-3 * np.abs(st_ref).max()
+    # a prefix of the sequence gives the same outputs for those steps, bit for bit
+    y_half, _ = run(slice(0, 1024 + 40))
+    assert torch.equal(y_half, y[:, :1024 + 40])
+
+
+def _sampled_rows_w8a8(dev, M, N, K, out_dtype, seed):
+    a, w = _ri(dev, M, K, seed=seed), _ri(dev, N, K, seed=seed + 1)
+    g = torch.Generator(device=dev).manual_seed(seed + 2)
+    sa = (torch.rand(M, device=dev, generator=g) + 0.5) * (0.4 / np.sqrt(K))
+    sb = (torch.rand(N, device=dev, generator=g) + 0.5) * 0.02
+    c = torch.empty((M, N), dtype=out_dtype, device=dev)
+    ops.scaled_mm_dq(c, a, w.t(), sa, sb)
+    rows = np.sort(np.random.default_rng(seed).choice(M, 48, replace=False))
+    rt = torch.from_numpy(rows).to(dev)
+    _, f, q = oracle.gemm_w8a8(_np(a[rt]), _np(w), _np(sa[rt]), _np(sb))
+    got = _np(c[rt])
+    if out_dtype == torch.int8:
+        np.testing.assert_array_equal(got, q)
+        assert np.abs(q).max() > 20
+    else:
+        np.testing.assert_array_equal(got, f.astype(np.float16))
+    # a row does not depend on the other rows: the same rows alone (the few-rows kernel) give the same bytes
+    c2 = torch.empty((len(rows), N), dtype=out_dtype, device=dev)
+    ops.scaled_mm_dq(c2, a[rt].contiguous(), w.t(), sa[rt].contiguous(), sb)
+    assert torch.equal(c2, c[rt])
+
+
+def test_w8a8_in_proj_full_size(dev):
+    _sampled_rows_w8a8(dev, B1 * L1, 2 * D1, 2560, torch.int8, seed=20)
+
+
+def test_w8a8_out_proj_full_size(dev):
+    _sampled_rows_w8a8(dev, B1 * L1, 2560, D1, torch.float16, seed=30)
+
+
+# ---------------------------------------------------------------- decode: batch 64, 1000 steps
+def test_decode_1000_steps(dev):
+    Bd, steps = 64, 1000
+    conv = QCausalConv1D(D1, D1, 4, groups=D1, device=dev)
+    conv.weight, conv.bias = _ri(dev, D1, 4, seed=40), _ri(dev, D1, seed=41)
+    conv.weight_scale, conv.bias_scale, conv.input_scale, conv.output_scale = 0.004, 0.004, 0.04, 0.03
+    conv_state = _ri(dev, Bd, D1, 3, seed=42)
+    g = torch.Generator(device=dev).manual_seed(43)
+    ssm_state = torch.randn(Bd, D1, N1, device=dev, generator=g) * 0.1
+    A, Dq, db = _ri(dev, D1, N1, seed=44), _ri(dev, D1, seed=45), _ri(dev, D1, seed=46)
+    ring = [tuple(_ri(dev, *shape, seed=100 + 5 * i + j) for j, shape in
+                  enumerate(((Bd, D1), (Bd, D1), (Bd, N1), (Bd, N1), (Bd, D1)))) for i in range(16)]
+    sc = dict(s_x=0.03, s_dt=0.02, s_A=0.02, s_B=0.03, s_C=0.03, s_D=0.008, s_z=0.04, s_db=0.01)
+    # the sampled rows the oracle follows
+    rows = torch.tensor([0, 17, 63], device=dev)
+    ch = torch.from_numpy(np.sort(np.random.default_rng(1).choice(D1, 16, replace=False))).to(dev)
+    cs_ref = _np(conv_state[rows][:, ch])
+    st_ref = _np(ssm_state[rows][:, ch])
+    w_s, b_s, A_s, D_s, db_s = _np(conv.weight[ch]), _np(conv.bias[ch]), _np(A[ch]), _np(Dq[ch]), _np(db[ch])
+    ring_s = [tuple(_np(t[rows][:, ch]) if t.shape[1] == D1 else _np(t[rows]) for t in r) for r in ring]
+    y = None
+    for i in range(steps):
+        x, dt, Bv, Cv, z = ring[i % 16]
+        xc = conv.update(x, conv_state)
+        y = ops.sscan_update(ssm_state, xc, _s(sc["s_x"], dev), dt, _s(sc["s_dt"], dev), A, _s(sc["s_A"], dev), None, Bv,
+                             _s(sc["s_B"], dev), Cv, _s(sc["s_C"], dev), Dq, _s(sc["s_D"], dev), z, _s(sc["s_z"], dev), db,
+                             _s(sc["s_db"], dev), True)
+    y_ref = None
+    for i in range(steps):
+        x, dt, Bv, Cv, z = ring_s[i % 16]
+        xc, cs_ref = oracle.conv1d_update(x, cs_ref, w_s, b_s, 0.04, 0.004, 0.004, 0.03)
+        y_ref, st_ref = oracle.sscan_update(st_ref, xc, dt, A_s, Bv, Cv, D_s, db_s, z, **sc)
+    np.testing.assert_array_equal(_np(conv_state[rows][:, ch]), cs_ref)
+    got_st = _np(ssm_state[rows][:, ch])
+    assert np.abs(got_st - st_ref).max() <= 1e-3 * np.abs(st_ref).max()
+    got_y = y[rows][:, ch].float().cpu().numpy()
+    np.testing.assert_allclose(got_y, y_ref.astype(np.float16).astype(np.float32), rtol=1e-2, atol=1e-2)
+
+
+# ---------------------------------------------------------------- Mamba2-2.7b SSD: batch 4 x 4096, 80 heads, d_state 128
+def _ssd(dev, x, dt, A, Bm, Cm, Dq, bias, Q, sc, **kw):
+    return ops.ssd_chunk_scan_combined_fwd(x, sc["x"], dt, _s(sc["dt"], dev), A, _s(sc["A"], dev), Bm, sc["B"], Cm, sc["C"], None, Q,
+                                           q_D=Dq, D_scale=_s(sc["D"], dev), dt_bias=bias, dt_softplus=True,
+                                           final_state_dtype=torch.float32, **kw)
+
+
+def test_ssd_full_size(dev):
+    B, L, H, N, G = 4, 4096, 80, 128, 1
+    x, dt = _ri(dev, B, L, H, 64, seed=50), _ri(dev, B, L, H, seed=51)
+    Bm, Cm = _ri(dev, B, L, G, N, seed=52), _ri(dev, B, L, G, N, seed=53)
+    A, Dq = _ri(dev, H, seed=54), _ri(dev, H, seed=55)
+    bias = torch.full((H,), -3.0, dtype=torch.float16, device=dev)          # step sizes around 1e-2 .. 3e-1
+    sc = dict(x=_s(0.03, dev), dt=0.02, A=0.02, B=_s(0.03, dev), C=_s(0.03, dev), D=0.008)
+    y, final = _ssd(dev, x, dt, A, Bm, Cm, Dq, bias, 256, sc)
+    # the result does not depend on the chunk size
+    y128, final128 = _ssd(dev, x, dt, A, Bm, Cm, Dq, bias, 128, sc)
+    scale = float(y.float().abs().max())
+    assert float((y.float() - y128.float()).abs().max()) <= 2e-2 * scale
+    assert float((final - final128).abs().max()) <= 2e-3 * float(final.abs().max())
+    # oracle on two heads of one batch entry
+    for bi, h in ((1, 3), (3, 77)):
+        hs = slice(h, h + 1)
+        ref = oracle.ssd_fwd(_np(x[bi:bi + 1, :, hs]), _np(dt[bi:bi + 1, :, hs]), _np(A[hs]), _np(Bm[bi:bi + 1]), _np(Cm[bi:bi + 1]),
+                             _np(Dq[hs]), None, _np(bias[hs]), chunk_size=256, x_scale=0.03, s_dt=0.02, s_A=0.02, s_B=0.03,
+                             s_C=0.03, s_D=0.008)
+        got = y[bi:bi + 1, :, hs].float().cpu().numpy()
+        s_ref = np.abs(ref["y"]).max()
+        np.testing.assert_allclose(got / s_ref, ref["y"].astype(np.float16).astype(np.float32) / s_ref, rtol=1e-2, atol=1e-2)
+        got_f = final[bi:bi + 1, hs].cpu().numpy()
+        assert np.abs(got_f - ref["final_f32"]).max() <= 1e-3 * np.abs(ref["final_f32"]).max()
+
+
+# ---------------------------------------------------------------- Mamba2-8b W4A8 layer: 16 x 1024 tokens
+def _sampled_rows_w4a8(dev, M, N, K, out8, seed):
+    a = _ri(dev, M, K, seed=seed)
+    g = torch.Generator(device=dev).manual_seed(seed + 1)
+    codes = torch.randint(0, 16, (N, K), dtype=torch.uint8, device=dev, generator=g)
+    sg = (torch.rand(K // 128, N, device=dev, generator=g) * 13.8 + 2.0).half()
+    sch = (torch.rand(N, device=dev, generator=g) + 0.5) * (0.06 / np.sqrt(K) / 8)
+    st = torch.rand(M, device=dev, generator=g) + 0.5
+    packed = wu.pack_w4a8(codes.t())
+    fn = ops.w4a8o8_gemm if out8 else ops.w4a8o16_gemm
+    c = fn(a, packed, st, sch[None], sg, None, M, N, K, False)
+    rows = np.sort(np.random.default_rng(seed).choice(M, 32, replace=False))
+    rt = torch.from_numpy(rows).to(dev)
+    _, _, f, q = oracle.gemm_w4a8(_np(a[rt]), _np(codes), _np(sg), _np(sch), _np(st[rt]))
+    got = _np(c[rt])
+    if out8:
+        np.testing.assert_array_equal(got, q)
+        assert np.abs(q).max() > 20
+    else:
+        np.testing.assert_array_equal(got, f.astype(np.float16))
+
+
+def test_w4a8_in_proj_full_size(dev):
+    _sampled_rows_w4a8(dev, 16 * 1024, 18560, 4096, True, seed=60)
+
+
+def test_w4a8_out_proj_full_size(dev):
+    _sampled_rows_w4a8(dev, 16 * 1024, 4096, 8192, False, seed=70)
+
+
+def test_ssd_8b_shape_chunk_independence(dev):
+    B, L, H, N, G = 16, 1024, 128, 128, 8
+    x, dt = _ri(dev, B, L, H, 64, seed=80), _ri(dev, B, L, H, seed=81)
+    Bm, Cm = _ri(dev, B, L, G, N, seed=82), _ri(dev, B, L, G, N, seed=83)
+    A, Dq = _ri(dev, H, seed=84), _ri(dev, H, seed=85)
+    bias = torch.full((H,), -3.0, dtype=torch.float16, device=dev)
+    g = torch.Generator(device=dev).manual_seed(86)
+    # grouped scales: four head groups and four dim groups per ssd group
+    xs = torch.rand(G, 4, 4, device=dev, generator=g) * 0.02 + 0.02
+    hr = (torch.arange(1, 5, dtype=torch.int32, device=dev) * 4).repeat(G, 1)
+    dr = (torch.arange(1, 5, dtype=torch.int32, device=dev) * 16).repeat(G, 4, 1)
+    sc = dict(x=xs, dt=0.02, A=0.02, B=torch.rand(G, device=dev, generator=g) * 0.02 + 0.02,
+              C=torch.rand(G, device=dev, generator=g) * 0.02 + 0.02, D=0.008)
+    kw = dict(x_head_group_range=hr, x_dim_group_range=dr)
+    y, final = _ssd(dev, x, dt, A, Bm, Cm, Dq, bias, 256, sc, **kw)
+    y64, final64 = _ssd(dev, x, dt, A, Bm, Cm, Dq, bias, 64, sc, **kw)
+    scale = float(y.float().abs().max())
+    assert float((y.float() - y64.float()).abs().max()) <= 2e-2 * scale
+    assert float((final - final64).abs().max()) <= 2e-3 * float(final.abs().max())
