@@ -344,6 +344,45 @@ def other_workloads(dev, steps, warmup):
     out.append(dict(workload="gated RMS norm, 16384 rows x 8192 (fp16 in, int8 gate, fp16 out)", us=ms * 1e3,
                     tokens_per_s=16384 / ms * 1e3, bound="hbm", achieved_GBs=nbytes / ms / 1e6,
                     frac=nbytes / ms / 1e6 / HBM_PEAK_GBS))
+    del xn, zn, wn
+    torch.cuda.empty_cache()
+    # the whole Mamba2-8b W4A8 mixer over a prompt (W4A8QMamba2.forward: in_proj, xBC conv, SSD chunk scan, gated
+    # norm, Hadamard, out_proj), 16 x 1024 tokens, d_model 4096, 128 heads of 64, d_state 128, 8 groups, chunk 256
+    from quamba_amd import W4A8QMamba2
+    G = 8
+    m2 = W4A8QMamba2(4096, 128, 4, 2, 64, ngroups=G, chunk_size=256, device=dev, state_dtype=torch.float32)
+    gen = torch.Generator(device=dev).manual_seed(5)
+    for lin, s_ch in ((m2.in_proj, 2e-4), (m2.out_proj, 1e-5)):
+        n, k = lin.size_n, lin.size_k
+        lin.weight = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device=dev, generator=gen)
+        lin.s_group = (torch.rand(k // 128, n, device=dev, generator=gen) * 13.8 + 2.0).half()
+        lin.s_channel = torch.full((1, n), s_ch, device=dev)
+        lin.input_scale = torch.tensor(0.05, device=dev)
+    c2 = m2.conv1d
+    dim = c2.weight.shape[0]
+    c2.weight, c2.bias = ri(dim, 4), ri(dim)
+    c2.x_scale = c2.B_scale = c2.C_scale = 0.03
+    c2.wx_scale = c2.wB_scale = c2.wC_scale = 0.004
+    c2.bx_scale = c2.bB_scale = c2.bC_scale = 0.002
+    c2.x_out_scales = torch.full((G, 4, 4), 0.02, device=dev)
+    c2.B_out_scales = c2.C_out_scales = torch.full((G,), 0.02, device=dev)
+    c2.x_head_group_range = (torch.arange(1, 5, dtype=torch.int32, device=dev) * 4).repeat(G, 1)
+    c2.x_dim_group_range = (torch.arange(1, 5, dtype=torch.int32, device=dev) * 16).repeat(G, 4, 1)
+    q2 = m2.qchunk_scan
+    q2.A_log, q2.D = ri(m2.nheads), ri(m2.nheads)
+    q2.dt_bias = torch.full((m2.nheads,), -3.0, dtype=torch.float16, device=dev)
+    q2.A_log_scale, q2.D_scale, q2.dt_scale = (torch.tensor(v, device=dev) for v in (0.02, 0.008, 0.02))
+    q2.x_scales, q2.B_scale, q2.C_scale = c2.x_out_scales, c2.B_out_scales, c2.C_out_scales
+    q2.x_head_group_range, q2.x_dim_group_range = c2.x_head_group_range, c2.x_dim_group_range
+    m2.norm.weight = torch.ones(m2.d_ssm, dtype=torch.float16, device=dev)
+    m2.norm.z_scale = 0.03
+    m2.had.x_H_scale = 0.04
+    u2 = ri(16, 1024, 4096)
+    ms = _time_fn(lambda: m2.forward(u2), min(steps, 10), 3)
+    gemm_ops = 2.0 * 16384 * (4096 * m2.in_proj.size_n + 8192 * 4096)
+    out.append(dict(workload="Mamba2-8b W4A8 mixer forward over a prompt (all six kernels), 16 x 1024 tokens",
+                    us=ms * 1e3, tokens_per_s=16384 / ms * 1e3, bound="mfma", achieved_TOPs=gemm_ops / ms / 1e9,
+                    frac=gemm_ops / ms / 1e9 / INT8_PEAK_TOPS))
     return out
 
 
