@@ -131,6 +131,7 @@ class QaGemmW4A8Params(C.Structure):
         ("tok_scale_numel", i32), ("output_transpose", i32), ("reserved0", i32),
         ("lda", i64), ("ldd", i64),
         ("a", vp), ("w_packed", vp), ("s_group", vp), ("s_channel", vp), ("s_token", vp), ("d", vp),
+        ("w8_workspace", vp), ("w8_workspace_bytes", i64),
     ]
 
 

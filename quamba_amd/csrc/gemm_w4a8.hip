@@ -378,6 +378,32 @@ int dispatch_skinny(const QaGemmW4A8Params& p, hipStream_t stream) {
     return (wide || p.k >= 16 * 2 * kBK) ? launch_skinny<2, 4, 8, 2>(p, stream) : launch_skinny<2, 4, 4, 2>(p, stream);
 }
 
+// ---------------------------------------------------------------------------------------------
+// The weights expanded to int8 once: w8 (N, K) row-major, the layout the int8 x int8 kernel reads.
+// One thread = 32 codes (16 packed bytes in, 32 bytes out), with the same expansion as the fused kernel.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void w4_expand_kernel(QaGemmW4A8Params p, int8_t* w8) {
+    const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    const int per_row = p.k / 32;
+    if (idx >= static_cast<int64_t>(p.n) * per_row) return;
+    const int n = static_cast<int>(idx / per_row), piece = static_cast<int>(idx % per_row);
+    const uint4 v = *reinterpret_cast<const uint4*>(p.w_packed + static_cast<int64_t>(n) * (p.k / 2) + piece * 16);
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    uint2 e[4];
+    if (p.group_size > 0) {
+        const __half sc = static_cast<const __half*>(p.s_group)[static_cast<int64_t>(piece / 4) * p.n + n];
+        const __half2 s2 = __half2half2(sc);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) e[t] = expand_grouped(w[t], s2);
+    } else {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) e[t] = expand_per_channel(w[t]);
+    }
+    int8_t* dst = w8 + static_cast<int64_t>(n) * p.k + piece * 32;
+    *reinterpret_cast<uint4*>(dst) = make_uint4(e[0].x, e[0].y, e[1].x, e[1].y);
+    *reinterpret_cast<uint4*>(dst + 16) = make_uint4(e[2].x, e[2].y, e[3].x, e[3].y);
+}
+
 }  // namespace
 }  // namespace qa
 
@@ -396,6 +422,23 @@ extern "C" int qa_gemm_w4a8(const QaGemmW4A8Params* p, void* stream_) {
     if (static_cast<int64_t>(p->m) * p->lda >= 0x70000000LL) return QA_ERR_SHAPE;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     if (p->m <= 64 && static_cast<int64_t>(p->n) * (p->k / 2) < 0x70000000LL) return dispatch_skinny(*p, stream);
+    const int64_t w8_bytes = static_cast<int64_t>(p->n) * p->k;
+    if (p->w8_workspace && !p->output_transpose && p->w8_workspace_bytes >= w8_bytes && aligned16(p->w8_workspace) &&
+        w8_bytes < 0x70000000LL) {
+        int8_t* w8 = static_cast<int8_t*>(p->w8_workspace);
+        const int64_t threads = static_cast<int64_t>(p->n) * (p->k / 32);
+        hipLaunchKernelGGL(w4_expand_kernel, dim3(static_cast<unsigned>((threads + 255) / 256)), dim3(256), 0, stream, *p, w8);
+        // (acc * s_channel[n]) * s_token[m] and s_token[m] * (s_channel[n] * acc) round the same two products
+        QaGemmW8A8Params q = {};
+        q.m = p->m; q.n = p->n; q.k = p->k;
+        q.lda = p->lda; q.ldw = p->k; q.ldd = p->ldd;
+        q.a = p->a; q.w = w8; q.d = p->d;
+        q.a_scale = p->s_token; q.a_scale_numel = p->tok_scale_numel;
+        q.w_scale = p->s_channel; q.w_scale_numel = p->n;
+        q.out_type = p->out_type;
+        q.round_mode = QA_ROUND_RNE;
+        return qa_gemm_w8a8(&q, stream_);
+    }
     const int64_t big_tiles = static_cast<int64_t>((p->m + 255) / 256) * ((p->n + 255) / 256);
     if (big_tiles >= 192) return launch_gemm<4, 2, 2, 4>(*p, stream);
     return launch_gemm<2, 2, 2, 2>(*p, stream);

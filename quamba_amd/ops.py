@@ -541,6 +541,10 @@ def w8a8o8_gemv(y, w, x, b_scales, a_scale):
 # ----------------------------------------------------------------------------------------------
 # W4A8 linear
 # ----------------------------------------------------------------------------------------------
+# products at least this large get a scratch buffer for expanding the 4-bit weights once per call
+W4A8_EXPAND_ONCE_OPS = 4e11
+
+
 def _w4a8_gemm(a, b_q_weight, s_tok, s_ch, s_group, m, n, k, output_transpose, out_dtype):
     _require(a.dtype == torch.int8 and a.is_cuda and a.dim() == 2 and a.is_contiguous(), "a must be a contiguous int8 GPU matrix")
     _require(tuple(a.shape) == (m, k), "a must have shape (m, k)")
@@ -565,6 +569,11 @@ def _w4a8_gemm(a, b_q_weight, s_tok, s_ch, s_group, m, n, k, output_transpose, o
     s_ch_c, s_tok_c = s_ch.contiguous(), s_tok.contiguous()
     p.a, p.w_packed, p.s_group = ptr(a), ptr(b_q_weight), ptr(s_group) if grouped else None
     p.s_channel, p.s_token, p.d = ptr(s_ch_c), ptr(s_tok_c), ptr(d)
+    w8 = None
+    if not output_transpose and 2.0 * m * n * k >= W4A8_EXPAND_ONCE_OPS:
+        # many rows: scratch for the weights expanded to int8 once (see QaGemmW4A8Params.w8_workspace)
+        w8 = torch.empty(n * k, dtype=torch.int8, device=a.device)
+        p.w8_workspace, p.w8_workspace_bytes = ptr(w8), w8.numel()
     with torch.cuda.device(a.device):
         st = _lib.lib().qa_gemm_w4a8(ct.byref(p), _lib.current_stream(a.device))
     _lib.check(st, "gemm_w4a8")

@@ -158,3 +158,19 @@ def test_reference_checkpoint_loads_and_computes_the_same(dev):
     x = torch.randint(-128, 128, (3, 50, K), dtype=torch.int8, device=dev)
     assert torch.equal(m(x), native(x))
     assert m(x).float().abs().max() > 0.1
+
+
+@pytest.mark.parametrize("grouped", [True, False])
+@pytest.mark.parametrize("out8", [True, False])
+def test_expanding_the_weights_once_gives_the_same_bits(dev, monkeypatch, grouped, out8):
+    """With a scratch buffer the weights are expanded to int8 once and the int8 x int8 kernel runs on them;
+    the wrapper only passes the buffer for large products, so the threshold is lowered here."""
+    M, N, K = 300, 520, 512
+    a, codes, sg, sc, st = _case(M, N, K, seed=9, grouped=grouped)
+    fused = _run(dev, a, codes, sg, sc, st, out8)
+    monkeypatch.setattr(ops, "W4A8_EXPAND_ONCE_OPS", 0.0)
+    once = _run(dev, a, codes, sg, sc, st, out8)
+    assert torch.equal(fused, once)
+    per_tensor = _run(dev, a, codes, sg, sc, st, out8, per_token=False)
+    monkeypatch.setattr(ops, "W4A8_EXPAND_ONCE_OPS", 1e30)
+    assert torch.equal(per_tensor, _run(dev, a, codes, sg, sc, st, out8, per_token=False))
