@@ -19,11 +19,14 @@ import torch.nn.functional as F
 
 from .conv import QCausalConv1D
 from .hadamard import QHadamard
-from .linear import W8A8B8O8Linear, W8A8B16O16Linear
+from .linear import (W4A8B8O8Linear, W4A8B8O8LinearParallel, W4A8B16O16Linear, W8A8B8O8Linear, W8A8B8O8LinearParallel,
+                     W8A8B16O16Linear)
 from .sscan import QSScan
 
 
 class W8A8QMamba(nn.Module):
+    # the linear layers of this precision (W4A8QMamba overrides them); dt_proj is W8A8 in both
+    _in_proj_cls, _x_proj_cls, _out_proj_cls = W8A8B8O8Linear, W8A8B8O8Linear, W8A8B16O16Linear
 
     def __init__(self, d_model, d_state=16, d_conv=4, expand=2, dt_rank="auto", conv_bias=True, bias=False,
                  use_had_transform=True, layer_idx=None, device=None, state_dtype=torch.int8, **kwargs):
@@ -39,14 +42,14 @@ class W8A8QMamba(nn.Module):
         self.dt_rank = math.ceil(d_model / 16) if dt_rank == "auto" else dt_rank
         self.layer_idx = layer_idx
         self.state_dtype = state_dtype        # int8 (the reference) or fp32 recurrent state
-        self.in_proj = W8A8B8O8Linear(d_model, self.d_inner * 2, device=device)
+        self.in_proj = self._in_proj_cls(d_model, self.d_inner * 2, device=device)
         self.conv1d = QCausalConv1D(self.d_inner, self.d_inner, d_conv, groups=self.d_inner, padding=d_conv - 1,
                                     bias=conv_bias, device=device)
-        self.x_proj = W8A8B8O8Linear(self.d_inner, self.dt_rank + 2 * d_state, device=device)
+        self.x_proj = self._x_proj_cls(self.d_inner, self.dt_rank + 2 * d_state, device=device)
         self.dt_proj = W8A8B8O8Linear(self.dt_rank, self.d_inner, device=device)
         self.selective_scan = QSScan(d_state, self.d_inner, delta_softplus=True, device=device)
         self.had = QHadamard(self.d_inner, x_H_scale=1.0)
-        self.out_proj = W8A8B16O16Linear(self.d_inner, d_model, device=device)
+        self.out_proj = self._out_proj_cls(self.d_inner, d_model, device=device)
 
     @classmethod
     def from_fp16(cls, originalLayer, act_scales, use_had_transform=True):
@@ -58,9 +61,11 @@ class W8A8QMamba(nn.Module):
                 originalLayer.dt_rank, use_had_transform=use_had_transform, layer_idx=getattr(originalLayer, "layer_idx", None),
                 device=dev)
         s = lambda k: float(torch.as_tensor(act_scales[k]).item())
-        q.in_proj = W8A8B8O8Linear.from_fp16(copy.deepcopy(originalLayer.in_proj), s("in_proj:input"), s("in_proj:output"))
+        q.in_proj = cls._in_proj_cls.from_fp16(copy.deepcopy(originalLayer.in_proj), cls._scale(act_scales, "in_proj:input"),
+                                               cls._scale(act_scales, "in_proj:output"))
         q.conv1d = QCausalConv1D.from_fp16(copy.deepcopy(originalLayer.conv1d), s("in_proj:output"), s("x_proj:input"))
-        q.x_proj = W8A8B8O8Linear.from_fp16(copy.deepcopy(originalLayer.x_proj), s("x_proj:input"), s("x_proj:output"))
+        q.x_proj = cls._x_proj_cls.from_fp16(copy.deepcopy(originalLayer.x_proj), cls._scale(act_scales, "x_proj:input"),
+                                             cls._scale(act_scales, "x_proj:output"))
         q.dt_proj = W8A8B8O8Linear.from_fp16(copy.deepcopy(originalLayer.dt_proj), s("x_proj:output"), s("dt_proj:output"))
         q.selective_scan = QSScan.from_fp16(
             originalLayer.d_state, originalLayer.d_inner, originalLayer.A_log.clone(), D=originalLayer.D.clone(),
@@ -69,8 +74,13 @@ class W8A8QMamba(nn.Module):
             dt_scale=act_scales["dt_proj:output"], B_scale=act_scales["x_proj:output"],
             C_scale=act_scales["x_proj:output"], z_scale=act_scales["in_proj:output"])
         q.had.x_H_scale = s("out_proj:input")
-        q.out_proj = W8A8B16O16Linear.from_fp16(copy.deepcopy(originalLayer.out_proj), s("out_proj:input"))
+        q.out_proj = cls._out_proj_cls.from_fp16(copy.deepcopy(originalLayer.out_proj), cls._scale(act_scales, "out_proj:input"))
         return q
+
+    @staticmethod
+    def _scale(act_scales, key):
+        """The form the linear classes of this precision take an activation scale in (a float here)."""
+        return float(torch.as_tensor(act_scales[key]).item())
 
     @torch.no_grad()
     def forward(self, hidden_states, inference_params=None, conv_state=None, ssm_state=None):
@@ -140,12 +150,24 @@ class W8A8QMamba(nn.Module):
         return conv_state, ssm_state
 
 
+class W4A8QMamba(W8A8QMamba):
+    """The W4A8 Mamba1 mixer of quamba/qMambaLayer.py:512-756: the same chain with 4-bit in_proj, x_proj and
+    out_proj (group size 128); dt_proj stays W8A8 as there."""
+    _in_proj_cls, _x_proj_cls, _out_proj_cls = W4A8B8O8Linear, W4A8B8O8Linear, W4A8B16O16Linear
+
+    @staticmethod
+    def _scale(act_scales, key):
+        return torch.as_tensor(act_scales[key])
+
+
 class W4A8QMamba2(nn.Module):
     """The quantized Mamba2 mixer of quamba/qMamba2.py:735-1068 (``W4A8QMamba2``) on this package's
     operators: in_proj (W4A8, int8 out with one output scale per z | x | B | C | dt segment) -> xBC conv
     (three int8 outputs) -> SSD chunk scan -> gated RMS norm (fp16) -> Hadamard + quantisation -> out_proj
     (W4A8, fp16).  ``step`` is the one-token form.  ``from_fp16`` is not provided: it needs the grouping
     tables produced by the reference's calibration pipeline; the sub-modules' own ``from_fp16`` exist."""
+
+    _in_proj_cls, _out_proj_cls = W4A8B8O8LinearParallel, W4A8B16O16Linear      # W8A8QMamba2 overrides them
 
     def __init__(self, d_model, d_state=128, d_conv=4, expand=2, headdim=64, d_ssm=None, ngroups=1, D_has_hdim=False,
                  rmsnorm=True, norm_before_gate=False, dt_limit=(0.0, float("inf")), bias=False, conv_bias=True,
@@ -154,7 +176,6 @@ class W4A8QMamba2(nn.Module):
         super().__init__()
         from .chunk_scan import Quamba2ChunkScan
         from .conv import Quamb2Conv1D
-        from .linear import W4A8B8O8LinearParallel, W4A8B16O16Linear
         from .norm import QRMSNormGated
         assert bias is False, "Only support bias=False for now"
         assert rmsnorm, "Only support Mamba2 block with rmsnorm"
@@ -171,7 +192,7 @@ class W4A8QMamba2(nn.Module):
         self.layer_idx = layer_idx
         self.state_dtype = state_dtype
         d_in_proj = 2 * self.d_inner + 2 * ngroups * d_state + self.nheads      # order: z, x, B, C, dt
-        self.in_proj = W4A8B8O8LinearParallel(d_model, d_in_proj, group_size=128, device=device)
+        self.in_proj = self._in_proj_cls(d_model, d_in_proj, device=device)
         conv_dim = self.d_ssm + 2 * ngroups * d_state
         self.conv1d = Quamb2Conv1D(self.d_ssm, headdim, d_state, ngroups, x_nhead_group, x_ndim_group, conv_dim, conv_dim,
                                    d_conv, groups=conv_dim, padding=d_conv - 1, bias=conv_bias, device=device)
@@ -180,7 +201,7 @@ class W4A8QMamba2(nn.Module):
         self.norm = QRMSNormGated(self.d_ssm, eps=1e-5, norm_before_gate=norm_before_gate, group_size=self.d_ssm // ngroups,
                                   use_float16_output=True, device=device)
         self.had = QHadamard(self.d_inner, x_H_scale=1.0)
-        self.out_proj = W4A8B16O16Linear(self.d_inner, d_model, group_size=128, device=device)
+        self.out_proj = self._out_proj_cls(self.d_inner, d_model, device=device)
 
     def _split(self, zxbcdt):
         return torch.split(zxbcdt, [self.d_ssm, self.d_ssm + 2 * self.ngroups * self.d_state, self.nheads], dim=-1)
@@ -223,3 +244,9 @@ class W4A8QMamba2(nn.Module):
         conv_state = torch.zeros(batch_size, self.d_conv, conv_dim, device=device, dtype=torch.int8).transpose(1, 2)
         ssm_state = torch.zeros(batch_size, self.nheads, self.headdim, self.d_state, device=device, dtype=self.state_dtype)
         return conv_state, ssm_state
+
+
+class W8A8QMamba2(W4A8QMamba2):
+    """The W8A8 Mamba2 mixer of quamba/qMamba2.py:1071-1400: the same chain with int8 weights in in_proj (one
+    output scale per z | x | B | C | dt segment) and out_proj."""
+    _in_proj_cls, _out_proj_cls = W8A8B8O8LinearParallel, W8A8B16O16Linear
