@@ -97,23 +97,36 @@ struct ScanCfg {
     static constexpr int kOutPitch = kCh + 8;              // halves; keeps rows 16-byte aligned
 };
 
+// LDS of one workgroup
+template <class Cfg, int T>
+struct ScanSmem {
+    __attribute__((aligned(16))) uint32_t in[3][Cfg::kCh * Cfg::kRow / 4];
+    __attribute__((aligned(16))) float bc[T][2][Cfg::kNP];
+    __attribute__((aligned(16))) __half out[T][Cfg::kOutPitch];
+    float gate[256];                   // SiLU gate per z code (indexed by the raw byte)
+};
+
+// One workgroup: channels c0 .. c0 + kCh - 1 of batch entry b.
 template <int NPL, int NSPLIT, int T, int WAVES>
-__global__ __launch_bounds__(64 * WAVES) void sscan_fwd_kernel(QaSScanParams p, int vec_in, int vec_bc, int vec_out) {
+__device__ __forceinline__ void sscan_fwd_body(const QaSScanParams& p, int vec_in, int vec_bc, int vec_out, int c0, int b,
+                                               ScanSmem<ScanCfg<NPL, NSPLIT, T, WAVES>, T>& sm) {
     using Cfg = ScanCfg<NPL, NSPLIT, T, WAVES>;
     constexpr int kThreads = Cfg::kThreads, kCh = Cfg::kCh, kNP = Cfg::kNP, kRow = Cfg::kRow;
-    constexpr int kInPieces = Cfg::kInPieces, kBcPieces = Cfg::kBcPieces, kOutPitch = Cfg::kOutPitch;
+    constexpr int kInPieces = Cfg::kInPieces, kBcPieces = Cfg::kBcPieces;
     constexpr int kPiecesPerRow = T / 16;
-
-    __shared__ __attribute__((aligned(16))) uint32_t s_in[3][kCh * kRow / 4];
-    __shared__ __attribute__((aligned(16))) float s_bc[T][2][kNP];
-    __shared__ __attribute__((aligned(16))) __half s_out[T][kOutPitch];
-    __shared__ float s_gate[256];      // SiLU gate per z code (indexed by the raw byte)
+    // Lanes that share the per-step work and reduce together: the NSPLIT lanes of a channel, at most a quad.
+    // With eight lanes per channel the two quads each do the per-step work for themselves (it costs a lane
+    // what it costs with four) and their partial sums meet in one cross-lane add per four steps.
+    constexpr int QS = NSPLIT < 4 ? NSPLIT : 4;
+    auto& s_in = sm.in;
+    auto& s_bc = sm.bc;
+    auto& s_out = sm.out;
+    auto& s_gate = sm.gate;
 
     const int tid = threadIdx.x;
     const int c_local = tid / NSPLIT;
     const int slice = tid % NSPLIT;
-    const int c0 = blockIdx.x * kCh;
-    const int b = blockIdx.y;
+    const int qslice = slice % QS;
     const int c = c0 + c_local;
     const bool c_ok = c < p.dim;
     const int cc = c_ok ? c : p.dim - 1;                   // clamped channel for parameter loads
@@ -226,15 +239,15 @@ __global__ __launch_bounds__(64 * WAVES) void sscan_fwd_kernel(QaSScanParams p, 
         for (int tq = 0; tq < n_quads; ++tq) {
             const uint32_t u4 = su[tq], d4 = sd[tq];
             const uint32_t z4 = has_z ? sz[tq] : 0u;
-            if constexpr (NSPLIT <= 4) {
+            if constexpr (NSPLIT <= 4 || (NSPLIT == 8 && NPL == 2)) {
                 // The per-step work that does not depend on the state index (dequantise, softplus,
                 // gate) is shared out: of the 4 steps in this dword, the lane with slice s does
                 // steps o*NSPLIT + s and the others read its results through quad DPP.
-                constexpr int OWN = 4 / NSPLIT;
+                constexpr int OWN = 4 / QS;
                 float own_u[OWN], own_dt[OWN], own_du[OWN];
 #pragma unroll
                 for (int o = 0; o < OWN; ++o) {
-                    const int j = o * NSPLIT + slice;
+                    const int j = o * QS + qslice;
                     own_u[o] = s_u * i8_of(u4, j);
                     float dt = __builtin_fmaf(s_dt, i8_of(d4, j), db);
                     if (p.delta_softplus) dt = softplus20(dt);
@@ -248,34 +261,49 @@ __global__ __launch_bounds__(64 * WAVES) void sscan_fwd_kernel(QaSScanParams p, 
                 for (int j = 0; j < 4; ++j) {
                     const int t = tq * 4 + j;
                     acc[j] = 0.0f;
-                    const float dt = quad_bcast_sel<NSPLIT>(own_dt[j / NSPLIT], j % NSPLIT);
-                    const float du = quad_bcast_sel<NSPLIT>(own_du[j / NSPLIT], j % NSPLIT);
-                    const float4* bf = reinterpret_cast<const float4*>(&s_bc[t][0][slice * NPL]);
-                    const float4* cf = reinterpret_cast<const float4*>(&s_bc[t][1][slice * NPL]);
+                    const float dt = quad_bcast_sel<QS>(own_dt[j / QS], j % QS);
+                    const float du = quad_bcast_sel<QS>(own_du[j / QS], j % QS);
+                    if constexpr (NPL == 2) {
+                        const float2 Bv = *reinterpret_cast<const float2*>(&s_bc[t][0][slice * NPL]);
+                        const float2 Cv = *reinterpret_cast<const float2*>(&s_bc[t][1][slice * NPL]);
+                        const float Bs[2] = {Bv.x, Bv.y};
+                        const float Cs[2] = {Cv.x, Cv.y};
 #pragma unroll
-                    for (int q = 0; q < NPL / 4; ++q) {
-                        const float4 Bv = bf[q];
-                        const float4 Cv = cf[q];
-                        const float Bs[4] = {Bv.x, Bv.y, Bv.z, Bv.w};
-                        const float Cs[4] = {Cv.x, Cv.y, Cv.z, Cv.w};
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            const int n = q * 4 + e;
+                        for (int n = 0; n < 2; ++n) {
                             const float a = fast_exp2(dt * A2[n]);
-                            h[n] = __builtin_fmaf(a, h[n], Bs[e] * du);
-                            acc[j] = __builtin_fmaf(h[n], Cs[e], acc[j]);
+                            h[n] = __builtin_fmaf(a, h[n], Bs[n] * du);
+                            acc[j] = __builtin_fmaf(h[n], Cs[n], acc[j]);
+                        }
+                    } else {
+                        const float4* bf = reinterpret_cast<const float4*>(&s_bc[t][0][slice * NPL]);
+                        const float4* cf = reinterpret_cast<const float4*>(&s_bc[t][1][slice * NPL]);
+#pragma unroll
+                        for (int q = 0; q < NPL / 4; ++q) {
+                            const float4 Bv = bf[q];
+                            const float4 Cv = cf[q];
+                            const float Bs[4] = {Bv.x, Bv.y, Bv.z, Bv.w};
+                            const float Cs[4] = {Cv.x, Cv.y, Cv.z, Cv.w};
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                const int n = q * 4 + e;
+                                const float a = fast_exp2(dt * A2[n]);
+                                h[n] = __builtin_fmaf(a, h[n], Bs[e] * du);
+                                acc[j] = __builtin_fmaf(h[n], Cs[e], acc[j]);
+                            }
                         }
                     }
                 }
                 // each lane needs the full sum of the steps it owns only: a transposing reduction
                 // (keep one half, hand the other half to the neighbour) instead of four full ones
                 float own_sum[OWN];
-                if constexpr (NSPLIT == 4) {
-                    const bool odd = slice & 1, hi = slice & 2;
+                if constexpr (QS == 4) {
+                    const bool odd = qslice & 1, hi = qslice & 2;
                     const float w01 = (odd ? acc[1] : acc[0]) + quad_xor<1>(odd ? acc[0] : acc[1]);
                     const float w23 = (odd ? acc[3] : acc[2]) + quad_xor<1>(odd ? acc[2] : acc[3]);
                     own_sum[0] = (hi ? w23 : w01) + quad_xor<2>(hi ? w01 : w23);
-                } else if constexpr (NSPLIT == 2) {
+                    // eight lanes per channel: the other quad holds the other half of the states
+                    if constexpr (NSPLIT == 8) own_sum[0] += __shfl_xor(own_sum[0], 4);
+                } else if constexpr (QS == 2) {
 #pragma unroll
                     for (int o = 0; o < OWN; ++o) {
                         own_sum[o] = (slice ? acc[o * 2 + 1] : acc[o * 2]) + quad_xor<1>(slice ? acc[o * 2] : acc[o * 2 + 1]);
@@ -286,11 +314,11 @@ __global__ __launch_bounds__(64 * WAVES) void sscan_fwd_kernel(QaSScanParams p, 
                 }
 #pragma unroll
                 for (int o = 0; o < OWN; ++o) {
-                    const int j = o * NSPLIT + slice;
+                    const int j = o * QS + qslice;
                     const int t = tq * 4 + j;
                     float y = __builtin_fmaf(D_f, own_u[o], own_sum[o]);
                     if (has_z) y *= s_gate[(z4 >> (8 * j)) & 0xffu];
-                    if (t < nt) s_out[t][c_local] = __float2half(y);
+                    if (t < nt && slice < QS) s_out[t][c_local] = __float2half(y);
                 }
             } else {
 #pragma unroll
@@ -364,12 +392,49 @@ __global__ __launch_bounds__(64 * WAVES) void sscan_fwd_kernel(QaSScanParams p, 
 }
 
 template <int NPL, int NSPLIT, int T, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void sscan_fwd_kernel(QaSScanParams p, int vec_in, int vec_bc, int vec_out) {
+    using Cfg = ScanCfg<NPL, NSPLIT, T, WAVES>;
+    __shared__ ScanSmem<Cfg, T> sm;
+    sscan_fwd_body<NPL, NSPLIT, T, WAVES>(p, vec_in, vec_bc, vec_out, blockIdx.x * Cfg::kCh, blockIdx.y, sm);
+}
+
+// Two kinds of workgroup in one launch, for d_state 16: the first `blocks_a` workgroups of a batch entry take
+// 64 channels each with four lanes per channel, the others 32 channels each with eight lanes per channel (half
+// the states per lane, a little more than half the time).  The kernel is bound by vector-ALU issue and a wave's
+// time does not depend on how many of its lanes are busy, so what counts is the number of waves per SIMD: when
+// the four-lane mapping alone would leave half of the SIMDs with one wave more than the others, the tail of the
+// channels goes to the short kind and every SIMD gets the same mix.
+__global__ __launch_bounds__(256) void sscan_fwd_mixed_kernel(QaSScanParams p, int vec_in, int vec_bc, int vec_out, int blocks_a) {
+    using CfgA = ScanCfg<4, 4, 64, 4>;
+    using CfgB = ScanCfg<2, 8, 64, 4>;
+    __shared__ union Smem {
+        ScanSmem<CfgA, 64> a;
+        ScanSmem<CfgB, 64> b;
+        __device__ Smem() {}
+    } sm;
+    const int bx = blockIdx.x;
+    if (bx < blocks_a) {
+        sscan_fwd_body<4, 4, 64, 4>(p, vec_in, vec_bc, vec_out, bx * CfgA::kCh, blockIdx.y, sm.a);
+    } else {
+        sscan_fwd_body<2, 8, 64, 4>(p, vec_in, vec_bc, vec_out, blocks_a * CfgA::kCh + (bx - blocks_a) * CfgB::kCh, blockIdx.y, sm.b);
+    }
+}
+
+template <int NPL, int NSPLIT, int T, int WAVES>
 int launch_fwd(const QaSScanParams& p, hipStream_t stream, int vec_in, int vec_bc, int vec_out) {
     using Cfg = ScanCfg<NPL, NSPLIT, T, WAVES>;
     if (p.n_groups > 1 && (p.dim / p.n_groups) % Cfg::kCh != 0) return QA_ERR_UNSUPPORTED;
     dim3 grid((p.dim + Cfg::kCh - 1) / Cfg::kCh, p.batch);
     hipLaunchKernelGGL((sscan_fwd_kernel<NPL, NSPLIT, T, WAVES>), grid, dim3(Cfg::kThreads), 0, stream, p, vec_in,
                        vec_bc, vec_out);
+    return check_launch();
+}
+
+// Channels [0, 64 * blocks_a) with four lanes per channel, the rest with eight.
+int launch_fwd_mixed(const QaSScanParams& p, hipStream_t stream, int vec_in, int vec_bc, int vec_out, int blocks_a) {
+    const int rest = p.dim - 64 * blocks_a;
+    dim3 grid(blocks_a + (rest + 31) / 32, p.batch);
+    hipLaunchKernelGGL(sscan_fwd_mixed_kernel, grid, dim3(256), 0, stream, p, vec_in, vec_bc, vec_out, blocks_a);
     return check_launch();
 }
 
@@ -591,6 +656,24 @@ extern "C" int qa_sscan_fwd(const QaSScanParams* p, void* stream_) {
             // the channel count allows, four waves per workgroup sharing one staged B/C tile.
             nsplit = 4;
             waves = p->dim % 64 == 0 ? 4 : (p->dim % 32 == 0 ? 2 : 1);
+            // Waves per SIMD with four lanes per channel: q + f.  With 0 < f <= 1/2 the last f/(q+f) of the
+            // channels of every batch entry go to the eight-lane kind (see sscan_fwd_mixed_kernel), as long as
+            // both parts stay whole workgroups and, with channel groups, whole groups.
+            int dev = 0, cus = 256;
+            if (hipGetDevice(&dev) != hipSuccess ||
+                hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) {
+                cus = 256;
+            }
+            const int64_t simds = 4LL * cus;
+            const int64_t waves_a = static_cast<int64_t>(p->batch) * p->dim / 16;
+            const int64_t q = waves_a / simds, rem_waves = waves_a % simds;
+            if (waves == 4 && p->n_groups == 1 && q >= 1 && rem_waves > 0 && 2 * rem_waves <= simds) {
+                const int64_t short_channels = rem_waves * 16 / p->batch;      // channels per batch entry for the short kind
+                const int blocks_a = static_cast<int>((p->dim - short_channels) / 64);
+                if (short_channels % 32 == 0 && (p->dim - short_channels) % 64 == 0 && blocks_a > 0) {
+                    return launch_fwd_mixed(*p, stream, vec_in, vec_bc, vec_out, blocks_a);
+                }
+            }
         }
         if (nsplit == 1 && waves == 1) return launch_fwd<16, 1, 64, 1>(*p, stream, vec_in, vec_bc, vec_out);
         if (nsplit == 2 && waves == 1) return launch_fwd<8, 2, 64, 1>(*p, stream, vec_in, vec_bc, vec_out);
@@ -598,6 +681,8 @@ extern "C" int qa_sscan_fwd(const QaSScanParams* p, void* stream_) {
         if (nsplit == 4 && waves == 1) return launch_fwd<4, 4, 64, 1>(*p, stream, vec_in, vec_bc, vec_out);
         if (nsplit == 4 && waves == 2) return launch_fwd<4, 4, 64, 2>(*p, stream, vec_in, vec_bc, vec_out);
         if (nsplit == 4 && waves == 4) return launch_fwd<4, 4, 64, 4>(*p, stream, vec_in, vec_bc, vec_out);
+        if (nsplit == 8 && waves == 4) return launch_fwd<2, 8, 64, 4>(*p, stream, vec_in, vec_bc, vec_out);
+        if (nsplit == 0 && waves > 0) return launch_fwd_mixed(*p, stream, vec_in, vec_bc, vec_out, waves);
         return QA_ERR_UNSUPPORTED;
     }
     if (N <= 32) return launch_fwd<8, 4, 64, 1>(*p, stream, vec_in, vec_bc, vec_out);

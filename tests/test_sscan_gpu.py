@@ -65,7 +65,9 @@ def test_fwd_matches_oracle(dev, B, L, D, N):
     assert diff.max() <= 1 and (diff != 0).mean() < 0.02
 
 
-@pytest.mark.parametrize("variant", ["1x1", "2x1", "2x2", "4x1", "4x2", "4x4"])
+# "<lanes per channel>x<waves>"; "8x4" is the eight-lane mapping, "0x<n>" the mixed launch (n workgroups of 64
+# channels with four lanes per channel, the remaining channels with eight)
+@pytest.mark.parametrize("variant", ["1x1", "2x1", "2x2", "4x1", "4x2", "4x4", "8x4", "0x1", "0x2"])
 def test_every_lane_mapping_gives_the_same_answer(dev, variant, monkeypatch):
     monkeypatch.setenv("QA_SSCAN_VARIANT", variant)
     d = synth.mamba1_scan_inputs(2, 300, 200, 16, seed=21)
@@ -181,3 +183,23 @@ def test_errors(dev):
     with pytest.raises(RuntimeError, match="<= 256"):
         ops.sscan_fwd(_t(d["u"], dev), _s(1, dev), _t(d["dt"], dev), _s(1, dev), big_A, _s(1, dev),
                       _t(d["B"][:, None], dev), _s(1, dev), _t(d["C"][:, None], dev), _s(1, dev), _s(1, dev))
+
+
+def test_mixed_launch_is_chosen_when_it_evens_out_the_waves(dev):
+    """Batch 8 x 5120 channels is 2.5 waves per SIMD with four lanes per channel: the last fifth of the channels
+    goes to the eight-lane kind.  Same answer as every channel with four lanes (the default for 4096 channels)."""
+    B, L, D, N = 8, 96, 5120, 16
+    g = torch.Generator(device=dev).manual_seed(3)
+    ri = lambda *s: torch.randint(-128, 128, s, dtype=torch.int8, device=dev, generator=g)
+    u, dt, z, Bm, Cm = ri(B, D, L), ri(B, D, L), ri(B, D, L), ri(B, 1, N, L), ri(B, 1, N, L)
+    A, Dq, db = ri(D, N), ri(D), ri(D)
+    s = lambda v: torch.tensor([v], dtype=torch.float32, device=dev)
+    run = lambda sl: ops.sscan_fwd(u[:, sl], s(0.03), dt[:, sl], s(0.02), A[sl], s(0.02), Bm, s(0.03), Cm, s(0.03), s(1.0), Dq[sl],
+                                   s(0.008), z[:, sl], s(0.03), db[sl], s(0.01), True, state_dtype=torch.float32)
+    y, st = run(slice(None))
+    y_a, st_a = run(slice(0, 4096))
+    y_b, st_b = run(slice(4096, 5120))
+    np.testing.assert_allclose(y[:, :, :4096].float().cpu().numpy(), y_a.float().cpu().numpy(), rtol=1e-2, atol=1e-2)
+    np.testing.assert_allclose(y[:, :, 4096:].float().cpu().numpy(), y_b.float().cpu().numpy(), rtol=1e-2, atol=1e-2)
+    full = torch.cat([st_a, st_b], dim=1)
+    assert float((st - full).abs().max()) <= 1e-3 * float(full.abs().max())
