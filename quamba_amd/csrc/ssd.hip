@@ -480,6 +480,12 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_kernel(QaSsdParams p, c
         xq[q] = p.D ? *reinterpret_cast<const uint2*>(p.x + at) : make_uint2(0u, 0u);
         zq[q] = p.z ? *reinterpret_cast<const uint2*>(p.z + at) : make_uint2(0u, 0u);
     };
+    // skip-term and gate parameters: requested with everything else, used in the epilogue
+    const float D_scale = p.D ? *p.D_scale : 0.0f;
+    const float z_scale = p.z ? *p.z_scale : 0.0f;
+    int8_t e_Dq[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) e_Dq[e] = p.D ? p.D[p.D_has_hdim ? h * kP + ecol + e : h] : int8_t(0);
     if (wave * PER_WAVE < NMT) {
         const int mt = tile_of(0);
 #pragma unroll
@@ -549,15 +555,10 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_kernel(QaSsdParams p, c
     }
     __syncthreads();
 
-    const float D_scale = p.D ? *p.D_scale : 0.0f;
-    const float z_scale = p.z ? *p.z_scale : 0.0f;
     __half* out = static_cast<__half*>(p.out);
     float e_Dv[8];                                           // D of the eight columns this lane writes
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-        const int pp = ecol + e;
-        e_Dv[e] = p.D ? D_scale * static_cast<float>(p.D[p.D_has_hdim ? h * kP + pp : h]) : 0.0f;
-    }
+    for (int e = 0; e < 8; ++e) e_Dv[e] = D_scale * static_cast<float>(e_Dq[e]);
 
 #pragma unroll
     for (int s = 0; s < PER_WAVE; ++s) {
@@ -610,14 +611,26 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_kernel(QaSsdParams p, c
             acc[0][r] *= e_ref;
             acc[1][r] *= e_ref;
         }
-        // term 2
+        // term 2.  The LDS operands of k-step ks+1 (decay table piece, two x fragments) are requested before
+        // the products of k-step ks; the addresses are valid for every ks, so the requests need no condition.
+        v8h gh_n = *reinterpret_cast<const v8h*>(g_tab + fhalf * 8);
+        v8h fx_n[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) fx_n[j] = *reinterpret_cast<const v8h*>(s_xt + (j * 32 + frow) * PITCH + fhalf * 8);
 #pragma unroll
         for (int ks = 0; ks < KSMAX; ++ks) {
+            const v8h gh = gh_n;
+            const v8h fx_c[2] = {fx_n[0], fx_n[1]};
+            if (ks + 1 < KSMAX) {
+                const int k1 = (ks + 1) * 16 + fhalf * 8;
+                gh_n = *reinterpret_cast<const v8h*>(g_tab + k1);
+#pragma unroll
+                for (int j = 0; j < 2; ++j) fx_n[j] = *reinterpret_cast<const v8h*>(s_xt + (j * 32 + frow) * PITCH + k1);
+            }
             if (ks < nks) {
                 const int k0 = ks * 16 + fhalf * 8;
                 v8h fl;
                 if (ks < n_off) {
-                    const v8h gh = *reinterpret_cast<const v8h*>(g_tab + k0);
                     fl = cbf[ks] * gh;
                 } else {
                     if (ks == n_off) {
@@ -643,10 +656,7 @@ __global__ __launch_bounds__(256, 2) void ssd_chunk_scan_kernel(QaSsdParams p, c
                     }
                 }
 #pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    const v8h fx = *reinterpret_cast<const v8h*>(s_xt + (j * 32 + frow) * PITCH + k0);
-                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fl, fx, acc[j], 0, 0, 0);
-                }
+                for (int j = 0; j < 2; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fl, fx_c[j], acc[j], 0, 0, 0);
             }
             if (ks < nks_next) cbf[ks] = *reinterpret_cast<const v8h*>(cb_ptr(mt_next, ks));
         }
