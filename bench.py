@@ -344,10 +344,18 @@ def other_workloads(dev, steps, warmup):
     out.append(dict(workload="gated RMS norm, 16384 rows x 8192 (fp16 in, int8 gate, fp16 out)", us=ms * 1e3,
                     tokens_per_s=16384 / ms * 1e3, bound="hbm", achieved_GBs=nbytes / ms / 1e6,
                     frac=nbytes / ms / 1e6 / HBM_PEAK_GBS))
+    # the same norm in groups of 1024 with the Hadamard transform + quantisation in the same kernel (what the
+    # Mamba2-8b mixer runs between the SSD scan and out_proj): fp16 and int8 gate in, int8 out
+    ms = _time_fn(lambda: ops.qlayer_normgated_hadamard_quant(xn, wn, 1e-5, 0.2, q_z=zn, z_scale=0.02, group_size=1024,
+                                                              norm_before_gate=False), steps, warmup)
+    nbytes = 16384 * 8192 * (2 + 1 + 1)
+    out.append(dict(workload="gated RMS norm (groups of 1024) + Hadamard + int8 quantisation in one kernel, 16384 rows x 8192",
+                    us=ms * 1e3, tokens_per_s=16384 / ms * 1e3, bound="hbm", achieved_GBs=nbytes / ms / 1e6,
+                    frac=nbytes / ms / 1e6 / HBM_PEAK_GBS))
     del xn, zn, wn
     torch.cuda.empty_cache()
     # the whole Mamba2-8b W4A8 mixer over a prompt (W4A8QMamba2.forward: in_proj, xBC conv, SSD chunk scan, gated
-    # norm, Hadamard, out_proj), 16 x 1024 tokens, d_model 4096, 128 heads of 64, d_state 128, 8 groups, chunk 256
+    # norm + Hadamard, out_proj), 16 x 1024 tokens, d_model 4096, 128 heads of 64, d_state 128, 8 groups, chunk 256
     from quamba_amd import W4A8QMamba2
     G = 8
     m2 = W4A8QMamba2(4096, 128, 4, 2, 64, ngroups=G, chunk_size=256, device=dev, state_dtype=torch.float32)
@@ -380,7 +388,7 @@ def other_workloads(dev, steps, warmup):
     u2 = ri(16, 1024, 4096)
     ms = _time_fn(lambda: m2.forward(u2), min(steps, 10), 3)
     gemm_ops = 2.0 * 16384 * (4096 * m2.in_proj.size_n + 8192 * 4096)
-    out.append(dict(workload="Mamba2-8b W4A8 mixer forward over a prompt (all six kernels), 16 x 1024 tokens",
+    out.append(dict(workload="Mamba2-8b W4A8 mixer forward over a prompt (in_proj, conv, SSD scan, norm + Hadamard, out_proj), 16 x 1024 tokens",
                     us=ms * 1e3, tokens_per_s=16384 / ms * 1e3, bound="mfma", achieved_TOPs=gemm_ops / ms / 1e9,
                     frac=gemm_ops / ms / 1e9 / INT8_PEAK_TOPS))
     return out

@@ -168,6 +168,18 @@ typedef struct QaHadamardParams {
 
 int qa_hadamard_quant(const QaHadamardParams* p, void* stream);
 
+/* The gated RMS norm and the Hadamard transform + quantisation of its fp16 output in one pass over the
+ * rows: out = qa_hadamard_quant(qa_rmsnorm_gated(...)) bit for bit, without the fp16 matrix between them.
+ * Replaces the pair QRMSNormGated.forward (quamba/qNorm.py:93-177, fp16 output) -> HadLinear's
+ * transform (quamba/qHadamard.py, quant_hadamard.fast_hadamard_transform) in the Mamba2 mixer
+ * (quamba/qMamba2.py, `y = self.norm(y, z)` then `self.out_proj(y)`).
+ * `norm`: rows, dim, group_size, norm_before_gate, eps, z_scale, x, weight, qz and their strides as for
+ * qa_rmsnorm_gated; out_mode must be QA_NORM_OUT_F16; out, out_row_stride, out_scale, dyn_scale unused.
+ * `had`: rows, dim (equal to the norm's), scale, out, out_row_stride; x, x_row_stride, in_type unused.
+ * Supported: dim 2048, 4096 or 8192 with group_size 512, 1024 or 2048, 16-byte aligned rows;
+ * anything else returns QA_ERR_UNSUPPORTED (callers then make the two calls). */
+int qa_rmsnorm_gated_hadamard_quant(const QaNormGatedParams* norm, const QaHadamardParams* had, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * Mamba1 int8 selective scan, forward over a sequence.
  * Replaces quant_sscan_cuda.fwd (csrc/selective_scan/quant_sscan.cpp:122-265; parameter block

@@ -162,6 +162,7 @@ SYMBOLS = {
     "qa_quamba2_conv1d_update": (C.c_int, [C.POINTER(QaConv2Params), vp]),
     "qa_hadamard_quant": (C.c_int, [C.POINTER(QaHadamardParams), vp]),
     "qa_rmsnorm_gated": (C.c_int, [C.POINTER(QaNormGatedParams), vp]),
+    "qa_rmsnorm_gated_hadamard_quant": (C.c_int, [C.POINTER(QaNormGatedParams), C.POINTER(QaHadamardParams), vp]),
     "qa_sscan_fwd": (C.c_int, [C.POINTER(QaSScanParams), vp]),
     "qa_ssm_state_update": (C.c_int, [C.POINTER(QaSsmUpdateParams), vp]),
     "qa_gemm_w8a8": (C.c_int, [C.POINTER(QaGemmW8A8Params), vp]),

@@ -14,7 +14,7 @@
 // (W waves per group), so every load and store of a wave is one contiguous run.
 // The gate has 256 possible values (one per int8 code): a workgroup evaluates them once into LDS and
 // every element looks its gate up, which gives the same bits as evaluating it per element.
-#include "qa_common.hpp"
+#include "normgated_core.hpp"
 
 namespace qa {
 namespace {
@@ -22,24 +22,12 @@ namespace {
 constexpr int kWavesPerBlock = 4;
 constexpr int kMaxPieces = 16;      // per lane: 16 pieces * 4 waves * 64 lanes * 8 columns = 32768 columns per group
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m);
-    return v;
-}
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m));
-    return v;
-}
-__device__ __forceinline__ float silu_of(float z) { return z * (1.0f / (1.0f + expf(-z))); }
-
 template <int PIECES, int WPI, bool GATE_LAST>
 __global__ __launch_bounds__(64 * kWavesPerBlock) void rmsnorm_gated_kernel(QaNormGatedParams p) {
     __shared__ float s_gate[256];
     __shared__ float s_part[2][kWavesPerBlock];
     if (p.qz) {
-        for (int i = threadIdx.x; i < 256; i += 64 * kWavesPerBlock) s_gate[i] = silu_of(p.z_scale * static_cast<float>(i - 128));
+        for (int i = threadIdx.x; i < 256; i += 64 * kWavesPerBlock) s_gate[i] = gate_of_code(i, p.z_scale);
         __syncthreads();
     }
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -82,7 +70,7 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) void rmsnorm_gated_kernel(QaNo
                 }
             }
 #pragma unroll
-            for (int j = 0; j < 8; ++j) ssq += v[c][j] * v[c][j];
+            for (int j = 0; j < 8; ++j) ssq = ssq_step(ssq, v[c][j]);
         }
     }
     ssq = wave_sum(ssq);
@@ -93,8 +81,7 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) void rmsnorm_gated_kernel(QaNo
 #pragma unroll
         for (int i = 0; i < WPI; ++i) ssq += s_part[0][i];
     }
-    const float var = ssq / static_cast<float>(N);
-    const float rstd = 1.0f / sqrtf(var + p.eps);
+    const float rstd = rstd_of(ssq, N, p.eps);
 
     float ymax = -INFINITY;
 #pragma unroll
@@ -105,7 +92,7 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) void rmsnorm_gated_kernel(QaNo
             const __half* wh = reinterpret_cast<const __half*>(&wraw);
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                float y = (v[c][j] * rstd) * __half2float(wh[j]);
+                float y = norm_value(v[c][j], rstd, __half2float(wh[j]));
                 if (GATE_LAST && qz) y *= gate[c][j];
                 v[c][j] = y;
                 ymax = fmaxf(ymax, y);
@@ -132,7 +119,7 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) void rmsnorm_gated_kernel(QaNo
             if (p.out_mode == QA_NORM_OUT_F16) {
                 __half o[8];
 #pragma unroll
-                for (int j = 0; j < 8; ++j) o[j] = __float2half(v[c][j]);
+                for (int j = 0; j < 8; ++j) o[j] = half_of_f32(v[c][j]);
                 *reinterpret_cast<uint4*>(static_cast<__half*>(p.out) + row * p.out_row_stride + col0 + e0) =
                     *reinterpret_cast<const uint4*>(o);
             } else {

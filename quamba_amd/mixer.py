@@ -225,8 +225,13 @@ class W4A8QMamba2(nn.Module):
         if want_state:
             y, last_state = y
             ssm_state.copy_(last_state)
-        y = self.norm(y.reshape(batch, seqlen, self.d_ssm), z)
-        return self.out_proj(self.had(y))
+        return self.out_proj(self._norm_had(y.reshape(batch, seqlen, self.d_ssm), z))
+
+    def _norm_had(self, y, z):
+        """Gated norm, then the Hadamard transform + quantisation: one kernel where the shape allows."""
+        if self.norm.fuses_with(self.had):
+            return self.norm.forward_hadamard(y, z, self.had)
+        return self.had(self.norm(y, z))
 
     @torch.no_grad()
     def step(self, hidden_states, conv_state, ssm_state):
@@ -234,8 +239,7 @@ class W4A8QMamba2(nn.Module):
         z, xBC, dt = self._split(self.in_proj(hidden_states.squeeze(1)))
         x, B, C = self.conv1d.update(xBC, conv_state)
         y = self.qchunk_scan.update(ssm_state, x, dt, B, C, z=None)
-        y = self.norm(y.reshape(y.shape[0], self.d_ssm), z)
-        out = self.out_proj(self.had(y))
+        out = self.out_proj(self._norm_had(y.reshape(y.shape[0], self.d_ssm), z))
         return out.unsqueeze(1), conv_state, ssm_state
 
     def allocate_inference_cache(self, batch_size, max_seqlen=None, dtype=None, **kwargs):

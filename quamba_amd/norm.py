@@ -70,6 +70,31 @@ class QRMSNormGated(torch.nn.Module):
         ngroups = 1 if self.group_size is None else shape[-1] // self.group_size
         return y.reshape(shape), scales.reshape(shape[:-1]) if ngroups == 1 else scales.reshape(ngroups, *shape[:-1])
 
+    def fuses_with(self, had):
+        """True when ``had(self(x, q_z))`` can run as one kernel: fp16 output feeding a power-of-two transform
+        of a shape the fused kernel covers."""
+        dim = self.weight.shape[0]
+        group = dim if self.group_size is None else self.group_size
+        return self.use_float16_output and had.dim == dim and ops.normgated_hadamard_supported(dim, group)
+
+    @torch.no_grad()
+    def forward_hadamard(self, x, q_z, had):
+        """``had(self(x, q_z))`` bit for bit, in one kernel (``had`` a QHadamard of the same width)."""
+        assert self.fuses_with(had)
+        shape = x.shape
+        x2 = x.reshape(-1, shape[-1])
+        if x2.stride(-1) != 1:
+            x2 = x2.contiguous()
+        if q_z is not None:
+            assert q_z.shape == shape
+            q_z = q_z.reshape(-1, shape[-1])
+            if q_z.stride(-1) != 1:
+                q_z = q_z.contiguous()
+        out = ops.qlayer_normgated_hadamard_quant(x2, self.weight, self.eps, had.had_scale / float(had.x_H_scale), q_z=q_z,
+                                                  z_scale=self.z_scale, group_size=self.group_size,
+                                                  norm_before_gate=self.norm_before_gate)
+        return out.reshape(shape)
+
     def __repr__(self):
         return (f"QRMSNormGated(dim={self.weight.shape[0]}, eps={self.eps}, z_scale={self.z_scale}, "
                 f"output_scale={self.output_scale}, use_float16_output={self.use_float16_output})")

@@ -303,6 +303,49 @@ def qlayer_normgated_fwd(x, weight, bias, eps, q_z=None, z_scale=None, static_ou
     return out, per_token_scale
 
 
+def normgated_hadamard_supported(dim, group_size):
+    """Shapes for which the gated norm and the Hadamard transform run as one kernel."""
+    return dim in (2048, 4096, 8192) and group_size in (512, 1024, 2048) and dim % group_size == 0
+
+
+def qlayer_normgated_hadamard_quant(x, weight, eps, had_scale, q_z=None, z_scale=None, group_size=None,
+                                    norm_before_gate=True):
+    """hadamard_quant(qlayer_normgated_fwd(..., use_float16_output=True)[0], had_scale) in one kernel, bit for
+    bit (QRMSNormGated.forward, quamba/qNorm.py:93-177, followed by the transform in front of out_proj,
+    quamba/qHadamard.py).  x fp16 (M, N); q_z int8 (M, N) or None.  Returns int8 (M, N).  Only for shapes
+    accepted by ``normgated_hadamard_supported``."""
+    _require(x.dtype == torch.float16 and x.dim() == 2, "x must be fp16 (M, N)")
+    _require_gpu(x, "x")
+    M, N = x.shape
+    group_size = N if group_size is None else group_size
+    _require(normgated_hadamard_supported(N, group_size), "shape not covered by the fused kernel")
+    _require(x.stride(-1) == 1, "x must be contiguous along the last dimension")
+    _require(weight.dtype == torch.float16 and tuple(weight.shape) == (N,) and weight.stride(-1) == 1 and weight.is_cuda,
+             "weight must be a contiguous fp16 GPU tensor of shape (N,)")
+    if q_z is not None:
+        _require(q_z.dtype == torch.int8 and tuple(q_z.shape) == (M, N) and q_z.stride(-1) == 1 and q_z.is_cuda,
+                 "q_z must be an int8 GPU tensor of shape (M, N), contiguous along the last dimension")
+    out = torch.empty((M, N), dtype=torch.int8, device=x.device)
+    n = _lib.QaNormGatedParams()
+    n.rows, n.dim, n.group_size = M, N, group_size
+    n.norm_before_gate = int(bool(norm_before_gate))
+    n.out_mode = 0
+    n.eps = float(eps)
+    n.z_scale = float(z_scale) if z_scale is not None else 0.0
+    n.x_row_stride = x.stride(0) if M > 1 else N
+    n.z_row_stride = (q_z.stride(0) if M > 1 else N) if q_z is not None else 0
+    n.x, n.weight, n.qz = ptr(x), ptr(weight), ptr(q_z)
+    h = _lib.QaHadamardParams()
+    h.rows, h.dim = M, N
+    h.scale = float(had_scale)
+    h.out_row_stride = N
+    h.out = ptr(out)
+    with torch.cuda.device(x.device):
+        st = _lib.lib().qa_rmsnorm_gated_hadamard_quant(ct.byref(n), ct.byref(h), _lib.current_stream(x.device))
+    _lib.check(st, "rmsnorm_gated_hadamard_quant")
+    return out
+
+
 def sscan_fwd(u, scale_u, delta, scale_delta, A, scale_A, B, scale_B, C, scale_C, scale_ssm_state,
               D=None, scale_D=None, z=None, scale_z=None, delta_bias=None, scale_delta_bias=None,
               delta_softplus=False, state_dtype=torch.int8):

@@ -50,6 +50,37 @@ def test_many_rows_take_the_one_lane_per_column_path(dev, dim):
     np.testing.assert_array_equal(got[:100], few)
 
 
+@pytest.mark.parametrize("dim", [2048, 4096, 8192])
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_many_power_of_two_rows_take_the_32_values_per_lane_path(dev, dim, dtype):
+    """More than 128 aligned rows of 2048, 4096 or 8192 columns: eight LDS planes, two round trips.  Same
+    bits as the oracle, whose rows are a sample to keep the test short, and as the general kernel that
+    rows off the 16-byte grid fall back to."""
+    rows = 261
+    x = _rows(rows, dim, seed=dim + 2).astype(dtype)
+    scale = np.float32(1.0 / math.sqrt(dim) / 0.06)
+    got = ops.hadamard_quant(torch.from_numpy(x).to(dev), float(scale)).cpu().numpy()
+    pick = np.array([0, 1, 127, 128, 129, 260])
+    np.testing.assert_array_equal(got[pick], oracle.hadamard_quant(x[pick], scale))
+    assert np.abs(got).max() > 60
+    shifted = torch.zeros((rows, dim + 8), dtype=torch.from_numpy(x).dtype, device=dev)
+    shifted[:, 1:dim + 1] = torch.from_numpy(x).to(dev)
+    np.testing.assert_array_equal(ops.hadamard_quant(shifted[:, 1:dim + 1], float(scale)).cpu().numpy(), got)
+
+
+def test_rounding_at_ties_and_saturation_on_the_32_values_per_lane_path(dev):
+    """Rows whose transform lands exactly on k + 1/2 and beyond the int8 range: half away from zero, then
+    saturation, as the general kernel does."""
+    dim, rows = 2048, 256
+    x = np.zeros((rows, dim), dtype=np.float16)
+    x[:, 0] = (np.arange(rows) - 128).astype(np.float16) * 0.5 + 0.25      # every output of row r is x[r, 0]
+    x[200:, 0] *= 8.0
+    got = ops.hadamard_quant(torch.from_numpy(x).to(dev), 2.0).cpu().numpy()
+    want = oracle.hadamard_quant(x, np.float32(2.0))
+    np.testing.assert_array_equal(got, want)
+    assert want.min() == -128 and want.max() == 127 and (np.abs(2.0 * x[:200, 0].astype(np.float32)) % 1 == 0.5).all()
+
+
 def test_fp32_input_and_leading_dims(dev):
     x = _rows(24, 5120, seed=3).astype(np.float32).reshape(2, 12, 5120)
     scale = np.float32(1.0 / math.sqrt(5120) / 0.05)

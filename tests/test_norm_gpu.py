@@ -95,3 +95,42 @@ def test_state_dict_and_errors(dev):
     assert m2.z_scale == 0.03 and m2.output_scale == 0.04
     with pytest.raises(NotImplementedError):
         _module(dev, 100, np.ones(100, np.float16), 20, True, False, 0.03, 0.04)(torch.zeros((2, 100), dtype=torch.float16, device=dev))
+
+
+# (rows, dim, group_size): the Mamba2-8b form, one group per wave, a whole wave's span per group, decode rows
+FUSED = [(300, 8192, 1024), (70, 8192, 512), (150, 4096, 2048), (131, 2048, 512), (9, 2048, 1024), (1, 8192, 1024)]
+
+
+@pytest.mark.parametrize("M,N,group_size", FUSED)
+@pytest.mark.parametrize("nbg", [True, False])
+@pytest.mark.parametrize("gated", [True, False])
+def test_norm_fused_with_hadamard_gives_the_bits_of_the_two_kernels(dev, M, N, group_size, nbg, gated):
+    """QRMSNormGated.forward_hadamard == QHadamard(QRMSNormGated(x, z)) bit for bit: the fused kernel reduces
+    every group in the order of the stand-alone norm and transforms the fp16 value of its output."""
+    from quamba_amd import QHadamard
+    x, w, qz = _inputs(M, N, seed=3 * M + N)
+    m = _module(dev, N, w, group_size, nbg, True, 0.03, None)
+    had = QHadamard(N, x_H_scale=0.07)
+    assert m.fuses_with(had)
+    xd = torch.from_numpy(x).to(dev)
+    zd = torch.from_numpy(qz).to(dev) if gated else None
+    want = had(m(xd, zd))
+    got = m.forward_hadamard(xd, zd, had)
+    assert got.dtype == torch.int8 and got.shape == (M, N)
+    np.testing.assert_array_equal(got.cpu().numpy(), want.cpu().numpy())
+    assert np.abs(want.cpu().numpy()).max() > 40
+    # z as the leading columns of a wider matrix, as the mixer hands it over
+    if gated:
+        wide = torch.zeros((M, N + 264), dtype=torch.int8, device=dev)
+        wide[:, :N] = zd
+        np.testing.assert_array_equal(m.forward_hadamard(xd, wide[:, :N], had).cpu().numpy(), want.cpu().numpy())
+
+
+def test_fused_norm_is_refused_for_other_shapes(dev):
+    from quamba_amd import QHadamard, ops
+    assert not _module(dev, 5120, np.ones(5120, np.float16), None, False, True, 0.03, None).fuses_with(QHadamard(5120))
+    assert not _module(dev, 4096, np.ones(4096, np.float16), None, False, True, 0.03, None).fuses_with(QHadamard(4096))
+    assert not _module(dev, 8192, np.ones(8192, np.float16), 1024, False, False, 0.03, 0.05).fuses_with(QHadamard(8192))
+    with pytest.raises(RuntimeError):
+        ops.qlayer_normgated_hadamard_quant(torch.zeros((4, 4096), dtype=torch.float16, device=dev),
+                                            torch.ones(4096, dtype=torch.float16, device=dev), 1e-5, 1.0, group_size=4096)
