@@ -63,6 +63,23 @@ __host__ __device__ inline Ws ws_layout(const QaSsdParams& p) {
     return w;
 }
 
+// Workgroups are handed to the eight XCDs (each with an L2 of its own) in turn by linear index.  The
+// heads of one ssd group share the packed B operand and neighbouring heads share the 128-byte lines
+// of x, so in the state kernel the heads of one (batch, group) unit get linear indices that land on one
+// XCD: index L -> XCD L % 8, position L / 8 there -> unit (L / 8) / hpg * 8 + L % 8, head (L / 8) % hpg
+// of the group.  Needs a unit count that is a multiple of eight; otherwise the natural order
+// (unit-major) is kept.  (The chunk scan measured the same either way and keeps the natural order.)
+__device__ __forceinline__ void unit_and_head(int linear, int units, int hpg, int& unit, int& head_in_group) {
+    if (units % 8 == 0) {
+        const int xcd = linear % 8, pos = linear / 8;
+        unit = (pos / hpg) * 8 + xcd;
+        head_in_group = pos % hpg;
+    } else {
+        unit = linear / hpg;
+        head_in_group = linear % hpg;
+    }
+}
+
 // x scale of channel p of head h (per-tensor, or looked up from the cumulative group ranges,
 // quamba/triton/quant_chunk_state.py:202-214)
 __device__ __forceinline__ void group_of(const QaSsdParams& p, int h, int& g, int& hg) {
@@ -164,43 +181,61 @@ __global__ __launch_bounds__(64) void ssd_cb_kernel(QaSsdParams p, __half* cb_ou
         for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
-    for (int ks = 0; ks < N / 32; ++ks) {
-        v4i fc[2], fb[2];
+    // every operand piece of the tile pair is requested before the first product: one memory round trip
+    constexpr int KSMAX = 4;                                  // dstate 128
+    const int nks = N / 32;
+    v4i fc[KSMAX][2], fb[KSMAX][2];
+#pragma unroll
+    for (int ks = 0; ks < KSMAX; ++ks) {
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
             const int m = mt * 64 + i * 32 + frow, k = kt * 64 + i * 32 + frow;
-            fc[i] = m < lim ? *reinterpret_cast<const v4i*>(p.C + ((static_cast<int64_t>(b) * p.seqlen + t0 + m) * G + g) * N + ks * 32 + fhalf * 16)
-                            : v4i{0, 0, 0, 0};
-            fb[i] = k < lim ? *reinterpret_cast<const v4i*>(p.B + ((static_cast<int64_t>(b) * p.seqlen + t0 + k) * G + g) * N + ks * 32 + fhalf * 16)
-                            : v4i{0, 0, 0, 0};
+            const bool on = ks < nks;
+            fc[ks][i] = (on && m < lim) ? *reinterpret_cast<const v4i*>(p.C + ((static_cast<int64_t>(b) * p.seqlen + t0 + m) * G + g) * N + ks * 32 + fhalf * 16)
+                                        : v4i{0, 0, 0, 0};
+            fb[ks][i] = (on && k < lim) ? *reinterpret_cast<const v4i*>(p.B + ((static_cast<int64_t>(b) * p.seqlen + t0 + k) * G + g) * N + ks * 32 + fhalf * 16)
+                                        : v4i{0, 0, 0, 0};
+        }
+    }
+#pragma unroll
+    for (int ks = 0; ks < KSMAX; ++ks) {
+        if (ks >= nks) break;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int m = mt * 64 + i * 32 + frow;
             if (mt == kt && m < lim) {
                 v8h lo, hi;
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
-                    lo[e] = static_cast<_Float16>(sC * static_cast<float>(byte_of(static_cast<uint32_t>(fc[i][e >> 2]), e & 3)));
-                    hi[e] = static_cast<_Float16>(sC * static_cast<float>(byte_of(static_cast<uint32_t>(fc[i][2 + (e >> 2)]), e & 3)));
+                    lo[e] = static_cast<_Float16>(sC * static_cast<float>(byte_of(static_cast<uint32_t>(fc[ks][i][e >> 2]), e & 3)));
+                    hi[e] = static_cast<_Float16>(sC * static_cast<float>(byte_of(static_cast<uint32_t>(fc[ks][i][2 + (e >> 2)]), e & 3)));
                 }
                 __half* dst = c16_out + ((static_cast<int64_t>(b) * p.seqlen + t0 + m) * G + g) * N + ks * 32 + fhalf * 16;
                 *reinterpret_cast<v8h*>(dst) = lo;
                 *reinterpret_cast<v8h*>(dst + 8) = hi;
             }
         }
+        // B rows as the first operand: the products come out with a lane per row m of C B^T and four
+        // consecutive columns k per register group, which leave as 8-byte pieces
 #pragma unroll
         for (int i = 0; i < 2; ++i)
 #pragma unroll
-            for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fc[i], fb[j], acc[i][j], 0, 0, 0);
+            for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[ks][j], fc[ks][i], acc[i][j], 0, 0, 0);
     }
-    // acc[i][j]: lane holds column k = kt*64 + j*32 + (lane & 31), register r row m = mt*64 + i*32 + 8*(r/4) + 4*(lane/32) + r%4
+    // acc[i][j]: lane holds row m = mt*64 + i*32 + (lane & 31), register r column k = kt*64 + j*32 + 8*(r/4) + 4*(lane/32) + r%4
     __half* tile = cb_out + ((static_cast<int64_t>(b) * nc + c) * G + g) * Q * Q;
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int m = mt * 64 + i * 32 + 8 * (r / 4) + 4 * fhalf + (r % 4);
-                const int k = kt * 64 + j * 32 + frow;
-                tile[static_cast<int64_t>(m) * Q + k] = __float2half((scale * static_cast<float>(acc[i][j][r])) * kCbShift);
+            for (int q = 0; q < 4; ++q) {
+                const int m = mt * 64 + i * 32 + frow;
+                const int k = kt * 64 + j * 32 + 8 * q + 4 * fhalf;
+                v4h o;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = static_cast<_Float16>((scale * static_cast<float>(acc[i][j][4 * q + e])) * kCbShift);
+                *reinterpret_cast<v4h*>(tile + static_cast<int64_t>(m) * Q + k) = o;
             }
 }
 
@@ -266,8 +301,10 @@ __global__ __launch_bounds__(256, 2) void ssd_state_kernel(QaSsdParams p, const 
     __shared__ __attribute__((aligned(16))) _Float16 s_patch[4 * 32 * kPatchPitch];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, frow = lane & 31, fhalf = lane >> 5;
-    const int h = blockIdx.x % p.nheads;
-    const int b = blockIdx.x / p.nheads;
+    int unit, hig;
+    unit_and_head(blockIdx.x, p.batch * p.ngroups, p.nheads / p.ngroups, unit, hig);
+    const int h = (unit % p.ngroups) * (p.nheads / p.ngroups) + hig;
+    const int b = unit / p.ngroups;
     const int G = p.ngroups, H = p.nheads;
     int g, hg;
     group_of(p, h, g, hg);
