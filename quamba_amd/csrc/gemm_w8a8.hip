@@ -283,5 +283,10 @@ extern "C" int qa_gemm_w8a8(const QaGemmW8A8Params* p, void* stream_) {
         if (cost(256, 320) < cost(256, 256)) return launch_gemm<2, 5, 4, 2, 2, false>(*p, stream);
         return launch_gemm<4, 2, 2, 4, 2, false>(*p, stream);                        // 256x256 tile, 8 waves
     }
-    return launch_gemm<2, 2, 2, 2, 2, false>(*p, stream);                            // 128x128 tile, 4 waves
+    // 128x128 tile, 4 waves.  Two stages (64 KB) let two workgroups share a CU; when there is at most one
+    // workgroup per CU anyway and K is long (x_proj: 16384 x 5120 -> 192), four stages keep three k-tiles
+    // in flight instead of one (36 -> 28 us for that shape).
+    const int64_t small_tiles = static_cast<int64_t>((p->m + 127) / 128) * ((p->n + 127) / 128);
+    if (small_tiles <= 256 && p->k >= 8 * gemm::kBK) return launch_gemm<2, 2, 2, 2, 4, false>(*p, stream);
+    return launch_gemm<2, 2, 2, 2, 2, false>(*p, stream);
 }
