@@ -13,9 +13,14 @@ __device__ __forceinline__ int8_t conv_epilogue(float v, float s_out, int silu) 
 
 // Requantised output by the cheap route (hardware exp2 / rcp, multiply by 1/s_out, round to nearest)
 // whenever that provably equals the exact route, else by the exact route.  The cheap value y differs
-// from the exactly-evaluated one by less than 2e-4 for |y| < 129 (a few ulp of relative error), so if
-// y is further than 2e-3 from every half-integer both round to the same integer; values beyond
-// +-129 saturate either way.  Only lanes inside that margin (about 0.4 %) take the exact route.
+// from the exactly-evaluated one by less than 2e-4 for |y| < 129 and v >= -16: the exponent argument
+// carries a relative error of 6e-8 |v|, exp2, rcp and the exact route's own steps are each within
+// 1-1.5 ulp, together below 1.4e-6 relative.  So if y is further than 5e-4 from every half-integer both
+// round to the same integer; values beyond +-129 saturate either way.  Lanes inside that margin (about
+// 0.1 %) and lanes with v < -16 (where the bound no longer holds; the output is then zero for any sane
+// output scale) take the exact route - but a wave takes it whenever one of its 64 lanes does, which is
+// why the margin is kept as narrow as the error bound allows (at 2e-3 a quarter of all wave-elements
+// went through the exact route's ~100 instructions).
 __device__ __forceinline__ int conv_quant(float v, float s_out, float inv_s_out, int silu) {
     float y = v;
     if (silu) {
@@ -26,7 +31,7 @@ __device__ __forceinline__ int conv_quant(float v, float s_out, float inv_s_out,
     const float yr = __builtin_rintf(y);
     const float d = __builtin_fabsf(y - yr);
     int q = static_cast<int>(__builtin_amdgcn_fmed3f(yr, -128.0f, 127.0f));
-    if (!(d <= 0.498f) && !(__builtin_fabsf(y) >= 129.0f)) q = conv_epilogue(v, s_out, silu);
+    if ((!(d <= 0.4995f) && !(__builtin_fabsf(y) >= 129.0f)) || (silu && v < -16.0f)) q = conv_epilogue(v, s_out, silu);
     return q;
 }
 

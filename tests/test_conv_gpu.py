@@ -35,6 +35,23 @@ def test_fwd_seqlen_contiguous_bit_exact(dev, B, D, L, k, silu):
     np.testing.assert_array_equal(got.cpu().numpy(), want)
 
 
+@pytest.mark.parametrize("s_in,s_out", [(0.02, 0.02), (0.004, 0.001), (0.3, 0.05), (0.05, 2.0), (0.01, 1e-5)])
+def test_fwd_bit_exact_over_wide_ranges_of_the_pre_activation(dev, s_in, s_out):
+    """Uniform int8 inputs and taps: the accumulator sweeps +-65000, so with these scales the SiLU argument
+    covers fractions of a unit up to several hundred units either side of zero, and the outputs run from
+    all-saturated to all-zero.  Two million outputs per case land on every side of the rounding margins of
+    the fast epilogue and of its switch to the exact route for very negative arguments."""
+    g = np.random.default_rng(int(s_in * 1e4) + 7)
+    B, D, L = 2, 256, 4096
+    qx = g.integers(-128, 128, (B, D, L)).astype(np.int8)
+    qw = g.integers(-128, 128, (D, 4)).astype(np.int8)
+    qb = g.integers(-128, 128, D).astype(np.int8)
+    sw, sb = 0.01, 0.02
+    want = oracle.conv1d_fwd(qx, qw, qb, s_in, sw, sb, s_out)
+    got = ops.causal_conv1d_fwd(_t(qx, dev), s_in, _t(qw, dev), sw, s_out, sb, _t(qb, dev))
+    np.testing.assert_array_equal(got.cpu().numpy(), want)
+
+
 def test_fwd_no_bias(dev):
     qx, sx, qw, sw, qb, sb, so = _case(2, 128, 256, 4, seed=5, bias=False)
     want = oracle.conv1d_fwd(qx, qw, None, sx, sw, sb, so)
