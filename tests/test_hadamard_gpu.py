@@ -68,6 +68,24 @@ def test_many_power_of_two_rows_take_the_32_values_per_lane_path(dev, dim, dtype
     np.testing.assert_array_equal(ops.hadamard_quant(shifted[:, 1:dim + 1], float(scale)).cpu().numpy(), got)
 
 
+@pytest.mark.parametrize("dim", [1536, 3072, 5120, 10240])
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_many_rows_of_12_or_40_times_128_or_256_columns_take_the_lane_per_column_path(dev, dim, dtype):
+    """More than 128 aligned rows of S * 128 or S * 256 columns: compile-time addressing, the S-point sums
+    quantised in registers.  Same bits as the oracle (a sample of the rows) and as the general kernel that
+    rows off the 16-byte grid fall back to."""
+    rows = 197
+    x = _rows(rows, dim, seed=dim + 3).astype(dtype)
+    scale = np.float32(1.0 / math.sqrt(dim) / 0.06)
+    got = ops.hadamard_quant(torch.from_numpy(x).to(dev), float(scale)).cpu().numpy()
+    pick = np.array([0, 1, 64, 127, 128, 196])
+    np.testing.assert_array_equal(got[pick], oracle.hadamard_quant(x[pick], scale))
+    assert np.abs(got).max() > 60
+    shifted = torch.zeros((rows, dim + 8), dtype=torch.from_numpy(x).dtype, device=dev)
+    shifted[:, 1:dim + 1] = torch.from_numpy(x).to(dev)
+    np.testing.assert_array_equal(ops.hadamard_quant(shifted[:, 1:dim + 1], float(scale)).cpu().numpy(), got)
+
+
 def test_rounding_at_ties_and_saturation_on_the_32_values_per_lane_path(dev):
     """Rows whose transform lands exactly on k + 1/2 and beyond the int8 range: half away from zero, then
     saturation, as the general kernel does."""
