@@ -297,7 +297,9 @@ typedef struct QaGemmW8A8Params {
     int32_t use_alpha;     /* 1: d = cast(alpha * float(acc)) with the host scalar below (the GEMV
                               rule of cutlass_scaled_mv_dq); the scale pointers are then ignored */
     float alpha;
-    int32_t reserved0;
+    int32_t scale_order;   /* 0: D = s_a[m] * (s_b[n] * acc) as above; 1: D = s_b[n] * (s_a[m] * acc), the
+                              association a caller needs when it exchanges the roles of the two operands
+                              to obtain the (N,M) output of a product defined the first way */
     int64_t lda, ldw, ldd; /* element strides between rows of a, w, d (d is (M,N) row-major) */
     const int8_t* a;
     const int8_t* w;
@@ -332,9 +334,9 @@ typedef struct QaGemmW4A8Params {
     const float* s_token;    /* fp32 (1) or (M) */
     void* d;
     /* Optional scratch of n*k bytes (16-byte aligned), or null.  With many activation rows every 256-row
-     * band of the output expands the same 4-bit weights again; given this buffer (and more than 64 rows, and
-     * the plain output layout) the weights are expanded once (same arithmetic, same int8 values) and the
-     * int8 x int8 kernel runs on the result.  It pays from about 4e11 operations (2*m*n*k) on; whether to pass
+     * band of the output expands the same 4-bit weights again; given this buffer (and more than 64 rows)
+     * the weights are expanded once (same arithmetic, same int8 values) and the int8 x int8 kernel runs on
+     * the result, for the (N,M) output with the roles of the operands exchanged.  It pays from about 4e11 operations (2*m*n*k) on; whether to pass
      * it is the caller's choice.  Results are bit-identical either way. */
     void* w8_workspace;
     int64_t w8_workspace_bytes;

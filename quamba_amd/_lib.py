@@ -119,7 +119,7 @@ class QaGemmW8A8Params(C.Structure):
     _fields_ = [
         ("m", i32), ("n", i32), ("k", i32), ("out_type", i32), ("round_mode", i32),
         ("a_scale_numel", i32), ("w_scale_numel", i32), ("use_alpha", i32),
-        ("alpha", f32), ("reserved0", i32),
+        ("alpha", f32), ("scale_order", i32),
         ("lda", i64), ("ldw", i64), ("ldd", i64),
         ("a", vp), ("w", vp), ("a_scale", vp), ("w_scale", vp), ("d", vp),
     ]

@@ -63,6 +63,7 @@ struct Epilogue {
     int use_alpha;            // d = cast(alpha * acc)
     float alpha;
     int round_mode;           // QaRound
+    int col_outer;            // d = cast(s_col * (s_row * acc)) instead of s_row * (s_col * acc)
     int64_t ldd;
     void* d;
 };
@@ -257,6 +258,7 @@ __device__ __forceinline__ void epilogue(const Epilogue& e, v16i (&acc)[TN][TM],
         float v;
         if (use_alpha) v = s_row[j] * accf;
         // GEMV rule (round-half-away mode): the two scales are multiplied first
+        else if (e.col_outer) v = s_col[i][q][t] * (s_row[j] * accf);
         else v = away ? (s_col[i][q][t] * s_row[j]) * accf : s_row[j] * (s_col[i][q][t] * accf);
         // keep the fp32 product a value of its own: folding the multiply into a mixed-precision
         // convert would round once instead of twice and change the fp16 result in rare cases
@@ -407,6 +409,7 @@ __device__ __forceinline__ void skinny_reduce_store(const Epilogue& e, v16i (&ac
             const float accf = static_cast<float>(red[(j * 16 + q * 4 + t) * 64 + ul]);
             const float s_col = use_alpha ? 1.0f : e.col_scale[e.col_numel == 1 ? 0 : min(nn + t, n - 1)];
             if (use_alpha) v[t] = s_row * accf;
+            else if (e.col_outer) v[t] = s_col * (s_row * accf);
             else v[t] = away ? (s_col * s_row) * accf : s_row * (s_col * accf);
             asm volatile("" : "+v"(v[t]));                 // the fp32 product is rounded on its own
         }

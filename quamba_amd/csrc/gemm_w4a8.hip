@@ -163,7 +163,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_w4a8_kernel(QaGemmW4A8Par
     Epilogue e;
     e.row_scale = p.s_token; e.col_scale = p.s_channel;
     e.row_numel = p.tok_scale_numel; e.col_numel = p.n;
-    e.use_alpha = 0; e.alpha = 0.0f; e.round_mode = QA_ROUND_RNE;
+    e.use_alpha = 0; e.alpha = 0.0f; e.round_mode = QA_ROUND_RNE; e.col_outer = 0;
     e.ldd = p.ldd; e.d = p.d;
     epilogue<TM, TN, OUT, false, TRANS>(e, acc, lds, p.m, p.n, m0 + wm * TM * 32, n0 + wn * TN * 32, wave, lane);
 }
@@ -338,7 +338,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_w4a8_skinny_kernel(QaGemmW4A8
     Epilogue e;
     e.row_scale = p.s_token; e.col_scale = p.s_channel;
     e.row_numel = p.tok_scale_numel; e.col_numel = p.n;
-    e.use_alpha = 0; e.alpha = 0.0f; e.round_mode = QA_ROUND_RNE;
+    e.use_alpha = 0; e.alpha = 0.0f; e.round_mode = QA_ROUND_RNE; e.col_outer = 0;
     e.ldd = p.ldd; e.d = p.d;
     skinny_reduce_store<TM, OUT, false, TRANS>(e, acc, red, p.m, p.n, n0, tid, kThreads);
 }
@@ -423,20 +423,32 @@ extern "C" int qa_gemm_w4a8(const QaGemmW4A8Params* p, void* stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     if (p->m <= 64 && static_cast<int64_t>(p->n) * (p->k / 2) < 0x70000000LL) return dispatch_skinny(*p, stream);
     const int64_t w8_bytes = static_cast<int64_t>(p->n) * p->k;
-    if (p->w8_workspace && !p->output_transpose && p->w8_workspace_bytes >= w8_bytes && aligned16(p->w8_workspace) &&
-        w8_bytes < 0x70000000LL) {
+    if (p->w8_workspace && p->w8_workspace_bytes >= w8_bytes && aligned16(p->w8_workspace) && w8_bytes < 0x70000000LL &&
+        (!p->output_transpose || p->n > 64)) {
         int8_t* w8 = static_cast<int8_t*>(p->w8_workspace);
         const int64_t threads = static_cast<int64_t>(p->n) * (p->k / 32);
         hipLaunchKernelGGL(w4_expand_kernel, dim3(static_cast<unsigned>((threads + 255) / 256)), dim3(256), 0, stream, *p, w8);
         // (acc * s_channel[n]) * s_token[m] and s_token[m] * (s_channel[n] * acc) round the same two products
         QaGemmW8A8Params q = {};
-        q.m = p->m; q.n = p->n; q.k = p->k;
-        q.lda = p->lda; q.ldw = p->k; q.ldd = p->ldd;
-        q.a = p->a; q.w = w8; q.d = p->d;
-        q.a_scale = p->s_token; q.a_scale_numel = p->tok_scale_numel;
-        q.w_scale = p->s_channel; q.w_scale_numel = p->n;
+        q.k = p->k; q.ldd = p->ldd; q.d = p->d;
         q.out_type = p->out_type;
         q.round_mode = QA_ROUND_RNE;
+        if (!p->output_transpose) {
+            q.m = p->m; q.n = p->n;
+            q.lda = p->lda; q.ldw = p->k;
+            q.a = p->a; q.w = w8;
+            q.a_scale = p->s_token; q.a_scale_numel = p->tok_scale_numel;
+            q.w_scale = p->s_channel; q.w_scale_numel = p->n;
+        } else {
+            // the (N,M) output is the product with the operands' roles exchanged; the column scale (the
+            // token's) is then applied last, which keeps the association s_token * (s_channel * acc)
+            q.m = p->n; q.n = p->m;
+            q.lda = p->k; q.ldw = p->lda;
+            q.a = w8; q.w = p->a;
+            q.a_scale = p->s_channel; q.a_scale_numel = p->n;
+            q.w_scale = p->s_token; q.w_scale_numel = p->tok_scale_numel;
+            q.scale_order = 1;
+        }
         return qa_gemm_w8a8(&q, stream_);
     }
     const int64_t big_tiles = static_cast<int64_t>((p->m + 255) / 256) * ((p->n + 255) / 256);

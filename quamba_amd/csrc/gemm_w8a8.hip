@@ -78,7 +78,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_w8a8_kernel(QaGemmW8A8Par
     Epilogue e;
     e.row_scale = p.a_scale; e.col_scale = p.w_scale;
     e.row_numel = p.a_scale_numel; e.col_numel = p.w_scale_numel;
-    e.use_alpha = p.use_alpha; e.alpha = p.alpha; e.round_mode = p.round_mode;
+    e.use_alpha = p.use_alpha; e.alpha = p.alpha; e.round_mode = p.round_mode; e.col_outer = p.scale_order;
     e.ldd = p.ldd; e.d = p.d;
     epilogue<TM, TN, OUT, FLEX, false>(e, acc, lds, p.m, p.n, m0 + wm * TM * 32, n0 + wn * TN * 32, wave, lane);
 }
@@ -209,7 +209,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_w8a8_skinny_kernel(QaGemmW8A8
     Epilogue e;
     e.row_scale = p.a_scale; e.col_scale = p.w_scale;
     e.row_numel = p.a_scale_numel; e.col_numel = p.w_scale_numel;
-    e.use_alpha = p.use_alpha; e.alpha = p.alpha; e.round_mode = p.round_mode;
+    e.use_alpha = p.use_alpha; e.alpha = p.alpha; e.round_mode = p.round_mode; e.col_outer = p.scale_order;
     e.ldd = p.ldd; e.d = p.d;
     skinny_reduce_store<TM, OUT, FLEX, false>(e, acc, red, p.m, p.n, n0, tid, kThreads);
 }
@@ -253,6 +253,7 @@ extern "C" int qa_gemm_w8a8(const QaGemmW8A8Params* p, void* stream_) {
     if (!p->use_alpha && (!p->a_scale || !p->w_scale)) return QA_ERR_NULL;
     if (p->m < 0 || p->n < 0 || p->k < 0) return QA_ERR_SHAPE;
     if (p->out_type != QA_OUT_I8 && p->out_type != QA_OUT_F16) return QA_ERR_UNSUPPORTED;
+    if (p->scale_order != 0 && p->scale_order != 1) return QA_ERR_UNSUPPORTED;
     if (!p->use_alpha && p->a_scale_numel != 1 && p->a_scale_numel != p->m) return QA_ERR_SHAPE;
     if (!p->use_alpha && p->w_scale_numel != 1 && p->w_scale_numel != p->n) return QA_ERR_SHAPE;
     // 16-byte operand chunks: the same alignment the reference's tensor-core path demands

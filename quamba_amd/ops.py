@@ -613,7 +613,7 @@ def _w4a8_gemm(a, b_q_weight, s_tok, s_ch, s_group, m, n, k, output_transpose, o
     p.a, p.w_packed, p.s_group = ptr(a), ptr(b_q_weight), ptr(s_group) if grouped else None
     p.s_channel, p.s_token, p.d = ptr(s_ch_c), ptr(s_tok_c), ptr(d)
     w8 = None
-    if not output_transpose and 2.0 * m * n * k >= W4A8_EXPAND_ONCE_OPS:
+    if 2.0 * m * n * k >= W4A8_EXPAND_ONCE_OPS:
         # many rows: scratch for the weights expanded to int8 once (see QaGemmW4A8Params.w8_workspace)
         w8 = torch.empty(n * k, dtype=torch.int8, device=a.device)
         p.w8_workspace, p.w8_workspace_bytes = ptr(w8), w8.numel()
