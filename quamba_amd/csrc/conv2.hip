@@ -99,6 +99,7 @@ __global__ __launch_bounds__(kThreads) void conv2_fwd_kernel(QaConv2Params p) {
     const Part part = part_of(p, ch0);          // the four channels of a lane never straddle two parts
     uint32_t taps[4];
     float bias_f[4], s_out[4], inv_s_out[4];
+    bool exact_only[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         const int ch = ch0 + e;
@@ -106,6 +107,7 @@ __global__ __launch_bounds__(kThreads) void conv2_fwd_kernel(QaConv2Params p) {
         bias_f[e] = p.bias ? part.s_bias * static_cast<float>(p.bias[ch]) : 0.0f;
         s_out[e] = out_scale_of(p, part, ch);
         inv_s_out[e] = 1.0f / s_out[e];
+        exact_only[e] = conv_needs_exact_route(s_out[e]);
     }
     int64_t out_ls, out_cs;
     int8_t* out = out_ptr(p, part, b, ch0, &out_ls, &out_cs);
@@ -139,7 +141,7 @@ __global__ __launch_bounds__(kThreads) void conv2_fwd_kernel(QaConv2Params p) {
             for (int e = 0; e < 4; ++e) {
                 const float acc = static_cast<float>(dot4(win[e], taps[e]));
                 const float v = __builtin_fmaf(part.s_in, acc, bias_f[e]);
-                const int q = conv_quant(v, s_out[e], inv_s_out[e], p.silu_activation);
+                const int q = conv_quant(v, s_out[e], inv_s_out[e], p.silu_activation, exact_only[e]);
                 packed |= static_cast<uint32_t>(q & 0xff) << (8 * e);
             }
             *reinterpret_cast<uint32_t*>(out + (tb + i) * out_ls) = packed;

@@ -16,22 +16,26 @@ __device__ __forceinline__ int8_t conv_epilogue(float v, float s_out, int silu) 
 // from the exactly-evaluated one by less than 2e-4 for |y| < 129 and v >= -16: the exponent argument
 // carries a relative error of 6e-8 |v|, exp2, rcp and the exact route's own steps are each within
 // 1-1.5 ulp, together below 1.4e-6 relative.  So if y is further than 5e-4 from every half-integer both
-// round to the same integer; values beyond +-129 saturate either way.  Lanes inside that margin (about
-// 0.1 %) and lanes with v < -16 (where the bound no longer holds; the output is then zero for any sane
-// output scale) take the exact route - but a wave takes it whenever one of its 64 lanes does, which is
-// why the margin is kept as narrow as the error bound allows (at 2e-3 a quarter of all wave-elements
-// went through the exact route's ~100 instructions).
-__device__ __forceinline__ int conv_quant(float v, float s_out, float inv_s_out, int silu) {
+// round to the same integer.  y is clamped to +-128.75 first: beyond that both routes saturate, and the
+// clamped value (a quarter away from 129) passes the test on its own.  For v < -16 the bound no longer
+// holds, but there |y| < 1.8e-6 / s_out: with s_out >= 1e-5 both routes give zero, and for smaller
+// output scales the caller sets `exact_only` and every lane takes the exact route.
+// A wave takes the exact route whenever one of its 64 lanes does, which is why the margin is kept as
+// narrow as the error bound allows (at 2e-3, 0.4 % of the lanes, a quarter of all wave-elements went
+// through the exact route's ~100 instructions).
+__device__ __forceinline__ bool conv_needs_exact_route(float s_out) { return !(s_out >= 1e-5f); }
+
+__device__ __forceinline__ int conv_quant(float v, float s_out, float inv_s_out, int silu, bool exact_only) {
     float y = v;
     if (silu) {
         const float e = __builtin_amdgcn_exp2f(v * -1.44269504088896341f);
         y = v * __builtin_amdgcn_rcpf(1.0f + e);
     }
-    y *= inv_s_out;
+    y = __builtin_amdgcn_fmed3f(y * inv_s_out, -128.75f, 128.75f);
     const float yr = __builtin_rintf(y);
     const float d = __builtin_fabsf(y - yr);
     int q = static_cast<int>(__builtin_amdgcn_fmed3f(yr, -128.0f, 127.0f));
-    if ((!(d <= 0.4995f) && !(__builtin_fabsf(y) >= 129.0f)) || (silu && v < -16.0f)) q = conv_epilogue(v, s_out, silu);
+    if (exact_only || !(d <= 0.4995f)) q = conv_epilogue(v, s_out, silu);
     return q;
 }
 

@@ -35,7 +35,7 @@ def test_fwd_seqlen_contiguous_bit_exact(dev, B, D, L, k, silu):
     np.testing.assert_array_equal(got.cpu().numpy(), want)
 
 
-@pytest.mark.parametrize("s_in,s_out", [(0.02, 0.02), (0.004, 0.001), (0.3, 0.05), (0.05, 2.0), (0.01, 1e-5)])
+@pytest.mark.parametrize("s_in,s_out", [(0.02, 0.02), (0.004, 0.001), (0.3, 0.05), (0.05, 2.0), (0.01, 1e-5), (0.0002, 2e-7)])
 def test_fwd_bit_exact_over_wide_ranges_of_the_pre_activation(dev, s_in, s_out):
     """Uniform int8 inputs and taps: the accumulator sweeps +-65000, so with these scales the SiLU argument
     covers fractions of a unit up to several hundred units either side of zero, and the outputs run from
