@@ -13,10 +13,11 @@ __device__ __forceinline__ int8_t conv_epilogue(float v, float s_out, int silu) 
 
 // Requantised output by the cheap route (hardware exp2 / rcp, multiply by 1/s_out, round to nearest)
 // whenever that provably equals the exact route, else by the exact route.  The cheap value y differs
-// from the exactly-evaluated one by less than 2e-4 for |y| < 129 and v >= -16: the exponent argument
-// carries a relative error of 6e-8 |v|, exp2, rcp and the exact route's own steps are each within
-// 1-1.5 ulp, together below 1.4e-6 relative.  So if y is further than 5e-4 from every half-integer both
-// round to the same integer.  y is clamped to +-128.75 first: beyond that both routes saturate, and the
+// from the exactly-evaluated one by less than 3.3e-4 for |y| < 129 and v >= -16: the exponent argument
+// v * log2(e) is rounded twice (a relative error of 1e-7 |v| in the exponential), exp2, rcp and the exact
+// route's own steps are each within 1-1.5 ulp, together below 2.5e-6 relative.  So if y is further than
+// 5e-4 from every half-integer both round to the same integer (a margin proportional to |y| was tried
+// and measured no faster).  y is clamped to +-128.75 first: beyond that both routes saturate, and the
 // clamped value (a quarter away from 129) passes the test on its own.  For v < -16 the bound no longer
 // holds, but there |y| < 1.8e-6 / s_out: with s_out >= 1e-5 both routes give zero, and for smaller
 // output scales the caller sets `exact_only` and every lane takes the exact route.
