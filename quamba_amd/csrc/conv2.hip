@@ -21,7 +21,7 @@ namespace qa {
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kRun = 32;          // time steps per wave
+constexpr int kRun = 64;          // time steps per wave
 constexpr int kBatchLoads = 8;    // loads in flight per lane
 
 struct Part {
@@ -126,12 +126,20 @@ __global__ __launch_bounds__(kThreads) void conv2_fwd_kernel(QaConv2Params p) {
         const int t = t0 - 3 + i;
         push(t >= 0 ? *reinterpret_cast<const uint32_t*>(src + t * p.xBC_l_stride) : 0u);
     }
-    for (int tb = t0; tb < t_end; tb += kBatchLoads) {
-        uint32_t d[kBatchLoads];
+    // the loads of the next batch of steps are in flight while the current batch is worked on
+    uint32_t d[kBatchLoads], dn[kBatchLoads];
+    auto fetch = [&](int tb, uint32_t (&dst)[kBatchLoads]) {
 #pragma unroll
         for (int i = 0; i < kBatchLoads; ++i) {
-            d[i] = tb + i < t_end ? *reinterpret_cast<const uint32_t*>(src + (tb + i) * p.xBC_l_stride) : 0u;
+            const int t = min(tb + i, p.seqlen - 1);              // in range for every lane; steps past the end are never used
+            dst[i] = *reinterpret_cast<const uint32_t*>(src + t * p.xBC_l_stride);
         }
+    };
+    fetch(t0, dn);
+    for (int tb = t0; tb < t_end; tb += kBatchLoads) {
+#pragma unroll
+        for (int i = 0; i < kBatchLoads; ++i) d[i] = dn[i];
+        if (tb + kBatchLoads < t_end) fetch(tb + kBatchLoads, dn);
 #pragma unroll
         for (int i = 0; i < kBatchLoads; ++i) {
             if (tb + i >= t_end) break;
