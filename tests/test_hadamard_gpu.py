@@ -86,6 +86,22 @@ def test_many_rows_of_12_or_40_times_128_or_256_columns_take_the_lane_per_column
     np.testing.assert_array_equal(ops.hadamard_quant(shifted[:, 1:dim + 1], float(scale)).cpu().numpy(), got)
 
 
+@pytest.mark.parametrize("rows,dim", [(2100, 8192), (4173, 2048)])
+def test_more_rows_than_resident_workgroups(dev, rows, dim):
+    """The 32-values-per-lane kernel launches as many workgroups as the chip holds and lets each walk several
+    rows with the next row's loads in flight: first, middle and last rows of such walks against the oracle."""
+    x = _rows(rows, dim, seed=rows)
+    scale = np.float32(1.0 / math.sqrt(dim) / 0.06)
+    got = ops.hadamard_quant(torch.from_numpy(x).to(dev), float(scale)).cpu().numpy()
+    pick = np.array([0, 1, 1023, 1024, 1025, 2047, 2048, 2049, rows - 2, rows - 1])
+    np.testing.assert_array_equal(got[pick], oracle.hadamard_quant(x[pick], scale))
+    # every row: the same bytes as when the row is transformed in a small call of its own
+    few = ops.hadamard_quant(torch.from_numpy(x[1000:1100]).to(dev), float(scale)).cpu().numpy()
+    np.testing.assert_array_equal(got[1000:1100], few)
+    tail = ops.hadamard_quant(torch.from_numpy(x[-150:]).to(dev), float(scale)).cpu().numpy()
+    np.testing.assert_array_equal(got[-150:], tail)
+
+
 def test_rounding_at_ties_and_saturation_on_the_32_values_per_lane_path(dev):
     """Rows whose transform lands exactly on k + 1/2 and beyond the int8 range: half away from zero, then
     saturation, as the general kernel does."""

@@ -98,7 +98,9 @@ def test_state_dict_and_errors(dev):
 
 
 # (rows, dim, group_size): the Mamba2-8b form, one group per wave, a whole wave's span per group, decode rows
-FUSED = [(300, 8192, 1024), (70, 8192, 512), (150, 4096, 2048), (131, 2048, 512), (9, 2048, 1024), (1, 8192, 1024)]
+FUSED = [(300, 8192, 1024), (70, 8192, 512), (150, 4096, 2048), (131, 2048, 512), (9, 2048, 1024), (1, 8192, 1024),
+         # more rows than workgroups in flight: a workgroup then walks several rows
+         (2100, 8192, 1024)]
 
 
 @pytest.mark.parametrize("M,N,group_size", FUSED)
