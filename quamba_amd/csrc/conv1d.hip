@@ -21,13 +21,13 @@ constexpr int kConvThreads = 256;
 // One thread = 16 consecutive time steps of one (batch, channel) row.  Rows are 16-byte aligned
 // (checked on the host); a ragged tail (seqlen % 16) is handled bytewise by the row's last thread.
 __global__ __launch_bounds__(kConvThreads) void conv_fwd_rows_kernel(QaConvParams p, int segs) {
-    const int64_t idx = static_cast<int64_t>(blockIdx.x) * kConvThreads + threadIdx.x;
-    const int64_t nrows = static_cast<int64_t>(p.batch) * p.dim;
-    if (idx >= nrows * segs) return;
-    const int seg = static_cast<int>(idx % segs);
-    const int64_t row = idx / segs;
-    const int c = static_cast<int>(row % p.dim);
-    const int b = static_cast<int>(row / p.dim);
+    // grid: x over runs of 64 segments of a row (one wave each), y over groups of four channels (one per
+    // wave), z = batch: no integer division on the way in, and the channel is the same for a whole wave,
+    // so its taps and bias are fetched and packed once per wave by scalar instructions
+    const int c = __builtin_amdgcn_readfirstlane(static_cast<int>(blockIdx.y * 4 + (threadIdx.x >> 6)));
+    const int b = blockIdx.z;
+    const int seg = blockIdx.x * 64 + (threadIdx.x & 63);
+    if (c >= p.dim || seg >= segs) return;
     const int8_t* x = p.x + b * p.x_batch_stride + c * p.x_c_stride;
     int8_t* out = p.out + b * p.out_batch_stride + c * p.out_c_stride;
 
@@ -248,11 +248,10 @@ extern "C" int qa_causal_conv1d_fwd(const QaConvParams* p, void* stream_) {
         }
         if (rows_ok) {
             const int segs = (p->seqlen + 15) / 16;
-            const int64_t threads = static_cast<int64_t>(p->batch) * p->dim * segs;
-            const int64_t blocks = (threads + kConvThreads - 1) / kConvThreads;
-            if (blocks > 0x7fffffffLL) return QA_ERR_SHAPE;
-            hipLaunchKernelGGL(conv_fwd_rows_kernel, dim3(static_cast<unsigned>(blocks)), dim3(kConvThreads), 0,
-                               stream, *p, segs);
+            const int64_t groups = (static_cast<int64_t>(p->dim) + 3) / 4;
+            if (groups > 65535 || p->batch > 65535) return QA_ERR_SHAPE;
+            const dim3 grid(static_cast<unsigned>((segs + 63) / 64), static_cast<unsigned>(groups), static_cast<unsigned>(p->batch));
+            hipLaunchKernelGGL(conv_fwd_rows_kernel, grid, dim3(kConvThreads), 0, stream, *p, segs);
             return check_launch();
         }
     }
