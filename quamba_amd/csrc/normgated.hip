@@ -34,10 +34,11 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) void rmsnorm_gated_kernel(QaNo
     const int ngroups = p.dim / p.group_size;
     constexpr int kItemsPerBlock = kWavesPerBlock / WPI;
     const int sub = wave % WPI;                               // this wave's share of the group
-    const int64_t item = static_cast<int64_t>(blockIdx.x) * kItemsPerBlock + wave / WPI;
-    if (item >= static_cast<int64_t>(p.rows) * ngroups) return;   // with WPI > 1 the whole workgroup leaves
-    const int64_t row = item / ngroups;
-    const int group = static_cast<int>(item % ngroups);
+    // the item is the same for a whole wave: scalar arithmetic, 32 bits (the host bounds the item count)
+    const unsigned item = __builtin_amdgcn_readfirstlane(blockIdx.x * kItemsPerBlock + wave / WPI);
+    if (item >= static_cast<unsigned>(p.rows) * static_cast<unsigned>(ngroups)) return;   // with WPI > 1 the whole workgroup leaves
+    const int64_t row = item / static_cast<unsigned>(ngroups);
+    const int group = static_cast<int>(item % static_cast<unsigned>(ngroups));
     const int N = p.group_size;
     const int col0 = group * N;
     const __half* x = static_cast<const __half*>(p.x) + row * p.x_row_stride + col0;
@@ -151,7 +152,7 @@ extern "C" int qa_rmsnorm_gated(const QaNormGatedParams* p, void* stream_) {
     const int64_t items = static_cast<int64_t>(p->rows) * (p->dim / p->group_size);
     const bool together = p->group_size > 2048;               // four waves per group
     const int64_t blocks = together ? items : (items + kWavesPerBlock - 1) / kWavesPerBlock;
-    if (blocks > 0x7fffffffLL) return QA_ERR_SHAPE;
+    if (blocks > 0x7fffffffLL || items > 0x7fffffffLL) return QA_ERR_SHAPE;
     const dim3 grid(static_cast<unsigned>(blocks)), block(64 * kWavesPerBlock);
     const int span = together ? 512 * kWavesPerBlock : 512;
     const int pieces = (p->group_size + span - 1) / span;
