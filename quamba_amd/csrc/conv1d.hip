@@ -36,6 +36,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_fwd_rows_kernel(QaConvParam
     const float bias_f = p.bias ? static_cast<float>(p.bias[c]) * p.scale_b : 0.0f;
     const float inv_s_out = 1.0f / p.scale_out;
     const bool exact_only = conv_needs_exact_route(p.scale_out);
+    const ConvQuantRegs kq;
 
     const int t0 = seg * 16;
     const int remaining = p.seqlen - t0;
@@ -60,7 +61,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_fwd_rows_kernel(QaConvParam
             const uint32_t win = j == 3 ? w[q + 1] : __builtin_amdgcn_alignbyte(w[q + 1], w[q], j + 1);
             const float acc = static_cast<float>(dot4(win, taps));
             const float v = __builtin_fmaf(s_wx, acc, bias_f);
-            const int r = conv_quant(v, p.scale_out, inv_s_out, p.silu_activation, exact_only);
+            const int r = conv_quant(v, p.scale_out, inv_s_out, p.silu_activation, exact_only, kq);
             packed |= static_cast<uint32_t>(r & 0xff) << (8 * j);
         }
         o[q] = packed;
@@ -98,6 +99,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_fwd_rows_dual_kernel(QaConv
         const float bias_f = p.bias ? static_cast<float>(p.bias[c]) * p.scale_b : 0.0f;
         const float inv_s_out = 1.0f / p.scale_out;
     const bool exact_only = conv_needs_exact_route(p.scale_out);
+    const ConvQuantRegs kq;
         uint32_t w[5];   // w[0] = x[t0-4 .. t0-1], w[1..4] = x[t0 .. t0+15]
         w[0] = t0 > 0 ? *reinterpret_cast<const uint32_t*>(x + t0 - 4) : 0u;
         if (remaining >= 16) {
@@ -117,7 +119,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_fwd_rows_dual_kernel(QaConv
                 const uint32_t win = j == 3 ? w[q + 1] : __builtin_amdgcn_alignbyte(w[q + 1], w[q], j + 1);
                 const float acc = static_cast<float>(dot4(win, taps));
                 const float v = __builtin_fmaf(s_wx, acc, bias_f);
-                const int r = conv_quant(v, p.scale_out, inv_s_out, p.silu_activation, exact_only);
+                const int r = conv_quant(v, p.scale_out, inv_s_out, p.silu_activation, exact_only, kq);
                 packed |= static_cast<uint32_t>(r & 0xff) << (8 * j);
             }
             o[q] = packed;

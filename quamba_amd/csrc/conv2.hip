@@ -100,6 +100,7 @@ __global__ __launch_bounds__(kThreads) void conv2_fwd_kernel(QaConv2Params p) {
     uint32_t taps[4];
     float bias_f[4], s_out[4], inv_s_out[4];
     bool exact_only[4];
+    const ConvQuantRegs kq;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         const int ch = ch0 + e;
@@ -149,7 +150,7 @@ __global__ __launch_bounds__(kThreads) void conv2_fwd_kernel(QaConv2Params p) {
             for (int e = 0; e < 4; ++e) {
                 const float acc = static_cast<float>(dot4(win[e], taps[e]));
                 const float v = __builtin_fmaf(part.s_in, acc, bias_f[e]);
-                const int q = conv_quant(v, s_out[e], inv_s_out[e], p.silu_activation, exact_only[e]);
+                const int q = conv_quant(v, s_out[e], inv_s_out[e], p.silu_activation, exact_only[e], kq);
                 packed |= static_cast<uint32_t>(q & 0xff) << (8 * e);
             }
             *reinterpret_cast<uint32_t*>(out + (tb + i) * out_ls) = packed;

@@ -26,16 +26,28 @@ __device__ __forceinline__ int8_t conv_epilogue(float v, float s_out, int silu) 
 // through the exact route's ~100 instructions).
 __device__ __forceinline__ bool conv_needs_exact_route(float s_out) { return !(s_out >= 1e-5f); }
 
-__device__ __forceinline__ int conv_quant(float v, float s_out, float inv_s_out, int silu, bool exact_only) {
+// The bounds of the two clamps, held in registers for the life of the thread.  They are not values an
+// instruction can carry inline, and the compiler would otherwise load each of them into a register
+// again for every output (three extra instructions on a path of under thirty).
+struct ConvQuantRegs {
+    float clamp_hi, q_hi;
+    __device__ __forceinline__ ConvQuantRegs() {
+        asm volatile("v_mov_b32 %0, 0x4300c000" : "=v"(clamp_hi));     // 128.75
+        asm volatile("v_mov_b32 %0, 0x42fe0000" : "=v"(q_hi));         // 127.0
+    }
+};
+
+__device__ __forceinline__ int conv_quant(float v, float s_out, float inv_s_out, int silu, bool exact_only,
+                                          const ConvQuantRegs& k) {
     float y = v;
     if (silu) {
         const float e = __builtin_amdgcn_exp2f(v * -1.44269504088896341f);
         y = v * __builtin_amdgcn_rcpf(1.0f + e);
     }
-    y = __builtin_amdgcn_fmed3f(y * inv_s_out, -128.75f, 128.75f);
+    y = __builtin_amdgcn_fmed3f(y * inv_s_out, -k.clamp_hi, k.clamp_hi);
     const float yr = __builtin_rintf(y);
     const float d = __builtin_fabsf(y - yr);
-    int q = static_cast<int>(__builtin_amdgcn_fmed3f(yr, -128.0f, 127.0f));
+    int q = static_cast<int>(__builtin_amdgcn_fmed3f(yr, -128.0f, k.q_hi));
     if (exact_only || !(d <= 0.4995f)) q = conv_epilogue(v, s_out, silu);
     return q;
 }
