@@ -20,6 +20,7 @@ constexpr int kConvThreads = 256;
 
 // One thread = 16 consecutive time steps of one (batch, channel) row.  Rows are 16-byte aligned
 // (checked on the host); a ragged tail (seqlen % 16) is handled bytewise by the row's last thread.
+template <bool SILU>
 __global__ __launch_bounds__(kConvThreads) void conv_fwd_rows_kernel(QaConvParams p, int segs) {
     // grid: x over runs of 64 segments of a row (one wave each), y over groups of four channels (one per
     // wave), z = batch: no integer division on the way in, and the channel is the same for a whole wave,
@@ -61,7 +62,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_fwd_rows_kernel(QaConvParam
             const uint32_t win = j == 3 ? w[q + 1] : __builtin_amdgcn_alignbyte(w[q + 1], w[q], j + 1);
             const float acc = static_cast<float>(dot4(win, taps));
             const float v = __builtin_fmaf(s_wx, acc, bias_f);
-            const int r = conv_quant(v, p.scale_out, inv_s_out, p.silu_activation, exact_only, kq);
+            const int r = conv_quant(v, p.scale_out, inv_s_out, SILU, exact_only, kq);
             packed |= static_cast<uint32_t>(r & 0xff) << (8 * j);
         }
         o[q] = packed;
@@ -79,6 +80,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_fwd_rows_kernel(QaConvParam
 // in the input's layout (16 bytes per thread, as above) and with channels contiguous, (batch, seqlen, dim).
 // Thread (channel tid/4, segment tid%4) computes 16 steps of one channel; the 64 x 64 byte tile then
 // passes through LDS and thread (step tid/4, piece tid%4) gathers 16 channels of one step.
+template <bool SILU>
 __global__ __launch_bounds__(kConvThreads) void conv_fwd_rows_dual_kernel(QaConvParams p, int tiles_l, int tiles_c) {
     constexpr int kPitch = 80;                       // bytes per staged channel row (16-byte aligned, 64 used)
     __shared__ __attribute__((aligned(16))) uint8_t s_tile[64 * kPitch];
@@ -119,7 +121,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_fwd_rows_dual_kernel(QaConv
                 const uint32_t win = j == 3 ? w[q + 1] : __builtin_amdgcn_alignbyte(w[q + 1], w[q], j + 1);
                 const float acc = static_cast<float>(dot4(win, taps));
                 const float v = __builtin_fmaf(s_wx, acc, bias_f);
-                const int r = conv_quant(v, p.scale_out, inv_s_out, p.silu_activation, exact_only, kq);
+                const int r = conv_quant(v, p.scale_out, inv_s_out, SILU, exact_only, kq);
                 packed |= static_cast<uint32_t>(r & 0xff) << (8 * j);
             }
             o[q] = packed;
@@ -244,8 +246,8 @@ extern "C" int qa_causal_conv1d_fwd(const QaConvParams* p, void* stream_) {
             const int tiles_l = (p->seqlen + 63) / 64, tiles_c = (p->dim + 63) / 64;
             const int64_t blocks = static_cast<int64_t>(p->batch) * tiles_l * tiles_c;
             if (blocks > 0x7fffffffLL) return QA_ERR_SHAPE;
-            hipLaunchKernelGGL(conv_fwd_rows_dual_kernel, dim3(static_cast<unsigned>(blocks)), dim3(kConvThreads), 0,
-                               stream, *p, tiles_l, tiles_c);
+            if (p->silu_activation) hipLaunchKernelGGL(conv_fwd_rows_dual_kernel<true>, dim3(static_cast<unsigned>(blocks)), dim3(kConvThreads), 0, stream, *p, tiles_l, tiles_c);
+            else hipLaunchKernelGGL(conv_fwd_rows_dual_kernel<false>, dim3(static_cast<unsigned>(blocks)), dim3(kConvThreads), 0, stream, *p, tiles_l, tiles_c);
             return check_launch();
         }
         if (rows_ok) {
@@ -253,7 +255,8 @@ extern "C" int qa_causal_conv1d_fwd(const QaConvParams* p, void* stream_) {
             const int64_t groups = (static_cast<int64_t>(p->dim) + 3) / 4;
             if (groups > 65535 || p->batch > 65535) return QA_ERR_SHAPE;
             const dim3 grid(static_cast<unsigned>((segs + 63) / 64), static_cast<unsigned>(groups), static_cast<unsigned>(p->batch));
-            hipLaunchKernelGGL(conv_fwd_rows_kernel, grid, dim3(kConvThreads), 0, stream, *p, segs);
+            if (p->silu_activation) hipLaunchKernelGGL(conv_fwd_rows_kernel<true>, grid, dim3(kConvThreads), 0, stream, *p, segs);
+            else hipLaunchKernelGGL(conv_fwd_rows_kernel<false>, grid, dim3(kConvThreads), 0, stream, *p, segs);
             return check_launch();
         }
     }
