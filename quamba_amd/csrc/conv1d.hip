@@ -20,15 +20,16 @@ constexpr int kConvThreads = 256;
 
 // One thread = 16 consecutive time steps of one (batch, channel) row.  Rows are 16-byte aligned
 // (checked on the host); a ragged tail (seqlen % 16) is handled bytewise by the row's last thread.
-template <bool SILU>
+template <bool SILU, int PIECES>
 __global__ __launch_bounds__(kConvThreads) void conv_fwd_rows_kernel(QaConvParams p, int segs) {
-    // grid: x over runs of 64 segments of a row (one wave each), y over groups of four channels (one per
-    // wave), z = batch: no integer division on the way in, and the channel is the same for a whole wave,
-    // so its taps and bias are fetched and packed once per wave by scalar instructions
+    // grid: x over runs of PIECES * 64 segments of a row (one wave each), y over groups of four channels
+    // (one per wave), z = batch: no integer division on the way in, and the channel is the same for a
+    // whole wave, so its taps and bias are fetched and packed once per wave by scalar instructions.
+    // A lane takes segment 64*k + lane of its wave's run, k < PIECES: every load of a wave is 1 KB in one piece.
     const int c = __builtin_amdgcn_readfirstlane(static_cast<int>(blockIdx.y * 4 + (threadIdx.x >> 6)));
     const int b = blockIdx.z;
-    const int seg = blockIdx.x * 64 + (threadIdx.x & 63);
-    if (c >= p.dim || seg >= segs) return;
+    const int seg0 = blockIdx.x * (64 * PIECES) + (threadIdx.x & 63);
+    if (c >= p.dim || seg0 >= segs) return;
     const int8_t* x = p.x + b * p.x_batch_stride + c * p.x_c_stride;
     int8_t* out = p.out + b * p.out_batch_stride + c * p.out_c_stride;
 
@@ -39,39 +40,51 @@ __global__ __launch_bounds__(kConvThreads) void conv_fwd_rows_kernel(QaConvParam
     const bool exact_only = conv_needs_exact_route(p.scale_out);
     const ConvQuantRegs kq;
 
-    const int t0 = seg * 16;
-    const int remaining = p.seqlen - t0;
-    uint32_t w[5];   // w[0] = x[t0-4 .. t0-1], w[1..4] = x[t0 .. t0+15]
-    w[0] = seg > 0 ? *reinterpret_cast<const uint32_t*>(x + t0 - 4) : 0u;
-    if (remaining >= 16) {
-        const uint4 v = *reinterpret_cast<const uint4*>(x + t0);
-        w[1] = v.x; w[2] = v.y; w[3] = v.z; w[4] = v.w;
-    } else {
-        w[1] = w[2] = w[3] = w[4] = 0u;
-        for (int i = 0; i < remaining; ++i) {
-            w[1 + (i >> 2)] |= static_cast<uint32_t>(static_cast<uint8_t>(x[t0 + i])) << (8 * (i & 3));
+    uint32_t w[PIECES][5];   // w[k][0] = x[t0-4 .. t0-1], w[k][1..4] = x[t0 .. t0+15]
+#pragma unroll
+    for (int k = 0; k < PIECES; ++k) {
+        const int seg = seg0 + 64 * k;
+        const int t0 = seg * 16;
+        const int remaining = p.seqlen - t0;
+        if (seg >= segs) break;
+        w[k][0] = seg > 0 ? *reinterpret_cast<const uint32_t*>(x + t0 - 4) : 0u;
+        if (remaining >= 16) {
+            const uint4 v = *reinterpret_cast<const uint4*>(x + t0);
+            w[k][1] = v.x; w[k][2] = v.y; w[k][3] = v.z; w[k][4] = v.w;
+        } else {
+            w[k][1] = w[k][2] = w[k][3] = w[k][4] = 0u;
+            for (int i = 0; i < remaining; ++i) {
+                w[k][1 + (i >> 2)] |= static_cast<uint32_t>(static_cast<uint8_t>(x[t0 + i])) << (8 * (i & 3));
+            }
         }
     }
-    uint32_t o[4];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        uint32_t packed = 0;
+    for (int k = 0; k < PIECES; ++k) {
+        const int seg = seg0 + 64 * k;
+        const int t0 = seg * 16;
+        const int remaining = p.seqlen - t0;
+        if (seg >= segs) break;
+        uint32_t o[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            // window ending at element 4q+j: bytes (4q+j-3 .. 4q+j) of the stream starting at w[1]
-            const uint32_t win = j == 3 ? w[q + 1] : __builtin_amdgcn_alignbyte(w[q + 1], w[q], j + 1);
-            const float acc = static_cast<float>(dot4(win, taps));
-            const float v = __builtin_fmaf(s_wx, acc, bias_f);
-            const int r = conv_quant(v, p.scale_out, inv_s_out, SILU, exact_only, kq);
-            packed |= static_cast<uint32_t>(r & 0xff) << (8 * j);
+        for (int q = 0; q < 4; ++q) {
+            uint32_t packed = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                // window ending at element 4q+j: bytes (4q+j-3 .. 4q+j) of the stream starting at w[k][1]
+                const uint32_t win = j == 3 ? w[k][q + 1] : __builtin_amdgcn_alignbyte(w[k][q + 1], w[k][q], j + 1);
+                const float acc = static_cast<float>(dot4(win, taps));
+                const float v = __builtin_fmaf(s_wx, acc, bias_f);
+                const int r = conv_quant(v, p.scale_out, inv_s_out, SILU, exact_only, kq);
+                packed |= static_cast<uint32_t>(r & 0xff) << (8 * j);
+            }
+            o[q] = packed;
         }
-        o[q] = packed;
-    }
-    if (remaining >= 16) {
-        *reinterpret_cast<uint4*>(out + t0) = make_uint4(o[0], o[1], o[2], o[3]);
-    } else {
-        for (int i = 0; i < remaining; ++i) {
-            out[t0 + i] = static_cast<int8_t>((o[i >> 2] >> (8 * (i & 3))) & 0xff);
+        if (remaining >= 16) {
+            *reinterpret_cast<uint4*>(out + t0) = make_uint4(o[0], o[1], o[2], o[3]);
+        } else {
+            for (int i = 0; i < remaining; ++i) {
+                out[t0 + i] = static_cast<int8_t>((o[i >> 2] >> (8 * (i & 3))) & 0xff);
+            }
         }
     }
 }
@@ -254,9 +267,13 @@ extern "C" int qa_causal_conv1d_fwd(const QaConvParams* p, void* stream_) {
             const int segs = (p->seqlen + 15) / 16;
             const int64_t groups = (static_cast<int64_t>(p->dim) + 3) / 4;
             if (groups > 65535 || p->batch > 65535) return QA_ERR_SHAPE;
-            const dim3 grid(static_cast<unsigned>((segs + 63) / 64), static_cast<unsigned>(groups), static_cast<unsigned>(p->batch));
-            if (p->silu_activation) hipLaunchKernelGGL(conv_fwd_rows_kernel<true>, grid, dim3(kConvThreads), 0, stream, *p, segs);
-            else hipLaunchKernelGGL(conv_fwd_rows_kernel<false>, grid, dim3(kConvThreads), 0, stream, *p, segs);
+            // two segments per lane once a row has at least 128 of them (2048 steps)
+            const int pieces = segs >= 128 ? 2 : 1;
+            const dim3 grid(static_cast<unsigned>((segs + 64 * pieces - 1) / (64 * pieces)), static_cast<unsigned>(groups),
+                            static_cast<unsigned>(p->batch));
+            auto go = [&](auto kernel) { hipLaunchKernelGGL(kernel, grid, dim3(kConvThreads), 0, stream, *p, segs); };
+            if (pieces == 2) p->silu_activation ? go(conv_fwd_rows_kernel<true, 2>) : go(conv_fwd_rows_kernel<false, 2>);
+            else p->silu_activation ? go(conv_fwd_rows_kernel<true, 1>) : go(conv_fwd_rows_kernel<false, 1>);
             return check_launch();
         }
     }
