@@ -226,7 +226,9 @@ __device__ __forceinline__ void wave_lds_sync() {
 // n = i*32 + 8*(r/4) + 4*(l/32) + (r%4).
 // FLEX = false compiles the common rule only (d = cast_rne(s_row * (s_col * acc))); FLEX = true also
 // honours use_alpha and the round-half-away GEMV rule at run time.  TRANS selects the (N,M) output.
-template <int TM, int TN, int OUT, bool FLEX, bool TRANS>
+// COL_OUTER (the column scale applied last) is a compile-time choice: selecting the association per
+// element costs two extra instructions on each of the 128 outputs of a lane.
+template <int TM, int TN, int OUT, bool FLEX, bool TRANS, bool COL_OUTER = false>
 __device__ __forceinline__ void epilogue(const Epilogue& e, v16i (&acc)[TN][TM], uint8_t* lds, int m, int n,
                                          int wave_m0, int wave_n0, int wave, int lane) {
     constexpr int kElt = OUT == QA_OUT_I8 ? 1 : 2;
@@ -258,7 +260,7 @@ __device__ __forceinline__ void epilogue(const Epilogue& e, v16i (&acc)[TN][TM],
         float v;
         if (use_alpha) v = s_row[j] * accf;
         // GEMV rule (round-half-away mode): the two scales are multiplied first
-        else if (e.col_outer) v = s_col[i][q][t] * (s_row[j] * accf);
+        else if (COL_OUTER) v = s_col[i][q][t] * (s_row[j] * accf);
         else v = away ? (s_col[i][q][t] * s_row[j]) * accf : s_row[j] * (s_col[i][q][t] * accf);
         // keep the fp32 product a value of its own: folding the multiply into a mixed-precision
         // convert would round once instead of twice and change the fp16 result in rare cases

@@ -13,7 +13,7 @@ namespace {
 
 using namespace gemm;
 
-template <int TM, int TN, int WGM, int WGN, int STAGES, int OUT, bool FLEX>
+template <int TM, int TN, int WGM, int WGN, int STAGES, int OUT, bool FLEX, bool COL_OUTER>
 __global__ __launch_bounds__(64 * WGM * WGN) void gemm_w8a8_kernel(QaGemmW8A8Params p) {
     using C = Cfg<TM, TN, WGM, WGN, STAGES>;
     constexpr int BM = C::kBM, BN = C::kBN, WAVES = C::kWaves;
@@ -80,15 +80,18 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_w8a8_kernel(QaGemmW8A8Par
     e.row_numel = p.a_scale_numel; e.col_numel = p.w_scale_numel;
     e.use_alpha = p.use_alpha; e.alpha = p.alpha; e.round_mode = p.round_mode; e.col_outer = p.scale_order;
     e.ldd = p.ldd; e.d = p.d;
-    epilogue<TM, TN, OUT, FLEX, false>(e, acc, lds, p.m, p.n, m0 + wm * TM * 32, n0 + wn * TN * 32, wave, lane);
+    epilogue<TM, TN, OUT, FLEX, false, COL_OUTER>(e, acc, lds, p.m, p.n, m0 + wm * TM * 32, n0 + wn * TN * 32, wave, lane);
 }
 
-template <int TM, int TN, int WGM, int WGN, int STAGES, int OUT, bool FLEX>
+template <int TM, int TN, int WGM, int WGN, int STAGES, int OUT, bool FLEX, bool COL_OUTER = false>
 int launch_one(const QaGemmW8A8Params& p, hipStream_t stream) {
     using C = Cfg<TM, TN, WGM, WGN, STAGES>;
+    if constexpr (!FLEX && !COL_OUTER) {
+        if (p.scale_order == 1) return launch_one<TM, TN, WGM, WGN, STAGES, OUT, FLEX, true>(p, stream);
+    }
     const int64_t tiles = static_cast<int64_t>((p.m + C::kBM - 1) / C::kBM) * ((p.n + C::kBN - 1) / C::kBN);
     if (tiles > 0x7fffffffLL) return QA_ERR_SHAPE;
-    auto kernel = gemm_w8a8_kernel<TM, TN, WGM, WGN, STAGES, OUT, FLEX>;
+    auto kernel = gemm_w8a8_kernel<TM, TN, WGM, WGN, STAGES, OUT, FLEX, COL_OUTER>;
     if (C::kLdsBytes > 65536) {
         // allowing more than 64 KiB of dynamic LDS is a per-function attribute; setting it is idempotent
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -254,6 +257,7 @@ extern "C" int qa_gemm_w8a8(const QaGemmW8A8Params* p, void* stream_) {
     if (p->m < 0 || p->n < 0 || p->k < 0) return QA_ERR_SHAPE;
     if (p->out_type != QA_OUT_I8 && p->out_type != QA_OUT_F16) return QA_ERR_UNSUPPORTED;
     if (p->scale_order != 0 && p->scale_order != 1) return QA_ERR_UNSUPPORTED;
+    if (p->scale_order == 1 && (p->use_alpha || p->round_mode != QA_ROUND_RNE)) return QA_ERR_UNSUPPORTED;
     if (!p->use_alpha && p->a_scale_numel != 1 && p->a_scale_numel != p->m) return QA_ERR_SHAPE;
     if (!p->use_alpha && p->w_scale_numel != 1 && p->w_scale_numel != p->n) return QA_ERR_SHAPE;
     // 16-byte operand chunks: the same alignment the reference's tensor-core path demands
