@@ -240,15 +240,26 @@ __device__ __forceinline__ void epilogue(const Epilogue& e, v16i (&acc)[TN][TM],
 
     // this lane's column scales: 4 consecutive columns per (i, q), loaded once
     float s_col[TN][4][4];
+    if (use_alpha || e.col_numel == 1) {
+        // one scale for every column: a single (scalar) fetch instead of one per column and lane
+        const float one = use_alpha ? 1.0f : e.col_scale[0];
 #pragma unroll
-    for (int i = 0; i < TN; ++i)
+        for (int i = 0; i < TN; ++i)
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
+            for (int q = 0; q < 4; ++q)
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                const int nn = wave_n0 + i * 32 + 8 * q + 4 * fhalf + t;
-                s_col[i][q][t] = use_alpha ? 1.0f : e.col_scale[e.col_numel == 1 ? 0 : min(nn, n - 1)];
-            }
+                for (int t = 0; t < 4; ++t) s_col[i][q][t] = one;
+    } else {
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const int nn = wave_n0 + i * 32 + 8 * q + 4 * fhalf + t;
+                    s_col[i][q][t] = e.col_scale[min(nn, n - 1)];
+                }
+    }
     float s_row[TM];
 #pragma unroll
     for (int j = 0; j < TM; ++j) {
