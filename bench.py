@@ -419,6 +419,32 @@ def mfma_calibration(dev):
     return out
 
 
+def valu_calibration(dev):
+    """Issue time of plain and transcendental vector instructions: eight waves per SIMD on every CU, each lane with
+    eight independent chains of one instruction; ns per wave-instruction per SIMD and the clock during the loop."""
+    from quamba_amd import _lib
+    lib = _lib.lib()
+    wgs, iters = 2048, 20000
+    sink = torch.empty(wgs * 256, dtype=torch.float32, device=dev)
+    ticks = torch.zeros(2, dtype=torch.int64, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    simds = 4 * torch.cuda.get_device_properties(dev).multi_processor_count
+    out = {}
+    for name, op in (("v_mul_f32", 0), ("v_exp_f32", 1), ("v_rcp_f32", 2), ("v_log_f32", 3), ("v_fmac_f32", 4), ("v_mul_f32_dpp", 5)):
+        for _ in range(4):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            _lib.check(lib.qa_diag_valu(sink.data_ptr(), sink.numel(), ticks.data_ptr(), wgs, iters, op, stream), "diag")
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1)
+        t = ticks.tolist()
+        per_simd = wgs * 4.0 / simds * iters * 8
+        out[name] = {"ns_per_wave_instruction_per_simd": round(ms * 1e6 / per_simd, 3), "ms": round(ms, 3),
+                     "clock_MHz": round(100.0 * t[0] / max(t[1], 1), 1)}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -434,6 +460,8 @@ def main():
     ap.add_argument("--mfma-calibration", action="store_true",
                     help="also measure the int8 matrix rate the part sustains in a register-only loop, with constant and "
                          "with random operand bytes (extra key in the JSON line)")
+    ap.add_argument("--valu-calibration", action="store_true",
+                    help="also measure the issue time of plain and transcendental vector instructions (extra key in the JSON line)")
     ap.add_argument("--traffic-json", default=os.path.join(ROOT, "profiles", "traffic.json"),
                     help="HBM bytes per launch measured with rocprofv3 --pmc (written by hand from profiles/)")
     args = ap.parse_args()
@@ -507,6 +535,8 @@ def main():
         del src, dst
     if args.mfma_calibration:
         line["mfma_calibration"] = mfma_calibration(dev)
+    if args.valu_calibration:
+        line["valu_calibration"] = valu_calibration(dev)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(mixer)
     if args.other_workloads:

@@ -395,6 +395,13 @@ int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream);
 int qa_diag_mfma_i8(int* sink, int64_t sink_elems, long long* ticks, int workgroups, int iters,
                     int random_operands, void* stream);
 
+/* Diagnostic, no counterpart in the reference: `workgroups` x 256 threads each issue iters x 8 independent
+ * instructions of one kind (op 0: v_mul_f32, 1: v_exp_f32, 2: v_rcp_f32, 3: v_log_f32, 4: v_fmac_f32,
+ * 5: v_mul_f32 with a quad-broadcast DPP operand); `sink` and `ticks` as
+ * above.  Used by bench.py to report the issue rate of plain and transcendental vector instructions, which
+ * bounds the selective scan. */
+int qa_diag_valu(float* sink, int64_t sink_elems, long long* ticks, int workgroups, int iters, int op, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

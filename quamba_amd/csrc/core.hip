@@ -67,8 +67,51 @@ __global__ __launch_bounds__(256) void diag_mfma_i8_kernel(int* sink, long long*
         ticks[1] = wall_clock64() - w0;
     }
 }
+// op 0: v_mul_f32, 1: v_exp_f32, 2: v_rcp_f32, 3: v_log_f32, 4: v_fmac_f32, 5: v_mul_f32 with a quad broadcast (DPP);
+// eight chains per lane
+template <int OP>
+__global__ __launch_bounds__(256) void diag_valu_kernel(float* sink, long long* ticks, int iters) {
+    const unsigned t = blockIdx.x * 256 + threadIdx.x;
+    float v[8];
+    for (int i = 0; i < 8; ++i) v[i] = 0.001f * static_cast<float>((t & 255u) + i + 1);
+    const long long c0 = clock64(), w0 = wall_clock64();
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            if (OP == 0) asm volatile("v_mul_f32 %0, 0.5, %0" : "+v"(v[i]));
+            else if (OP == 1) asm volatile("v_exp_f32 %0, %0" : "+v"(v[i]));
+            else if (OP == 2) asm volatile("v_rcp_f32 %0, %0" : "+v"(v[i]));
+            else if (OP == 3) asm volatile("v_log_f32 %0, %0" : "+v"(v[i]));
+            else if (OP == 4) asm volatile("v_fmac_f32 %0, %1, %1" : "+v"(v[i]) : "v"(v[(i + 1) & 7]));
+            else asm volatile("v_mul_f32_dpp %0, %0, %1 quad_perm:[0,0,0,0] row_mask:0xf bank_mask:0xf bound_ctrl:1" : "+v"(v[i]) : "v"(v[(i + 1) & 7]));
+        }
+    }
+    float s = 0.0f;
+    for (int i = 0; i < 8; ++i) s += v[i];
+    sink[t] = s;
+    if (t == 0 && ticks) {
+        ticks[0] = clock64() - c0;
+        ticks[1] = wall_clock64() - w0;
+    }
+}
 }  // namespace
 }  // namespace qa
+
+extern "C" int qa_diag_valu(float* sink, int64_t sink_elems, long long* ticks, int workgroups, int iters, int op,
+                            void* stream) {
+    if (!sink) return QA_ERR_NULL;
+    if (workgroups < 1 || iters < 0 || sink_elems < static_cast<int64_t>(workgroups) * 256) return QA_ERR_SHAPE;
+    if (op < 0 || op > 5) return QA_ERR_UNSUPPORTED;
+    const dim3 grid(static_cast<unsigned>(workgroups)), block(256);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (op == 0) hipLaunchKernelGGL(qa::diag_valu_kernel<0>, grid, block, 0, st, sink, ticks, iters);
+    else if (op == 1) hipLaunchKernelGGL(qa::diag_valu_kernel<1>, grid, block, 0, st, sink, ticks, iters);
+    else if (op == 2) hipLaunchKernelGGL(qa::diag_valu_kernel<2>, grid, block, 0, st, sink, ticks, iters);
+    else if (op == 3) hipLaunchKernelGGL(qa::diag_valu_kernel<3>, grid, block, 0, st, sink, ticks, iters);
+    else if (op == 4) hipLaunchKernelGGL(qa::diag_valu_kernel<4>, grid, block, 0, st, sink, ticks, iters);
+    else hipLaunchKernelGGL(qa::diag_valu_kernel<5>, grid, block, 0, st, sink, ticks, iters);
+    return qa::check_launch();
+}
 
 extern "C" int qa_diag_mfma_i8(int* sink, int64_t sink_elems, long long* ticks, int workgroups, int iters,
                                int random_operands, void* stream) {
