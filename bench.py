@@ -391,6 +391,29 @@ def other_workloads(dev, steps, warmup):
     out.append(dict(workload="Mamba2-8b W4A8 mixer forward over a prompt (in_proj, conv, SSD scan, norm + Hadamard, out_proj), 16 x 1024 tokens",
                     us=ms * 1e3, tokens_per_s=16384 / ms * 1e3, bound="mfma", achieved_TOPs=gemm_ops / ms / 1e9,
                     frac=gemm_ops / ms / 1e9 / INT8_PEAK_TOPS))
+    del u2
+    # the same module for one token (W4A8QMamba2.step: in_proj, xBC conv update, state update, norm + Hadamard,
+    # out_proj), captured eight times into one HIP graph; bytes = the packed weights + the fp32 state, read and written
+    w_bytes = sum(l.weight.numel() + l.s_group.numel() * 2 for l in (m2.in_proj, m2.out_proj))
+    for B in (1, 64):
+        caches = [m2.allocate_inference_cache(B) for _ in range(8)]
+        h1 = ri(B, 1, 4096)
+
+        def token2():
+            for cs, ss in caches:
+                m2.step(h1, cs, ss)
+        for _ in range(3):
+            token2()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            token2()
+        ms = _time_fn(graph.replay, 64, 4) / len(caches)
+        nbytes = w_bytes + B * (2 * m2.nheads * m2.headdim * m2.d_state * 4 + 4096 + 2 * 4096)
+        out.append(dict(workload=f"Mamba2-8b W4A8 mixer, one token (five kernels), batch {B}, HIP graph of 8 steps on one layer's weights",
+                        us=ms * 1e3, tokens_per_s=B / ms * 1e3, bound="hbm", achieved_GBs=nbytes / ms / 1e6,
+                        frac=nbytes / ms / 1e6 / HBM_PEAK_GBS))
+        del graph, caches
     return out
 
 

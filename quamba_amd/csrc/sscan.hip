@@ -512,8 +512,15 @@ __global__ __launch_bounds__(256) void ssm_update_kernel(QaSsmUpdateParams p) {
         const int n0 = (sub + k * LPR) * 4;
         if (n0 >= p.dstate) continue;
         if constexpr (VEC) {
-            // dstate is a multiple of four here, so the piece is whole
-            *reinterpret_cast<int32_t*>(a8[k]) = *reinterpret_cast<const int32_t*>(Ap + n0);
+            // dstate is a multiple of four here, so the piece is whole.  A_log alone may be a broadcast view
+            // (one value per head, stride 0 along the states, as Mamba2 passes it): it is read through its
+            // stride, the state and B, C with one load per piece
+            if (p.A_dstate_stride == 1 && (reinterpret_cast<uintptr_t>(Ap + n0) & 3u) == 0) {
+                *reinterpret_cast<int32_t*>(a8[k]) = *reinterpret_cast<const int32_t*>(Ap + n0);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) a8[k][e] = Ap[(n0 + e) * p.A_dstate_stride];
+            }
             *reinterpret_cast<int32_t*>(b8v[k]) = *reinterpret_cast<const int32_t*>(Bp + n0);
             *reinterpret_cast<int32_t*>(c8[k]) = *reinterpret_cast<const int32_t*>(Cp + n0);
             if constexpr (FP32) {
@@ -599,12 +606,11 @@ int launch_update(const QaSsmUpdateParams& p, hipStream_t stream) {
     const int64_t st_align = p.state_is_fp32 ? 16 : 4;      // bytes of one lane's four states
     const int64_t st_el = p.state_is_fp32 ? 4 : 1;
     auto mult = [](int64_t v, int64_t m) { return v % m == 0; };
-    const bool vec = p.dstate % 4 == 0 && p.state_dstate_stride == 1 && p.A_dstate_stride == 1 &&
+    const bool vec = p.dstate % 4 == 0 && p.state_dstate_stride == 1 &&
                      p.B_dstate_stride == 1 && p.C_dstate_stride == 1 &&
                      reinterpret_cast<uintptr_t>(p.state) % st_align == 0 &&
                      mult(p.state_batch_stride * st_el, st_align) && mult(p.state_head_stride * st_el, st_align) &&
                      mult(p.state_dim_stride * st_el, st_align) &&
-                     aligned4(p.A_log) && mult(p.A_head_stride, 4) && mult(p.A_dim_stride, 4) &&
                      aligned4(p.B) && mult(p.B_batch_stride, 4) && mult(p.B_group_stride, 4) &&
                      aligned4(p.C) && mult(p.C_batch_stride, 4) && mult(p.C_group_stride, 4);
     auto go = [&](auto kernel) { hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, p); };
