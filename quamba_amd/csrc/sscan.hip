@@ -673,6 +673,16 @@ extern "C" int qa_sscan_fwd(const QaSScanParams* p, void* stream_) {
             const int64_t simds = 4LL * cus;
             const int64_t waves_a = static_cast<int64_t>(p->batch) * p->dim / 16;
             const int64_t q = waves_a / simds, rem_waves = waves_a % simds;
+            // Few waves (small batches): a launch takes about as long as the busiest SIMD's waves one after the
+            // other, and with so few of them latency, not issue, sets a wave's pace - so twice as many waves
+            // of two thirds the length (eight lanes per channel) finish sooner.  Measured at 5120 channels x
+            // 2048 steps, by waves per SIMD (eight-lane kind: 1: 228, 2: 255, 3: 309, 4: 378, 5: 456 us;
+            // four-lane kind: 1: 284, 2: 358, 3: 455 us): the eight-lane kind wins up to 1.5 four-lane waves
+            // per SIMD.
+            if (waves == 4 && 2 * waves_a <= 3 * simds && p->dim % 32 == 0 &&
+                (p->n_groups <= 1 || (p->dim / p->n_groups) % 32 == 0)) {
+                return launch_fwd<2, 8, 64, 4>(*p, stream, vec_in, vec_bc, vec_out);
+            }
             if (waves == 4 && p->n_groups == 1 && q >= 1 && rem_waves > 0 && 2 * rem_waves <= simds) {
                 const int64_t short_channels = rem_waves * 16 / p->batch;      // channels per batch entry for the short kind
                 const int blocks_a = static_cast<int>((p->dim - short_channels) / 64);
