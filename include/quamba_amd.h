@@ -222,6 +222,21 @@ typedef struct QaSScanParams {
     void* out;                     /* fp16 */
     int8_t* last_state_i8;         /* int8 (batch, dim, dstate) contiguous, or null */
     float* last_state_f32;         /* fp32 (batch, dim, dstate) contiguous, or null */
+    /* Optional (all null / 0 otherwise): one long sequence scanned as several segments side by side - no
+     * counterpart in the reference, whose kernel splits the sequence inside a thread block instead
+     * (csrc/selective_scan/quant_sscan_fwd_kernel.cuh, BlockScan over (a, b) pairs).
+     * dt_sum_out: fp32 (batch, dim), receives the sum over the steps of each channel's step size after bias
+     *   and softplus; the decay of the whole run of steps is exp(A * that).
+     * carry_dt_sum fp32 (n, dim), carry_state fp32 (n, dim, dstate), carry_first: the batch entries are
+     *   segments carry_first, carry_first + 1, ... of one sequence; carry_* hold, for the segments before
+     *   them, the step-size sums and the end states of a scan from a zero state.  Entry b starts from
+     *   the state obtained by chaining segments 0 .. carry_first + b - 1:
+     *   h <- exp(A * carry_dt_sum[s]) * h + carry_state[s]. */
+    float* dt_sum_out;
+    const float* carry_dt_sum;
+    const float* carry_state;
+    int32_t carry_first;
+    int32_t reserved1;
 } QaSScanParams;
 
 int qa_sscan_fwd(const QaSScanParams* p, void* stream);

@@ -148,6 +148,22 @@ __device__ __forceinline__ void sscan_fwd_body(const QaSScanParams& p, int vec_i
                     ? -expf(s_A * static_cast<float>(p.A_log[cc * p.A_d_stride + n * p.A_dstate_stride])) * kLog2e
                     : 0.0f;
     }
+    // Segments of one sequence scanned in parallel: this batch entry is segment carry_first + b and starts from
+    // the state that the earlier segments (scanned from a zero state) chain up to:
+    // h <- exp(A * (sum of the segment's step sizes)) h + (the segment's own end state)
+    if (p.carry_state) {
+        const int seg = p.carry_first + b;
+        for (int sp = 0; sp < seg; ++sp) {
+            const float sd = p.carry_dt_sum[static_cast<int64_t>(sp) * p.dim + cc];
+#pragma unroll
+            for (int j = 0; j < NPL; ++j) {
+                const int n = min(slice * NPL + j, p.dstate - 1);
+                h[j] = __builtin_fmaf(fast_exp2(sd * A2[j]), h[j],
+                                      p.carry_state[(static_cast<int64_t>(sp) * p.dim + cc) * p.dstate + n]);
+            }
+        }
+    }
+    float dt_sum = 0.0f;                 // of the steps this lane evaluates the step size for
 
     const int8_t* in_base[3] = {p.u + b * p.u_batch_stride, p.delta + b * p.delta_batch_stride,
                                 has_z ? p.z + b * p.z_batch_stride : nullptr};
@@ -254,6 +270,7 @@ __device__ __forceinline__ void sscan_fwd_body(const QaSScanParams& p, int vec_i
                     // steps past the end of the sequence must leave the state alone: a = 1, b = 0
                     dt = tq * 4 + j < nt ? dt : 0.0f;
                     own_dt[o] = dt;
+                    dt_sum += dt;
                     own_du[o] = dt * own_u[o];
                 }
                 float acc[4];
@@ -328,6 +345,7 @@ __device__ __forceinline__ void sscan_fwd_body(const QaSScanParams& p, int vec_i
                     const float u_val = s_u * i8_of(u4, j);
                     float dt = __builtin_fmaf(s_dt, i8_of(d4, j), db);
                     if (p.delta_softplus) dt = softplus20(dt);
+                    dt_sum += dt;
                     const float du = dt * u_val;
                     const float4* bf = reinterpret_cast<const float4*>(&s_bc[t][0][slice * NPL]);
                     const float4* cf = reinterpret_cast<const float4*>(&s_bc[t][1][slice * NPL]);
@@ -377,6 +395,14 @@ __device__ __forceinline__ void sscan_fwd_body(const QaSScanParams& p, int vec_i
         __syncthreads();
     }
 
+    if (p.dt_sum_out) {
+        // shared-out steps: the lanes of a quad hold the sums of different steps
+        if constexpr (NSPLIT <= 4 || (NSPLIT == 8 && NPL == 2)) {
+            if constexpr (QS >= 2) dt_sum += quad_xor<1>(dt_sum);
+            if constexpr (QS == 4) dt_sum += quad_xor<2>(dt_sum);
+        }
+        if (c_ok && slice == 0) p.dt_sum_out[static_cast<int64_t>(b) * p.dim + c] = dt_sum;
+    }
     if (c_ok) {
         const int64_t base = (static_cast<int64_t>(b) * p.dim + c) * p.dstate;
         const float s_state = p.last_state_i8 ? *p.scale_ssm_state : 1.0f;

@@ -414,10 +414,58 @@ def sscan_fwd(u, scale_u, delta, scale_delta, A, scale_A, B, scale_B, C, scale_C
     p.u, p.delta, p.A_log, p.B, p.C, p.out = ptr(u), ptr(delta), ptr(A), ptr(B), ptr(C), ptr(out)
     p.scale_u, p.scale_delta, p.scale_A = ptr(scale_u), ptr(scale_delta), ptr(scale_A)
     p.scale_B, p.scale_C = ptr(scale_B), ptr(scale_C)
+    segments = _sscan_segments(batch, dim, seqlen)
     with torch.cuda.device(u.device):
-        st = _lib.lib().qa_sscan_fwd(ct.byref(p), _lib.current_stream(u.device))
+        stream = _lib.current_stream(u.device)
+        if segments <= 1:
+            st = _lib.lib().qa_sscan_fwd(ct.byref(p), stream)
+        else:
+            # One sequence alone leaves most of the chip idle (a wave walks all of its steps), so it is scanned as
+            # `segments` pieces side by side: every piece from a zero state, which also yields each piece's end
+            # state and the sum of its step sizes; then the pieces after the first once more, each from the state
+            # its predecessors chain up to.  Twice the arithmetic on `segments` times the waves.
+            seg = seqlen // segments
+            local = torch.empty((segments, dim, dstate), dtype=torch.float32, device=u.device)
+            dt_sum = torch.empty((segments, dim), dtype=torch.float32, device=u.device)
+            p1 = _lib.QaSScanParams.from_buffer_copy(p)
+            p1.batch, p1.seqlen = segments, seg
+            p1.u_batch_stride = p1.delta_batch_stride = p1.z_batch_stride = seg
+            p1.B_batch_stride = p1.C_batch_stride = seg
+            p1.out_batch_stride = seg * out.stride(1)
+            p1.last_state_i8, p1.last_state_f32, p1.dt_sum_out = None, ptr(local), ptr(dt_sum)
+            st = _lib.lib().qa_sscan_fwd(ct.byref(p1), stream)
+            if st == 0:
+                tail = torch.empty((segments - 1, dim, dstate), dtype=state_dtype, device=u.device)
+                p2 = _lib.QaSScanParams.from_buffer_copy(p1)
+                p2.batch = segments - 1
+                p2.u, p2.delta = u.data_ptr() + seg, delta.data_ptr() + seg
+                p2.B, p2.C = B.data_ptr() + seg, C.data_ptr() + seg
+                if z is not None:
+                    p2.z = z.data_ptr() + seg
+                p2.out = out.data_ptr() + seg * out.stride(1) * 2
+                p2.dt_sum_out, p2.carry_dt_sum, p2.carry_state, p2.carry_first = None, ptr(dt_sum), ptr(local), 1
+                if state_dtype == torch.int8:
+                    p2.last_state_i8, p2.last_state_f32 = ptr(tail), None
+                else:
+                    p2.last_state_i8, p2.last_state_f32 = None, ptr(tail)
+                st = _lib.lib().qa_sscan_fwd(ct.byref(p2), stream)
+                x = tail[-1].reshape(1, dim, 1, dstate)
     _lib.check(st, "sscan_fwd")
     return out, x
+
+
+# A single sequence of at least this many steps is scanned in segments (see sscan_fwd); 0 disables it.
+SSCAN_SEGMENT_MIN_STEPS = 1024
+
+
+def _sscan_segments(batch, dim, seqlen):
+    if batch != 1 or not SSCAN_SEGMENT_MIN_STEPS or seqlen < SSCAN_SEGMENT_MIN_STEPS:
+        return 1
+    for segments in (8, 4, 2):
+        # equal pieces whose rows keep the 16-byte alignment of the whole, at least 128 steps each
+        if seqlen % (segments * 16) == 0 and seqlen // segments >= 128:
+            return segments
+    return 1
 
 
 

@@ -65,6 +65,34 @@ def test_fwd_matches_oracle(dev, B, L, D, N):
     assert diff.max() <= 1 and (diff != 0).mean() < 0.02
 
 
+# (seqlen, dim, dstate, variant): a single sequence is scanned as 8, 8, 4 or 2 segments side by side, each segment
+# a second time from the state its predecessors chain up to; with every lane mapping that can meet it
+@pytest.mark.parametrize("L,D,N,variant", [(2048, 256, 16, None), (1536, 96, 16, "4x4"), (1024, 200, 16, "8x4"),
+                                           (1024, 64, 16, "2x2"), (1056, 40, 32, None), (1024, 24, 64, None),
+                                           (2048, 5120, 16, None)])
+def test_one_sequence_scanned_in_segments(dev, L, D, N, variant, monkeypatch):
+    if variant:
+        monkeypatch.setenv("QA_SSCAN_VARIANT", variant)
+    assert ops._sscan_segments(1, D, L) > 1
+    d = synth.mamba1_scan_inputs(1, L, D, N, seed=L + D + 1)
+    y_ref, _, st32_ref = _oracle(d, s_state=1.0)
+    s_state = max(float(np.abs(st32_ref).max()), 1e-5) / 127.0
+    _, st8_ref, _ = _oracle(d, s_state=s_state)
+    y, x32 = _gpu(d, dev, s_state, torch.float32)
+    assert y.shape == (1, L, D) and x32.shape == (1, D, 1, N)
+    _check(y, y_ref)
+    assert np.abs(x32[:, :, 0].cpu().numpy() - st32_ref).max() <= STATE_REL * np.abs(st32_ref).max()
+    y8, x8 = _gpu(d, dev, s_state, torch.int8)
+    assert torch.equal(y, y8) and x8.shape == (1, D, 1, N) and x8.dtype == torch.int8
+    diff = np.abs(x8[:, :, 0].cpu().numpy().astype(int) - st8_ref.astype(int))
+    assert diff.max() <= 1 and (diff != 0).mean() < 0.02
+    # and against the same kernel walking the sequence in one piece
+    monkeypatch.setattr(ops, "SSCAN_SEGMENT_MIN_STEPS", 0)
+    y1, x1 = _gpu(d, dev, s_state, torch.float32)
+    np.testing.assert_allclose(y.float().cpu().numpy(), y1.float().cpu().numpy(), rtol=2e-3, atol=2e-3)
+    assert (x32 - x1).abs().max().item() <= 1e-4 * x1.abs().max().item()
+
+
 # "<lanes per channel>x<waves>"; "8x4" is the eight-lane mapping, "0x<n>" the mixed launch (n workgroups of 64
 # channels with four lanes per channel, the remaining channels with eight)
 @pytest.mark.parametrize("variant", ["1x1", "2x1", "2x2", "4x1", "4x2", "4x4", "8x4", "0x1", "0x2"])
