@@ -351,8 +351,8 @@ typedef struct QaGemmW4A8Params {
     /* Optional scratch of n*k bytes (16-byte aligned), or null.  With many activation rows every 256-row
      * band of the output expands the same 4-bit weights again; given this buffer (and more than 64 rows)
      * the weights are expanded once (same arithmetic, same int8 values) and the int8 x int8 kernel runs on
-     * the result, for the (N,M) output with the roles of the operands exchanged.  It pays from about 4e11 operations (2*m*n*k) on; whether to pass
-     * it is the caller's choice.  Results are bit-identical either way. */
+     * the result, for the (N,M) output with the roles of the operands exchanged.  It pays from about 1000
+     * activation rows on; whether to pass it is the caller's choice.  Results are bit-identical either way. */
     void* w8_workspace;
     int64_t w8_workspace_bytes;
 } QaGemmW4A8Params;

@@ -168,12 +168,12 @@ def test_expanding_the_weights_once_gives_the_same_bits(dev, monkeypatch, groupe
     M, N, K = 300, 520, 512
     a, codes, sg, sc, st = _case(M, N, K, seed=9, grouped=grouped)
     fused = _run(dev, a, codes, sg, sc, st, out8)
-    monkeypatch.setattr(ops, "W4A8_EXPAND_ONCE_OPS", 0.0)
+    monkeypatch.setattr(ops, "W4A8_EXPAND_ONCE_ROWS", 0)
     once = _run(dev, a, codes, sg, sc, st, out8)
     assert torch.equal(fused, once)
     per_tensor = _run(dev, a, codes, sg, sc, st, out8, per_token=False)
     once_t = _run(dev, a, codes, sg, sc, st, out8, transpose=True)         # (N, M): the operands' roles exchanged
     assert once_t.shape == (N, M) and torch.equal(once_t.t(), once)
-    monkeypatch.setattr(ops, "W4A8_EXPAND_ONCE_OPS", 1e30)
+    monkeypatch.setattr(ops, "W4A8_EXPAND_ONCE_ROWS", 1 << 30)
     assert torch.equal(per_tensor, _run(dev, a, codes, sg, sc, st, out8, per_token=False))
     assert torch.equal(once_t, _run(dev, a, codes, sg, sc, st, out8, transpose=True))
