@@ -255,7 +255,7 @@ __device__ __forceinline__ void sscan_fwd_body(const QaSScanParams& p, int vec_i
         for (int tq = 0; tq < n_quads; ++tq) {
             const uint32_t u4 = su[tq], d4 = sd[tq];
             const uint32_t z4 = has_z ? sz[tq] : 0u;
-            if constexpr (NSPLIT <= 4 || (NSPLIT == 8 && NPL == 2)) {
+            if constexpr (NSPLIT <= 4 || NSPLIT == 8) {
                 // The per-step work that does not depend on the state index (dequantise, softplus,
                 // gate) is shared out: of the 4 steps in this dword, the lane with slice s does
                 // steps o*NSPLIT + s and the others read its results through quad DPP.
@@ -397,7 +397,7 @@ __device__ __forceinline__ void sscan_fwd_body(const QaSScanParams& p, int vec_i
 
     if (p.dt_sum_out) {
         // shared-out steps: the lanes of a quad hold the sums of different steps
-        if constexpr (NSPLIT <= 4 || (NSPLIT == 8 && NPL == 2)) {
+        if constexpr (NSPLIT <= 4 || NSPLIT == 8) {
             if constexpr (QS >= 2) dt_sum += quad_xor<1>(dt_sum);
             if constexpr (QS == 4) dt_sum += quad_xor<2>(dt_sum);
         }
@@ -727,9 +727,25 @@ extern "C" int qa_sscan_fwd(const QaSScanParams* p, void* stream_) {
         if (nsplit == 0 && waves > 0) return launch_fwd_mixed(*p, stream, vec_in, vec_bc, vec_out, waves);
         return QA_ERR_UNSUPPORTED;
     }
-    if (N <= 32) return launch_fwd<8, 4, 64, 1>(*p, stream, vec_in, vec_bc, vec_out);
-    if (N <= 64) return launch_fwd<8, 8, 32, 1>(*p, stream, vec_in, vec_bc, vec_out);
-    if (N <= 128) return launch_fwd<8, 16, 16, 1>(*p, stream, vec_in, vec_bc, vec_out);
+    // Wider states: eight states per lane, or sixteen.  A workgroup converts its B/C tile once for all of its
+    // channels, so with enough channels to fill the part four waves share one tile (64 or 32 channels per
+    // workgroup); few channels keep one wave per workgroup, which gives more workgroups.
+    auto many = [&](int channels_per_wg) {
+        const int64_t wgs = static_cast<int64_t>(p->batch) * ((p->dim + channels_per_wg - 1) / channels_per_wg);
+        return wgs >= 128 && (p->n_groups <= 1 || (p->dim / p->n_groups) % channels_per_wg == 0);
+    };
+    if (N <= 32) {
+        if (many(64)) return launch_fwd<8, 4, 64, 4>(*p, stream, vec_in, vec_bc, vec_out);
+        return launch_fwd<8, 4, 64, 1>(*p, stream, vec_in, vec_bc, vec_out);
+    }
+    if (N <= 64) {
+        if (many(32)) return launch_fwd<8, 8, 32, 4>(*p, stream, vec_in, vec_bc, vec_out);
+        return launch_fwd<8, 8, 32, 1>(*p, stream, vec_in, vec_bc, vec_out);
+    }
+    if (N <= 128) {
+        if (many(32)) return launch_fwd<16, 8, 32, 4>(*p, stream, vec_in, vec_bc, vec_out);
+        return launch_fwd<8, 16, 16, 1>(*p, stream, vec_in, vec_bc, vec_out);
+    }
     return launch_fwd<16, 16, 16, 1>(*p, stream, vec_in, vec_bc, vec_out);
 }
 

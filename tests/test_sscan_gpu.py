@@ -43,9 +43,13 @@ def _check(y_gpu, y_ref):
     assert r2 < 1e-5
 
 
-# (batch, seqlen, dim, dstate): 130m/2.8b-shaped rows, ragged lengths, channel tails, wide states
+# (batch, seqlen, dim, dstate): 130m/2.8b-shaped rows, ragged lengths, channel tails, wide states, and the
+# 128-state rows of the reference's own list (test_qsscan.py:51-54: dims 5120 and 8192, here with fewer steps)
 SHAPES = [(1, 512, 1536, 16), (2, 33, 1536, 16), (2, 89, 100, 16), (1, 1, 64, 16), (2, 2048 + 7, 96, 16),
-          (2, 130, 72, 8), (1, 200, 40, 32), (1, 100, 24, 64), (1, 70, 8, 128), (1, 40, 6, 256)]
+          (2, 130, 72, 8), (1, 200, 40, 32), (1, 100, 24, 64), (1, 70, 8, 128), (1, 40, 6, 256),
+          (4, 96, 5120, 128), (4, 40, 8192, 128),
+          # wide states with many channels (four waves share a B/C tile): ragged channel tails, a padded state count
+          (2, 70, 4170, 32), (2, 50, 2100, 64), (3, 33, 1400, 100)]
 
 
 @pytest.mark.parametrize("B,L,D,N", SHAPES)
@@ -139,7 +143,8 @@ def test_fwd_unaligned_rows(dev):
 
 
 @pytest.mark.parametrize("B,D,N,fp32_state", [(1, 1536, 16, False), (64, 5120, 16, True), (3, 100, 16, False),
-                                              (2, 64, 128, True), (2, 30, 8, False)])
+                                              (2, 64, 128, True), (2, 30, 8, False),
+                                              (4, 5120, 128, False), (4, 8192, 128, True)])
 def test_update_matches_oracle_over_several_steps(dev, B, D, N, fp32_state):
     steps = 5
     d = synth.mamba1_scan_inputs(B, steps, D, N, seed=D + N)
