@@ -723,6 +723,13 @@ def ssd_chunk_scan_combined_fwd(q_x, x_scale, q_dt, dt_scale, q_A_log, A_log_sca
         keep.append(t)
         return ptr(t)
 
+    # The kernels are built for 64 and 128 states.  Fewer (the reference's tests use 16) run as the next of
+    # the two with zero codes in the added B and C columns: those states stay zero and add exactly nothing.
+    dstate_given = dstate
+    if dstate not in (64, 128) and dstate < 128:
+        dstate = 64 if dstate < 64 else 128
+        q_B = torch.nn.functional.pad(q_B, (0, dstate - dstate_given))
+        q_C = torch.nn.functional.pad(q_C, (0, dstate - dstate_given))
     q_x, q_B, q_C, q_dt = q_x.contiguous(), q_B.contiguous(), q_C.contiguous(), q_dt.contiguous()
     p = _lib.QaSsdParams()
     p.batch, p.seqlen, p.nheads, p.headdim, p.dstate, p.ngroups = batch, seqlen, nheads, headdim, dstate, ngroups
@@ -771,6 +778,8 @@ def ssd_chunk_scan_combined_fwd(q_x, x_scale, q_dt, dt_scale, q_A_log, A_log_sca
     with torch.cuda.device(dev):
         st = lib.qa_ssd_chunk_scan_fwd(ct.byref(p), _lib.current_stream(dev))
     _lib.check(st, "ssd_chunk_scan_fwd")
+    if dstate != dstate_given:
+        final = final[..., :dstate_given].contiguous()
     if return_workspace:
         return out, final, ws
     return out, final
