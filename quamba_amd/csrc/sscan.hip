@@ -744,7 +744,7 @@ extern "C" int qa_sscan_fwd(const QaSScanParams* p, void* stream_) {
     }
     if (N <= 128) {
         if (many(32)) return launch_fwd<16, 8, 32, 4>(*p, stream, vec_in, vec_bc, vec_out);
-        return launch_fwd<8, 16, 16, 1>(*p, stream, vec_in, vec_bc, vec_out);
+        return launch_fwd<16, 8, 32, 1>(*p, stream, vec_in, vec_bc, vec_out);
     }
     return launch_fwd<16, 16, 16, 1>(*p, stream, vec_in, vec_bc, vec_out);
 }
