@@ -73,7 +73,9 @@ def test_fwd_matches_oracle(dev, B, L, D, N):
 # a second time from the state its predecessors chain up to; with every lane mapping that can meet it
 @pytest.mark.parametrize("L,D,N,variant", [(2048, 256, 16, None), (1536, 96, 16, "4x4"), (1024, 200, 16, "8x4"),
                                            (1024, 64, 16, "2x2"), (1056, 40, 32, None), (1024, 24, 64, None),
-                                           (2048, 5120, 16, None)])
+                                           (2048, 5120, 16, None),
+                                           # wide states: four waves per workgroup (128 workgroups and more) and one
+                                           (1024, 512, 128, None), (1024, 544, 64, None), (1024, 100, 100, None)])
 def test_one_sequence_scanned_in_segments(dev, L, D, N, variant, monkeypatch):
     if variant:
         monkeypatch.setenv("QA_SSCAN_VARIANT", variant)
