@@ -285,7 +285,10 @@ extern "C" int qa_gemm_w8a8(const QaGemmW8A8Params* p, void* stream_) {
             const int64_t tiles = ((p->m + bm - 1) / bm) * ((p->n + bn - 1) / bn);
             return ((tiles + cus - 1) / cus) * bm * bn;
         };
-        if (cost(256, 320) < cost(256, 256)) return launch_gemm<2, 5, 4, 2, 2, false>(*p, stream);
+        const int64_t c_sq = cost(256, 256), c_wide = cost(256, 320), c_tall = cost(320, 256);
+        if (c_wide < c_sq && c_wide <= c_tall) return launch_gemm<2, 5, 4, 2, 2, false>(*p, stream);
+        // at equal arithmetic the larger tile has fewer rounds, each with its own start and epilogue
+        if (c_tall <= c_sq) return launch_gemm<5, 2, 2, 4, 2, false>(*p, stream);
         return launch_gemm<4, 2, 2, 4, 2, false>(*p, stream);                        // 256x256 tile, 8 waves
     }
     // 128x128 tile, 4 waves.  Two stages (64 KB) let two workgroups share a CU; when there is at most one
