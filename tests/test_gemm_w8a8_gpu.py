@@ -31,7 +31,9 @@ SHAPES = [(256, 256, 128), (128, 128, 64), (300, 200, 208), (1, 48, 64), (17, 33
           # a K that ends inside a 32-byte step, fewer K tiles than waves
           (33, 100, 5120), (5, 200, 2064), (64, 5120, 160), (1, 2560, 5120), (32, 10240, 2560), (65, 96, 4096),
           # few 128x128 tiles and a long K: the four-stage form of the small tile, K ending inside a tile
-          (130, 136, 1104), (1000, 192, 5120)]
+          (130, 136, 1104), (1000, 192, 5120),
+          # one round of 320x256 tiles where 256x256 tiles would need two: whole tiles, and ragged in both directions
+          (2560, 8192, 64), (2400, 8100, 80)]
 
 
 @pytest.mark.parametrize("M,N,K", SHAPES)
