@@ -236,8 +236,15 @@ typedef struct QaSScanParams {
     const float* carry_dt_sum;
     const float* carry_state;
     int32_t carry_first;
-    int32_t reserved1;
+    /* 0: the library picks how lanes are laid over channels and states.  Tests name a mapping to cover every
+     * kernel variant on one shape: QA_SSCAN_MAPPING(lanes per channel, waves per workgroup) for d_state <= 16
+     * (lanes 1, 2, 4, 8); lanes == 0 is the launch with two kinds of workgroup, the second argument then being
+     * the number of 64-channel workgroups per batch entry that take four lanes per channel.  A mapping the
+     * shape does not admit returns QA_ERR_SHAPE or QA_ERR_UNSUPPORTED.  Results agree to fp32 rounding. */
+    int32_t mapping;
 } QaSScanParams;
+
+#define QA_SSCAN_MAPPING(lanes, arg) (0x10000 | ((lanes) << 8) | (arg))
 
 int qa_sscan_fwd(const QaSScanParams* p, void* stream);
 

@@ -223,6 +223,50 @@ def sscan_update(state, x, dt, A_log, B, C_, D=None, dt_bias=None, z=None, *, s_
     return y, state
 
 
+def ssm_update_heads(state, x, dt, A_log, B, C_, D=None, dt_bias=None, z=None, *, x_scale, s_dt, s_A, s_B, s_C,
+                     s_D=0.0, s_z=0.0, state_scale=1.0, head_range=None, dim_range=None, softplus=True):
+    """One recurrence step in the layout with heads (Mamba2, and Mamba1 as one head).
+    state int8 or float32 (B,H,P,N) (not modified; the new state is returned); x, z int8 (B,H,P);
+    dt int8 broadcastable to (B,H,P); A_log int8 broadcastable to (H,P,N); B, C int8 (B,G,N); D int8
+    broadcastable to (H,P); dt_bias float broadcastable to (H,P), holding the value that is added to dt.
+    Without head_range / dim_range: x_scale, s_B, s_C, state_scale scalars (requantisation factor 1e2);
+    with them: x_scale (G,hg,dg), s_B / s_C (G), state_scale (G,hg,dg,N), int32 cumulative end indices
+    head_range (G,hg) and dim_range (G,hg,dg) (factor 1e6).  Returns (y float32 (B,H,P), new state)."""
+    x, xp = _req(x)
+    Bsz, H, P = x.shape
+    state = np.array(state, order="C", copy=True)
+    N = state.shape[-1]
+    assert state.shape == (Bsz, H, P, N)
+    B, bp = _req(B)
+    C_, cp = _req(C_)
+    G = B.shape[1]
+    dt, dp = _req(np.broadcast_to(np.asarray(dt, np.int8), (Bsz, H, P)))
+    A_log, ap = _req(np.broadcast_to(np.asarray(A_log, np.int8), (H, P, N)))
+    f32 = lambda a: np.ascontiguousarray(np.asarray(a, np.float32).reshape(-1))
+    vp = lambda a: None if a is None else a.ctypes.data_as(C.c_void_p)
+    Dd = None if D is None else np.ascontiguousarray(np.broadcast_to(np.asarray(D, np.int8), (H, P)))
+    db = None if dt_bias is None else np.ascontiguousarray(np.broadcast_to(np.asarray(dt_bias, np.float32), (H, P)))
+    grouped = head_range is not None
+    xs, sB, sC, ss = f32(x_scale), f32(s_B), f32(s_C), f32(state_scale)
+    hr = None if not grouped else np.ascontiguousarray(head_range, np.int32)
+    dr = None if not grouped else np.ascontiguousarray(dim_range, np.int32)
+    nhg, ndg = (hr.shape[1], dr.shape[2]) if grouped else (0, 0)
+    if grouped:
+        assert xs.size == G * nhg * ndg and sB.size == G and sC.size == G and ss.size == G * nhg * ndg * N
+    else:
+        assert xs.size == 1 and sB.size == 1 and sC.size == 1 and ss.size == 1
+    y = np.empty((Bsz, H, P), np.float32)
+    if state.dtype == np.float32:
+        s8, s32 = None, vp(state)
+    else:
+        assert state.dtype == np.int8
+        s8, s32 = vp(state), None
+    lib().qo_ssm_update_heads(s8, s32, xp, dp, ap, bp, cp, vp(Dd), vp(db), _opt(z), vp(xs), vp(ss), vp(sB), vp(sC),
+                              vp(hr), vp(dr), _f(s_dt), _f(s_A), _f(s_D), _f(s_z), Bsz, H, P, N, G, nhg, ndg,
+                              int(softplus), vp(y))
+    return y, state
+
+
 def gemm_w8a8(a, w, s_a, s_b, round_half_away=False):
     """a int8 (M,K), w int8 (N,K), s_a fp32 (1|M), s_b fp32 (1|N).
     Returns (acc int32 (M,N), fp32 value before the cast, int8 cast)."""

@@ -290,6 +290,75 @@ void qo_sscan_update(int8_t* state_i8, float* state_f32, const int8_t* x, const 
 }
 
 /* ---------------------------------------------------------------------------------------------
+ * Single-step state update with heads, quamba/triton/selective_state_update.py:23-126 (per-tensor
+ * scales, requantisation factor 1e2, :119) and :236-362 (Mamba2: x scale per (ssd group, head group,
+ * dim group), state scale per (ssd group, head group, dim group, state), B / C scale per ssd group,
+ * factor 1e6, :355).  Dense arrays: state (batch, nheads, dim, dstate) int8 or fp32, x / dt / z int8
+ * (batch, nheads, dim), A_log int8 (nheads, dim, dstate), B / C int8 (batch, ngroups, dstate), D int8
+ * (nheads, dim), dt_bias fp32 (nheads, dim) holding the value the kernel adds (:90-92 / :327).  The
+ * kernel's TIE_HDIM branch (:98-105 / :333-340: dt, dt_bias and A_log are one value per head, passed
+ * as stride-0 views) evaluates the same expressions on those values, so the caller expands the views.
+ * Group lookup (:303-315): hg = #{j : h mod (H/G) >= head_range[g,j]}, dg = #{j : p >= dim_range[g,hg,j]}.
+ * y fp32 (batch, nheads, dim) is the value stored as fp16, from the un-requantised state (:357).
+ * ------------------------------------------------------------------------------------------- */
+void qo_ssm_update_heads(int8_t* state_i8, float* state_f32, const int8_t* x, const int8_t* dt, const int8_t* A_log,
+                         const int8_t* B, const int8_t* C, const int8_t* D, const float* dt_bias, const int8_t* z,
+                         const float* x_scale, const float* state_scale, const float* s_B, const float* s_C,
+                         const int32_t* head_range, const int32_t* dim_range,
+                         float s_dt, float s_A, float s_D, float s_z,
+                         int batch, int nheads, int dim, int dstate, int ngroups, int nhead_groups, int ndim_groups,
+                         int softplus, float* y) {
+    const int hpg = nheads / ngroups;
+    const int grouped = nhead_groups > 0;
+    const float K = grouped ? 1e6f : 1e2f;
+    for (int b = 0; b < batch; ++b) {
+        for (int h = 0; h < nheads; ++h) {
+            const int g = h / hpg;
+            int hg = 0;
+            if (grouped) {
+                for (int j = 0; j < nhead_groups; ++j) hg += (h % hpg) >= head_range[g * nhead_groups + j];   /* :306 */
+            }
+            const float sB = s_B[grouped ? g : 0], sC = s_C[grouped ? g : 0];                    /* :277-279 */
+            for (int p = 0; p < dim; ++p) {
+                int sidx = 0;
+                if (grouped) {
+                    int dg = 0;
+                    const int32_t* dr = dim_range + (g * nhead_groups + hg) * ndim_groups;
+                    for (int j = 0; j < ndim_groups; ++j) dg += p >= dr[j];                       /* :312 */
+                    sidx = (g * nhead_groups + hg) * ndim_groups + dg;
+                }
+                const int64_t i = ((int64_t)b * nheads + h) * dim + p;
+                const int64_t hp = (int64_t)h * dim + p;
+                const float xv = x_scale[sidx] * (float)x[i];                                     /* :83 / :316 */
+                float dtv = s_dt * (float)dt[i];                                                  /* :87 / :325 */
+                if (dt_bias) dtv += dt_bias[hp];                                                  /* :90-92 / :327 */
+                if (softplus) dtv = softplus20(dtv);
+                float acc = 0.0f;
+                for (int n = 0; n < dstate; ++n) {
+                    const int64_t si = i * dstate + n;
+                    const float sc = grouped ? state_scale[(int64_t)sidx * dstate + n] : state_scale[0];
+                    float hv = state_f32 ? state_f32[si] : sc * (float)state_i8[si];              /* :85 / :323 */
+                    const float A = -expf(s_A * (float)A_log[hp * dstate + n]);                   /* :96 / :331 */
+                    const float dA = expf(A * dtv);                                               /* :97 / :332 */
+                    const float Bv = sB * (float)B[((int64_t)b * ngroups + g) * dstate + n];      /* :107 / :342 */
+                    const float Cv = sC * (float)C[((int64_t)b * ngroups + g) * dstate + n];
+                    hv = hv * dA + (Bv * dtv) * xv;                                               /* :118 / :353 */
+                    if (state_f32) state_f32[si] = hv;
+                    else state_i8[si] = sat8_rne((hv * K) / (sc * K));                            /* :119 / :355 */
+                    acc += hv * Cv;                                                               /* :121 / :357 */
+                }
+                if (D) acc += xv * (s_D * (float)D[hp]);                                          /* :123 / :359 */
+                if (z) {
+                    const float zv = s_z * (float)z[i];
+                    acc *= zv * (1.0f / (1.0f + expf(-zv)));                                      /* :125 / :361 */
+                }
+                y[i] = acc;
+            }
+        }
+    }
+}
+
+/* ---------------------------------------------------------------------------------------------
  * W8A8 GEMM, csrc/linear/quant_linear_fwd_kernel.cuh:63-130:
  *   acc = int32 sum_k a[m,k]*w[n,k];  d = s_a[m|0] * (s_b[n|0] * float(acc))  (:85-97)
  * out_f32 receives the fp32 value before the final cast; out_i8 its int8 cast (round to nearest

@@ -87,7 +87,7 @@ class QaSScanParams(C.Structure):
         ("scale_u", vp), ("scale_delta", vp), ("scale_A", vp), ("scale_B", vp), ("scale_C", vp),
         ("scale_D", vp), ("scale_delta_bias", vp), ("scale_z", vp), ("scale_ssm_state", vp),
         ("out", vp), ("last_state_i8", vp), ("last_state_f32", vp),
-        ("dt_sum_out", vp), ("carry_dt_sum", vp), ("carry_state", vp), ("carry_first", i32), ("reserved1", i32),
+        ("dt_sum_out", vp), ("carry_dt_sum", vp), ("carry_state", vp), ("carry_first", i32), ("mapping", i32),
     ]
 
 

@@ -40,6 +40,16 @@ __device__ __forceinline__ float softplus20(float x) {
     return e < 0.015625f ? series : big;
 }
 
+// The same function without a branch (the early return above becomes a jump around the rest, which keeps a
+// batch of independent evaluations from overlapping): softplus(x) = max(x, 0) + log1p(exp(-|x|)).  Above the
+// threshold the second term is below half an ulp of x, so x comes back exactly, as the reference returns it.
+__device__ __forceinline__ float softplus20_flat(float x) {
+    const float e = fast_exp2(-__builtin_fabsf(x) * kLog2e);
+    const float series = e * __builtin_fmaf(e, __builtin_fmaf(e, __builtin_fmaf(e, -0.25f, 1.0f / 3.0f), -0.5f), 1.0f);
+    const float big = fast_log2(1.0f + e) * 0.693147180559945309f;
+    return __builtin_fmaxf(x, 0.0f) + (e < 0.015625f ? series : big);
+}
+
 __device__ __forceinline__ float silu_gate(float z) {
     return z * fast_rcp(1.0f + fast_exp2(-z * kLog2e));
 }
@@ -424,25 +434,335 @@ __global__ __launch_bounds__(64 * WAVES) void sscan_fwd_kernel(QaSScanParams p, 
     sscan_fwd_body<NPL, NSPLIT, T, WAVES>(p, vec_in, vec_bc, vec_out, blockIdx.x * Cfg::kCh, blockIdx.y, sm);
 }
 
+// ---------------------------------------------------------------------------------------------
+// d_state <= 16, many channels: the same walk with everything that does not depend on the state index taken out
+// of the time loop.  While a tile of T = 32 steps is staged, the thread that loaded a channel's bytes also
+// evaluates the step size (bias, softplus) and step size x input for those steps and leaves them in LDS as
+// fp32; all of these evaluations are independent, so their long dependent chains (two transcendentals each)
+// overlap instead of standing at the head of every group of four steps, and the time loop reads them with two
+// 16-byte loads that every lane of a channel shares - no cross-lane operands in the multiplications.
+//   lanes of a channel: NSPLIT in {4, 8}; states per lane: NPL = 16 / NSPLIT; a lane stages T / NSPLIT steps
+//   of its own channel per tile.
+// ---------------------------------------------------------------------------------------------
+template <int NPL, int NSPLIT, int WAVES>
+struct PreCfg {
+    static constexpr int T = 32;
+    static constexpr int kThreads = 64 * WAVES;
+    static constexpr int kCh = kThreads / NSPLIT;
+    static constexpr int kNP = NPL * NSPLIT;               // 16
+    static constexpr int kStage = T / NSPLIT;              // steps (= bytes per tensor) a lane stages per tile
+    static constexpr int kPitch = T + 4;                   // floats per row of per-step values: rows 16-byte
+                                                           // aligned, eight rows cover the 32 banks
+    static constexpr int kBcPitch = 2 * kNP + 4;           // floats per step of B | C
+    static constexpr int kOutPitch = kCh + 8;              // halves; keeps rows 16-byte aligned
+    static constexpr int kBcPieces = (2 * kNP * T / 4 + kThreads - 1) / kThreads;   // dwords of B/C per thread
+};
+
+template <class Cfg>
+struct PreSmem {
+    __attribute__((aligned(16))) float d[Cfg::kCh][Cfg::kPitch];     // step size
+    __attribute__((aligned(16))) float du[Cfg::kCh][Cfg::kPitch];    // step size x input
+    float skip[Cfg::kCh][Cfg::kPitch];                               // D x input
+    float gate[Cfg::kCh][Cfg::kPitch];                               // SiLU gate of the step
+    __attribute__((aligned(16))) float bc[Cfg::T][Cfg::kBcPitch];    // B (kNP) | C (kNP) of a step, scaled
+    __attribute__((aligned(16))) __half out[Cfg::T][Cfg::kOutPitch];
+    float gate_table[256];             // SiLU gate per z code (indexed by the raw byte)
+};
+
+// BYTES bytes starting at row[t]; bytes at or beyond t_end read as zero.
+template <int BYTES>
+__device__ __forceinline__ void load_bytes(uint32_t (&w)[BYTES / 4], const int8_t* row, int t, int t_end, bool vec) {
+    if (vec && t + BYTES <= t_end) {
+        if constexpr (BYTES == 8) {
+            const uint2 v = *reinterpret_cast<const uint2*>(row + t);
+            w[0] = v.x; w[1] = v.y;
+        } else {
+            w[0] = *reinterpret_cast<const uint32_t*>(row + t);
+        }
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < BYTES / 4; ++i) w[i] = 0u;
+    for (int i = 0; i < BYTES; ++i) {
+        if (t + i < t_end) w[i >> 2] |= static_cast<uint32_t>(static_cast<uint8_t>(row[t + i])) << (8 * (i & 3));
+    }
+}
+
+template <int NPL, int NSPLIT, int WAVES, bool HAS_Z>
+__device__ __forceinline__ void sscan_fwd_pre_body(const QaSScanParams& p, int vec_in, int vec_bc, int vec_out, int c0, int b,
+                                                   PreSmem<PreCfg<NPL, NSPLIT, WAVES>>& sm) {
+    using Cfg = PreCfg<NPL, NSPLIT, WAVES>;
+    constexpr int T = Cfg::T, kThreads = Cfg::kThreads, kCh = Cfg::kCh, kNP = Cfg::kNP, kStage = Cfg::kStage;
+    constexpr int kBcPieces = Cfg::kBcPieces;
+    static_assert(NSPLIT == 4 || NSPLIT == 8, "four or eight lanes per channel");
+    static_assert(kNP == 16 && (NPL == 4 || NPL == 2), "sixteen states");
+
+    const int tid = threadIdx.x;
+    const int c_local = tid / NSPLIT;
+    const int slice = tid % NSPLIT;
+    const int qslice = slice & 3;
+    const int c = c0 + c_local;
+    const bool c_ok = c < p.dim;
+    const int cc = c_ok ? c : p.dim - 1;                   // clamped channel for parameter loads
+    const int g = c0 / (p.dim / p.n_groups);
+    const int L = p.seqlen;
+    const bool softplus = p.delta_softplus != 0;
+
+    const float s_u = *p.scale_u, s_dt = *p.scale_delta, s_A = *p.scale_A, s_B = *p.scale_B, s_C = *p.scale_C;
+    const float s_z = HAS_Z ? *p.scale_z : 0.0f;
+    const float D_f = p.D ? *p.scale_D * static_cast<float>(p.D[cc]) : 0.0f;
+    const float db = p.delta_bias ? *p.scale_delta_bias * static_cast<float>(p.delta_bias[cc]) : 0.0f;
+
+    float A2[NPL], h[NPL];
+#pragma unroll
+    for (int j = 0; j < NPL; ++j) {
+        const int n = slice * NPL + j;
+        h[j] = 0.0f;
+        A2[j] = n < p.dstate
+                    ? -expf(s_A * static_cast<float>(p.A_log[cc * p.A_d_stride + n * p.A_dstate_stride])) * kLog2e
+                    : 0.0f;
+    }
+    if (p.carry_state) {                 // segments of one sequence side by side, see sscan_fwd_body
+        const int seg = p.carry_first + b;
+        for (int sp = 0; sp < seg; ++sp) {
+            const float sd = p.carry_dt_sum[static_cast<int64_t>(sp) * p.dim + cc];
+#pragma unroll
+            for (int j = 0; j < NPL; ++j) {
+                const int n = min(slice * NPL + j, p.dstate - 1);
+                h[j] = __builtin_fmaf(fast_exp2(sd * A2[j]), h[j],
+                                      p.carry_state[(static_cast<int64_t>(sp) * p.dim + cc) * p.dstate + n]);
+            }
+        }
+    }
+    float dt_sum = 0.0f;                 // of the steps this lane stages
+
+    const int8_t* u_row = p.u + b * p.u_batch_stride + static_cast<int64_t>(cc) * p.u_d_stride;
+    const int8_t* d_row = p.delta + b * p.delta_batch_stride + static_cast<int64_t>(cc) * p.delta_d_stride;
+    const int8_t* z_row = HAS_Z ? p.z + b * p.z_batch_stride + static_cast<int64_t>(cc) * p.z_d_stride : nullptr;
+    const int8_t* bc_base[2] = {p.B + b * p.B_batch_stride + g * p.B_group_stride,
+                                p.C + b * p.C_batch_stride + g * p.C_group_stride};
+    const int64_t bc_nstride[2] = {p.B_dstate_stride, p.C_dstate_stride};
+    const float bc_scale[2] = {s_B, s_C};
+
+    uint32_t r_u[kStage / 4], r_d[kStage / 4], r_z[kStage / 4];
+    uint32_t r_bc[kBcPieces];
+
+    // B / C dword `piece` of a tile: the state index varies fastest over the lanes, so that the four scattered
+    // LDS writes of stage() spread over the banks
+    auto bc_piece = [&](int piece, int& which, int& n, int& col) {
+        which = piece / (kNP * T / 4);
+        n = piece % kNP;
+        col = (piece / kNP) % (T / 4);
+    };
+
+    auto issue_loads = [&](int t0) {
+        const int t = t0 + slice * kStage;
+        // rows past the last channel read the last channel's bytes; nothing of theirs is stored
+        load_bytes<kStage>(r_u, u_row, t, L, vec_in);
+        load_bytes<kStage>(r_d, d_row, t, L, vec_in);
+        if constexpr (HAS_Z) load_bytes<kStage>(r_z, z_row, t, L, vec_in);
+#pragma unroll
+        for (int i = 0; i < kBcPieces; ++i) {
+            int which, n, col;
+            bc_piece(tid + i * kThreads, which, n, col);
+            uint32_t v[1] = {0u};
+            if (which < 2 && n < p.dstate) load_bytes<4>(v, bc_base[which] + n * bc_nstride[which], t0 + col * 4, L, vec_bc);
+            r_bc[i] = v[0];
+        }
+    };
+
+    // Writes the staged tile.  Per step of this lane's share of its channel: step size (bias, softplus), step
+    // size x input, skip term and gate - everything the time loop needs that does not depend on the state.
+    auto stage = [&](int t0) {
+        float dv[kStage], duv[kStage], sk[kStage], gt[kStage];
+#pragma unroll
+        for (int e = 0; e < kStage; ++e) {
+            const float u_val = s_u * i8_of(r_u[e >> 2], e & 3);
+            float dt = __builtin_fmaf(s_dt, i8_of(r_d[e >> 2], e & 3), db);
+            if (softplus) dt = softplus20_flat(dt);
+            dv[e] = dt;
+            sk[e] = D_f * u_val;
+            duv[e] = u_val;
+            gt[e] = HAS_Z ? sm.gate_table[(r_z[e >> 2] >> (8 * (e & 3))) & 0xffu] : 1.0f;
+        }
+        if (t0 + T > L) {
+            // ragged last tile: steps past the end of the sequence must leave the state alone (a = 1, b = 0)
+#pragma unroll
+            for (int e = 0; e < kStage; ++e) dv[e] = t0 + slice * kStage + e < L ? dv[e] : 0.0f;
+        }
+#pragma unroll
+        for (int e = 0; e < kStage; ++e) {
+            dt_sum += dv[e];
+            duv[e] *= dv[e];
+        }
+#pragma unroll
+        for (int q = 0; q < kStage / 4; ++q) {
+            const int t = slice * kStage + q * 4;
+            *reinterpret_cast<float4*>(&sm.d[c_local][t]) = make_float4(dv[q * 4], dv[q * 4 + 1], dv[q * 4 + 2], dv[q * 4 + 3]);
+            *reinterpret_cast<float4*>(&sm.du[c_local][t]) = make_float4(duv[q * 4], duv[q * 4 + 1], duv[q * 4 + 2], duv[q * 4 + 3]);
+            *reinterpret_cast<float4*>(&sm.skip[c_local][t]) = make_float4(sk[q * 4], sk[q * 4 + 1], sk[q * 4 + 2], sk[q * 4 + 3]);
+            if constexpr (HAS_Z) {
+                *reinterpret_cast<float4*>(&sm.gate[c_local][t]) = make_float4(gt[q * 4], gt[q * 4 + 1], gt[q * 4 + 2], gt[q * 4 + 3]);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kBcPieces; ++i) {
+            int which, n, col;
+            bc_piece(tid + i * kThreads, which, n, col);
+            if (which < 2) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) sm.bc[col * 4 + e][which * kNP + n] = bc_scale[which] * i8_of(r_bc[i], e);
+            }
+        }
+    };
+
+    // operands of one group of four steps
+    struct Group {
+        float d[4], du[4], B[4][NPL], C[4][NPL], skip, gate;
+    };
+    auto fetch = [&](Group& o, int tq) {
+        const float4 d4 = *reinterpret_cast<const float4*>(&sm.d[c_local][tq * 4]);
+        const float4 du4 = *reinterpret_cast<const float4*>(&sm.du[c_local][tq * 4]);
+        o.d[0] = d4.x; o.d[1] = d4.y; o.d[2] = d4.z; o.d[3] = d4.w;
+        o.du[0] = du4.x; o.du[1] = du4.y; o.du[2] = du4.z; o.du[3] = du4.w;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float* row = sm.bc[tq * 4 + j];
+            if constexpr (NPL == 2) {
+                const float2 Bv = *reinterpret_cast<const float2*>(row + slice * NPL);
+                const float2 Cv = *reinterpret_cast<const float2*>(row + kNP + slice * NPL);
+                o.B[j][0] = Bv.x; o.B[j][1] = Bv.y; o.C[j][0] = Cv.x; o.C[j][1] = Cv.y;
+            } else {
+                const float4 Bv = *reinterpret_cast<const float4*>(row + slice * NPL);
+                const float4 Cv = *reinterpret_cast<const float4*>(row + kNP + slice * NPL);
+                o.B[j][0] = Bv.x; o.B[j][1] = Bv.y; o.B[j][2] = Bv.z; o.B[j][3] = Bv.w;
+                o.C[j][0] = Cv.x; o.C[j][1] = Cv.y; o.C[j][2] = Cv.z; o.C[j][3] = Cv.w;
+            }
+        }
+        o.skip = sm.skip[c_local][tq * 4 + qslice];
+        o.gate = HAS_Z ? sm.gate[c_local][tq * 4 + qslice] : 1.0f;
+    };
+
+    const int n_tiles = (L + T - 1) / T;
+    issue_loads(0);
+    if constexpr (HAS_Z) {
+        for (int i = tid; i < 256; i += kThreads) sm.gate_table[i] = silu_gate(s_z * static_cast<float>(static_cast<int8_t>(i)));
+        __syncthreads();
+    }
+    stage(0);
+    __syncthreads();
+
+    for (int tile = 0; tile < n_tiles; ++tile) {
+        const int t0 = tile * T;
+        const int nt = min(T, L - t0);
+        if (tile + 1 < n_tiles) issue_loads(t0 + T);
+
+        // All T / 4 groups of four steps, also in a ragged last tile: steps past the end have step size 0 and leave
+        // the state alone, and their output rows are never stored.  No branch in the body and constant LDS
+        // offsets; the operands of a group are fetched while the group before is being computed.
+        Group grp[2];
+        fetch(grp[0], 0);
+#pragma unroll
+        for (int tq = 0; tq < T / 4; ++tq) {
+            Group& o = grp[tq & 1];
+            if (tq + 1 < T / 4) fetch(grp[(tq + 1) & 1], tq + 1);
+            // keep the reads of the next group ahead of this group's arithmetic (the scheduler would sink them
+            // to their first use, and a wave would then wait for LDS once per group)
+            __builtin_amdgcn_sched_barrier(0);
+            float acc[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                acc[j] = 0.0f;
+#pragma unroll
+                for (int n = 0; n < NPL; ++n) {
+                    const float a = fast_exp2(o.d[j] * A2[n]);
+                    h[n] = __builtin_fmaf(a, h[n], o.B[j][n] * o.du[j]);
+                    acc[j] = __builtin_fmaf(h[n], o.C[j][n], acc[j]);
+                }
+            }
+            // each lane of a quad completes the step it owns: a transposing reduction (keep one half, hand the
+            // other half to the neighbour) instead of four full ones
+            const bool odd = qslice & 1, hi = qslice & 2;
+            const float w01 = (odd ? acc[1] : acc[0]) + quad_xor<1>(odd ? acc[0] : acc[1]);
+            const float w23 = (odd ? acc[3] : acc[2]) + quad_xor<1>(odd ? acc[2] : acc[3]);
+            float own_sum = (hi ? w23 : w01) + quad_xor<2>(hi ? w01 : w23);
+            // eight lanes per channel: the other quad holds the other half of the states (both quads then hold
+            // the same sums and store the same values)
+            if constexpr (NSPLIT == 8) own_sum += __shfl_xor(own_sum, 4);
+            float y = own_sum + o.skip;
+            if constexpr (HAS_Z) y *= o.gate;
+            sm.out[tq * 4 + qslice][c_local] = __float2half(y);
+        }
+        __syncthreads();   // out complete; everyone is done reading the staged tile
+
+        // write the tile's output rows: (t, kCh channels) contiguous along channels
+        {
+            constexpr int kChunksPerRow = kCh / 8;
+            __half* out_b = static_cast<__half*>(p.out) + b * p.out_batch_stride;
+            for (int piece = tid; piece < nt * kChunksPerRow; piece += kThreads) {
+                const int t = piece / kChunksPerRow, ch8 = (piece % kChunksPerRow) * 8;
+                __half* dst = out_b + (t0 + t) * p.out_l_stride + (c0 + ch8) * p.out_d_stride;
+                if (vec_out && c0 + ch8 + 8 <= p.dim) {
+                    *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(&sm.out[t][ch8]);
+                } else {
+                    for (int e = 0; e < 8; ++e) {
+                        if (c0 + ch8 + e < p.dim) dst[e * p.out_d_stride] = sm.out[t][ch8 + e];
+                    }
+                }
+            }
+        }
+        if (tile + 1 < n_tiles) stage(t0 + T);
+        __syncthreads();
+    }
+
+    if (p.dt_sum_out) {
+        // the lanes of a channel staged different steps
+        dt_sum += quad_xor<1>(dt_sum);
+        dt_sum += quad_xor<2>(dt_sum);
+        if constexpr (NSPLIT == 8) dt_sum += __shfl_xor(dt_sum, 4);
+        if (c_ok && slice == 0) p.dt_sum_out[static_cast<int64_t>(b) * p.dim + c] = dt_sum;
+    }
+    if (c_ok) {
+        const int64_t base = (static_cast<int64_t>(b) * p.dim + c) * p.dstate;
+        const float s_state = p.last_state_i8 ? *p.scale_ssm_state : 1.0f;
+#pragma unroll
+        for (int j = 0; j < NPL; ++j) {
+            const int n = slice * NPL + j;
+            if (n < p.dstate) {
+                if (p.last_state_f32) p.last_state_f32[base + n] = h[j];
+                if (p.last_state_i8) p.last_state_i8[base + n] = sat8_half_away(h[j] / s_state);
+            }
+        }
+    }
+}
+
+template <int NPL, int NSPLIT, int WAVES, bool HAS_Z>
+__global__ __launch_bounds__(64 * WAVES) void sscan_fwd_pre_kernel(QaSScanParams p, int vec_in, int vec_bc, int vec_out) {
+    using Cfg = PreCfg<NPL, NSPLIT, WAVES>;
+    __shared__ PreSmem<Cfg> sm;
+    sscan_fwd_pre_body<NPL, NSPLIT, WAVES, HAS_Z>(p, vec_in, vec_bc, vec_out, blockIdx.x * Cfg::kCh, blockIdx.y, sm);
+}
+
 // Two kinds of workgroup in one launch, for d_state 16: the first `blocks_a` workgroups of a batch entry take
 // 64 channels each with four lanes per channel, the others 32 channels each with eight lanes per channel (half
 // the states per lane, a little more than half the time).  The kernel is bound by vector-ALU issue and a wave's
 // time does not depend on how many of its lanes are busy, so what counts is the number of waves per SIMD: when
 // the four-lane mapping alone would leave half of the SIMDs with one wave more than the others, the tail of the
 // channels goes to the short kind and every SIMD gets the same mix.
+template <bool HAS_Z>
 __global__ __launch_bounds__(256) void sscan_fwd_mixed_kernel(QaSScanParams p, int vec_in, int vec_bc, int vec_out, int blocks_a) {
-    using CfgA = ScanCfg<4, 4, 64, 4>;
-    using CfgB = ScanCfg<2, 8, 64, 4>;
+    using CfgA = PreCfg<4, 4, 4>;
+    using CfgB = PreCfg<2, 8, 4>;
     __shared__ union Smem {
-        ScanSmem<CfgA, 64> a;
-        ScanSmem<CfgB, 64> b;
+        PreSmem<CfgA> a;
+        PreSmem<CfgB> b;
         __device__ Smem() {}
     } sm;
     const int bx = blockIdx.x;
     if (bx < blocks_a) {
-        sscan_fwd_body<4, 4, 64, 4>(p, vec_in, vec_bc, vec_out, bx * CfgA::kCh, blockIdx.y, sm.a);
+        sscan_fwd_pre_body<4, 4, 4, HAS_Z>(p, vec_in, vec_bc, vec_out, bx * CfgA::kCh, blockIdx.y, sm.a);
     } else {
-        sscan_fwd_body<2, 8, 64, 4>(p, vec_in, vec_bc, vec_out, blocks_a * CfgA::kCh + (bx - blocks_a) * CfgB::kCh, blockIdx.y, sm.b);
+        sscan_fwd_pre_body<2, 8, 4, HAS_Z>(p, vec_in, vec_bc, vec_out, blocks_a * CfgA::kCh + (bx - blocks_a) * CfgB::kCh, blockIdx.y, sm.b);
     }
 }
 
@@ -456,11 +776,27 @@ int launch_fwd(const QaSScanParams& p, hipStream_t stream, int vec_in, int vec_b
     return check_launch();
 }
 
+template <int NPL, int NSPLIT, int WAVES>
+int launch_fwd_pre(const QaSScanParams& p, hipStream_t stream, int vec_in, int vec_bc, int vec_out) {
+    using Cfg = PreCfg<NPL, NSPLIT, WAVES>;
+    if (p.n_groups > 1 && (p.dim / p.n_groups) % Cfg::kCh != 0) return QA_ERR_UNSUPPORTED;
+    dim3 grid((p.dim + Cfg::kCh - 1) / Cfg::kCh, p.batch);
+    if (p.z) {
+        hipLaunchKernelGGL((sscan_fwd_pre_kernel<NPL, NSPLIT, WAVES, true>), grid, dim3(Cfg::kThreads), 0, stream, p, vec_in,
+                           vec_bc, vec_out);
+    } else {
+        hipLaunchKernelGGL((sscan_fwd_pre_kernel<NPL, NSPLIT, WAVES, false>), grid, dim3(Cfg::kThreads), 0, stream, p, vec_in,
+                           vec_bc, vec_out);
+    }
+    return check_launch();
+}
+
 // Channels [0, 64 * blocks_a) with four lanes per channel, the rest with eight.
 int launch_fwd_mixed(const QaSScanParams& p, hipStream_t stream, int vec_in, int vec_bc, int vec_out, int blocks_a) {
     const int rest = p.dim - 64 * blocks_a;
     dim3 grid(blocks_a + (rest + 31) / 32, p.batch);
-    hipLaunchKernelGGL(sscan_fwd_mixed_kernel, grid, dim3(256), 0, stream, p, vec_in, vec_bc, vec_out, blocks_a);
+    if (p.z) hipLaunchKernelGGL(sscan_fwd_mixed_kernel<true>, grid, dim3(256), 0, stream, p, vec_in, vec_bc, vec_out, blocks_a);
+    else hipLaunchKernelGGL(sscan_fwd_mixed_kernel<false>, grid, dim3(256), 0, stream, p, vec_in, vec_bc, vec_out, blocks_a);
     return check_launch();
 }
 
@@ -648,13 +984,6 @@ int launch_update(const QaSsmUpdateParams& p, hipStream_t stream) {
 }  // namespace
 }  // namespace qa
 
-// Variant override for tuning runs: QA_SSCAN_VARIANT = "<nsplit>x<waves>" (e.g. "4x2").
-static int sscan_variant_from_env(int* nsplit, int* waves) {
-    const char* s = getenv("QA_SSCAN_VARIANT");
-    if (!s) return 0;
-    return sscanf(s, "%dx%d", nsplit, waves) == 2;
-}
-
 extern "C" int qa_sscan_fwd(const QaSScanParams* p, void* stream_) {
     using namespace qa;
     if (!p || !p->u || !p->delta || !p->A_log || !p->B || !p->C || !p->out) return QA_ERR_NULL;
@@ -680,14 +1009,32 @@ extern "C" int qa_sscan_fwd(const QaSScanParams* p, void* stream_) {
                         p->out_l_stride % 8 == 0;
 
     const int N = p->dstate;
+    const int per_group = p->dim / p->n_groups;
+    if (p->mapping != 0) {
+        // a lane mapping named by the caller (tests): only d_state <= 16 has more than one
+        if (N > 16) return QA_ERR_UNSUPPORTED;
+        const int lanes = (p->mapping >> 8) & 0xff, arg = p->mapping & 0xff;
+        if (lanes == 0) {
+            // mixed launch: `arg` workgroups of 64 channels with four lanes per channel, the rest with eight
+            if (arg < 1 || p->n_groups != 1 || 64LL * arg > p->dim) return QA_ERR_SHAPE;
+            return launch_fwd_mixed(*p, stream, vec_in, vec_bc, vec_out, arg);
+        }
+        if (lanes == 1 && arg == 1) return launch_fwd<16, 1, 64, 1>(*p, stream, vec_in, vec_bc, vec_out);
+        if (lanes == 2 && arg == 1) return launch_fwd<8, 2, 64, 1>(*p, stream, vec_in, vec_bc, vec_out);
+        if (lanes == 2 && arg == 2) return launch_fwd<8, 2, 64, 2>(*p, stream, vec_in, vec_bc, vec_out);
+        if (lanes == 4 && arg == 1) return launch_fwd_pre<4, 4, 1>(*p, stream, vec_in, vec_bc, vec_out);
+        if (lanes == 4 && arg == 2) return launch_fwd_pre<4, 4, 2>(*p, stream, vec_in, vec_bc, vec_out);
+        if (lanes == 4 && arg == 4) return launch_fwd_pre<4, 4, 4>(*p, stream, vec_in, vec_bc, vec_out);
+        if (lanes == 8 && arg == 4) return launch_fwd_pre<2, 8, 4>(*p, stream, vec_in, vec_bc, vec_out);
+        return QA_ERR_UNSUPPORTED;
+    }
     if (N <= 16) {
-        int nsplit = 0, waves = 0;
-        if (!sscan_variant_from_env(&nsplit, &waves)) {
-            // The kernel is bound by vector-ALU issue, so the mapping that wastes the fewest issue slots
-            // wins: four lanes per channel (the per-step work is shared out over the quad) and, when
-            // the channel count allows, four waves per workgroup sharing one staged B/C tile.
-            nsplit = 4;
-            waves = p->dim % 64 == 0 ? 4 : (p->dim % 32 == 0 ? 2 : 1);
+        // The kernel is bound by vector-ALU issue, so the mapping that wastes the fewest issue slots wins: four
+        // lanes per channel and, when the channel count allows, four waves per workgroup sharing one staged
+        // B/C tile.  With channel groups a workgroup must stay inside one group.
+        int waves = p->dim % 64 == 0 ? 4 : (p->dim % 32 == 0 ? 2 : 1);
+        while (waves > 1 && p->n_groups > 1 && per_group % (16 * waves) != 0) waves >>= 1;
+        if (waves == 4) {
             // Waves per SIMD with four lanes per channel: q + f.  With 0 < f <= 1/2 the last f/(q+f) of the
             // channels of every batch entry go to the eight-lane kind (see sscan_fwd_mixed_kernel), as long as
             // both parts stay whole workgroups and, with channel groups, whole groups.
@@ -701,31 +1048,21 @@ extern "C" int qa_sscan_fwd(const QaSScanParams* p, void* stream_) {
             const int64_t q = waves_a / simds, rem_waves = waves_a % simds;
             // Few waves (small batches): a launch takes about as long as the busiest SIMD's waves one after the
             // other, and with so few of them latency, not issue, sets a wave's pace - so twice as many waves
-            // of two thirds the length (eight lanes per channel) finish sooner.  Measured at 5120 channels x
-            // 2048 steps, by waves per SIMD (eight-lane kind: 1: 228, 2: 255, 3: 309, 4: 378, 5: 456 us;
-            // four-lane kind: 1: 284, 2: 358, 3: 455 us): the eight-lane kind wins up to 1.5 four-lane waves
-            // per SIMD.
-            if (waves == 4 && 2 * waves_a <= 3 * simds && p->dim % 32 == 0 &&
-                (p->n_groups <= 1 || (p->dim / p->n_groups) % 32 == 0)) {
-                return launch_fwd<2, 8, 64, 4>(*p, stream, vec_in, vec_bc, vec_out);
+            // of two thirds the length (eight lanes per channel) finish sooner: up to 1.5 four-lane waves per SIMD.
+            if (2 * waves_a <= 3 * simds && (p->n_groups <= 1 || per_group % 32 == 0)) {
+                return launch_fwd_pre<2, 8, 4>(*p, stream, vec_in, vec_bc, vec_out);
             }
-            if (waves == 4 && p->n_groups == 1 && q >= 1 && rem_waves > 0 && 2 * rem_waves <= simds) {
+            if (p->n_groups == 1 && q >= 1 && rem_waves > 0 && 2 * rem_waves <= simds) {
                 const int64_t short_channels = rem_waves * 16 / p->batch;      // channels per batch entry for the short kind
                 const int blocks_a = static_cast<int>((p->dim - short_channels) / 64);
                 if (short_channels % 32 == 0 && (p->dim - short_channels) % 64 == 0 && blocks_a > 0) {
                     return launch_fwd_mixed(*p, stream, vec_in, vec_bc, vec_out, blocks_a);
                 }
             }
+            return launch_fwd_pre<4, 4, 4>(*p, stream, vec_in, vec_bc, vec_out);
         }
-        if (nsplit == 1 && waves == 1) return launch_fwd<16, 1, 64, 1>(*p, stream, vec_in, vec_bc, vec_out);
-        if (nsplit == 2 && waves == 1) return launch_fwd<8, 2, 64, 1>(*p, stream, vec_in, vec_bc, vec_out);
-        if (nsplit == 2 && waves == 2) return launch_fwd<8, 2, 64, 2>(*p, stream, vec_in, vec_bc, vec_out);
-        if (nsplit == 4 && waves == 1) return launch_fwd<4, 4, 64, 1>(*p, stream, vec_in, vec_bc, vec_out);
-        if (nsplit == 4 && waves == 2) return launch_fwd<4, 4, 64, 2>(*p, stream, vec_in, vec_bc, vec_out);
-        if (nsplit == 4 && waves == 4) return launch_fwd<4, 4, 64, 4>(*p, stream, vec_in, vec_bc, vec_out);
-        if (nsplit == 8 && waves == 4) return launch_fwd<2, 8, 64, 4>(*p, stream, vec_in, vec_bc, vec_out);
-        if (nsplit == 0 && waves > 0) return launch_fwd_mixed(*p, stream, vec_in, vec_bc, vec_out, waves);
-        return QA_ERR_UNSUPPORTED;
+        if (waves == 2) return launch_fwd_pre<4, 4, 2>(*p, stream, vec_in, vec_bc, vec_out);
+        return launch_fwd_pre<4, 4, 1>(*p, stream, vec_in, vec_bc, vec_out);
     }
     // Wider states: eight states per lane, or sixteen.  A workgroup converts its B/C tile once for all of its
     // channels, so with enough channels to fill the part four waves share one tile (64 or 32 channels per

@@ -414,6 +414,7 @@ def sscan_fwd(u, scale_u, delta, scale_delta, A, scale_A, B, scale_B, C, scale_C
     p.u, p.delta, p.A_log, p.B, p.C, p.out = ptr(u), ptr(delta), ptr(A), ptr(B), ptr(C), ptr(out)
     p.scale_u, p.scale_delta, p.scale_A = ptr(scale_u), ptr(scale_delta), ptr(scale_A)
     p.scale_B, p.scale_C = ptr(scale_B), ptr(scale_C)
+    p.mapping = SSCAN_MAPPING
     segments = _sscan_segments(batch, dim, seqlen)
     with torch.cuda.device(u.device):
         stream = _lib.current_stream(u.device)
@@ -456,6 +457,15 @@ def sscan_fwd(u, scale_u, delta, scale_delta, A, scale_A, B, scale_B, C, scale_C
 
 # A single sequence of at least this many steps is scanned in segments (see sscan_fwd); 0 disables it.
 SSCAN_SEGMENT_MIN_STEPS = 1024
+# QaSScanParams.mapping of every call: 0 lets the library choose; tests set sscan_mapping(lanes, arg) to reach each
+# kernel variant on one shape.
+SSCAN_MAPPING = 0
+
+
+def sscan_mapping(lanes, arg):
+    """QA_SSCAN_MAPPING(lanes per channel, waves per workgroup); lanes == 0: the launch with two kinds of
+    workgroup, ``arg`` 64-channel workgroups per batch entry taking four lanes per channel."""
+    return 0x10000 | (int(lanes) << 8) | int(arg)
 
 
 def _sscan_segments(batch, dim, seqlen):
@@ -768,6 +778,16 @@ def ssd_chunk_scan_combined_fwd(q_x, x_scale, q_dt, dt_scale, q_A_log, A_log_sca
     p.final_state_is_fp32 = int(final_state_dtype == torch.float32)
     if not p.final_state_is_fp32:
         _require(final_state_dtype == torch.int8, "final_state_dtype must be torch.int8 or torch.float32")
+        ssm_state_scale = torch.as_tensor(ssm_state_scale, device=dev).to(torch.float32)
+        if p.nhead_groups:
+            _require(tuple(ssm_state_scale.shape) == (ngroups, p.nhead_groups, p.ndim_groups, dstate_given),
+                     "ssm_state_scale must be [ngroups, nhead_groups, ndim_groups, dstate]")
+            if dstate != dstate_given:
+                # the kernel walks the scale rows with the padded state count; the added states are zero, so
+                # any finite scale serves for them
+                ssm_state_scale = torch.nn.functional.pad(ssm_state_scale, (0, dstate - dstate_given), value=1.0)
+        else:
+            _require(ssm_state_scale.numel() == 1, "ssm_state_scale must have one element without group ranges")
         p.state_scale = f32(ssm_state_scale)
     lib = _lib.lib()
     nbytes = lib.qa_ssd_workspace_bytes(ct.byref(p))

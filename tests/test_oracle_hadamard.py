@@ -29,6 +29,15 @@ def test_special_matrices_are_hadamard_with_the_reference_normalisation(S):
         np.testing.assert_array_equal(H, H.T)                      # the construction is symmetric
 
 
+@pytest.mark.parametrize("S,name", [(12, "had_12_paley"), (40, "had_40_tpal")])
+def test_special_matrices_equal_the_tables_the_reference_generates_its_code_from(S, name):
+    # tests/golden/hadamard_tables.npz holds the +/- tables of the reference's csrc/hadamard/code_gen.py, parsed
+    # as text by tests/golden/make_hadamard_tables.py; H H^T = n I alone would admit any Hadamard matrix
+    import os
+    tables = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "hadamard_tables.npz"))
+    np.testing.assert_array_equal(oracle.hadamard_special(S), tables[name])
+
+
 def _dense(dim):
     S, M = oracle.hadamard_split(dim)
     W = scipy.linalg.hadamard(M).astype(np.float64) if M > 1 else np.ones((1, 1))

@@ -78,7 +78,7 @@ def test_fwd_matches_oracle(dev, B, L, D, N):
                                            (1024, 512, 128, None), (1024, 544, 64, None), (1024, 100, 100, None)])
 def test_one_sequence_scanned_in_segments(dev, L, D, N, variant, monkeypatch):
     if variant:
-        monkeypatch.setenv("QA_SSCAN_VARIANT", variant)
+        monkeypatch.setattr(ops, "SSCAN_MAPPING", ops.sscan_mapping(*map(int, variant.split("x"))))
     assert ops._sscan_segments(1, D, L) > 1
     d = synth.mamba1_scan_inputs(1, L, D, N, seed=L + D + 1)
     y_ref, _, st32_ref = _oracle(d, s_state=1.0)
@@ -103,7 +103,7 @@ def test_one_sequence_scanned_in_segments(dev, L, D, N, variant, monkeypatch):
 # channels with four lanes per channel, the remaining channels with eight)
 @pytest.mark.parametrize("variant", ["1x1", "2x1", "2x2", "4x1", "4x2", "4x4", "8x4", "0x1", "0x2"])
 def test_every_lane_mapping_gives_the_same_answer(dev, variant, monkeypatch):
-    monkeypatch.setenv("QA_SSCAN_VARIANT", variant)
+    monkeypatch.setattr(ops, "SSCAN_MAPPING", ops.sscan_mapping(*map(int, variant.split("x"))))
     d = synth.mamba1_scan_inputs(2, 300, 200, 16, seed=21)
     y_ref, _, st32_ref = _oracle(d, s_state=1.0)
     y, x32 = _gpu(d, dev, 1.0, torch.float32)

@@ -1,5 +1,6 @@
 """GPU parity of the Mamba2 SSD chunk scan and its single-step update against the CPU oracle.
-fp16 outputs: rtol 1e-2 / atol 1e-2 (relative to the output scale); fp32 states 1e-3 relative."""
+fp16 outputs: rtol 1e-2 / atol 1e-2 on the values themselves; fp32 states 1e-3 relative; int8 states at most
+one step off, and only where the un-rounded quotient lies within 2e-3 of a rounding tie."""
 import numpy as np
 import pytest
 import torch
@@ -31,9 +32,9 @@ def _gpu(d, dev, chunk, state_scale=None, dt=None, final_dtype=torch.float32, **
 
 
 def _check_y(y_gpu, y_ref):
+    # the bar of the fp16 scan outputs, on the values themselves: |got - want| <= 1e-2 + 1e-2 |want|
     got = y_gpu.float().cpu().numpy()
-    scale = np.abs(y_ref).max()
-    np.testing.assert_allclose(got / scale, y_ref.astype(np.float16).astype(np.float32) / scale, rtol=1e-2, atol=1e-2)
+    np.testing.assert_allclose(got, y_ref.astype(np.float16).astype(np.float32), rtol=1e-2, atol=1e-2)
     assert np.sum((got - y_ref) ** 2) / np.sum(y_ref ** 2) < 1e-4
 
 
@@ -123,6 +124,107 @@ def test_module_forward_then_update_continue_the_sequence(dev):
         want = ref["y"][:, t]
         np.testing.assert_allclose(yt.float().cpu().numpy() / np.abs(want).max(), want / np.abs(want).max(), rtol=1e-2, atol=1e-2)
     assert np.abs(state.cpu().numpy() - ref["final_f32"]).max() <= 2e-3 * np.abs(ref["final_f32"]).max()
+
+
+def _update_step_inputs(B, H, N, G, steps, seed):
+    d = synth.mamba2_ssd_inputs(B, steps, H, 64, N, G, seed=seed, grouped=True, nhead_groups=4, ndim_groups=4, with_z=True)
+    g = np.random.default_rng(seed)
+    d["state_scale"] = (0.004 * g.uniform(0.5, 1.5, (G, 4, 4, N))).astype(np.float32)
+    d["state0"] = g.integers(-127, 128, (B, H, 64, N)).astype(np.int8)
+    return d
+
+
+def _oracle_step(d, t, state):
+    return oracle.ssm_update_heads(state, d["x"][:, t], d["dt"][:, t, :, None], d["A_log"][:, None, None], d["B"][:, t],
+                                   d["C"][:, t], d["D"][:, None], d["dt_bias"].astype(np.float32)[:, None], d["z"][:, t],
+                                   x_scale=d["x_scale"], s_dt=d["s_dt"], s_A=d["s_A"], s_B=d["s_B"], s_C=d["s_C"],
+                                   s_D=d["s_D"], s_z=d["s_z"], state_scale=d["state_scale"], head_range=d["head_range"],
+                                   dim_range=d["dim_range"])
+
+
+def _expand_state_scale(d, H, G):
+    """state scale per (head, p, n) from the group tables, for the tie test below"""
+    hpg, hs, ds = H // G, (H // G) // 4, 64 // 4
+    h = np.arange(H)
+    return d["state_scale"][h[:, None] // hpg, (h[:, None] % hpg) // hs, np.arange(64)[None, :] // ds]      # (H, 64, N)
+
+
+def _check_int8_state(got, want_i8, h_f32, scale_hpn):
+    """at most one step off, and only where the quotient the rounding sees is within 2e-3 of a tie (the kernel's exp is
+    the hardware's, the oracle's is libm's)"""
+    diff = np.abs(got.astype(int) - want_i8.astype(int))
+    assert diff.max() <= 1
+    q = h_f32.astype(np.float64) / scale_hpn[None].astype(np.float64)
+    near_tie = np.abs(np.abs(q - np.floor(q)) - 0.5) < 2e-3
+    assert not (diff != 0)[~near_tie].any()
+    assert (diff != 0).mean() < 0.01
+
+
+# the three rows of the reference's test_qchunkscan_group_heads_update (quamba/tests/test_ssd_combined.py:40-44)
+@pytest.mark.parametrize("B,H,N,G", [(1, 24, 16, 1), (4, 80, 128, 1), (4, 128, 128, 8)])
+def test_grouped_int8_state_update_matches_oracle(dev, B, H, N, G):
+    steps = 6
+    d = _update_step_inputs(B, H, N, G, steps, seed=H + N)
+    s = lambda v: torch.tensor(np.asarray(v, np.float32)).to(dev)
+    nheads = H
+    state = _t(d["state0"], dev)
+    ref_state = d["state0"]
+    scale_hpn = _expand_state_scale(d, H, G)
+    A3 = _t(d["A_log"], dev).view(nheads, 1, 1).expand(nheads, 64, N)
+    D2 = _t(d["D"], dev).view(nheads, 1).expand(nheads, 64)
+    b2 = _t(d["dt_bias"], dev).view(nheads, 1).expand(nheads, 64)
+    saw_big = False
+    for t in range(steps):
+        deq = (ref_state.astype(np.float32) * scale_hpn[None]).astype(np.float32)
+        _, h_f32 = _oracle_step(d, t, deq)                     # the fp32 state the requantisation rounds
+        y_ref, ref_state = _oracle_step(d, t, ref_state)
+        dt3 = _t(d["dt"][:, t], dev).unsqueeze(-1).expand(B, nheads, 64)
+        y = ops.sscan_update(state, _t(d["x"][:, t], dev), s(d["x_scale"]), dt3, s(d["s_dt"]), A3, s(d["s_A"]),
+                             s(d["state_scale"]), _t(d["B"][:, t], dev), s(d["s_B"]), _t(d["C"][:, t], dev), s(d["s_C"]),
+                             D2, s(d["s_D"]), _t(d["z"][:, t], dev), s(d["s_z"]), b2, None, True,
+                             x_head_group_range=_t(d["head_range"], dev), x_dim_group_range=_t(d["dim_range"], dev))
+        assert state.dtype == torch.int8 and y.dtype == torch.float16
+        np.testing.assert_allclose(y.float().cpu().numpy(), y_ref.astype(np.float16).astype(np.float32), rtol=1e-2, atol=1e-2)
+        _check_int8_state(state.cpu().numpy(), ref_state, h_f32, scale_hpn)
+        saw_big = saw_big or np.abs(ref_state).max() > 100
+        state.copy_(_t(ref_state, dev))                        # both sides take the next step from the same state
+    assert saw_big
+
+
+def test_grouped_int8_state_update_strided_state_and_odd_state_count(dev):
+    # dstate % 4 != 0 and a state tensor that is a slice of a wider one: the element-wise kernel
+    B, H, N, G, steps = 3, 8, 30, 2, 5
+    d = _update_step_inputs(B, H, N, G, steps, seed=41)
+    s = lambda v: torch.tensor(np.asarray(v, np.float32)).to(dev)
+    wide = torch.zeros((B, H, 64, N + 3), dtype=torch.int8, device=dev)
+    state = wide[..., 1:N + 1]
+    state.copy_(_t(d["state0"], dev))
+    ref_state = d["state0"]
+    scale_hpn = _expand_state_scale(d, H, G)
+    A3 = _t(d["A_log"], dev).view(H, 1, 1).expand(H, 64, N)
+    b2 = _t(d["dt_bias"], dev).view(H, 1).expand(H, 64)
+    d["D"] = None
+    for t in range(steps):
+        deq = (ref_state.astype(np.float32) * scale_hpn[None]).astype(np.float32)
+        _, h_f32 = _oracle_step_noD(d, t, deq)
+        y_ref, ref_state = _oracle_step_noD(d, t, ref_state)
+        dt3 = _t(d["dt"][:, t], dev).unsqueeze(-1).expand(B, H, 64)
+        y = ops.sscan_update(state, _t(d["x"][:, t], dev), s(d["x_scale"]), dt3, s(d["s_dt"]), A3, s(d["s_A"]),
+                             s(d["state_scale"]), _t(d["B"][:, t], dev), s(d["s_B"]), _t(d["C"][:, t], dev), s(d["s_C"]),
+                             None, None, _t(d["z"][:, t], dev), s(d["s_z"]), b2, None, True,
+                             x_head_group_range=_t(d["head_range"], dev), x_dim_group_range=_t(d["dim_range"], dev))
+        np.testing.assert_allclose(y.float().cpu().numpy(), y_ref.astype(np.float16).astype(np.float32), rtol=1e-2, atol=1e-2)
+        _check_int8_state(state.cpu().numpy(), ref_state, h_f32, scale_hpn)
+        state.copy_(_t(ref_state, dev))
+    assert (wide[..., 0] == 0).all() and (wide[..., N + 1:] == 0).all()        # nothing written outside the view
+
+
+def _oracle_step_noD(d, t, state):
+    return oracle.ssm_update_heads(state, d["x"][:, t], d["dt"][:, t, :, None], d["A_log"][:, None, None], d["B"][:, t],
+                                   d["C"][:, t], None, d["dt_bias"].astype(np.float32)[:, None], d["z"][:, t],
+                                   x_scale=d["x_scale"], s_dt=d["s_dt"], s_A=d["s_A"], s_B=d["s_B"], s_C=d["s_C"],
+                                   s_z=d["s_z"], state_scale=d["state_scale"], head_range=d["head_range"],
+                                   dim_range=d["dim_range"])
 
 
 def test_errors(dev):
