@@ -417,12 +417,27 @@ def other_workloads(dev, steps, warmup):
     return out
 
 
+def _probes():
+    """ctypes handle of the bench-only probe library (quamba_amd/libqa_bench_probes.so, built by quamba_amd.build)."""
+    import ctypes as C
+    path = os.path.join(ROOT, "quamba_amd", "libqa_bench_probes.so")
+    if not os.path.exists(path):
+        sys.exit(f"{path} is missing: build it with `python -m quamba_amd.build`")
+    h = C.CDLL(path)
+    vp = C.c_void_p
+    for name in ("qa_probe_mfma_i8", "qa_probe_valu"):
+        fn = getattr(h, name)
+        fn.restype = C.c_int
+        fn.argtypes = [vp, C.c_int64, vp, C.c_int, C.c_int, C.c_int, vp]
+    return h
+
+
 def mfma_calibration(dev):
     """Sustained v_mfma_i32_32x32x32_i8 rate of a register-only loop (two waves per SIMD on every CU) for
     constant and for pseudo-random operand bytes, six launches of about 5 ms each; the last one is reported.
     The clock is the ratio of the shader-clock and 100 MHz counters over the loop."""
     from quamba_amd import _lib
-    lib = _lib.lib()
+    lib = _probes()
     wgs, iters = 512, 20000
     sink = torch.empty(wgs * 256, dtype=torch.int32, device=dev)
     ticks = torch.zeros(2, dtype=torch.int64, device=dev)
@@ -432,7 +447,7 @@ def mfma_calibration(dev):
         for _ in range(6):
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
-            _lib.check(lib.qa_diag_mfma_i8(sink.data_ptr(), sink.numel(), ticks.data_ptr(), wgs, iters, rnd, stream), "diag")
+            _lib.check(lib.qa_probe_mfma_i8(sink.data_ptr(), sink.numel(), ticks.data_ptr(), wgs, iters, rnd, stream), "diag")
             e1.record()
             torch.cuda.synchronize()
             ms = e0.elapsed_time(e1)
@@ -446,7 +461,7 @@ def valu_calibration(dev):
     """Issue time of plain and transcendental vector instructions: eight waves per SIMD on every CU, each lane with
     eight independent chains of one instruction; ns per wave-instruction per SIMD and the clock during the loop."""
     from quamba_amd import _lib
-    lib = _lib.lib()
+    lib = _probes()
     wgs, iters = 2048, 20000
     sink = torch.empty(wgs * 256, dtype=torch.float32, device=dev)
     ticks = torch.zeros(2, dtype=torch.int64, device=dev)
@@ -457,7 +472,7 @@ def valu_calibration(dev):
         for _ in range(4):
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
-            _lib.check(lib.qa_diag_valu(sink.data_ptr(), sink.numel(), ticks.data_ptr(), wgs, iters, op, stream), "diag")
+            _lib.check(lib.qa_probe_valu(sink.data_ptr(), sink.numel(), ticks.data_ptr(), wgs, iters, op, stream), "diag")
             e1.record()
             torch.cuda.synchronize()
             ms = e0.elapsed_time(e1)

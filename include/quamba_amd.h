@@ -408,22 +408,6 @@ typedef struct QaSsdParams {
 int64_t qa_ssd_workspace_bytes(const QaSsdParams* p);
 int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream);
 
-/* Diagnostic, no counterpart in the reference: launches `workgroups` x 256 threads that each issue
- * iters x 8 v_mfma_i32_32x32x32_i8 (65536 integer operations per instruction and wave) on operands held
- * in registers, one repeated byte (random_operands = 0) or pseudo-random bytes (1).  `sink` (device,
- * >= workgroups * 256 ints) receives throw-away sums; `ticks` (device-visible, two 64-bit values, or
- * null) receives the shader-clock and 100 MHz-clock counts of workgroup 0's loop.  Used by bench.py to
- * report the int8 matrix rate the part sustains for a given operand activity. */
-int qa_diag_mfma_i8(int* sink, int64_t sink_elems, long long* ticks, int workgroups, int iters,
-                    int random_operands, void* stream);
-
-/* Diagnostic, no counterpart in the reference: `workgroups` x 256 threads each issue iters x 8 independent
- * instructions of one kind (op 0: v_mul_f32, 1: v_exp_f32, 2: v_rcp_f32, 3: v_log_f32, 4: v_fmac_f32,
- * 5: v_mul_f32 with a quad-broadcast DPP operand); `sink` and `ticks` as
- * above.  Used by bench.py to report the issue rate of plain and transcendental vector instructions, which
- * bounds the selective scan. */
-int qa_diag_valu(float* sink, int64_t sink_elems, long long* ticks, int workgroups, int iters, int op, void* stream);
-
 #ifdef __cplusplus
 }
 #endif

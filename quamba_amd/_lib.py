@@ -170,8 +170,6 @@ SYMBOLS = {
     "qa_gemm_w4a8": (C.c_int, [C.POINTER(QaGemmW4A8Params), vp]),
     "qa_ssd_workspace_bytes": (C.c_int64, [C.POINTER(QaSsdParams)]),
     "qa_ssd_chunk_scan_fwd": (C.c_int, [C.POINTER(QaSsdParams), vp]),
-    "qa_diag_mfma_i8": (C.c_int, [vp, C.c_int64, vp, C.c_int, C.c_int, C.c_int, vp]),
-    "qa_diag_valu": (C.c_int, [vp, C.c_int64, vp, C.c_int, C.c_int, C.c_int, vp]),
 }
 
 _lib = None
