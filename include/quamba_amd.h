@@ -25,7 +25,8 @@ typedef enum QaStatus {
     QA_ERR_SHAPE = -2,       /* a size is out of the supported range */
     QA_ERR_STRIDE = -3,      /* a stride / alignment requirement is violated */
     QA_ERR_UNSUPPORTED = -4, /* valid request the library has no kernel for */
-    QA_ERR_LAUNCH = -5       /* the HIP runtime refused the launch */
+    QA_ERR_LAUNCH = -5,      /* the HIP runtime refused the launch */
+    QA_ERR_SCRATCH = -6      /* the problem needs more scratch than the library's fixed buffer holds */
 } QaStatus;
 
 /* Human-readable text for a status code (static storage). */
@@ -407,6 +408,18 @@ typedef struct QaSsdParams {
 
 int64_t qa_ssd_workspace_bytes(const QaSsdParams* p);
 int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream);
+
+/* qa_ssd_chunk_scan_fwd for callers that cannot allocate device memory: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference (its launcher allocates its
+ * intermediates with torch.empty on every call, quamba/triton/quant_ssd_combined.py:61-77).  The caller passes
+ * inputs and outputs as usual; `workspace` and `workspace_bytes` are ignored: the intermediates live in a fixed
+ * buffer of QA_SSD_STATIC_SCRATCH_BYTES (64 MiB) that is part of the library's device image - every GPU the
+ * library runs on holds it until the process ends.  A problem whose qa_ssd_workspace_bytes() exceeds that size
+ * returns QA_ERR_SCRATCH.  The call allocates nothing and frees nothing; same kernels, same results as
+ * qa_ssd_chunk_scan_fwd.  All calls on one GPU share the buffer: calls that overlap on one GPU (two streams, two
+ * threads) race; calls on one stream, or ordered by events, do not.  Nothing in the buffer has to start at zero. */
+#define QA_SSD_STATIC_SCRATCH_BYTES (64ll << 20)
+int qa_ssd_chunk_scan_fwd_noalloc(const QaSsdParams* p, void* stream);
 
 #ifdef __cplusplus
 }

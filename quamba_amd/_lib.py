@@ -170,6 +170,7 @@ SYMBOLS = {
     "qa_gemm_w4a8": (C.c_int, [C.POINTER(QaGemmW4A8Params), vp]),
     "qa_ssd_workspace_bytes": (C.c_int64, [C.POINTER(QaSsdParams)]),
     "qa_ssd_chunk_scan_fwd": (C.c_int, [C.POINTER(QaSsdParams), vp]),
+    "qa_ssd_chunk_scan_fwd_noalloc": (C.c_int, [C.POINTER(QaSsdParams), vp]),
 }
 
 _lib = None

@@ -16,6 +16,7 @@ extern "C" const char* qa_status_string(int status) {
         case QA_ERR_STRIDE: return "stride or alignment requirement violated";
         case QA_ERR_UNSUPPORTED: return "unsupported configuration";
         case QA_ERR_LAUNCH: return "HIP launch failed";
+        case QA_ERR_SCRATCH: return "the problem needs more scratch memory than the library's fixed buffer holds";
         default: return "unknown status";
     }
 }

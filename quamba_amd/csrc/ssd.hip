@@ -15,6 +15,9 @@
 // while memory has channels fastest; x tiles are transposed once on the way into LDS (4x4 blocks:
 // four dword loads, four 8-byte LDS stores) and then read as 16-byte MFMA operands, B is packed in
 // operand order once per ssd group.
+#include <atomic>
+#include <mutex>
+
 #include "qa_common.hpp"
 
 namespace qa {
@@ -818,4 +821,58 @@ extern "C" int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream_) {
         else launch_scan(ssd_chunk_scan_kernel<64, 64>);
     }
     return check_launch();
+}
+
+// ---------------------------------------------------------------------------------------------
+// The same scan for callers that cannot allocate (code under HIP graph capture, serving loops and harnesses that
+// forbid hipMalloc): the workspace is a fixed array in the device image instead of a caller's buffer.  Every GPU
+// holds its own copy of the array at its own address, so the address is looked up once per device, with that
+// device current, and kept.  In host code the array's name is only a handle for that lookup, never a pointer.
+// ---------------------------------------------------------------------------------------------
+namespace qa {
+namespace {
+constexpr int64_t kStaticScratchBytes = QA_SSD_STATIC_SCRATCH_BYTES;
+constexpr int kMaxDevices = 64;
+}  // namespace
+}  // namespace qa
+
+static __device__ __align__(256) unsigned char scratch[qa::kStaticScratchBytes];
+
+namespace qa {
+namespace {
+std::mutex g_scratch_mutex;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// Device address of `scratch` on the current device (null: the runtime refused the lookup).
+void* static_scratch_of_current_device() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (ptr) return ptr;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    ptr = g_scratch_ptr[dev].load(std::memory_order_relaxed);
+    if (ptr) return ptr;
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+        set_last_hip_error(static_cast<int>(e));
+        return nullptr;
+    }
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+    return ptr;
+}
+}  // namespace
+}  // namespace qa
+
+extern "C" int qa_ssd_chunk_scan_fwd_noalloc(const QaSsdParams* p, void* stream_) {
+    using namespace qa;
+    const int st = validate(p);
+    if (st != QA_OK) return st;
+    if (p->batch == 0 || p->seqlen == 0) return QA_OK;
+    if (ws_layout(*p).total > kStaticScratchBytes) return QA_ERR_SCRATCH;
+    void* ptr = static_scratch_of_current_device();
+    if (!ptr) return QA_ERR_LAUNCH;
+    QaSsdParams q = *p;
+    q.workspace = ptr;
+    q.workspace_bytes = kStaticScratchBytes;
+    return qa_ssd_chunk_scan_fwd(&q, stream_);
 }

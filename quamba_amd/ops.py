@@ -701,7 +701,7 @@ def ssd_chunk_scan_combined_fwd(q_x, x_scale, q_dt, dt_scale, q_A_log, A_log_sca
                                 ssm_state_scale, chunk_size, q_D=None, D_scale=None, q_z=None, z_scale=None,
                                 dt_bias=None, initial_states=None, seq_idx=None, cu_seqlens=None, dt_softplus=False,
                                 dt_limit=(0.0, float("inf")), x_head_group_range=None, x_dim_group_range=None,
-                                final_state_dtype=torch.int8, return_workspace=False):
+                                final_state_dtype=torch.int8, return_workspace=False, static_scratch=False):
     """Quantized SSD forward; interface of _quant_mamba_chunk_scan_combined_fwd and, with the group
     ranges, of _quamba2_mamba_chunk_scan_combined_fwd (quamba/triton/quant_ssd_combined.py:11-166).
 
@@ -709,6 +709,9 @@ def ssd_chunk_scan_combined_fwd(q_x, x_scale, q_dt, dt_scale, q_A_log, A_log_sca
     already processed step sizes; q_A_log int8 (nheads); q_B, q_C int8 (batch, seqlen, ngroups,
     dstate); q_D int8 (nheads) or (nheads, headdim); dt_bias fp16 (nheads).
     Returns (out fp16 like q_x, final_states (batch, nheads, headdim, dstate) int8 or fp32).
+    With ``static_scratch`` the intermediates live in the library's fixed device buffer instead of a workspace
+    allocated here (qa_ssd_chunk_scan_fwd_noalloc: for callers that must not allocate; calls on one GPU must
+    not overlap); problems that need more than the buffer holds raise RuntimeError.
     """
     if initial_states is not None:
         raise NotImplementedError("initial_states is not supported")
@@ -793,11 +796,18 @@ def ssd_chunk_scan_combined_fwd(q_x, x_scale, q_dt, dt_scale, q_A_log, A_log_sca
     nbytes = lib.qa_ssd_workspace_bytes(ct.byref(p))
     if nbytes <= 0:
         _lib.check(lib.qa_ssd_chunk_scan_fwd(ct.byref(p), None) or -4, "ssd_chunk_scan_fwd")
-    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
-    p.workspace, p.workspace_bytes = ptr(ws), nbytes
-    with torch.cuda.device(dev):
-        st = lib.qa_ssd_chunk_scan_fwd(ct.byref(p), _lib.current_stream(dev))
-    _lib.check(st, "ssd_chunk_scan_fwd")
+    if static_scratch:
+        _require(not return_workspace, "the library's own scratch buffer cannot be returned")
+        with torch.cuda.device(dev):
+            st = lib.qa_ssd_chunk_scan_fwd_noalloc(ct.byref(p), _lib.current_stream(dev))
+        _lib.check(st, "ssd_chunk_scan_fwd_noalloc")
+        ws = None
+    else:
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        p.workspace, p.workspace_bytes = ptr(ws), nbytes
+        with torch.cuda.device(dev):
+            st = lib.qa_ssd_chunk_scan_fwd(ct.byref(p), _lib.current_stream(dev))
+        _lib.check(st, "ssd_chunk_scan_fwd")
     if dstate != dstate_given:
         final = final[..., :dstate_given].contiguous()
     if return_workspace:
