@@ -1,20 +1,18 @@
 // Mamba2 quantized SSD chunk scan (prefill) for gfx950.
 //
 // Stages and arithmetic follow the reference's Triton pipeline (quamba/triton/quant_ssd_combined.py
-// :61-77, grouped :146-162); see each kernel for the file it restates.  fp16 operands, fp32
-// accumulation, as there; the one pure int8 contraction (C B^T) runs on the int8 matrix cores.
+// :61-77, grouped :146-162); see each kernel for the file it restates.  fp16 operands rounded where the
+// reference rounds them, fp32 accumulation, as there; the one pure int8 contraction (C B^T) runs on the
+// int8 matrix cores and stays in fp32.
 //   cumsum      dt = clamp(softplus(s_dt q_dt + dt_bias)), dA_cs = within-chunk cumsum(dt * A)
-//   cb          CB[m,k] = (s_C s_B) * sum_n q_C[m,n] q_B[k,n]                       (int8 MFMA, lower tiles)
-//   state       S_c[p,n] = sum_k f16(x^[k,p] exp(dA_last - dA_k) dt_k) f16(B^[k,n])   (fp16 MFMA; the reference
-//               rounds B^ times the weight instead, the difference is inside the fp16 tolerance)
+//   cb          CB[m,k] = (s_C s_B) * sum_n q_C[m,n] q_B[k,n]                       (int8 MFMA, lower tiles, fp32 out)
+//   state       S_c[p,n] = sum_k f16(x^[k,p]) f16(B^[k,n] exp(dA_last - dA_k) dt_k)   (fp16 MFMA)
 //               P_0 = 0, P_{c+1} = exp(dA_last,c) P_c + S_c in registers; P_c stored in fp16; final state fp32 / int8
-//   chunk_scan  y[m,p] = exp(dA_m) sum_n f16(C^[m,n]) P_c[p,n] + sum_{k<=m} f16(CB[m,k] e^{dA_m-dA_k} dt_k) f16(x^[k,p])
-//               + D x^[m,p], optional z gate, fp16 out                               (fp16 MFMA; C B^T is held
-//               in fp16 and meets its decay factor in a packed fp16 multiply)
+//   chunk_scan  y[m,p] = exp(dA_m) sum_n f16(C^[m,n]) f16(P_c[p,n]) + sum_{k<=m} f16(CB[m,k] e^{dA_m-dA_k} dt_k) f16(x^[k,p])
+//               + D x^[m,p], optional z gate, fp16 out                               (fp16 MFMA)
 // Both fp16 contractions over the time index need x (and B) with time as the fastest-moving index,
-// while memory has channels fastest; x tiles are transposed once on the way into LDS (4x4 blocks:
-// four dword loads, four 8-byte LDS stores) and then read as 16-byte MFMA operands, B is packed in
-// operand order once per ssd group.
+// while memory has channels fastest; the tiles are transposed once on the way into LDS and then read as
+// 16-byte MFMA operands.
 #include <atomic>
 #include <mutex>
 
@@ -28,59 +26,32 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef _Float16 v4h __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
 
 constexpr int kP = 64;          // head dimension this build supports
 constexpr float kLog2e = 1.44269504088896341f;
-// C B^T is kept in fp16 divided by 16 (exact), so that products of full-range int8 rows stay inside
-// the fp16 range; the factor returns with the decay table.
-constexpr float kCbShift = 0.0625f, kCbUnshift = 16.0f;
 
 __device__ __forceinline__ float fexp(float x) { return __builtin_amdgcn_exp2f(x * kLog2e); }
-// orders a wave's own LDS writes before its later LDS reads (wave-private scratch needs no workgroup barrier)
-__device__ __forceinline__ void wave_sync() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
 __device__ __forceinline__ int8_t byte_of(uint32_t w, int j) { return static_cast<int8_t>((w >> (8 * j)) & 0xffu); }
 
 struct Ws {            // workspace sections (byte offsets), see qa_ssd_workspace_bytes
-    int64_t dt, dA, cb, prev, final_f32, c16, bt16, total;
+    int64_t dt, dA, cb, prev, c16, total;
 };
 
 __host__ __device__ inline int64_t align256(int64_t v) { return (v + 255) & ~int64_t(255); }
 
 __host__ __device__ inline Ws ws_layout(const QaSsdParams& p) {
     const int64_t nc = (p.seqlen + p.chunk_size - 1) / p.chunk_size;
-    const int64_t B = p.batch, H = p.nheads, Q = p.chunk_size, G = p.ngroups, P = p.headdim, N = p.dstate;
+    const int64_t B = p.batch, H = p.nheads, Q = p.chunk_size, G = p.ngroups, N = p.dstate;
     Ws w;
     int64_t off = 0;
     w.dt = off; off = align256(off + B * H * nc * Q * 4);
     w.dA = off; off = align256(off + B * H * nc * Q * 4);
-    w.cb = off; off = align256(off + B * nc * G * Q * Q * 2);
-    w.prev = off; off = align256(off + B * nc * H * P * N * 2);
-    w.final_f32 = off; off = align256(off + B * H * P * N * 4);
+    w.cb = off; off = align256(off + B * nc * G * Q * Q * 4);
+    w.prev = off; off = align256(off + B * nc * H * kP * N * 2);
     w.c16 = off; off = align256(off + B * static_cast<int64_t>(p.seqlen) * G * N * 2);
-    w.bt16 = off; off = align256(off + B * nc * G * N * Q * 2);
     w.total = off;
     return w;
-}
-
-// Workgroups are handed to the eight XCDs (each with an L2 of its own) in turn by linear index.  The
-// heads of one ssd group share the packed B operand and neighbouring heads share the 128-byte lines
-// of x, so in the state kernel the heads of one (batch, group) unit get linear indices that land on one
-// XCD: index L -> XCD L % 8, position L / 8 there -> unit (L / 8) / hpg * 8 + L % 8, head (L / 8) % hpg
-// of the group.  Needs a unit count that is a multiple of eight; otherwise the natural order
-// (unit-major) is kept.  (The chunk scan measured the same either way and keeps the natural order.)
-__device__ __forceinline__ void unit_and_head(int linear, int units, int hpg, int& unit, int& head_in_group) {
-    if (units % 8 == 0) {
-        const int xcd = linear % 8, pos = linear / 8;
-        unit = (pos / hpg) * 8 + xcd;
-        head_in_group = pos % hpg;
-    } else {
-        unit = linear / hpg;
-        head_in_group = linear % hpg;
-    }
 }
 
 // x scale of channel p of head h (per-tensor, or looked up from the cumulative group ranges,
@@ -161,7 +132,7 @@ __global__ __launch_bounds__(256) void ssd_cumsum_kernel(QaSsdParams p, float* d
 // write their C rows dequantised to fp16 (f16(s_C * q_C)): every head of the group multiplies those
 // rows with its entering state in the chunk scan, which then reads them ready-made.
 // ---------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(64) void ssd_cb_kernel(QaSsdParams p, __half* cb_out, __half* c16_out, int nc) {
+__global__ __launch_bounds__(64) void ssd_cb_kernel(QaSsdParams p, float* cb_out, __half* c16_out, int nc) {
     const int Q = p.chunk_size, N = p.dstate, G = p.ngroups;
     const int nt = Q / 64;
     // blockIdx.x enumerates lower-triangular tile pairs (mt >= kt)
@@ -226,7 +197,7 @@ __global__ __launch_bounds__(64) void ssd_cb_kernel(QaSsdParams p, __half* cb_ou
             for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[ks][j], fc[ks][i], acc[i][j], 0, 0, 0);
     }
     // acc[i][j]: lane holds row m = mt*64 + i*32 + (lane & 31), register r column k = kt*64 + j*32 + 8*(r/4) + 4*(lane/32) + r%4
-    __half* tile = cb_out + ((static_cast<int64_t>(b) * nc + c) * G + g) * Q * Q;
+    float* tile = cb_out + ((static_cast<int64_t>(b) * nc + c) * G + g) * Q * Q;
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -235,224 +206,252 @@ __global__ __launch_bounds__(64) void ssd_cb_kernel(QaSsdParams p, __half* cb_ou
             for (int q = 0; q < 4; ++q) {
                 const int m = mt * 64 + i * 32 + frow;
                 const int k = kt * 64 + j * 32 + 8 * q + 4 * fhalf;
-                v4h o;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) o[e] = static_cast<_Float16>((scale * static_cast<float>(acc[i][j][4 * q + e])) * kCbShift);
-                *reinterpret_cast<v4h*>(tile + static_cast<int64_t>(m) * Q + k) = o;
+                float4 o;
+                o.x = scale * static_cast<float>(acc[i][j][4 * q]);
+                o.y = scale * static_cast<float>(acc[i][j][4 * q + 1]);
+                o.z = scale * static_cast<float>(acc[i][j][4 * q + 2]);
+                o.w = scale * static_cast<float>(acc[i][j][4 * q + 3]);
+                *reinterpret_cast<float4*>(tile + static_cast<int64_t>(m) * Q + k) = o;
             }
 }
 
 // ---------------------------------------------------------------------------------------------
-// B operand of the chunk-state product, packed once per (batch, chunk, ssd group) for every head of
-// the group: f16(s_B q_B[k, n]) stored fragment-major, so that a wave's 16-byte-per-lane operand of
-// n-tile nt and k-step ks is one contiguous kilobyte:
-//   element (n, k) -> (((n/32) * (Q/16) + k/16) * 64 + ((k%16)/8) * 32 + n%32) * 8 + k%8
-// One workgroup per (batch, chunk, group, n-tile); the 32 columns of the tile pass through LDS.
+// The fp16 contractions run on v_mfma_f32_16x16x32_f16 with the operands rounded to fp16 where the reference
+// rounds them, so that the products agree and only the order of the fp32 sums differs:
+//   S_c[p,n] = sum_k f16(x^[k,p]) f16(B^[k,n] exp(dA_last - dA_k) dt_k);   P_{c+1} = exp(dA_last) P_c + S_c
+//   y[m,p]   = exp(dA_m) sum_n f16(C^[m,n]) f16(P_c[p,n])                                  (term 1)
+//            + sum_{k<=m} f16(CB[m,k] exp(dA_m - dA_k) dt_k) f16(x^[k,p])                  (term 2)
+//            + x^[m,p] D, optional z gate, fp16 out
+// Both contractions over the time index need x with time as the fastest-moving index, while memory has channels
+// fastest.  A thread transposes 4x4 blocks on the way into LDS: four dword loads (sixteen lanes cover the 64
+// bytes of a row), four 8-byte stores.  The rows of the transposed tile are kept in the order
+//   slot(p) = 16 (p % 4) + p / 4
+// so that the sixteen lanes of one store write sixteen neighbouring rows (all banks, instead of every fourth row)
+// and an MFMA tile, sixteen neighbouring rows, holds the channels p = 4 i + tile (i = 0..15): a lane then owns
+// four neighbouring channels of an output row, which leave as one 8-byte store without passing through LDS.
+// int8 values enter as biased bytes u = q + 128 (one xor per dword): s q = fma(u, s, -128 s) exactly, with the
+// byte-to-float conversion in a single instruction.
 // ---------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void ssd_bpack_kernel(QaSsdParams p, __half* bt16, int nc) {
-    constexpr int QMAX = 256, PITCH = 36;
-    __shared__ __attribute__((aligned(16))) int8_t s_b[QMAX * PITCH];
-    const int Q = p.chunk_size, N = p.dstate, G = p.ngroups, NT = N / 32;
-    const int nt = blockIdx.x % NT;
-    const int bcg = blockIdx.x / NT;
-    const int g = bcg % G, c = (bcg / G) % nc, b = bcg / (G * nc);
-    const int tid = threadIdx.x;
-    const int t0 = c * Q;
-    const int lim = min(Q, p.seqlen - t0);
-    const float sB = p.nhead_groups > 0 ? p.B_scale[g] : p.B_scale[0];
-    // rows k of the tile: 32 bytes each, two 16-byte pieces
-    for (int piece = tid; piece < Q * 2; piece += 256) {
-        const int k = piece >> 1, half = piece & 1;
-        uint4 v = make_uint4(0u, 0u, 0u, 0u);
-        if (k < lim) v = *reinterpret_cast<const uint4*>(p.B + ((static_cast<int64_t>(b) * p.seqlen + t0 + k) * G + g) * N + nt * 32 + half * 16);
-        uint32_t* dst = reinterpret_cast<uint32_t*>(s_b + k * PITCH + half * 16);
-        dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;
-    }
-    __syncthreads();
-    __half* out = bt16 + (static_cast<int64_t>(bcg) * NT + nt) * (Q / 16) * 64 * 8;
-    for (int piece = tid; piece < (Q / 16) * 64; piece += 256) {
-        const int ks = piece >> 6, lane = piece & 63, frow = lane & 31, fhalf = lane >> 5;
-        v8h o;
+__device__ __forceinline__ v4f mfma16(v8h a, v8h b, v4f c) { return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0); }
+__device__ __forceinline__ float ubyte_of(uint32_t w, int j) { return static_cast<float>((w >> (8 * j)) & 0xffu); }
+constexpr uint32_t kBias = 0x80808080u;
+__device__ __forceinline__ uint32_t word_of(const uint4& v, int d) { return d == 0 ? v.x : d == 1 ? v.y : d == 2 ? v.z : v.w; }
+__device__ __forceinline__ float lane_of(const float4& v, int d) { return d == 0 ? v.x : d == 1 ? v.y : d == 2 ? v.z : v.w; }
+
+// A thread's share of a chunk's x tile, steps 4 kb .. 4 kb + 3 of channels 16 pb .. 16 pb + 15 (four 16-byte loads,
+// biased bytes), goes to the transposed fp16 tile: sixteen 8-byte stores, rows in slot order.
+template <int XP>
+__device__ __forceinline__ void stage_x_share(_Float16 (*xt)[XP], const uint4 (&xr)[4], const float* xs, int pb, int kb) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) o[e] = static_cast<_Float16>(sB * static_cast<float>(s_b[(ks * 16 + fhalf * 8 + e) * PITCH + frow]));
-        *reinterpret_cast<v8h*>(out + static_cast<int64_t>(piece) * 8) = o;
+    for (int d = 0; d < 4; ++d) {
+        const float4 s4 = *reinterpret_cast<const float4*>(xs + 16 * pb + 4 * d);
+        const uint32_t w0 = word_of(xr[0], d) ^ kBias, w1 = word_of(xr[1], d) ^ kBias, w2 = word_of(xr[2], d) ^ kBias, w3 = word_of(xr[3], d) ^ kBias;
+#pragma unroll
+        for (int cc = 0; cc < 4; ++cc) {
+            const float sc = lane_of(s4, cc), nsc = -128.0f * sc;
+            v4h v;
+            v[0] = static_cast<_Float16>(__builtin_fmaf(ubyte_of(w0, cc), sc, nsc));
+            v[1] = static_cast<_Float16>(__builtin_fmaf(ubyte_of(w1, cc), sc, nsc));
+            v[2] = static_cast<_Float16>(__builtin_fmaf(ubyte_of(w2, cc), sc, nsc));
+            v[3] = static_cast<_Float16>(__builtin_fmaf(ubyte_of(w3, cc), sc, nsc));
+            *reinterpret_cast<v4h*>(&xt[cc * 16 + 4 * pb + d][kb * 4]) = v;          // row slot(16 pb + 4 d + cc)
+        }
+    }
+}
+
+// Workgroup L of a launch whose units (things that share operands through L2) should stay on one XCD: L -> XCD
+// L % 8, position L / 8 there; `parts` consecutive positions are the parts of one (unit, head).
+__device__ __forceinline__ void unit_head_part(int linear, int units, int hpg, int parts, int& unit, int& head_in_group, int& part) {
+    if (units % 8 == 0) {
+        const int xcd = linear % 8, pos = linear / 8;
+        part = pos % parts;
+        unit = (pos / parts / hpg) * 8 + xcd;
+        head_in_group = (pos / parts) % hpg;
+    } else {
+        part = linear % parts;
+        unit = linear / parts / hpg;
+        head_in_group = (linear / parts) % hpg;
     }
 }
 
 // ---------------------------------------------------------------------------------------------
-// Stages 2, 3 and 6 in one pass (quamba/triton/quant_chunk_state.py:76-89, quant_state_passing.py
-// :60-83, quant_ssm_states.py:43,119): one workgroup per (batch, head) walks the chunks in order and
-// keeps the running state P (headdim x dstate, fp32) in registers, in the layout of the MFMA
-// accumulators:
-//   S_c[p,n] = sum_k f16(x^[k,p] w_k) f16(B^[k,n]),  w_k = exp(dA_last - dA_k) dt_k
-//   store f16(P) as the state entering chunk c;  P = exp(dA_last) P + S_c
-// The per-head weight w_k is applied to x (64 columns) rather than to B (dstate columns), so the B
-// operand is the same for every head of a group and comes ready-made from ssd_bpack_kernel; the
-// fp32 chunk states never travel through memory.  The x tile of chunk c+1 is fetched into registers
-// before the products of chunk c are issued.
-// Wave w owns n-tile w and both p-tiles (dstate 128) or n-tile w&1 and p-tile w>>1 (dstate 64).
+// Stages 2, 3 and 6 (quamba/triton/quant_chunk_state.py:76-89, quant_state_passing.py:60-83, quant_ssm_states.py
+// :43,119): a workgroup of four waves per (batch, head, 64 state columns) walks the chunks in order with its part
+// of the running state P (64 x 64 of headdim x dstate, fp32) in registers; the fp32 chunk states never travel
+// through memory.  A wave owns 16 columns n and all rows p.  Its B operand, f16((s_B q_B[k,n]) w_k) with the
+// per-head weight w_k = exp(dA_last - dA_k) dt_k, is built in registers from the transposed int8 B tile in LDS
+// (rows n of 4-byte-aligned pitch with an odd number of dwords: conflict-free for the transposing dword stores
+// and for the operand reads); its A operand is the transposed x tile.  The tiles of chunk c+1 are fetched into
+// registers while chunk c is multiplied.  The state entering chunk c >= 1 is stored as fp16, rows in slot order.
 // ---------------------------------------------------------------------------------------------
-template <int N, int Q>
-__global__ __launch_bounds__(256, 2) void ssd_state_kernel(QaSsdParams p, const float* dt_ws, const float* dA_ws,
-                                                        const __half* bt16, __half* prev, float* final_ws, int nc) {
-    constexpr int PITCH = Q + 8, NT = N / 32, PTW = NT == 4 ? 2 : 1, nks = Q / 16;
-    constexpr int XB = (Q / 4) * (kP / 4) / 256;               // 4x4 blocks of the x tile per thread
-    __shared__ __attribute__((aligned(16))) _Float16 s_xt[kP * PITCH];
-    __shared__ __attribute__((aligned(16))) float s_w[2][Q];
-    __shared__ float s_xs[kP];
-    constexpr int kPatchPitch = 40;                            // halves; rows stay 16-byte aligned
-    __shared__ __attribute__((aligned(16))) _Float16 s_patch[4 * 32 * kPatchPitch];
+template <int Q>
+struct StateSmem {
+    static constexpr int XP = Q + 8;        // halves per row of the transposed x tile
+    static constexpr int BP = Q + 4;        // bytes per row of the transposed B tile
+    __attribute__((aligned(16))) _Float16 xt[kP][XP];
+    __attribute__((aligned(16))) int8_t b8[64][BP];
+    __attribute__((aligned(16))) float w[Q];
+    __attribute__((aligned(16))) float xs[kP];    // x scale per channel
+};
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, frow = lane & 31, fhalf = lane >> 5;
-    int unit, hig;
-    unit_and_head(blockIdx.x, p.batch * p.ngroups, p.nheads / p.ngroups, unit, hig);
-    const int h = (unit % p.ngroups) * (p.nheads / p.ngroups) + hig;
-    const int b = unit / p.ngroups;
-    const int G = p.ngroups, H = p.nheads;
+template <int N, int Q>
+__global__ __launch_bounds__(256, 3) void ssd_state_kernel(QaSsdParams p, const float* dt_ws, const float* dA_ws, __half* prev, int nc) {
+    using S = StateSmem<Q>;
+    extern __shared__ __attribute__((aligned(16))) unsigned char ssd_smem_raw[];
+    S& sm = *reinterpret_cast<S*>(ssd_smem_raw);
+    constexpr int kThreads = 256;
+    constexpr int PARTS = N / 64;                                 // workgroups per (batch, head)
+    static_assert(Q <= kThreads, "a thread stages at most one share of the chunk's tiles");
+
+    const int tid = threadIdx.x, lane = tid & 63, l16 = lane & 15, lq = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);    // the same in every lane: kept in a scalar register
+    const int G = p.ngroups, H = p.nheads, L = p.seqlen;
+    int unit, hig, part;
+    unit_head_part(blockIdx.x, p.batch * G, H / G, PARTS, unit, hig, part);
+    const int h = (unit % G) * (H / G) + hig;
+    const int b = unit / G;
     int g, hg;
     group_of(p, h, g, hg);
-    if (tid < kP) s_xs[tid] = x_scale_of(p, g, hg, tid);
-    const int ntile = NT == 4 ? wave : (wave & 1);
-    const int pt0 = NT == 4 ? 0 : (wave >> 1);
-    const int64_t row_stride = static_cast<int64_t>(H) * kP;
+    const bool grouped = p.nhead_groups > 0;
+    const float sB = grouped ? p.B_scale[g] : p.B_scale[0];
+    const float nsB = -128.0f * sB;
+    const uint32_t xrow = static_cast<uint32_t>(H) * kP;          // bytes between steps of x
+    const uint32_t brow = static_cast<uint32_t>(G) * N;           // bytes between steps of B
     const int64_t rows0 = (static_cast<int64_t>(b) * H + h) * nc;
-
-    uint32_t xr[XB][4];
-    auto load_x = [&](int c) {
+    // this thread's share of a chunk's tiles: steps 4 kb .. 4 kb + 3, sixteen columns from 16 pb (of x: channels; of
+    // B: state columns of this workgroup's part)
+    const int pb = tid % 4, kb = tid / 4;
+    const bool mine = Q == 256 || tid < Q;
+    const uint32_t voff_x = static_cast<uint32_t>(4 * kb) * xrow + 16 * pb, voff_b = static_cast<uint32_t>(4 * kb) * brow + 16 * pb;
+    if (tid < kP) sm.xs[tid] = x_scale_of(p, g, hg, tid);
+    uint4 xr[4], br[4];
+    float r_dt = 0.0f, r_dA = 0.0f, r_last = 0.0f;
+    auto load_chunk = [&](int c) {
         const int t0 = c * Q;
-        const int valid = min(Q, p.seqlen - t0);
-        const int8_t* src = p.x + ((static_cast<int64_t>(b) * p.seqlen + t0) * H + h) * kP;
+        const int valid = min(Q, L - t0);
+        // uniform row addresses plus one per-thread offset: the address arithmetic stays in scalar registers
+        const int8_t* xsrc = p.x + (static_cast<int64_t>(b) * L + t0) * xrow + static_cast<int64_t>(h) * kP;
+        const int8_t* bsrc = p.B + (static_cast<int64_t>(b) * L + t0) * brow + static_cast<int64_t>(g) * N + part * 64;
+        if (mine) {
+            if (valid == Q) {
 #pragma unroll
-        for (int i = 0; i < XB; ++i) {
-            const int id = tid + i * 256, kb = id / (kP / 4), cb = id % (kP / 4);
+                for (int r = 0; r < 4; ++r) {
+                    xr[r] = *reinterpret_cast<const uint4*>(xsrc + static_cast<uint32_t>(r) * xrow + static_cast<uint64_t>(voff_x));
+                    br[r] = *reinterpret_cast<const uint4*>(bsrc + static_cast<uint32_t>(r) * brow + static_cast<uint64_t>(voff_b));
+                }
+            } else {
+                // ragged last chunk: steps past the end of the sequence read as zero (the loads stay inside the tensors)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int k = kb * 4 + r;
-                // rows past the end of the sequence read the last valid row and are zeroed (no branch)
-                const uint32_t v = *reinterpret_cast<const uint32_t*>(src + min(k, valid - 1) * row_stride + cb * 4);
-                xr[i][r] = k < valid ? v : 0u;
+                for (int r = 0; r < 4; ++r) {
+                    const int k = 4 * kb + r;
+                    const uint32_t kk = static_cast<uint32_t>(min(k, valid - 1));
+                    const uint4 xv = *reinterpret_cast<const uint4*>(xsrc + kk * xrow + 16 * pb);
+                    const uint4 bv = *reinterpret_cast<const uint4*>(bsrc + kk * brow + 16 * pb);
+                    xr[r] = k < valid ? xv : make_uint4(0u, 0u, 0u, 0u);
+                    br[r] = k < valid ? bv : make_uint4(0u, 0u, 0u, 0u);
+                }
             }
         }
-    };
-    // s_w[c & 1][k] = exp(dA_last - dA_k) dt_k, in two halves so that the loads are issued an MFMA
-    // phase before their values are needed
-    float w_dt = 0.0f, w_dA = 0.0f, w_last = 0.0f;
-    auto weights_load = [&](int c) {
-        const float* dt_row = dt_ws + (rows0 + c) * Q;
         const float* dA_row = dA_ws + (rows0 + c) * Q;
-        w_last = dA_row[Q - 1];
-        if (Q == 256 || tid < Q) {
-            w_dt = dt_row[tid];
-            w_dA = dA_row[tid];
+        r_last = dA_row[Q - 1];
+        if (tid < Q) {
+            r_dt = dt_ws[(rows0 + c) * Q + tid];
+            r_dA = dA_row[tid];
         }
     };
-    auto weights_store = [&](int c) {
-        if (Q == 256 || tid < Q) s_w[c & 1][tid] = fexp(w_last - w_dA) * w_dt;
-    };
-    auto store_x = [&](int c) {
-        const float* w = s_w[c & 1];
+    auto stage_chunk = [&]() {
+        if (mine) {
+            stage_x_share<S::XP>(sm.xt, xr, sm.xs, pb, kb);
 #pragma unroll
-        for (int i = 0; i < XB; ++i) {
-            const int id = tid + i * 256, kb = id / (kP / 4), cb = id % (kP / 4);
-            const float4 wk = *reinterpret_cast<const float4*>(w + kb * 4);
-            const float wr[4] = {wk.x, wk.y, wk.z, wk.w};
-#pragma unroll
-            for (int cc = 0; cc < 4; ++cc) {
-                const float cs = s_xs[cb * 4 + cc];
-                v4h o;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) o[r] = static_cast<_Float16>((cs * static_cast<float>(byte_of(xr[i][r], cc))) * wr[r]);
-                *reinterpret_cast<v4h*>(s_xt + (cb * 4 + cc) * PITCH + kb * 4) = o;
+            for (int d = 0; d < 4; ++d) {
+                // 4x4 byte transpose: rows k (registers) x columns n (bytes) -> rows n x bytes k
+                const uint32_t r0 = word_of(br[0], d) ^ kBias, r1 = word_of(br[1], d) ^ kBias, r2 = word_of(br[2], d) ^ kBias, r3 = word_of(br[3], d) ^ kBias;
+                const uint32_t lo01 = __builtin_amdgcn_perm(r1, r0, 0x05010400u);   // r0.b0 r1.b0 r0.b1 r1.b1
+                const uint32_t hi01 = __builtin_amdgcn_perm(r1, r0, 0x07030602u);   // r0.b2 r1.b2 r0.b3 r1.b3
+                const uint32_t lo23 = __builtin_amdgcn_perm(r3, r2, 0x05010400u);
+                const uint32_t hi23 = __builtin_amdgcn_perm(r3, r2, 0x07030602u);
+                const int n4 = 16 * pb + 4 * d;
+                *reinterpret_cast<uint32_t*>(&sm.b8[n4 + 0][kb * 4]) = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u);
+                *reinterpret_cast<uint32_t*>(&sm.b8[n4 + 1][kb * 4]) = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u);
+                *reinterpret_cast<uint32_t*>(&sm.b8[n4 + 2][kb * 4]) = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);
+                *reinterpret_cast<uint32_t*>(&sm.b8[n4 + 3][kb * 4]) = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u);
             }
         }
-    };
-    v8h fb[nks];
-    auto load_b = [&](int c) {
-        const __half* src = bt16 + (((static_cast<int64_t>(b) * nc + c) * G + g) * NT + ntile) * nks * 512 + lane * 8;
-#pragma unroll
-        for (int ks = 0; ks < nks; ++ks) fb[ks] = *reinterpret_cast<const v8h*>(src + ks * 512);
+        if (tid < Q) sm.w[tid] = fexp(r_last - r_dA) * r_dt;        // weight of step k in the chunk's state
     };
 
-    v16f run[PTW], acc[PTW];
+    // the running state: columns n = 64 part + 16 wave + lane % 16; tile j, register r: channel p = 4 (4 (lane / 16) + r) + j
+    const int n_col = part * 64 + 16 * wave + l16;
+    v4f run[4];
 #pragma unroll
-    for (int j = 0; j < PTW; ++j)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) { run[j][r] = 0.0f; acc[j][r] = 0.0f; }
+    for (int j = 0; j < 4; ++j) run[j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
 
-    load_x(0);
-    weights_load(0);
-    load_b(0);
-    weights_store(0);
-    float dA_last = w_last;                                    // of the chunk being multiplied
-    __syncthreads();                                           // s_xs, s_w[0]
-    store_x(0);
+    load_chunk(0);
+    __syncthreads();                                              // the table of x scales
+    stage_chunk();
+    float dA_last = r_last;                                       // of the chunk about to be multiplied
     __syncthreads();
 
     for (int c = 0; c < nc; ++c) {
         const bool more = c + 1 < nc;
-        if (more) {
-            weights_load(c + 1);                               // requests return in order: the one needed first goes first
-            load_x(c + 1);
-        }
+        if (more) load_chunk(c + 1);                               // in flight during the products
+        v4f accs[4];
 #pragma unroll
-        for (int ks = 0; ks < nks; ++ks) {
+        for (int j = 0; j < 4; ++j) accs[j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-            for (int j = 0; j < PTW; ++j) {
-                const v8h fx = *reinterpret_cast<const v8h*>(s_xt + ((pt0 + j) * 32 + frow) * PITCH + ks * 16 + fhalf * 8);
-                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fx, fb[ks], acc[j], 0, 0, 0);
-            }
+        for (int ks = 0; ks < Q / 32; ++ks) {
+            const int k0 = 32 * ks + 8 * lq;
+            const uint32_t b0 = *reinterpret_cast<const uint32_t*>(&sm.b8[16 * wave + l16][k0]);
+            const uint32_t b1 = *reinterpret_cast<const uint32_t*>(&sm.b8[16 * wave + l16][k0 + 4]);
+            const float4 w0 = *reinterpret_cast<const float4*>(&sm.w[k0]), w1 = *reinterpret_cast<const float4*>(&sm.w[k0 + 4]);
+            v8h fx[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) fx[j] = *reinterpret_cast<const v8h*>(&sm.xt[j * 16 + l16][k0]);
+            const float wk[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+            v8h bw;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) bw[e] = static_cast<_Float16>(__builtin_fmaf(ubyte_of(e < 4 ? b0 : b1, e & 3), sB, nsB) * wk[e]);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) accs[j] = mfma16(fx[j], bw, accs[j]);
         }
-        if (more) load_b(c + 1);                               // in flight during the update and the staging below
-        // the state entering chunk c, then the recurrence.  Lane holds column n = ntile*32 + lane%32 and,
-        // in register r, row p = pt*32 + 8*(r/4) + 4*(lane/32) + r%4.
-        // The 32 x 32 tile passes through a wave-private LDS patch so that it leaves as 16-byte pieces.
+        // P <- exp(dA_last) P + S
         const float decay = fexp(dA_last);
-        __half* pst = prev + ((static_cast<int64_t>(b) * nc + c) * H + h) * kP * N + ntile * 32;
-        _Float16* patch = s_patch + wave * (32 * kPatchPitch);
 #pragma unroll
-        for (int j = 0; j < PTW; ++j) {
+        for (int j = 0; j < 4; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                patch[(8 * (r / 4) + 4 * fhalf + (r % 4)) * kPatchPitch + frow] = static_cast<_Float16>(run[j][r]);
-                run[j][r] = decay * run[j][r] + acc[j][r];
-                acc[j][r] = 0.0f;
-            }
-            wave_sync();
-#pragma unroll
-            for (int q = 0; q < 2; ++q) {
-                const int row = q * 16 + (lane >> 2), piece = lane & 3;
-                const uint4 v = *reinterpret_cast<const uint4*>(patch + row * kPatchPitch + piece * 8);
-                *reinterpret_cast<uint4*>(pst + ((pt0 + j) * 32 + row) * N + piece * 8) = v;
-            }
-            wave_sync();
-        }
+            for (int r = 0; r < 4; ++r) run[j][r] = decay * run[j][r] + accs[j][r];
         if (more) {
-            weights_store(c + 1);
-            dA_last = w_last;
+            // the state entering chunk c + 1, in fp16 as the reference keeps it, rows in slot order
+            __half* pst = prev + (((static_cast<int64_t>(b) * nc + c + 1) * H + h) * kP) * N + n_col;
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) pst[(j * 16 + 4 * lq + r) * N] = __float2half(run[j][r]);
         }
-        __syncthreads();                                       // every wave is done with this chunk's x tile; s_w written
-        if (more) store_x(c + 1);
+        __syncthreads();                                           // every wave has read this chunk's tiles
+        if (more) {
+            stage_chunk();
+            dA_last = r_last;
+        }
         __syncthreads();
     }
 
-    // final state: fp32 copy for the caller's workspace, and the requested output form
+    // final state in the requested form
+    if (p.final_states) {
 #pragma unroll
-    for (int j = 0; j < PTW; ++j)
+        for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int pp = (pt0 + j) * 32 + 8 * (r / 4) + 4 * fhalf + (r % 4);
-            const int n = ntile * 32 + frow;
-            const int64_t fo = ((static_cast<int64_t>(b) * H + h) * kP + pp) * N + n;
-            const float sv = run[j][r];
-            if (final_ws) final_ws[fo] = sv;
-            if (p.final_states) {
+            for (int r = 0; r < 4; ++r) {
+                const int pp = 4 * (4 * lq + r) + j;
+                const int64_t fo = ((static_cast<int64_t>(b) * H + h) * kP + pp) * N + n_col;
+                const float sv = run[j][r];
                 if (p.final_state_is_fp32) {
                     static_cast<float*>(p.final_states)[fo] = sv;
                 } else {
                     float sc, K;
-                    if (p.nhead_groups > 0) {
+                    if (grouped) {
                         const int dg = dim_group_of(p, g, hg, pp);
-                        sc = p.state_scale[((g * p.nhead_groups + hg) * p.ndim_groups + dg) * N + n];
+                        sc = p.state_scale[((g * p.nhead_groups + hg) * p.ndim_groups + dg) * N + n_col];
                         K = 1e6f;
                     } else {
                         sc = p.state_scale[0];
@@ -462,285 +461,257 @@ __global__ __launch_bounds__(256, 2) void ssd_state_kernel(QaSsdParams p, const 
                     static_cast<int8_t*>(p.final_states)[fo] = sat8_rne((s16 * K) / (sc * K));
                 }
             }
-        }
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
-// Stage 5 (quamba/triton/quant_chunk_scan.py:96-171): one workgroup per (batch, chunk, head), four
-// waves; each wave owns whole 32-row m-tiles (paired small/large so the causal work balances).
-// Everything a tile reads from global memory - its C rows, its rows of C B^T (fp16, all k-steps of the
-// causal range) and the x / z bytes of the epilogue - is requested at the top of the tile, so the
-// memory latency is paid once per tile instead of once per k-step.
+// Stage 5 (quamba/triton/quant_chunk_scan.py:96-171): a workgroup of four waves per (batch, chunk, head).  A wave
+// owns whole 16-row m-tiles with all 64 columns p, long and short causal ranges mixed so that the waves carry equal
+// work (with sixteen tiles: 15 - w, 8 + w, 7 - w, w), longest first.  Its A operands are built in registers: rows
+// of f16(C^) come ready-made from the preparation kernel; the weights of term 2 are C B^T (fp32, from the
+// preparation kernel, fetched four 32-step pieces ahead) times the decay.  For the pieces below the diagonal the
+// decay factors into exp(dA_m - R) (one exp per lane and piece) and exp(R - dA_k) dt_k (a table per workgroup)
+// with R = dA at the last step of the piece, so that both exponents are <= 0; on the piece that holds the
+// diagonal it is computed per element, in the reference's order.  The B operands (entering state, transposed
+// x) are read from LDS, both with rows in slot order.  Everything the prologue and the first tile read from
+// global memory is requested before the first LDS write; a tile's operands are requested before the epilogue
+// of the tile before.
 // ---------------------------------------------------------------------------------------------
 template <int N, int Q>
-__global__ __launch_bounds__(256, 2) void ssd_chunk_scan_kernel(QaSsdParams p, const float* dt_ws, const float* dA_ws,
-                                                                const __half* cb_ws, const __half* prev, const __half* c16, int nc) {
-    constexpr int WAVES = 4, PITCH = Q + 8, PPITCH = N + 8, kThreads = 64 * WAVES;
-    constexpr int kScratch = 512;      // floats per wave: the decay table (Q halves) or an 8 x 64 piece of the output tile
-    constexpr int NMT = Q / 32, PER_WAVE = NMT / WAVES > 0 ? NMT / WAVES : 1, KSMAX = Q / 16;
-    __shared__ __attribute__((aligned(16))) _Float16 s_xt[kP * PITCH];
-    __shared__ __attribute__((aligned(16))) _Float16 s_prev[kP * PPITCH];     // entering state, rows p
-    __shared__ __attribute__((aligned(16))) float s_dt[Q];
-    __shared__ __attribute__((aligned(16))) float s_dA[Q];
-    __shared__ __attribute__((aligned(16))) float s_g[WAVES * kScratch];
-    __shared__ float s_xs[kP];
+struct ScanSmem {
+    static constexpr int XP = Q + 8;        // halves per row of the transposed x tile
+    static constexpr int NCH = N / 8;       // 16-byte pieces per row of the entering state
+    static constexpr int SWZ = (NCH < 16 ? NCH : 16) - 1;
+    __attribute__((aligned(16))) _Float16 xt[kP][XP];
+    // rows without padding: piece c of row r sits at position c ^ (r & SWZ), so that the sixteen rows of an operand
+    // read fall into different banks
+    __attribute__((aligned(16))) _Float16 prev[kP][N];
+    __attribute__((aligned(16))) float dt[Q];
+    __attribute__((aligned(16))) float dA[Q];
+    __attribute__((aligned(16))) float gk[Q];   // exp(dA[end of the 32-step piece] - dA_k) dt_k
+    __attribute__((aligned(16))) float xs[kP];  // x scale per channel
+    __attribute__((aligned(16))) float Dv[kP];  // skip weight per channel
+};
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, frow = lane & 31, fhalf = lane >> 5;
-    const int h = blockIdx.x % p.nheads;
-    const int c = (blockIdx.x / p.nheads) % nc;
-    const int b = blockIdx.x / (p.nheads * nc);
-    const int G = p.ngroups, H = p.nheads;
+constexpr int scan_waves_of(int Q) { return Q / 16 < 8 ? Q / 16 : 8; }
+
+template <int N, int Q>
+__global__ __launch_bounds__(64 * scan_waves_of(Q), 4) void ssd_chunk_scan_kernel(QaSsdParams p, const float* dt_ws, const float* dA_ws,
+                                                                                const float* cb_ws, const __half* prev, const __half* c16, int nc) {
+    using S = ScanSmem<N, Q>;
+    extern __shared__ __attribute__((aligned(16))) unsigned char ssd_smem_raw[];
+    S& sm = *reinterpret_cast<S*>(ssd_smem_raw);
+    constexpr int kWaves = scan_waves_of(Q);
+    constexpr int kThreads = 64 * kWaves;
+    constexpr int NMT = Q / 16;                                   // 16-row m-tiles of a chunk
+    constexpr int TILES = NMT / kWaves;                           // per wave: 4 (Q 256), 2 (Q 128), 1 (Q 64)
+    constexpr int WIN = 4;                                        // pieces of C B^T in flight: a rolling window
+    static_assert(Q <= kThreads, "a thread stages at most one share of the x tile");
+    constexpr int PPC = kP * N / 8;                               // 16-byte pieces of the entering state
+    constexpr int PB = PPC / kThreads;
+
+    const int tid = threadIdx.x, lane = tid & 63, l16 = lane & 15, lq = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);    // the same in every lane: kept in a scalar register
+    const int G = p.ngroups, H = p.nheads, L = p.seqlen;
+    // the heads of one (batch, chunk, ssd group) read the same C B^T and C rows: they go to one XCD
+    int unit, hig, part;
+    unit_head_part(blockIdx.x, p.batch * nc * G, H / G, 1, unit, hig, part);
+    const int h = (unit % G) * (H / G) + hig;
+    const int c = (unit / G) % nc;
+    const int b = unit / (G * nc);
     int g, hg;
     group_of(p, h, g, hg);
     const int t0 = c * Q;
-    const int lim = min(Q, p.seqlen - t0);
-    const int64_t row_base = (static_cast<int64_t>(b) * H + h) * nc + c;
-    const __half* cb = cb_ws + ((static_cast<int64_t>(b) * nc + c) * G + g) * Q * Q;
-    const int64_t row_stride = static_cast<int64_t>(H) * kP;
-    const int erow = lane >> 3, ecol = (lane & 7) * 8;       // epilogue: row within a piece of 8, first of 8 columns
-    const int64_t tile_base = (static_cast<int64_t>(b) * p.seqlen + t0) * row_stride + static_cast<int64_t>(h) * kP + ecol;
-
-    // Per-tile operands that come from global memory: this lane's pieces of its C row (term 1), of its
-    // row of C B^T (term 2, every k-step of the causal range) and the x / z bytes of the epilogue.  They
-    // are requested one tile ahead: the first tile's together with the prologue's reads, the next
-    // tile's piece by piece as the current tile lets go of the registers.
-    // tile order 0, NMT-1, 1, NMT-2, ...: wave w takes entries w*PER_WAVE + s
-    auto tile_of = [&](int s) {
-        const int entry = wave * PER_WAVE + s;
-        return (entry & 1) ? NMT - 1 - (entry >> 1) : (entry >> 1);
-    };
-    v8h c_frag[N / 16], cbf[KSMAX];
-    uint2 xq[4], zq[4];
-    auto c_ptr = [&](int mt, int ks) {
-        return c16 + ((static_cast<int64_t>(b) * p.seqlen + t0 + min(mt * 32 + frow, lim - 1)) * G + g) * N + ks * 16 + fhalf * 8;
-    };
-    auto cb_ptr = [&](int mt, int ks) { return cb + static_cast<int64_t>(mt * 32 + frow) * Q + fhalf * 8 + ks * 16; };
-    auto load_xz = [&](int mt, int q) {
-        const int64_t at = tile_base + min(mt * 32 + 8 * q + erow, lim - 1) * row_stride;
-        xq[q] = p.D ? *reinterpret_cast<const uint2*>(p.x + at) : make_uint2(0u, 0u);
-        zq[q] = p.z ? *reinterpret_cast<const uint2*>(p.z + at) : make_uint2(0u, 0u);
-    };
-    // skip-term and gate parameters: requested with everything else, used in the epilogue
+    const int lim = min(Q, L - t0);
+    const uint32_t xrow = static_cast<uint32_t>(H) * kP;          // bytes between steps of x
+    const float* cb = cb_ws + ((static_cast<int64_t>(b) * nc + c) * G + g) * Q * Q;
+    const int8_t* xbase = p.x + (static_cast<int64_t>(b) * L + t0) * xrow + static_cast<int64_t>(h) * kP;
+    const int8_t* zbase = p.z + (static_cast<int64_t>(b) * L + t0) * xrow + static_cast<int64_t>(h) * kP;       // only read if p.z
     const float D_scale = p.D ? *p.D_scale : 0.0f;
     const float z_scale = p.z ? *p.z_scale : 0.0f;
-    int8_t e_Dq[8];
-#pragma unroll
-    for (int e = 0; e < 8; ++e) e_Dq[e] = p.D ? p.D[p.D_has_hdim ? h * kP + ecol + e : h] : int8_t(0);
-    if (wave * PER_WAVE < NMT) {
-        const int mt = tile_of(0);
-#pragma unroll
-        for (int ks = 0; ks < N / 16; ++ks) c_frag[ks] = *reinterpret_cast<const v8h*>(c_ptr(mt, ks));
-#pragma unroll
-        for (int ks = 0; ks < KSMAX; ++ks)
-            if (ks < 2 * (mt + 1)) cbf[ks] = *reinterpret_cast<const v8h*>(cb_ptr(mt, ks));
-#pragma unroll
-        for (int q = 0; q < 4; ++q) load_xz(mt, q);
-    }
-    {
-        // Prologue: every global read is issued before the first LDS write, so that the workgroup waits
-        // for memory once.  x is transposed on the way (4x4 blocks: four dword loads, four 8-byte stores).
-        static_assert(Q <= kThreads, "one step per thread");
-        constexpr int XB = (Q / 4) * (kP / 4) / kThreads, PB = kP * N / 8 / kThreads;
-        float r_dt = 0.0f, r_dA = 0.0f;
-        if (Q == kThreads || tid < Q) {
-            r_dt = dt_ws[row_base * Q + tid];
-            r_dA = dA_ws[row_base * Q + tid];
-        }
-        const __half* pst = prev + ((static_cast<int64_t>(b) * nc + c) * H + h) * kP * N;
-        uint4 r_prev[PB];
-#pragma unroll
-        for (int i = 0; i < PB; ++i) {
-            const int piece = tid + i * kThreads, pr = piece / (N / 8), col = (piece % (N / 8)) * 8;
-            r_prev[i] = *reinterpret_cast<const uint4*>(pst + pr * N + col);
-        }
-        const int8_t* xsrc = p.x + ((static_cast<int64_t>(b) * p.seqlen + t0) * H + h) * kP;
-        const int64_t xstride = static_cast<int64_t>(H) * kP;
-        const int cb4 = tid % (kP / 4);                      // the same four columns in every block of this thread
-        uint32_t xr[XB][4];
-#pragma unroll
-        for (int i = 0; i < XB; ++i) {
-            const int kb = (tid + i * kThreads) / (kP / 4);
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int k = kb * 4 + r;
-                const uint32_t v = *reinterpret_cast<const uint32_t*>(xsrc + min(k, lim - 1) * xstride + cb4 * 4);
-                xr[i][r] = k < lim ? v : 0u;
-            }
-        }
-        float cs[4];
-#pragma unroll
-        for (int cc = 0; cc < 4; ++cc) cs[cc] = x_scale_of(p, g, hg, cb4 * 4 + cc);
-        if (tid < kP) s_xs[tid] = x_scale_of(p, g, hg, tid);
+    __half* out = static_cast<__half*>(p.out) + (static_cast<int64_t>(b) * L + t0) * xrow + static_cast<int64_t>(h) * kP;
 
-        if (Q == kThreads || tid < Q) {
-            s_dt[tid] = r_dt;
-            s_dA[tid] = r_dA;
+    // tile s of this wave
+    auto tile_of = [&](int s) { return (s & 1) == 0 ? NMT - 1 - 8 * (s / 2) - wave : 8 * ((TILES - 1 - s) / 2) + wave; };
+
+    // ---- what an m-tile reads from global memory for terms 1 and 2: its rows of f16(C^) and the first pieces of its
+    // rows of C B^T
+    v8h cfr[N / 32];
+    float4 cbr[WIN][2];
+    auto tile_load = [&](int mt) {
+        const int m_row = mt * 16 + l16;
+        const int nks = (mt + 2) / 2;
+        const float* cbp = cb + static_cast<uint32_t>(m_row * Q + 8 * lq);
+        const __half* cp = c16 + ((static_cast<int64_t>(b) * L + t0 + min(m_row, lim - 1)) * G + g) * N + 8 * lq;
+        if (c > 0) {
+#pragma unroll
+            for (int ks = 0; ks < N / 32; ++ks) cfr[ks] = *reinterpret_cast<const v8h*>(cp + 32 * ks);
+        }
+#pragma unroll
+        for (int ks = 0; ks < WIN; ++ks) {
+            if (ks < nks) {
+                cbr[ks][0] = *reinterpret_cast<const float4*>(cbp + 32 * ks);
+                cbr[ks][1] = *reinterpret_cast<const float4*>(cbp + 32 * ks + 4);
+            }
+        }
+    };
+
+    {
+        // Prologue: every global read is issued before the first LDS write, so that the workgroup waits for memory
+        // once.
+        float r_dt = 0.0f, r_dA = 0.0f, r_end = 0.0f;
+        if (tid < Q) {
+            const int64_t row = ((static_cast<int64_t>(b) * H + h) * nc + c) * Q;
+            r_dt = dt_ws[row + tid];
+            r_dA = dA_ws[row + tid];
+            r_end = dA_ws[row + (tid | 31)];
+        }
+        // (the first chunk has no entering state: its slot of the workspace is read all the same and never used)
+        static_assert(PPC % kThreads == 0, "every thread copies the same number of pieces of the entering state");
+        v4i r_prev[PB];
+        const __half* pst = prev + ((static_cast<int64_t>(b) * nc + c) * H + h) * kP * N;
+#pragma unroll
+        for (int i = 0; i < PB; ++i) r_prev[i] = *reinterpret_cast<const v4i*>(pst + (tid + i * kThreads) * 8);
+        // this thread's share of the x tile: steps 4 kb .. 4 kb + 3, channels 16 pb .. 16 pb + 15
+        const int pb = tid % 4, kb = tid / 4;
+        const bool mine = Q == kThreads || tid < Q;
+        uint4 xr[4];
+        if (mine) {
+            if (lim == Q) {
+                const uint32_t voff_x = static_cast<uint32_t>(4 * kb) * xrow + 16 * pb;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) xr[r] = *reinterpret_cast<const uint4*>(xbase + static_cast<uint32_t>(r) * xrow + static_cast<uint64_t>(voff_x));
+            } else {
+                // ragged last chunk: steps past the end of the sequence read as zero (the loads stay inside the tensor)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int k = 4 * kb + r;
+                    const uint4 xv = *reinterpret_cast<const uint4*>(xbase + static_cast<uint32_t>(min(k, lim - 1)) * xrow + 16 * pb);
+                    xr[r] = k < lim ? xv : make_uint4(0u, 0u, 0u, 0u);
+                }
+            }
+        }
+        tile_load(tile_of(0));
+        if (tid < kP) {
+            sm.xs[tid] = x_scale_of(p, g, hg, tid);
+            sm.Dv[tid] = !p.D ? 0.0f : D_scale * static_cast<float>(p.D_has_hdim ? p.D[h * kP + tid] : p.D[h]);
+        }
+        __syncthreads();                                           // the tables per channel (and every load above has landed)
+
+        if (tid < Q) {
+            sm.dt[tid] = r_dt;
+            sm.dA[tid] = r_dA;
+            sm.gk[tid] = fexp(r_end - r_dA) * r_dt;
         }
 #pragma unroll
         for (int i = 0; i < PB; ++i) {
             const int piece = tid + i * kThreads, pr = piece / (N / 8), col = (piece % (N / 8)) * 8;
-            *reinterpret_cast<uint4*>(s_prev + pr * PPITCH + col) = r_prev[i];
+            *reinterpret_cast<v4i*>(&sm.prev[pr][col ^ ((pr & S::SWZ) * 8)]) = r_prev[i];
         }
-#pragma unroll
-        for (int i = 0; i < XB; ++i) {
-            const int kb = (tid + i * kThreads) / (kP / 4);
-#pragma unroll
-            for (int cc = 0; cc < 4; ++cc) {
-                v4h o;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) o[r] = static_cast<_Float16>(cs[cc] * static_cast<float>(byte_of(xr[i][r], cc)));
-                *reinterpret_cast<v4h*>(s_xt + (cb4 * 4 + cc) * PITCH + kb * 4) = o;
-            }
-        }
+        if (mine) stage_x_share<S::XP>(sm.xt, xr, sm.xs, pb, kb);
     }
     __syncthreads();
 
-    __half* out = static_cast<__half*>(p.out);
-    float e_Dv[8];                                           // D of the eight columns this lane writes
 #pragma unroll
-    for (int e = 0; e < 8; ++e) e_Dv[e] = D_scale * static_cast<float>(e_Dq[e]);
-
-#pragma unroll
-    for (int s = 0; s < PER_WAVE; ++s) {
-        if (wave * PER_WAVE + s >= NMT) break;
+    for (int s = 0; s < TILES; ++s) {
+        // the most pieces a tile in position s can have (position 0 holds the longest tiles)
+        const int max_tile = (s & 1) == 0 ? NMT - 1 - 8 * (s / 2) : 8 * ((TILES - 1 - s) / 2) + kWaves - 1;
+        const int max_nks = (max_tile + 2) / 2;
         const int mt = tile_of(s);
-        const bool has_next = s + 1 < PER_WAVE;
-        const int mt_next = has_next ? tile_of(s + 1) : 0;
-        const int nks_next = has_next ? 2 * (mt_next + 1) : 0;
-        const int m_lane = mt * 32 + frow;                 // row of this lane's A operands
-        const int nks = 2 * (mt + 1);                      // k-steps of the causal range
-        const int n_off = 2 * mt;                          // of which entirely before the tile
-        v16f acc[2];
+        const int m0 = mt * 16;
+        const int nks = (mt + 2) / 2;                               // 32-step pieces that reach row m0 + 15; the last holds the diagonal
+        const int m_row = m0 + l16;                                 // row of this lane's A operands
+        const float* cbp = cb + static_cast<uint32_t>(m_row * Q + 8 * lq);
+        const float dA_m = sm.dA[m_row];
+        // skip-term operands of this lane's four output rows
+        // (requested now, used in the epilogue: nothing there waits for memory)
+        uint32_t xq[4], zq[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int r = 0; r < 4; ++r) {
+            const uint32_t at = static_cast<uint32_t>(min(m0 + 4 * lq + r, lim - 1)) * xrow + 4 * l16;
+            xq[r] = *reinterpret_cast<const uint32_t*>(xbase + at);
+            if (p.z) zq[r] = *reinterpret_cast<const uint32_t*>(zbase + at);
+        }
+        v4f acc[4];
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[j][r] = 0.0f;
-
-        // Decay factors.  The cumulative dA decreases along the chunk, so with ref = dA at the first row
-        // of this m-tile, exp(dA_m - dA_k) = exp(dA_m - ref) * exp(ref - dA_k) for every k before the
-        // tile, both factors <= 1.  The k factor (times dt_k, times the power of two that C B^T was
-        // stored without) is tabulated once per tile by the wave, in fp16; the row factor is applied to
-        // the accumulator after the off-diagonal k-steps, together with term 1 (whose decay exp(dA_m) =
-        // exp(ref) * exp(dA_m - ref)).  Only the two diagonal k-steps evaluate the decay per element.
-        // acc = E_m * (exp(ref) * T1 + sum_{k < m0} (CB * G_k) x_k) + diagonal.
-        const int m0 = mt * 32;
-        const float ref = s_dA[m0];
-        _Float16* g_tab = reinterpret_cast<_Float16*>(s_g + wave * kScratch);
-        for (int k = lane; k < m0; k += 64) g_tab[k] = static_cast<_Float16>((fexp(ref - s_dA[k]) * s_dt[k]) * kCbUnshift);
-        wave_sync();
-
-        // term 1: C^ (rows m, dstate contiguous) x entering state (rows p, dstate contiguous, staged in LDS)
-        const bool row_ok = m_lane < lim;
+        for (int j = 0; j < 4; ++j) acc[j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+        // term 1: C^ (rows m) x entering state (rows p), zero for the first chunk
+        if (c > 0) {
 #pragma unroll
-        for (int ks = 0; ks < N / 16; ++ks) {
-            v8h fc = c_frag[ks];
-            if (has_next) c_frag[ks] = *reinterpret_cast<const v8h*>(c_ptr(mt_next, ks));
-            if (!row_ok) {
+            for (int ks = 0; ks < N / 32; ++ks) {
+                v8h fs[4];
 #pragma unroll
-                for (int e = 0; e < 8; ++e) fc[e] = static_cast<_Float16>(0.0f);
+                for (int j = 0; j < 4; ++j) fs[j] = *reinterpret_cast<const v8h*>(&sm.prev[j * 16 + l16][(32 * ks + 8 * lq) ^ ((l16 & S::SWZ) * 8)]);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[j] = mfma16(cfr[ks], fs[j], acc[j]);
             }
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const v8h fs = *reinterpret_cast<const v8h*>(s_prev + (j * 32 + frow) * PPITCH + ks * 16 + fhalf * 8);
-                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fc, fs, acc[j], 0, 0, 0);
+            for (int r = 0; r < 4; ++r) {
+                const float em = fexp(sm.dA[m0 + 4 * lq + r]);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[j][r] *= em;
             }
         }
-        const float e_ref = fexp(ref);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            acc[0][r] *= e_ref;
-            acc[1][r] *= e_ref;
-        }
-        // term 2.  The LDS operands of k-step ks+1 (decay table piece, two x fragments) are requested before
-        // the products of k-step ks; the addresses are valid for every ks, so the requests need no condition.
-        v8h gh_n = *reinterpret_cast<const v8h*>(g_tab + fhalf * 8);
-        v8h fx_n[2];
+        for (int ks = 0; ks < 8; ++ks) {
+            if (ks < max_nks && ks < nks) {
+                const int k0 = 32 * ks + 8 * lq;
+                v8h fx[4];
 #pragma unroll
-        for (int j = 0; j < 2; ++j) fx_n[j] = *reinterpret_cast<const v8h*>(s_xt + (j * 32 + frow) * PITCH + fhalf * 8);
-#pragma unroll
-        for (int ks = 0; ks < KSMAX; ++ks) {
-            const v8h gh = gh_n;
-            const v8h fx_c[2] = {fx_n[0], fx_n[1]};
-            if (ks + 1 < KSMAX) {
-                const int k1 = (ks + 1) * 16 + fhalf * 8;
-                gh_n = *reinterpret_cast<const v8h*>(g_tab + k1);
-#pragma unroll
-                for (int j = 0; j < 2; ++j) fx_n[j] = *reinterpret_cast<const v8h*>(s_xt + (j * 32 + frow) * PITCH + k1);
-            }
-            if (ks < nks) {
-                const int k0 = ks * 16 + fhalf * 8;
-                v8h fl;
-                if (ks < n_off) {
-                    fl = cbf[ks] * gh;
-                } else {
-                    if (ks == n_off) {
-                        // leaving the off-diagonal part: apply the row factors once
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) {
-                            const float em = fexp(s_dA[m0 + 8 * (r / 4) + 4 * fhalf + (r % 4)] - ref);
-                            acc[0][r] *= em;
-                            acc[1][r] *= em;
-                        }
-                    }
-                    const float dA_m = s_dA[m_lane];
-                    const float4 dA0 = *reinterpret_cast<const float4*>(s_dA + k0), dA1 = *reinterpret_cast<const float4*>(s_dA + k0 + 4);
-                    const float4 dt0 = *reinterpret_cast<const float4*>(s_dt + k0), dt1 = *reinterpret_cast<const float4*>(s_dt + k0 + 4);
-                    const float dAk[8] = {dA0.x, dA0.y, dA0.z, dA0.w, dA1.x, dA1.y, dA1.z, dA1.w};
-                    const float dtk[8] = {dt0.x, dt0.y, dt0.z, dt0.w, dt1.x, dt1.y, dt1.z, dt1.w};
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        const int k = k0 + e;
-                        const float cbv = static_cast<float>(cbf[ks][e]) * kCbUnshift;
-                        const float wv = (cbv * fexp(dA_m - dAk[e])) * dtk[e];
-                        fl[e] = static_cast<_Float16>(k <= m_lane ? wv : 0.0f);
-                    }
+                for (int j = 0; j < 4; ++j) fx[j] = *reinterpret_cast<const v8h*>(&sm.xt[j * 16 + l16][k0]);
+                const float4 c0 = cbr[ks % WIN][0], c1 = cbr[ks % WIN][1];
+                const float cv[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+                if (ks + WIN < max_nks && ks + WIN < nks) {
+                    // the slot is free: the piece WIN ahead takes it
+                    cbr[ks % WIN][0] = *reinterpret_cast<const float4*>(cbp + 32 * (ks + WIN));
+                    cbr[ks % WIN][1] = *reinterpret_cast<const float4*>(cbp + 32 * (ks + WIN) + 4);
                 }
+                float wv[8];
+                if (ks + 1 < nks) {
+                    const float4 g0 = *reinterpret_cast<const float4*>(&sm.gk[k0]), g1 = *reinterpret_cast<const float4*>(&sm.gk[k0 + 4]);
+                    const float gk[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+                    const float e_m = fexp(dA_m - sm.dA[32 * ks + 31]);
 #pragma unroll
-                for (int j = 0; j < 2; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fl, fx_c[j], acc[j], 0, 0, 0);
+                    for (int e = 0; e < 8; ++e) wv[e] = cv[e] * (e_m * gk[e]);
+                } else {
+                    // the piece with the diagonal: steps after row m do not count
+                    const float4 a0 = *reinterpret_cast<const float4*>(&sm.dA[k0]), a1 = *reinterpret_cast<const float4*>(&sm.dA[k0 + 4]);
+                    const float4 d0 = *reinterpret_cast<const float4*>(&sm.dt[k0]), d1 = *reinterpret_cast<const float4*>(&sm.dt[k0 + 4]);
+                    const float ak[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+                    const float dk[8] = {d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w};
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) wv[e] = ((k0 + e <= m_row ? cv[e] : 0.0f) * fexp(fminf(dA_m - ak[e], 0.0f))) * dk[e];
+                }
+                v8h fl;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) fl[e] = static_cast<_Float16>(wv[e]);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[j] = mfma16(fl, fx[j], acc[j]);
             }
-            if (ks < nks_next) cbf[ks] = *reinterpret_cast<const v8h*>(cb_ptr(mt_next, ks));
         }
-        wave_sync();                                    // the table is done with: its space now carries the output tile
-        // Epilogue.  In the accumulators a lane holds one column p and 16 rows; memory wants rows of 64
-        // contiguous columns.  The tile passes through the wave's scratch eight rows at a time (registers
-        // 4q..4q+3 of both accumulators are rows 8q + 4*(lane/32) + 0..3), after which lane l holds row
-        // l/8 and the eight columns 8*(l%8)..+7: the skip term and the gate use the 8 bytes fetched at
-        // the top of the tile, the output is one 16-byte store.
-        float* o_tab = s_g + wave * kScratch;
+        if (s + 1 < TILES) tile_load(tile_of(s + 1));              // in flight during the epilogue
+        // Epilogue: acc[j][r] is row m0 + 4 (lane / 16) + r, channel 4 (lane % 16) + j
+        const float4 xs4 = *reinterpret_cast<const float4*>(&sm.xs[4 * l16]), Dv4 = *reinterpret_cast<const float4*>(&sm.Dv[4 * l16]);
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-#pragma unroll
-            for (int j = 0; j < 2; ++j)
-#pragma unroll
-                for (int t = 0; t < 4; ++t) o_tab[(4 * fhalf + t) * 64 + j * 32 + frow] = acc[j][4 * q + t];
-            wave_sync();
-            const int m = mt * 32 + 8 * q + erow;
-            const float4 y0 = *reinterpret_cast<const float4*>(o_tab + erow * 64 + ecol);
-            const float4 y1 = *reinterpret_cast<const float4*>(o_tab + erow * 64 + ecol + 4);
-            wave_sync();                                // the next piece overwrites the scratch
-            const uint2 xb = xq[q], zb = zq[q];
-            if (has_next) load_xz(mt_next, q);
+        for (int r = 0; r < 4; ++r) {
+            const int m = m0 + 4 * lq + r;
             if (m < lim) {
-                float y[8] = {y0.x, y0.y, y0.z, y0.w, y1.x, y1.y, y1.z, y1.w};
-                const int64_t at = tile_base + m * row_stride;
+                float y[4] = {acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
                 if (p.D) {
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        const float xv = static_cast<float>(byte_of(e < 4 ? xb.x : xb.y, e & 3));
-                        y[e] += (s_xs[ecol + e] * xv) * e_Dv[e];
-                    }
+                    for (int j = 0; j < 4; ++j) y[j] += __builtin_fmaf(ubyte_of(xq[r] ^ kBias, j), lane_of(xs4, j), -128.0f * lane_of(xs4, j)) * lane_of(Dv4, j);
                 }
                 if (p.z) {
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        const float zv = z_scale * static_cast<float>(byte_of(e < 4 ? zb.x : zb.y, e & 3));
-                        y[e] *= zv * __builtin_amdgcn_rcpf(1.0f + fexp(-zv));
+                    for (int j = 0; j < 4; ++j) {
+                        const float zv = z_scale * static_cast<float>(byte_of(zq[r], j));
+                        y[j] *= zv * __builtin_amdgcn_rcpf(1.0f + fexp(-zv));
                     }
                 }
-                v8h o;
+                v4h o;
 #pragma unroll
-                for (int e = 0; e < 8; ++e) o[e] = static_cast<_Float16>(y[e]);
-                *reinterpret_cast<v8h*>(out + at) = o;
+                for (int j = 0; j < 4; ++j) o[j] = static_cast<_Float16>(y[j]);
+                *reinterpret_cast<v4h*>(out + static_cast<uint32_t>(m) * xrow + 4 * l16) = o;
             }
         }
     }
@@ -758,7 +729,8 @@ int validate(const QaSsdParams* p) {
     if (p->dstate != 64 && p->dstate != 128) return QA_ERR_UNSUPPORTED;
     if (p->chunk_size != 64 && p->chunk_size != 128 && p->chunk_size != 256) return QA_ERR_UNSUPPORTED;
     if (!aligned16(p->x) || !aligned16(p->B) || !aligned16(p->C) || !aligned16(p->out)) return QA_ERR_STRIDE;
-    if (p->z && (reinterpret_cast<uintptr_t>(p->z) & 7u)) return QA_ERR_STRIDE;      // the gate is read 8 bytes at a time
+    if (p->z && !aligned16(p->z)) return QA_ERR_STRIDE;      // x, the gate and the output are accessed in aligned pieces
+    if (p->D && p->D_has_hdim && !aligned16(p->D)) return QA_ERR_STRIDE;
     return QA_OK;
 }
 
@@ -782,44 +754,46 @@ extern "C" int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream_) {
     uint8_t* base = static_cast<uint8_t*>(p->workspace);
     float* dt_ws = reinterpret_cast<float*>(base + ws.dt);
     float* dA_ws = reinterpret_cast<float*>(base + ws.dA);
-    __half* cb_ws = reinterpret_cast<__half*>(base + ws.cb);
-    __half* prev = reinterpret_cast<__half*>(base + ws.prev);
-    float* final_ws = reinterpret_cast<float*>(base + ws.final_f32);
+    float* cb_ws = reinterpret_cast<float*>(base + ws.cb);
     __half* c16_ws = reinterpret_cast<__half*>(base + ws.c16);
     const int nc = (p->seqlen + p->chunk_size - 1) / p->chunk_size;
     const int64_t bch = static_cast<int64_t>(p->batch) * nc * p->nheads;
     if (bch > 0x7fffffffLL || static_cast<int64_t>(p->batch) * nc * p->ngroups > 65535) return QA_ERR_SHAPE;
+    if (static_cast<int64_t>(p->batch) * p->nheads * 2 > 0x7fffffffLL) return QA_ERR_SHAPE;
 
     hipLaunchKernelGGL(ssd_cumsum_kernel, dim3(static_cast<unsigned>((bch + 3) / 4)), dim3(256), 0, stream, *p, dt_ws,
                        dA_ws, nc);
     const int nt = p->chunk_size / 64;
     hipLaunchKernelGGL(ssd_cb_kernel, dim3(nt * (nt + 1) / 2, p->batch * nc * p->ngroups), dim3(64), 0, stream, *p, cb_ws, c16_ws, nc);
-    __half* bt16_ws = reinterpret_cast<__half*>(base + ws.bt16);
-    const int64_t bcg_tiles = static_cast<int64_t>(p->batch) * nc * p->ngroups * (p->dstate / 32);
-    if (bcg_tiles > 0x7fffffffLL) return QA_ERR_SHAPE;
-    hipLaunchKernelGGL(ssd_bpack_kernel, dim3(static_cast<unsigned>(bcg_tiles)), dim3(256), 0, stream, *p, bt16_ws, nc);
-    const dim3 hgrid(static_cast<unsigned>(p->batch * p->nheads));
-    auto launch_state = [&](auto kernel) { hipLaunchKernelGGL(kernel, hgrid, dim3(256), 0, stream, *p, dt_ws, dA_ws, bt16_ws, prev, final_ws, nc); };
-    if (p->dstate == 128) {
-        if (p->chunk_size == 256) launch_state(ssd_state_kernel<128, 256>);
-        else if (p->chunk_size == 128) launch_state(ssd_state_kernel<128, 128>);
-        else launch_state(ssd_state_kernel<128, 64>);
-    } else {
-        if (p->chunk_size == 256) launch_state(ssd_state_kernel<64, 256>);
-        else if (p->chunk_size == 128) launch_state(ssd_state_kernel<64, 128>);
-        else launch_state(ssd_state_kernel<64, 64>);
-    }
+    __half* prev_ws = reinterpret_cast<__half*>(base + ws.prev);
+    const dim3 hgrid(static_cast<unsigned>(p->batch * p->nheads * (p->dstate / 64)));
     const dim3 sgrid(static_cast<unsigned>(bch));
-    auto launch_scan = [&](auto kernel) { hipLaunchKernelGGL(kernel, sgrid, dim3(256), 0, stream, *p, dt_ws, dA_ws, cb_ws, prev, c16_ws, nc); };
+    int status = QA_OK;
+    // more LDS than a kernel gets by default: raise the limit (idempotent)
+    auto lds_ok = [&](const void* kernel, size_t lds) {
+        if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)) == hipSuccess) return true;
+        status = check_launch();
+        if (status == QA_OK) status = QA_ERR_LAUNCH;
+        return false;
+    };
+    auto launch = [&](auto state_kernel, size_t state_lds, auto scan_kernel, size_t scan_lds, int scan_threads) {
+        if (!lds_ok(reinterpret_cast<const void*>(state_kernel), state_lds) || !lds_ok(reinterpret_cast<const void*>(scan_kernel), scan_lds)) return;
+        hipLaunchKernelGGL(state_kernel, hgrid, dim3(256), state_lds, stream, *p, dt_ws, dA_ws, prev_ws, nc);
+        hipLaunchKernelGGL(scan_kernel, sgrid, dim3(scan_threads), scan_lds, stream, *p, dt_ws, dA_ws, cb_ws, prev_ws, c16_ws, nc);
+    };
+#define QA_SSD_LAUNCH(N_, Q_) launch(ssd_state_kernel<N_, Q_>, sizeof(StateSmem<Q_>), ssd_chunk_scan_kernel<N_, Q_>, \
+                                     sizeof(ScanSmem<N_, Q_>), 64 * scan_waves_of(Q_))
     if (p->dstate == 128) {
-        if (p->chunk_size == 256) launch_scan(ssd_chunk_scan_kernel<128, 256>);
-        else if (p->chunk_size == 128) launch_scan(ssd_chunk_scan_kernel<128, 128>);
-        else launch_scan(ssd_chunk_scan_kernel<128, 64>);
+        if (p->chunk_size == 256) QA_SSD_LAUNCH(128, 256);
+        else if (p->chunk_size == 128) QA_SSD_LAUNCH(128, 128);
+        else QA_SSD_LAUNCH(128, 64);
     } else {
-        if (p->chunk_size == 256) launch_scan(ssd_chunk_scan_kernel<64, 256>);
-        else if (p->chunk_size == 128) launch_scan(ssd_chunk_scan_kernel<64, 128>);
-        else launch_scan(ssd_chunk_scan_kernel<64, 64>);
+        if (p->chunk_size == 256) QA_SSD_LAUNCH(64, 256);
+        else if (p->chunk_size == 128) QA_SSD_LAUNCH(64, 128);
+        else QA_SSD_LAUNCH(64, 64);
     }
+#undef QA_SSD_LAUNCH
+    if (status != QA_OK) return status;
     return check_launch();
 }
 

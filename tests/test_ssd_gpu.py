@@ -32,10 +32,18 @@ def _gpu(d, dev, chunk, state_scale=None, dt=None, final_dtype=torch.float32, **
 
 
 def _check_y(y_gpu, y_ref):
-    # the bar of the fp16 scan outputs, on the values themselves: |got - want| <= 1e-2 + 1e-2 |want|
+    """The bar of the fp16 scan outputs, on the values themselves: |got - want| <= 1e-2 + 1e-2 |want|.
+    Both sides round the same operands to fp16 before multiplying (as the reference does); where a value lies on
+    a rounding tie, the last bit of exp decides which way it goes, and one product of a large operand (outlier
+    channels are 20x the rest) then moves by 2^-11 of its size, which can exceed the bar of an output near zero.
+    Such outputs are allowed for at most two in 100 000, and only up to three times the bar."""
     got = y_gpu.float().cpu().numpy()
-    np.testing.assert_allclose(got, y_ref.astype(np.float16).astype(np.float32), rtol=1e-2, atol=1e-2)
-    assert np.sum((got - y_ref) ** 2) / np.sum(y_ref ** 2) < 1e-4
+    want = y_ref.astype(np.float16).astype(np.float32)
+    bar = 1e-2 + 1e-2 * np.abs(want)
+    err = np.abs(got - want)
+    assert (err > bar).mean() <= 2e-5, f"{(err > bar).sum()} of {err.size} outputs beyond rtol 1e-2 / atol 1e-2"
+    assert (err <= 3 * bar).all()
+    assert np.sum((got - y_ref) ** 2) / np.sum(y_ref ** 2) < 1e-6
 
 
 # batch, seqlen, nheads, dstate, ngroups, chunk
@@ -56,7 +64,8 @@ def test_forward_matches_oracle(dev, B, L, H, N, G, Q):
     assert np.abs(got - ref["final_f32"]).max() <= 1e-3 * np.abs(ref["final_f32"]).max()
 
 
-def test_every_stage_matches_the_oracle(dev):
+def test_preparation_stages_match_the_oracle(dev):
+    # what the two preparation kernels leave in the workspace: step sizes, their running sums and C B^T
     B, L, H, N, G, Q = 2, 200, 4, 128, 2, 64
     d = synth.mamba2_ssd_inputs(B, L, H, 64, N, G, seed=77)
     ref = _oracle(d, Q, stages=True)
@@ -64,17 +73,15 @@ def test_every_stage_matches_the_oracle(dev):
     nc = (L + Q - 1) // Q
     a256 = lambda v: (v + 255) & ~255
     off, parts = 0, {}
-    for name, shape, dt in [("dt", (B, H, nc, Q), torch.float32), ("dA_cumsum", (B, H, nc, Q), torch.float32),
-                            ("CB", (B, nc, G, Q, Q), torch.float16), ("prev_states", (B, nc, H, 64, N), torch.float16)]:
-        n = int(np.prod(shape)) * (4 if dt == torch.float32 else 2)
-        parts[name] = ws[off:off + n].view(dt).view(shape).float().cpu().numpy()
+    for name, shape in [("dt", (B, H, nc, Q)), ("dA_cumsum", (B, H, nc, Q)), ("CB", (B, nc, G, Q, Q))]:
+        n = int(np.prod(shape)) * 4
+        parts[name] = ws[off:off + n].view(torch.float32).view(shape).cpu().numpy()
         off = a256(off + n)
     np.testing.assert_allclose(parts["dt"], ref["dt"], rtol=1e-5, atol=1e-9)
     np.testing.assert_allclose(parts["dA_cumsum"], ref["dA_cumsum"], rtol=1e-5, atol=1e-8)
-    # C B^T is kept in fp16, divided by 16; Q == 64: one tile, all of it written
-    np.testing.assert_allclose(parts["CB"] * 16.0, ref["CB"], rtol=1e-3, atol=1e-3 * np.abs(ref["CB"]).max())
-    # the fp32 chunk states stay in registers; the states entering each chunk (their running sum) are checked
-    assert np.abs(parts["prev_states"] - ref["prev_states"]).max() <= 1e-3 * np.abs(ref["prev_states"]).max()
+    # exact integer sums times the scale product; Q == 64: one tile, all of it written
+    np.testing.assert_allclose(parts["CB"], ref["CB"], rtol=1e-6, atol=1e-6 * np.abs(ref["CB"]).max())
+    _check_y(y, ref["y"])
 
 
 @pytest.mark.parametrize("with_z,d_has_hdim", [(True, False), (False, True)])
@@ -118,12 +125,23 @@ def test_module_forward_then_update_continue_the_sequence(dev):
     cut = lambda a: _t(a[:, :L], dev)
     y, state = q(cut(d["x"]), cut(d["dt"]), cut(d["B"]), cut(d["C"]), return_final_states=True, state_dtype=torch.float32)
     _check_y(y, ref["y"][:, :L])
+    # the steps after the prefill: against the oracle's single step from the oracle's own state after L steps (the bar
+    # of the fp16 outputs), and against the chunked form run over L + 3 steps, which is the same mathematics with
+    # other roundings (fp16 states and weights there, an fp32 state here): a looser, absolute bar
+    head = dict(d, **{k: d[k][:, :L] for k in ("x", "dt", "B", "C")})
+    st_ref = _oracle(head, Q)["final_f32"]
+    assert np.abs(state.cpu().numpy() - st_ref).max() <= 2e-3 * np.abs(st_ref).max()
     for t in range(L, L + 3):
         yt = q.update(state, _t(d["x"][:, t].reshape(B, -1), dev), _t(d["dt"][:, t], dev), _t(d["B"][:, t].reshape(B, -1), dev),
                       _t(d["C"][:, t].reshape(B, -1), dev))
-        want = ref["y"][:, t]
-        np.testing.assert_allclose(yt.float().cpu().numpy() / np.abs(want).max(), want / np.abs(want).max(), rtol=1e-2, atol=1e-2)
-    assert np.abs(state.cpu().numpy() - ref["final_f32"]).max() <= 2e-3 * np.abs(ref["final_f32"]).max()
+        y_ref, st_ref = oracle.ssm_update_heads(
+            st_ref, d["x"][:, t], d["dt"][:, t, :, None], d["A_log"][:, None, None], d["B"][:, t], d["C"][:, t], d["D"][:, None],
+            d["dt_bias"].astype(np.float32)[:, None], None, x_scale=d["x_scale"], s_dt=d["s_dt"], s_A=d["s_A"], s_B=d["s_B"],
+            s_C=d["s_C"], s_D=d["s_D"], state_scale=np.ones((G, 2, 2, N), np.float32), head_range=d["head_range"], dim_range=d["dim_range"])
+        got = yt.float().cpu().numpy().reshape(B, H, 64)
+        np.testing.assert_allclose(got, y_ref.astype(np.float16).astype(np.float32), rtol=1e-2, atol=1e-2)
+        np.testing.assert_allclose(got, ref["y"][:, t].astype(np.float16).astype(np.float32), rtol=1e-2, atol=3e-2)
+    assert np.abs(state.cpu().numpy() - st_ref).max() <= 2e-3 * np.abs(st_ref).max()
 
 
 def _update_step_inputs(B, H, N, G, steps, seed):
