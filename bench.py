@@ -55,12 +55,14 @@ class Mixer:
         q_hid, s_hid = synth.quantize_absmax(hid)
         self.hidden = _t(q_hid, dev).view(B, L, dm)
 
-        w_in_q, w_in_s, _ = synth.linear_weights(2 * D, dm, seed, "in_proj", per_channel=False)
+        # int8 weights with one scale per output channel (the [1, N] b_scales epilogue of the reference's
+        # W8A8B8O8LinearParallel, quamba/qLinearLayer.py:698-711)
+        w_in_q, w_in_s, _ = synth.linear_weights(2 * D, dm, seed, "in_proj", per_channel=True)
         self.in_proj = W8A8B8O8Linear(dm, 2 * D, device=dev)
         self.in_proj.weight = _t(w_in_q, dev).t()
         s_xz = 0.04                                          # int8 scale of in_proj's output
         self.in_proj.a = torch.tensor([[float(s_hid) / s_xz]], dtype=torch.float32, device=dev)
-        self.in_proj.b = torch.tensor([[float(w_in_s[0])]], dtype=torch.float32, device=dev)
+        self.in_proj.b = _t(w_in_s, dev).view(1, 2 * D)
 
         qw, sw, qb, sb = synth.conv_weights(D, k, seed)
         self.conv = QCausalConv1D(D, D, k, groups=D, device=dev)
@@ -84,11 +86,11 @@ class Mixer:
         self.Bm, self.Cm, self.s_B, self.s_C = _t(qB, dev), _t(qC, dev), _s(sB, dev), _s(sC, dev)
         self.s_state = _s(1.0, dev)
 
-        w_out_q, w_out_s, _ = synth.linear_weights(dm, D, seed, "out_proj", per_channel=False)
+        w_out_q, w_out_s, _ = synth.linear_weights(dm, D, seed, "out_proj", per_channel=True)
         self.out_proj = W8A8B16O16Linear(D, dm, device=dev)
         self.out_proj.weight = _t(w_out_q, dev).t()
         self.out_proj.a = torch.tensor([[0.02]], dtype=torch.float32, device=dev)
-        self.out_proj.b = torch.tensor([[float(w_out_s[0])]], dtype=torch.float32, device=dev)
+        self.out_proj.b = _t(w_out_s, dev).view(1, dm)
         y_q, _ = synth.quantize_absmax(synth.activations((B * L, D), 1, seed, "y_had"))
         self.y_q = _t(y_q, dev).view(B, L, D)
 
@@ -133,8 +135,9 @@ def cpu_baseline(dev_mixer, seconds_budget=30.0):
     w_in = m.in_proj.weight.t().cpu().float()
     y_q = m.y_q[:1].cpu().float().view(L, D)
     w_out = m.out_proj.weight.t().cpu().float()
-    x8 = np.ascontiguousarray(np.random.default_rng(0).integers(-128, 128, (1, D, L)).astype(np.int8))
-    z8 = np.ascontiguousarray(np.random.default_rng(1).integers(-128, 128, (1, D, L)).astype(np.int8))
+    # the conv and the scan take what in_proj produced for this batch entry (x | z halves), as on the GPU
+    xz = m.step()[0][:1].cpu().numpy()
+    x8, z8 = np.ascontiguousarray(xz[:, :D]), np.ascontiguousarray(xz[:, D:])
     dt8 = np.ascontiguousarray(m.dt[:1].cpu().numpy())
     B8, C8 = m.Bm[:1].cpu().numpy(), m.Cm[:1].cpu().numpy()
     A, Dq, db = m.A_log.cpu().numpy(), m.Dq.cpu().numpy(), m.dt_bias.cpu().numpy()
@@ -178,14 +181,14 @@ def _time_fn(fn, steps, warmup):
     return e0.elapsed_time(e1) / steps
 
 
-def other_workloads(dev, steps, warmup):
-    """Secondary shapes of the same path (not the headline line): Mamba1-2.8b decode step, Mamba2-2.7b SSD
-    chunk scan, Mamba2-8b W4A8 layer.  Returns a list of dicts with per-launch time and roofline fraction."""
-    from quamba_amd import Quamb2Conv1D
-    out = []
-    ri = lambda *s: torch.randint(-128, 128, s, dtype=torch.int8, device=dev)
+def _ri(dev):
+    return lambda *s: torch.randint(-128, 128, s, dtype=torch.int8, device=dev)
+
+
+def _wl_decode(dev):
+    """Mamba1-2.8b decode step: conv update + state update, batch 64, fp32 state, sixteen steps in one HIP graph."""
+    ri = _ri(dev)
     sc = lambda v: torch.tensor([v], dtype=torch.float32, device=dev)
-    # decode: batch 64, d_inner 5120, d_state 16, conv state width 3, fp32 recurrent state
     B, D, N = 64, 5120, 16
     conv = QCausalConv1D(D, D, 4, groups=D, device=dev)
     conv.weight, conv.bias = ri(D, 4), ri(D)
@@ -215,9 +218,81 @@ def other_workloads(dev, steps, warmup):
             decode()
     ms = _time_fn(graph.replay, 64, 4) / 16
     nbytes = 3 * B * D + 2 * B * D * 3 + 2 * B * D * N * 4 + 2 * B * D + D * N
-    out.append(dict(workload="Mamba1-2.8b decode step (conv update + state update), batch 64, fp32 state, HIP graph of 16 steps",
-                    us=ms * 1e3, us_eager_python=ms_eager * 1e3, tokens_per_s=B / ms * 1e3, bound="hbm",
-                    achieved_GBs=nbytes / ms / 1e6, frac=nbytes / ms / 1e6 / HBM_PEAK_GBS))
+    return dict(workload="Mamba1-2.8b decode step (conv update + state update), batch 64, fp32 state, HIP graph of 16 steps",
+                name="decode_step", us=ms * 1e3, us_eager_python=ms_eager * 1e3, tokens_per_s=B / ms * 1e3, bound="hbm",
+                bytes=nbytes, achieved_GBs=nbytes / ms / 1e6, frac=nbytes / ms / 1e6 / HBM_PEAK_GBS)
+
+
+def _wl_ssd(dev, steps, warmup, B, L, H, N, G, Q, name, label):
+    """SSD chunk scan of `label`: per-tensor scales for one group, grouped scales (four head groups x four dim groups
+    per ssd group) otherwise; fp32 final states."""
+    ri = _ri(dev)
+    sc = lambda v: torch.tensor([v], dtype=torch.float32, device=dev)
+    x, dt, Bm, Cm = ri(B, L, H, 64), ri(B, L, H), ri(B, L, G, N), ri(B, L, G, N)
+    A2, D2 = ri(H), ri(H)
+    bias = torch.zeros(H, dtype=torch.float16, device=dev)
+    # scales live on the device before the timed region (creating one is a blocking host-to-device copy)
+    k_dt, k_A, k_D = (sc(v) for v in (0.02, 0.02, 0.008))
+    kw = {}
+    if G == 1:
+        k_x, k_B, k_C = sc(0.03), sc(0.03), sc(0.03)
+    else:
+        hpg = H // G
+        k_x = torch.rand(G, 4, 4, device=dev) * 0.02 + 0.02
+        k_B, k_C = torch.rand(G, device=dev) * 0.02 + 0.02, torch.rand(G, device=dev) * 0.02 + 0.02
+        kw = dict(x_head_group_range=(torch.arange(1, 5, dtype=torch.int32, device=dev) * (hpg // 4)).repeat(G, 1),
+                  x_dim_group_range=(torch.arange(1, 5, dtype=torch.int32, device=dev) * 16).repeat(G, 4, 1))
+    ssd = lambda: ops.ssd_chunk_scan_combined_fwd(x, k_x, dt, k_dt, A2, k_A, Bm, k_B, Cm, k_C, None, Q,
+                                                  q_D=D2, D_scale=k_D, dt_bias=bias, dt_softplus=True,
+                                                  final_state_dtype=torch.float32, **kw)
+    ms = _time_fn(ssd, steps, warmup)
+    nbytes = B * L * H * 64 + 2 * B * L * G * N + B * L * H + 2 * B * L * H * 64 + 4 * B * H * 64 * N
+    # dense multiply-adds: C B^T (lower tiles), chunk states, C x entering state, causal part of (C B^T) x
+    nc = (L + Q - 1) // Q
+    flops = 2.0 * B * nc * (G * Q * Q * N / 2 + H * Q * 64 * N + H * Q * 64 * N + H * Q * Q * 64 / 2)
+    return dict(workload=label, name=name, us=ms * 1e3, tokens_per_s=B * L / ms * 1e3, bound="hbm", bytes=nbytes,
+                achieved_GBs=nbytes / ms / 1e6, frac=nbytes / ms / 1e6 / HBM_PEAK_GBS, dense_TFLOPs=flops / ms / 1e9)
+
+
+def _wl_w4a8(dev, steps, warmup, M, Nn, K, o8, name):
+    ri = _ri(dev)
+    a = ri(M, K)
+    w = torch.randint(0, 256, (Nn, K // 2), dtype=torch.uint8, device=dev)
+    sg = (torch.rand(K // 128, Nn, device=dev) * 10 + 2).half()
+    s_ch, s_tok = torch.full((1, Nn), 1e-4, device=dev), torch.ones(M, device=dev)
+    fn = ops.w4a8o8_gemm if o8 else ops.w4a8o16_gemm
+    ms = _time_fn(lambda: fn(a, w, s_tok, s_ch, sg, None, M, Nn, K, False), steps, warmup)
+    n_ops = 2.0 * M * Nn * K
+    tops = n_ops / ms / 1e9
+    return dict(workload=f"Mamba2-8b W4A8 {name} {M}x{K}->{Nn}", name=f"w4a8_{name}", us=ms * 1e3, tokens_per_s=M / ms * 1e3,
+                bound="mfma", ops=n_ops, achieved_TOPs=tops, frac=tops / INT8_PEAK_TOPS)
+
+
+SSD_27B = (4, 4096, 80, 128, 1, 256, "ssd_2p7b", "Mamba2-2.7b SSD chunk scan, batch 4 x 4096, 80 heads, d_state 128, chunk 256")
+SSD_8B = (16, 1024, 128, 128, 8, 256, "ssd_8b", "Mamba2-8b SSD chunk scan, batch 16 x 1024, 128 heads, d_state 128, 8 groups, chunk 256")
+
+
+def secondary_workloads(dev, steps, warmup):
+    """The other benchmark configurations on the same path, in short form for the default line: the Mamba1-2.8b decode
+    step, the Mamba2-2.7b SSD chunk scan, and the Mamba2-8b layer's three heavy kernels (W4A8 in_proj, SSD chunk scan,
+    W4A8 out_proj).  Per-launch time, algorithmic bytes or operations, fraction of the bounding peak."""
+    out = [_wl_decode(dev), _wl_ssd(dev, steps, warmup, *SSD_27B),
+           _wl_w4a8(dev, steps, warmup, 16384, 18560, 4096, True, "in_proj"),
+           _wl_ssd(dev, steps, warmup, *SSD_8B),
+           _wl_w4a8(dev, steps, warmup, 16384, 4096, 8192, False, "out_proj")]
+    torch.cuda.empty_cache()
+    return out
+
+
+def other_workloads(dev, steps, warmup):
+    """Secondary shapes of the same path, the long list: whole mixers for one token and over a prompt, the Mamba2 conv,
+    Hadamard and norm kernels, single-token W4A8 streams.  Returns a list of dicts with per-launch time and roofline
+    fraction."""
+    from quamba_amd import Quamb2Conv1D
+    out = []
+    ri = _ri(dev)
+    sc = lambda v: torch.tensor([v], dtype=torch.float32, device=dev)
+    D, N = 5120, 16
     # the whole Mamba1-2.8b mixer for one token (in_proj, conv update, x_proj, dt_proj, state update, Hadamard,
     # out_proj): eight layers with their own weights (330 MB, more than the last-level cache holds) in one graph
     from quamba_amd import W8A8QMamba
@@ -265,22 +340,6 @@ def other_workloads(dev, steps, warmup):
                     achieved_TOPs=2.0 * Bp * Lp * (2560 * 10240 + 5120 * 192 + 160 * 5120 + 5120 * 2560) / ms / 1e9,
                     frac=2.0 * Bp * Lp * (2560 * 10240 + 5120 * 192 + 160 * 5120 + 5120 * 2560) / ms / 1e9 / INT8_PEAK_TOPS))
     del layers, m, hp
-    # SSD: batch 4, seqlen 4096, 80 heads of 64, d_state 128, 1 group, chunk 256
-    B, L, H, N, G, Q = 4, 4096, 80, 128, 1, 256
-    x, dt, Bm, Cm = ri(B, L, H, 64), ri(B, L, H), ri(B, L, G, N), ri(B, L, G, N)
-    A2, D2 = ri(H), ri(H)
-    bias = torch.zeros(H, dtype=torch.float16, device=dev)
-    # scales live on the device before the timed region (creating one is a blocking host-to-device copy)
-    k_x, k_dt, k_A, k_B, k_C, k_D = (sc(v) for v in (0.03, 0.02, 0.02, 0.03, 0.03, 0.008))
-    ssd = lambda: ops.ssd_chunk_scan_combined_fwd(x, k_x, dt, k_dt, A2, k_A, Bm, k_B, Cm, k_C, None, Q,
-                                                  q_D=D2, D_scale=k_D, dt_bias=bias, dt_softplus=True,
-                                                  final_state_dtype=torch.float32)
-    ms = _time_fn(ssd, steps, warmup)
-    nbytes = B * L * H * 64 + 2 * B * L * G * N + B * L * H + 2 * B * L * H * 64 + 4 * B * H * 64 * N
-    out.append(dict(workload="Mamba2-2.7b SSD chunk scan, batch 4 x 4096, 80 heads, d_state 128, chunk 256", us=ms * 1e3,
-                    tokens_per_s=B * L / ms * 1e3, bound="hbm", achieved_GBs=nbytes / ms / 1e6, frac=nbytes / ms / 1e6 / HBM_PEAK_GBS,
-                    dense_TFLOPs=86.9e9 / ms / 1e9))
-    del x, dt, Bm, Cm
     # Mamba2-8b xBC conv: batch 16 x 1024, x 8192 channels (128 heads of 64), 8 groups of d_state 128, grouped scales
     B, L, H, N, G = 16, 1024, 128, 128, 8
     dim = H * 64 + 2 * G * N
@@ -308,19 +367,11 @@ def other_workloads(dev, steps, warmup):
         out.append(dict(workload=f"Hadamard + int8 quantisation, 16384 rows x {dim}", us=ms * 1e3, tokens_per_s=16384 / ms * 1e3,
                         bound="hbm", achieved_GBs=nbytes / ms / 1e6, frac=nbytes / ms / 1e6 / HBM_PEAK_GBS))
         del xh
-    # W4A8: in_proj 16384 x 4096 -> 18560 (int8 out), out_proj 16384 x 8192 -> 4096 (fp16 out)
+    # W4A8 layers for one token: a stream over the packed weights (eight copies in turn: 300 MB)
     for (M, Nn, K, o8, name) in ((16384, 18560, 4096, True, "in_proj"), (16384, 4096, 8192, False, "out_proj")):
-        a = ri(M, K)
-        w = torch.randint(0, 256, (Nn, K // 2), dtype=torch.uint8, device=dev)
         sg = (torch.rand(K // 128, Nn, device=dev) * 10 + 2).half()
-        s_ch, s_tok = torch.full((1, Nn), 1e-4, device=dev), torch.ones(M, device=dev)
+        s_ch = torch.full((1, Nn), 1e-4, device=dev)
         fn = ops.w4a8o8_gemm if o8 else ops.w4a8o16_gemm
-        ms = _time_fn(lambda: fn(a, w, s_tok, s_ch, sg, None, M, Nn, K, False), steps, warmup)
-        tops = 2.0 * M * Nn * K / ms / 1e9
-        out.append(dict(workload=f"Mamba2-8b W4A8 {name} {M}x{K}->{Nn}", us=ms * 1e3, tokens_per_s=M / ms * 1e3, bound="mfma",
-                        achieved_TOPs=tops, frac=tops / INT8_PEAK_TOPS))
-        # the same layer for one token: a stream over the packed weights (eight copies in turn: 300 MB)
-        del a, w
         ws = [torch.randint(0, 256, (Nn, K // 2), dtype=torch.uint8, device=dev) for _ in range(8)]
         a1, s_tok1 = ri(1, K), torch.ones(1, device=dev)
         for w in ws:
@@ -491,8 +542,12 @@ def main():
     ap.add_argument("--batch", type=int, default=CFG["batch"])
     ap.add_argument("--seqlen", type=int, default=CFG["seqlen"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="leave out the short list of the other benchmark configurations (decode step, Mamba2-2.7b SSD "
+                         "scan, Mamba2-8b in_proj / SSD scan / out_proj)")
     ap.add_argument("--other-workloads", action="store_true",
-                    help="also time the decode step, the Mamba2 SSD scan and the W4A8 GEMMs (extra key in the JSON line)")
+                    help="also time the long list: whole mixers, Mamba2 conv, Hadamard, norms, single-token W4A8 "
+                         "(key other_workloads_long in the JSON line)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain 1 GiB device copies (reference points for hardware-counter runs)")
     ap.add_argument("--mfma-calibration", action="store_true",
@@ -531,7 +586,7 @@ def main():
         if kinfo["bound"] == "hbm":
             kinfo.update(achieved=kinfo["bytes"] / dur_ms / 1e6, peak=HBM_PEAK_GBS, unit="GB/s")
         else:
-            kinfo.update(achieved=kinfo["ops"] / dur_ms / 1e9, peak=INT8_PEAK_TOPS, unit="TFLOP/s")
+            kinfo.update(achieved=kinfo["ops"] / dur_ms / 1e9, peak=INT8_PEAK_TOPS, unit="TOP/s")
         kinfo["frac"] = kinfo["achieved"] / kinfo["peak"]
     traffic = {}
     if os.path.exists(args.traffic_json):
@@ -577,11 +632,16 @@ def main():
         line["valu_calibration"] = valu_calibration(dev)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(mixer)
+    del mixer
+    torch.cuda.empty_cache()
+    rounded = lambda ws: [{k: (round(v, 4) if isinstance(v, float) else v) for k, v in w.items()} for w in ws]
+    if not args.no_other_workloads:
+        ws = secondary_workloads(dev, min(args.steps, 20), args.warmup)
+        for w in ws:
+            w["traffic"] = traffic.get(w["name"])
+        line["other_workloads"] = rounded(ws)
     if args.other_workloads:
-        del mixer
-        torch.cuda.empty_cache()
-        line["other_workloads"] = [{k: (round(v, 4) if isinstance(v, float) else v) for k, v in w.items()}
-                                   for w in other_workloads(dev, min(args.steps, 20), args.warmup)]
+        line["other_workloads_long"] = rounded(other_workloads(dev, min(args.steps, 20), args.warmup))
     print(json.dumps(line))
 
 
