@@ -40,14 +40,17 @@ __device__ __forceinline__ float softplus20(float x) {
     return e < 0.015625f ? series : big;
 }
 
-// The same function without a branch (the early return above becomes a jump around the rest, which keeps a
-// batch of independent evaluations from overlapping): softplus(x) = max(x, 0) + log1p(exp(-|x|)).  Above the
-// threshold the second term is below half an ulp of x, so x comes back exactly, as the reference returns it.
+// The same function without a branch and with one rounding compensated instead of a series:
+//   softplus(x) = max(x, 0) + log1p(e),  e = exp(-|x|) in (0, 1]
+//   u = fl(1 + e) = 1 + e + r with r = (u - 1) - e exact, so log1p(e) = ln(u - r) = ln u - r / u + ..., and with
+//   u in [1, 2] taking r for r / u is wrong by less than 2^-24 of the result.
+// Above the threshold the second term is below half an ulp of x, so x comes back exactly, as the reference returns it.
 __device__ __forceinline__ float softplus20_flat(float x) {
-    const float e = fast_exp2(-__builtin_fabsf(x) * kLog2e);
-    const float series = e * __builtin_fmaf(e, __builtin_fmaf(e, __builtin_fmaf(e, -0.25f, 1.0f / 3.0f), -0.5f), 1.0f);
-    const float big = fast_log2(1.0f + e) * 0.693147180559945309f;
-    return __builtin_fmaxf(x, 0.0f) + (e < 0.015625f ? series : big);
+    const float e = fast_exp2(__builtin_fabsf(x) * -kLog2e);
+    const float u = 1.0f + e;
+    const float r = (u - 1.0f) - e;
+    const float sp = __builtin_fmaf(fast_log2(u), 0.693147180559945309f, -r);
+    return __builtin_amdgcn_fmed3f(x, 0.0f, __builtin_inff()) + sp;
 }
 
 __device__ __forceinline__ float silu_gate(float z) {
@@ -510,8 +513,9 @@ __device__ __forceinline__ void sscan_fwd_pre_body(const QaSScanParams& p, int v
 
     const float s_u = *p.scale_u, s_dt = *p.scale_delta, s_A = *p.scale_A, s_B = *p.scale_B, s_C = *p.scale_C;
     const float s_z = HAS_Z ? *p.scale_z : 0.0f;
-    const float D_f = p.D ? *p.scale_D * static_cast<float>(p.D[cc]) : 0.0f;
+    const float D_u = p.D ? (*p.scale_D * static_cast<float>(p.D[cc])) * s_u : 0.0f;       // skip weight per input code
     const float db = p.delta_bias ? *p.scale_delta_bias * static_cast<float>(p.delta_bias[cc]) : 0.0f;
+    const bool want_dt_sum = p.dt_sum_out != nullptr;
 
     float A2[NPL], h[NPL];
 #pragma unroll
@@ -542,7 +546,7 @@ __device__ __forceinline__ void sscan_fwd_pre_body(const QaSScanParams& p, int v
     const int8_t* bc_base[2] = {p.B + b * p.B_batch_stride + g * p.B_group_stride,
                                 p.C + b * p.C_batch_stride + g * p.C_group_stride};
     const int64_t bc_nstride[2] = {p.B_dstate_stride, p.C_dstate_stride};
-    const float bc_scale[2] = {s_B, s_C};
+    const float bc_scale[2] = {s_B * s_u, s_C};
 
     uint32_t r_u[kStage / 4], r_d[kStage / 4], r_z[kStage / 4];
     uint32_t r_bc[kBcPieces];
@@ -576,24 +580,27 @@ __device__ __forceinline__ void sscan_fwd_pre_body(const QaSScanParams& p, int v
     auto stage = [&](int t0) {
         float dv[kStage], duv[kStage], sk[kStage], gt[kStage];
 #pragma unroll
-        for (int e = 0; e < kStage; ++e) {
-            const float u_val = s_u * i8_of(r_u[e >> 2], e & 3);
-            float dt = __builtin_fmaf(s_dt, i8_of(r_d[e >> 2], e & 3), db);
-            if (softplus) dt = softplus20_flat(dt);
-            dv[e] = dt;
-            sk[e] = D_f * u_val;
-            duv[e] = u_val;
-            gt[e] = HAS_Z ? sm.gate_table[(r_z[e >> 2] >> (8 * (e & 3))) & 0xffu] : 1.0f;
+        for (int e = 0; e < kStage; ++e) dv[e] = __builtin_fmaf(s_dt, i8_of(r_d[e >> 2], e & 3), db);
+        if (softplus) {                  // one uniform branch per tile: the evaluations below overlap
+#pragma unroll
+            for (int e = 0; e < kStage; ++e) dv[e] = softplus20_flat(dv[e]);
         }
         if (t0 + T > L) {
             // ragged last tile: steps past the end of the sequence must leave the state alone (a = 1, b = 0)
 #pragma unroll
             for (int e = 0; e < kStage; ++e) dv[e] = t0 + slice * kStage + e < L ? dv[e] : 0.0f;
         }
+        if (want_dt_sum) {
+#pragma unroll
+            for (int e = 0; e < kStage; ++e) dt_sum += dv[e];
+        }
 #pragma unroll
         for (int e = 0; e < kStage; ++e) {
-            dt_sum += dv[e];
-            duv[e] *= dv[e];
+            // the input scale rides with B and D: (s_B q_B) (dt (s_u q_u)) = ((s_B s_u) q_B) (dt q_u)
+            const float u_q = i8_of(r_u[e >> 2], e & 3);
+            sk[e] = D_u * u_q;
+            duv[e] = dv[e] * u_q;
+            gt[e] = HAS_Z ? sm.gate_table[(r_z[e >> 2] >> (8 * (e & 3))) & 0xffu] : 1.0f;
         }
 #pragma unroll
         for (int q = 0; q < kStage / 4; ++q) {
