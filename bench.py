@@ -508,7 +508,7 @@ def mfma_calibration(dev):
     return out
 
 
-def valu_calibration(dev):
+def valu_calibration(dev, ops_list=None, launches=4):
     """Issue time of plain and transcendental vector instructions: eight waves per SIMD on every CU, each lane with
     eight independent chains of one instruction; ns per wave-instruction per SIMD and the clock during the loop."""
     from quamba_amd import _lib
@@ -519,8 +519,11 @@ def valu_calibration(dev):
     stream = torch.cuda.current_stream().cuda_stream
     simds = 4 * torch.cuda.get_device_properties(dev).multi_processor_count
     out = {}
-    for name, op in (("v_mul_f32", 0), ("v_exp_f32", 1), ("v_rcp_f32", 2), ("v_log_f32", 3), ("v_fmac_f32", 4), ("v_mul_f32_dpp", 5)):
-        for _ in range(4):
+    all_ops = (("v_mul_f32", 0), ("v_exp_f32", 1), ("v_rcp_f32", 2), ("v_log_f32", 3), ("v_fmac_f32", 4), ("v_mul_f32_dpp", 5))
+    for name, op in all_ops:
+        if ops_list is not None and name not in ops_list:
+            continue
+        for _ in range(launches):
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
             _lib.check(lib.qa_probe_valu(sink.data_ptr(), sink.numel(), ticks.data_ptr(), wgs, iters, op, stream), "diag")
@@ -532,6 +535,34 @@ def valu_calibration(dev):
         out[name] = {"ns_per_wave_instruction_per_simd": round(ms * 1e6 / per_simd, 3), "ms": round(ms, 3),
                      "clock_MHz": round(100.0 * t[0] / max(t[1], 1), 1)}
     return out
+
+
+# Vector instructions a wave of the selective scan issues per group of four steps, counted in the compiled kernel
+# (time loop + staging of the next tile + output store, divided by the eight groups of a 32-step tile): the kind with
+# four lanes per channel and four states per lane, and the short kind with eight lanes per channel and two states.
+SCAN_MIX = {"four_lane": {"plain": 99, "transcendental": 18}, "eight_lane": {"plain": 58, "transcendental": 9}}
+
+
+def scan_issue_bound(dev, B, D, L):
+    """Lower bound of the scan launch from vector-ALU issue alone: every wave's instruction mix priced at the rates a
+    register-only loop reaches on this GPU now (measured here with the probe library), the waves spread evenly over
+    the SIMDs.  Follows the host's choice of the two kinds of workgroup for d_state 16 (qa_sscan_fwd)."""
+    rates = valu_calibration(dev, ("v_mul_f32", "v_exp_f32"), launches=2)
+    t_plain = rates["v_mul_f32"]["ns_per_wave_instruction_per_simd"]
+    t_trans = rates["v_exp_f32"]["ns_per_wave_instruction_per_simd"]
+    simds = 4 * torch.cuda.get_device_properties(dev).multi_processor_count
+    waves4 = B * D // 16
+    q, rem = divmod(waves4, simds)
+    short = 0
+    if 2 * waves4 <= 3 * simds:
+        short = D
+    elif q >= 1 and 0 < rem and 2 * rem <= simds and (rem * 16 // B) % 32 == 0 and (D - rem * 16 // B) % 64 == 0:
+        short = rem * 16 // B
+    waves = {"four_lane": B * (D - short) // 16, "eight_lane": B * short // 8}
+    groups = (L + 31) // 32 * 8
+    ns = sum(waves[k] * groups * (SCAN_MIX[k]["plain"] * t_plain + SCAN_MIX[k]["transcendental"] * t_trans) for k in waves)
+    return dict(issue_bound_us=ns / simds / 1e3, ns_plain=t_plain, ns_transcendental=t_trans, waves=waves,
+                instructions_per_four_steps=SCAN_MIX)
 
 
 def main():
@@ -595,6 +626,12 @@ def main():
     roofline = dict(kernel=dom["name"], bound=dom["bound"], achieved=round(dom["achieved"], 2), peak=dom["peak"],
                     unit=dom["unit"], frac=round(dom["frac"], 4), traffic=traffic.get(dom["name"]),
                     avg_us=round(dom["avg_us"], 2))
+    if dom["name"] == "sscan_fwd":
+        # the bound that binds this kernel is vector-ALU issue, not HBM: how far the launch is from it
+        ib = scan_issue_bound(dev, B, CFG["d_inner"], L)
+        roofline["issue_bound_us"] = round(ib["issue_bound_us"], 2)
+        roofline["frac_of_issue_bound"] = round(ib["issue_bound_us"] / dom["avg_us"], 4)
+        roofline["issue_bound_inputs"] = {k: ib[k] for k in ("ns_plain", "ns_transcendental", "waves", "instructions_per_four_steps")}
     per_kernel = [dict(kernel=k["name"], bound=k["bound"], avg_us=round(k["avg_us"], 2), achieved=round(k["achieved"], 2),
                        unit=k["unit"], peak=k["peak"], frac=round(k["frac"], 4), traffic=traffic.get(k["name"]))
                   for k in kernels]
