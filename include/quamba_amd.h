@@ -300,6 +300,16 @@ typedef struct QaSsmUpdateParams {
 
 int qa_ssm_state_update(const QaSsmUpdateParams* p, void* stream);
 
+/* One Mamba1 decode step in one launch: the conv's single-step update (qa_causal_conv1d_update on `conv`) and the
+ * state update (qa_ssm_state_update on `p`), the state update taking the conv's int8 output as its x (p->x is not
+ * read).  Replaces the pair quant_causal_conv1d_cuda.update (csrc/causal_conv1d/quant_causal_conv1d.cpp, kernel
+ * quant_causal_conv1d_update_kernel.cuh:34-75) + quant_sscan_cuda.update / selective_state_update
+ * (quamba/triton/selective_state_update.py:83-126) for callers whose dt, B and C do not depend on the conv output of
+ * the same step (a benchmark loop with given inputs; in the full Mamba1 layer x_proj sits between the two, so the
+ * layer calls them separately).  Same bits as the two calls: conv_state and state are updated in place, conv->out
+ * (may be null) receives the conv output.  One head (p->nheads == 1), d_state <= 16, per-tensor scales. */
+int qa_mamba1_decode_step(const QaConvParams* conv, const QaSsmUpdateParams* p, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * W8A8 GEMM with scale epilogue:  D[m,n] = cast( s_a[m|0] * ( s_b[n|0] * float(sum_k a[m,k] w[n,k]) ) )
  * Replaces quant_linear_cuda.cutlass_scaled_mm_dq / cutlass_scaled_mv_dq / w8a8o8_gemv

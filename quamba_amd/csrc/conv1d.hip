@@ -211,22 +211,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_update_kernel(QaConvParams 
     if (idx >= static_cast<int64_t>(p.batch) * p.dim) return;
     const int c = static_cast<int>(idx % p.dim);
     const int b = static_cast<int>(idx / p.dim);
-    int8_t* st = p.conv_state + b * p.conv_state_batch_stride + c * p.conv_state_c_stride;
-    const int8_t* w = p.weight + c * p.weight_c_stride;
-    const int width = p.width;
-    const int slen = p.conv_state_len;            // width (slot 0 is dropped) or width-1
-    const int drop = slen - (width - 1);          // 1 or 0
-    int8_t xs[4];
-    for (int i = 0; i < width - 1; ++i) xs[i] = st[(i + drop) * p.conv_state_l_stride];
-    xs[width - 1] = p.x[b * p.x_batch_stride + c * p.x_c_stride];
-    for (int i = 0; i < slen; ++i) st[i * p.conv_state_l_stride] = xs[i + (width - slen)];
-    const float s_wx = p.scale_w * p.scale_x;
-    float v = p.bias ? static_cast<float>(p.bias[c]) * p.scale_b : 0.0f;
-    for (int i = 0; i < width; ++i) {
-        const float wv = static_cast<float>(w[i * p.weight_width_stride]);
-        v = __builtin_fmaf(s_wx * wv, static_cast<float>(xs[i]), v);
-    }
-    p.out[b * p.out_batch_stride + c * p.out_c_stride] = conv_epilogue(v, p.scale_out, p.silu_activation);
+    conv_step_row(p, b, c, true);
 }
 
 int validate_common(const QaConvParams* p) {

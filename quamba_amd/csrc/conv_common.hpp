@@ -68,4 +68,49 @@ __device__ __forceinline__ int dot4(uint32_t a, uint32_t b) {
     return __builtin_amdgcn_sdot4(static_cast<int>(a), static_cast<int>(b), 0, false);
 }
 
+// One decode step of channel c of batch entry b (quant_causal_conv1d_update_kernel.cuh:34-75): the conv state moves
+// on by one step (in place), the window meets the taps, bias, SiLU, requantisation.  Returns the int8 output and,
+// with `store`, writes state and output.  Taps and a four-wide state row are fetched as one word when their layout
+// allows; the requantisation takes the cheap route whenever it provably equals the exact one (conv_quant).
+__device__ __forceinline__ int8_t conv_step_row(const QaConvParams& p, int b, int c, bool store) {
+    int8_t* st = p.conv_state + b * p.conv_state_batch_stride + c * p.conv_state_c_stride;
+    const int8_t* w = p.weight + c * p.weight_c_stride;
+    const int width = p.width;
+    const int slen = p.conv_state_len;            // width (slot 0 is dropped) or width-1
+    const int drop = slen - (width - 1);          // 1 or 0
+    __attribute__((aligned(4))) int8_t xs[4], ws[4] = {0, 0, 0, 0};
+    const bool w_word = width == 4 && p.weight_width_stride == 1 && (reinterpret_cast<uintptr_t>(w) & 3u) == 0;
+    const bool s_word = slen == 4 && p.conv_state_l_stride == 1 && (reinterpret_cast<uintptr_t>(st) & 3u) == 0;
+    if (w_word) {
+        *reinterpret_cast<uint32_t*>(ws) = *reinterpret_cast<const uint32_t*>(w);
+    } else {
+        for (int i = 0; i < width; ++i) ws[i] = w[i * p.weight_width_stride];
+    }
+    if (s_word) {
+        __attribute__((aligned(4))) int8_t row[4];
+        *reinterpret_cast<uint32_t*>(row) = *reinterpret_cast<const uint32_t*>(st);
+        for (int i = 0; i < width - 1; ++i) xs[i] = row[i + drop];
+    } else {
+        for (int i = 0; i < width - 1; ++i) xs[i] = st[(i + drop) * p.conv_state_l_stride];
+    }
+    xs[width - 1] = p.x[b * p.x_batch_stride + c * p.x_c_stride];
+    const float bias_f = p.bias ? static_cast<float>(p.bias[c]) * p.scale_b : 0.0f;
+    if (store) {
+        if (s_word) {
+            // state as long as the window: the whole window is the new state
+            *reinterpret_cast<uint32_t*>(st) = *reinterpret_cast<const uint32_t*>(xs);
+        } else {
+            for (int i = 0; i < slen; ++i) st[i * p.conv_state_l_stride] = xs[i + (width - slen)];
+        }
+    }
+    const float s_wx = p.scale_w * p.scale_x;
+    float v = bias_f;
+    for (int i = 0; i < width; ++i) v = __builtin_fmaf(s_wx * static_cast<float>(ws[i]), static_cast<float>(xs[i]), v);
+    const ConvQuantRegs kq;
+    const int8_t q = static_cast<int8_t>(conv_quant(v, p.scale_out, 1.0f / p.scale_out, p.silu_activation,
+                                                    conv_needs_exact_route(p.scale_out), kq));
+    if (store && p.out) p.out[b * p.out_batch_stride + c * p.out_c_stride] = q;
+    return q;
+}
+
 }  // namespace qa

@@ -20,6 +20,7 @@
 //   * global loads of tile i+1 are issued before the arithmetic of tile i and held in registers
 //     until the tile has been consumed, then written to LDS.
 #include "qa_common.hpp"
+#include "conv_common.hpp"
 
 namespace qa {
 namespace {
@@ -817,8 +818,12 @@ int launch_fwd_mixed(const QaSScanParams& p, hipStream_t stream, int vec_in, int
 // naturally aligned, so a lane moves its four states with one load and one store per operand.
 // A wave's life here is a chain of memory round trips, not arithmetic, so optional operands are read
 // through a stand-in address instead of behind a branch: every load of the row is in flight at once.
-template <int LPR, bool VEC, bool FP32>
-__global__ __launch_bounds__(256) void ssm_update_kernel(QaSsmUpdateParams p) {
+// CONV: the row's input code is not read from p.x but produced here by the causal conv's single-step update on
+// channel d of batch entry b (quant_causal_conv1d_update_kernel.cuh:34-75: shift the conv state, dot product with
+// the taps, bias, SiLU, requantise - the arithmetic of conv_update_kernel, same bits), for one lane per row.
+template <int LPR, bool VEC, bool FP32, bool CONV>
+__device__ __forceinline__ void ssm_update_body(const QaSsmUpdateParams& p, const QaConvParams* cp) {
+    static_assert(!CONV || LPR == 1, "the conv step needs one lane per row");
     // grid: x over the channels of one head, y = head, z = batch (no integer division on the way in)
     const int gid = blockIdx.x * 256 + threadIdx.x;
     const int sub = gid % LPR;
@@ -848,9 +853,10 @@ __global__ __launch_bounds__(256) void ssm_update_kernel(QaSsmUpdateParams p) {
     const int64_t bias_i = hd * p.dt_bias_head_stride + d * p.dt_bias_dim_stride;
     const int8_t* x_a = p.x + b * p.x_batch_stride + hd * p.x_head_stride + d * p.x_dim_stride;
     const int8_t* dt_a = p.dt + b * p.dt_batch_stride + hd * p.dt_head_stride + d * p.dt_dim_stride;
-    const int8_t* z_a = p.z ? p.z + b * p.z_batch_stride + hd * p.z_head_stride + d * p.z_dim_stride : x_a;
-    const int8_t* D_a = p.D ? p.D + hd * p.D_head_stride + d * p.D_dim_stride : x_a;
-    const int8_t* b8_a = bias_i8 ? static_cast<const int8_t*>(p.dt_bias) + bias_i : x_a;
+    const int8_t* standin8 = CONV ? dt_a : x_a;             // always readable, one byte (p.x is not used with CONV)
+    const int8_t* z_a = p.z ? p.z + b * p.z_batch_stride + hd * p.z_head_stride + d * p.z_dim_stride : standin8;
+    const int8_t* D_a = p.D ? p.D + hd * p.D_head_stride + d * p.D_dim_stride : standin8;
+    const int8_t* b8_a = bias_i8 ? static_cast<const int8_t*>(p.dt_bias) + bias_i : standin8;
     const __half* b16_a = bias_f16 ? static_cast<const __half*>(p.dt_bias) + bias_i : reinterpret_cast<const __half*>(standin);
 
     const float x_scale = p.x_scale[sidx];
@@ -862,7 +868,13 @@ __global__ __launch_bounds__(256) void ssm_update_kernel(QaSsmUpdateParams p) {
     const float D_scale = *(p.D ? p.D_scale : standin);
     const float z_scale = *(p.z ? p.z_scale : standin);
     const float bias_scale = *(bias_i8 ? p.dt_bias_scale : standin);
-    const float xq = static_cast<float>(*x_a), dtq = static_cast<float>(*dt_a);
+    float xq;
+    if constexpr (CONV) {
+        xq = static_cast<float>(conv_step_row(*cp, static_cast<int>(b), d, row_ok));
+    } else {
+        xq = static_cast<float>(*x_a);
+    }
+    const float dtq = static_cast<float>(*dt_a);
     const float zq = static_cast<float>(*z_a), Dq = static_cast<float>(*D_a);
     const float b8 = static_cast<float>(*b8_a), b16 = __half2float(*b16_a);
     const float requant_k = grouped ? 1e6f : 1e2f;
@@ -875,7 +887,10 @@ __global__ __launch_bounds__(256) void ssm_update_kernel(QaSsmUpdateParams p) {
     // (sub + k * LPR) * 4.  All loads first, then the arithmetic, then the stores.
     constexpr int kPieces = 4;
     float hv[kPieces][4], sc[kPieces][4];
-    int8_t a8[kPieces][4], b8v[kPieces][4], c8[kPieces][4], s8[kPieces][4];
+    __attribute__((aligned(16))) int8_t a8[kPieces][4];
+    __attribute__((aligned(4))) int8_t b8v[kPieces][4], c8[kPieces][4], s8[kPieces][4];
+    // one lane per row with sixteen states in a row of A_log: the lane's sixteen codes come as one 16-byte piece
+    const bool a_row16 = VEC && LPR == 1 && p.dstate == 16 && p.A_dstate_stride == 1 && (reinterpret_cast<uintptr_t>(Ap) & 15u) == 0;
 #pragma unroll
     for (int k = 0; k < kPieces; ++k) {
         const int n0 = (sub + k * LPR) * 4;
@@ -884,14 +899,23 @@ __global__ __launch_bounds__(256) void ssm_update_kernel(QaSsmUpdateParams p) {
             // dstate is a multiple of four here, so the piece is whole.  A_log alone may be a broadcast view
             // (one value per head, stride 0 along the states, as Mamba2 passes it): it is read through its
             // stride, the state and B, C with one load per piece
-            if (p.A_dstate_stride == 1 && (reinterpret_cast<uintptr_t>(Ap + n0) & 3u) == 0) {
+            if (a_row16) {
+                if (k == 0) *reinterpret_cast<uint4*>(&a8[0][0]) = *reinterpret_cast<const uint4*>(Ap);
+            } else if (p.A_dstate_stride == 1 && (reinterpret_cast<uintptr_t>(Ap + n0) & 3u) == 0) {
                 *reinterpret_cast<int32_t*>(a8[k]) = *reinterpret_cast<const int32_t*>(Ap + n0);
             } else {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) a8[k][e] = Ap[(n0 + e) * p.A_dstate_stride];
             }
-            *reinterpret_cast<int32_t*>(b8v[k]) = *reinterpret_cast<const int32_t*>(Bp + n0);
-            *reinterpret_cast<int32_t*>(c8[k]) = *reinterpret_cast<const int32_t*>(Cp + n0);
+            if constexpr (LPR == 1) {
+                // every lane of the wave reads the same B and C words (one batch entry per workgroup): scalar loads
+                typedef const __attribute__((address_space(4))) int32_t* const_words;
+                *reinterpret_cast<int32_t*>(b8v[k]) = reinterpret_cast<const_words>(reinterpret_cast<uintptr_t>(Bp))[n0 / 4];
+                *reinterpret_cast<int32_t*>(c8[k]) = reinterpret_cast<const_words>(reinterpret_cast<uintptr_t>(Cp))[n0 / 4];
+            } else {
+                *reinterpret_cast<int32_t*>(b8v[k]) = *reinterpret_cast<const int32_t*>(Bp + n0);
+                *reinterpret_cast<int32_t*>(c8[k]) = *reinterpret_cast<const int32_t*>(Cp + n0);
+            }
             if constexpr (FP32) {
                 const float4 v = *reinterpret_cast<const float4*>(static_cast<const float*>(p.state) + st_base + n0);
                 hv[k][0] = v.x; hv[k][1] = v.y; hv[k][2] = v.z; hv[k][3] = v.w;
@@ -917,7 +941,7 @@ __global__ __launch_bounds__(256) void ssm_update_kernel(QaSsmUpdateParams p) {
     const float xv = x_scale * xq;
     float dt = dt_scale * dtq;
     dt += bias_i8 ? bias_scale * b8 : (bias_f16 ? b16 : 0.0f);
-    if (p.dt_softplus) dt = dt <= 20.0f ? log1pf(expf(dt)) : dt;
+    if (p.dt_softplus) dt = softplus20_flat(dt);
     float acc = 0.0f;
 #pragma unroll
     for (int k = 0; k < kPieces; ++k) {
@@ -967,8 +991,19 @@ __global__ __launch_bounds__(256) void ssm_update_kernel(QaSsmUpdateParams p) {
     }
 }
 
+template <int LPR, bool VEC, bool FP32>
+__global__ __launch_bounds__(256) void ssm_update_kernel(QaSsmUpdateParams p) {
+    ssm_update_body<LPR, VEC, FP32, false>(p, nullptr);
+}
+
+// conv step + state update of one token in one launch (d_state <= 16, one head)
+template <bool VEC, bool FP32>
+__global__ __launch_bounds__(256) void decode_step_kernel(QaSsmUpdateParams p, QaConvParams cp) {
+    ssm_update_body<1, VEC, FP32, true>(p, &cp);
+}
+
 template <int LPR>
-int launch_update(const QaSsmUpdateParams& p, hipStream_t stream) {
+int launch_update(const QaSsmUpdateParams& p, hipStream_t stream, const QaConvParams* conv = nullptr) {
     const int64_t blocks = (static_cast<int64_t>(p.dim) * LPR + 255) / 256;
     if (blocks > 0x7fffffffLL / 256 || p.nheads > 65535 || p.batch > 65535) return QA_ERR_SHAPE;
     const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(p.nheads), static_cast<unsigned>(p.batch));
@@ -982,6 +1017,14 @@ int launch_update(const QaSsmUpdateParams& p, hipStream_t stream) {
                      mult(p.state_dim_stride * st_el, st_align) &&
                      aligned4(p.B) && mult(p.B_batch_stride, 4) && mult(p.B_group_stride, 4) &&
                      aligned4(p.C) && mult(p.C_batch_stride, 4) && mult(p.C_group_stride, 4);
+    if constexpr (LPR == 1) {
+        if (conv) {
+            auto fused = [&](auto kernel) { hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, p, *conv); };
+            if (p.state_is_fp32) vec ? fused(decode_step_kernel<true, true>) : fused(decode_step_kernel<false, true>);
+            else vec ? fused(decode_step_kernel<true, false>) : fused(decode_step_kernel<false, false>);
+            return check_launch();
+        }
+    }
     auto go = [&](auto kernel) { hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, p); };
     if (p.state_is_fp32) vec ? go(ssm_update_kernel<LPR, true, true>) : go(ssm_update_kernel<LPR, false, true>);
     else vec ? go(ssm_update_kernel<LPR, true, false>) : go(ssm_update_kernel<LPR, false, false>);
@@ -1093,9 +1136,10 @@ extern "C" int qa_sscan_fwd(const QaSScanParams* p, void* stream_) {
     return launch_fwd<16, 16, 16, 1>(*p, stream, vec_in, vec_bc, vec_out);
 }
 
-extern "C" int qa_ssm_state_update(const QaSsmUpdateParams* p, void* stream_) {
-    using namespace qa;
-    if (!p || !p->state || !p->x || !p->dt || !p->A_log || !p->B || !p->C || !p->out) return QA_ERR_NULL;
+namespace qa {
+namespace {
+int validate_update(const QaSsmUpdateParams* p, bool needs_x) {
+    if (!p || !p->state || (needs_x && !p->x) || !p->dt || !p->A_log || !p->B || !p->C || !p->out) return QA_ERR_NULL;
     if (!p->x_scale || !p->dt_scale || !p->A_log_scale || !p->B_scale || !p->C_scale) return QA_ERR_NULL;
     if (!p->state_is_fp32 && !p->state_scale) return QA_ERR_NULL;
     if ((p->D && !p->D_scale) || (p->z && !p->z_scale)) return QA_ERR_NULL;
@@ -1103,6 +1147,15 @@ extern "C" int qa_ssm_state_update(const QaSsmUpdateParams* p, void* stream_) {
     if (p->nhead_groups > 0 && (!p->x_head_group_range || !p->x_dim_group_range || p->ndim_groups < 1)) return QA_ERR_NULL;
     if (p->batch < 0 || p->nheads < 1 || p->dim < 0 || p->dstate < 1 || p->dstate > 256) return QA_ERR_SHAPE;
     if (p->ngroups < 1 || p->nheads % p->ngroups != 0) return QA_ERR_SHAPE;
+    return QA_OK;
+}
+}  // namespace
+}  // namespace qa
+
+extern "C" int qa_ssm_state_update(const QaSsmUpdateParams* p, void* stream_) {
+    using namespace qa;
+    const int st = validate_update(p, true);
+    if (st != QA_OK) return st;
     if (p->batch == 0 || p->dim == 0) return QA_OK;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const int N = p->dstate;
@@ -1112,4 +1165,18 @@ extern "C" int qa_ssm_state_update(const QaSsmUpdateParams* p, void* stream_) {
     if (N <= 64) return launch_update<4>(*p, stream);
     if (N <= 128) return launch_update<8>(*p, stream);
     return launch_update<16>(*p, stream);
+}
+
+extern "C" int qa_mamba1_decode_step(const QaConvParams* conv, const QaSsmUpdateParams* p, void* stream_) {
+    using namespace qa;
+    const int st = validate_update(p, false);
+    if (st != QA_OK) return st;
+    if (!conv || !conv->x || !conv->weight || !conv->conv_state) return QA_ERR_NULL;
+    if (conv->width < 2 || conv->width > 4) return QA_ERR_SHAPE;
+    if (conv->conv_state_len != conv->width && conv->conv_state_len != conv->width - 1) return QA_ERR_SHAPE;
+    if (conv->batch != p->batch || conv->dim != p->dim) return QA_ERR_SHAPE;
+    // one lane per (batch, channel) row carries both steps: one head, at most sixteen states, per-tensor scales
+    if (p->nheads != 1 || p->dstate > 16 || p->nhead_groups > 0) return QA_ERR_UNSUPPORTED;
+    if (p->batch == 0 || p->dim == 0) return QA_OK;
+    return launch_update<1>(*p, static_cast<hipStream_t>(stream_), conv);
 }

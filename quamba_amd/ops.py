@@ -75,10 +75,8 @@ def causal_conv1d_fwd(x, scale_x, weight, scale_w, scale_out, scale_b, bias=None
     return (out, out_t) if also_channel_last else out
 
 
-def causal_conv1d_update(x, conv_state, scale_x, weight, scale_w, scale_out, scale_b, bias=None,
-                         silu_activation=True):
-    """One decode step: x int8 (batch, dim); conv_state int8 (batch, dim, width) or
-    (batch, dim, width-1), shifted in place."""
+def _conv_update_params(x, conv_state, scale_x, weight, scale_w, scale_out, scale_b, bias, silu_activation):
+    """QaConvParams of one decode step and the output tensor they point at."""
     _require(x.dtype == torch.int8 and weight.dtype == torch.int8 and conv_state.dtype == torch.int8,
              "x, weight and conv_state must be int8")
     for t, n in ((x, "x"), (conv_state, "conv_state"), (weight, "weight")):
@@ -105,10 +103,35 @@ def causal_conv1d_update(x, conv_state, scale_x, weight, scale_w, scale_out, sca
     p.conv_state_len = conv_state.shape[2]
     p.x, p.weight, p.bias, p.out, p.conv_state = ptr(x), ptr(weight), ptr(bias), ptr(out), ptr(conv_state)
     p.scale_x, p.scale_w, p.scale_b, p.scale_out = float(scale_x), float(scale_w), float(scale_b), float(scale_out)
+    return p, out
+
+
+def causal_conv1d_update(x, conv_state, scale_x, weight, scale_w, scale_out, scale_b, bias=None,
+                         silu_activation=True):
+    """One decode step: x int8 (batch, dim); conv_state int8 (batch, dim, width) or
+    (batch, dim, width-1), shifted in place."""
+    p, out = _conv_update_params(x, conv_state, scale_x, weight, scale_w, scale_out, scale_b, bias, silu_activation)
     with torch.cuda.device(x.device):
         st = _lib.lib().qa_causal_conv1d_update(ct.byref(p), _lib.current_stream(x.device))
     _lib.check(st, "causal_conv1d_update")
     return out
+
+
+def mamba1_decode_step(x, conv_state, scale_x, weight, scale_w, scale_out, scale_b, bias, silu_activation,
+                       state, q_dt, dt_scale, q_A_log, A_log_scale, ssm_state_scale, q_B, B_scale, q_C, C_scale,
+                       q_D=None, D_scale=None, q_z=None, z_scale=None, dt_bias=None, dt_bias_scale=None,
+                       dt_softplus=False, x_scale=None):
+    """causal_conv1d_update followed by sscan_update on the conv's output, in one launch (qa_mamba1_decode_step):
+    for decode loops whose dt, B and C are given, i.e. do not come from a projection of this step's conv output.
+    Arguments as for the two calls; the scan's x scale is the conv's ``scale_out``: pass it again as ``x_scale``, a
+    one-element fp32 GPU tensor, to keep the call free of host-to-device copies (graph capture).  conv_state and
+    state are updated in place.  Returns (conv output int8, y fp16)."""
+    pc, xc = _conv_update_params(x, conv_state, scale_x, weight, scale_w, scale_out, scale_b, bias, silu_activation)
+    if x_scale is None:
+        x_scale = torch.tensor([float(scale_out)], dtype=torch.float32, device=x.device)
+    y = sscan_update(state, xc, x_scale, q_dt, dt_scale, q_A_log, A_log_scale, ssm_state_scale, q_B, B_scale, q_C,
+                     C_scale, q_D, D_scale, q_z, z_scale, dt_bias, dt_bias_scale, dt_softplus, _conv_step=pc)
+    return xc, y
 
 
 # ----------------------------------------------------------------------------------------------
@@ -481,7 +504,7 @@ def _sscan_segments(batch, dim, seqlen):
 
 def sscan_update(state, q_x, x_scale, q_dt, dt_scale, q_A_log, A_log_scale, ssm_state_scale, q_B, B_scale,
                  q_C, C_scale, q_D=None, D_scale=None, q_z=None, z_scale=None, dt_bias=None, dt_bias_scale=None,
-                 dt_softplus=False, x_head_group_range=None, x_dim_group_range=None):
+                 dt_softplus=False, x_head_group_range=None, x_dim_group_range=None, _conv_step=None):
     """One recurrence step; ``state`` (int8 with ssm_state_scale, or fp32) is updated in place.
 
     Shapes as quamba/triton/selective_state_update.py:129-160: state (batch, dim, dstate) or
@@ -577,8 +600,12 @@ def sscan_update(state, q_x, x_scale, q_dt, dt_scale, q_A_log, A_log_scale, ssm_
         p.dt_bias = ptr(dt_bias)
         p.dt_bias_head_stride, p.dt_bias_dim_stride = dt_bias.stride()
     with torch.cuda.device(q_x.device):
-        st = _lib.lib().qa_ssm_state_update(ct.byref(p), _lib.current_stream(q_x.device))
-    _lib.check(st, "ssm_state_update")
+        if _conv_step is not None:
+            # q_x is the buffer the conv step of the same launch writes (see mamba1_decode_step)
+            st = _lib.lib().qa_mamba1_decode_step(ct.byref(_conv_step), ct.byref(p), _lib.current_stream(q_x.device))
+        else:
+            st = _lib.lib().qa_ssm_state_update(ct.byref(p), _lib.current_stream(q_x.device))
+    _lib.check(st, "mamba1_decode_step" if _conv_step is not None else "ssm_state_update")
     return out if has_heads else out.squeeze(1)
 
 

@@ -113,7 +113,8 @@ def test_w8a8_out_proj_full_size(dev):
 
 
 # ---------------------------------------------------------------- decode: batch 64, 1000 steps
-def test_decode_1000_steps(dev):
+@pytest.mark.parametrize("one_launch", [False, True], ids=["two_launches", "one_launch"])
+def test_decode_1000_steps(dev, one_launch):
     Bd, steps = 64, 1000
     conv = QCausalConv1D(D1, D1, 4, groups=D1, device=dev)
     conv.weight, conv.bias = _ri(dev, D1, 4, seed=40), _ri(dev, D1, seed=41)
@@ -135,6 +136,12 @@ def test_decode_1000_steps(dev):
     y = None
     for i in range(steps):
         x, dt, Bv, Cv, z = ring[i % 16]
+        if one_launch:
+            _, y = ops.mamba1_decode_step(x, conv_state, conv.input_scale, conv.weight, conv.weight_scale, conv.output_scale,
+                                          conv.bias_scale, conv.bias, True, ssm_state, dt, _s(sc["s_dt"], dev), A, _s(sc["s_A"], dev),
+                                          None, Bv, _s(sc["s_B"], dev), Cv, _s(sc["s_C"], dev), Dq, _s(sc["s_D"], dev), z,
+                                          _s(sc["s_z"], dev), db, _s(sc["s_db"], dev), True)
+            continue
         xc = conv.update(x, conv_state)
         y = ops.sscan_update(ssm_state, xc, _s(sc["s_x"], dev), dt, _s(sc["s_dt"], dev), A, _s(sc["s_A"], dev), None, Bv,
                              _s(sc["s_B"], dev), Cv, _s(sc["s_C"], dev), Dq, _s(sc["s_D"], dev), z, _s(sc["s_z"], dev), db,

@@ -179,6 +179,41 @@ def test_update_matches_oracle_over_several_steps(dev, B, D, N, fp32_state):
             st_ref = got.copy()              # follow the GPU's state so a one-step tie does not compound
 
 
+@pytest.mark.parametrize("B,D,N,width,state_len,fp32_state", [(3, 100, 16, 4, 3, True), (64, 1536, 16, 4, 4, False),
+                                                              (2, 257, 8, 3, 2, True), (5, 64, 16, 2, 2, False)])
+def test_decode_step_in_one_launch_equals_conv_update_then_state_update(dev, B, D, N, width, state_len, fp32_state):
+    """qa_mamba1_decode_step against the two calls it stands for, bit for bit (conv output, conv state, y, state),
+    over several steps; the two-call path is the one the oracle tests pin."""
+    steps = 4
+    g = torch.Generator(device=dev).manual_seed(B * D + width)
+    ri = lambda *shape: torch.randint(-128, 128, shape, dtype=torch.int8, device=dev, generator=g)
+    w, bias = ri(D, width), ri(D)
+    A, Dq, db = ri(D, N), ri(D), ri(D)
+    conv_a = ri(B, D, state_len)
+    st_a = (torch.randn(B, D, N, device=dev, generator=g) * 0.1) if fp32_state else ri(B, D, N)
+    conv_b, st_b = conv_a.clone(), st_a.clone()
+    sc = [_s(v, dev) for v in (0.02, 0.02, 0.03, 0.03, 0.008, 0.04, 0.01, 0.004)]
+    s_dt, s_A, s_B, s_C, s_D, s_z, s_db, s_state = sc
+    for _ in range(steps):
+        x, dt, z, Bv, Cv = ri(B, D), ri(B, D), ri(B, D), ri(B, N), ri(B, N)
+        xc_a = ops.causal_conv1d_update(x, conv_a, 0.04, w, 0.004, 0.03, 0.004, bias, True)
+        y_a = ops.sscan_update(st_a, xc_a, _s(0.03, dev), dt, s_dt, A, s_A, s_state, Bv, s_B, Cv, s_C, Dq, s_D, z, s_z, db, s_db, True)
+        xc_b, y_b = ops.mamba1_decode_step(x, conv_b, 0.04, w, 0.004, 0.03, 0.004, bias, True, st_b, dt, s_dt, A, s_A, s_state,
+                                           Bv, s_B, Cv, s_C, Dq, s_D, z, s_z, db, s_db, True)
+        assert torch.equal(xc_a, xc_b) and torch.equal(conv_a, conv_b)
+        assert torch.equal(y_a, y_b) and torch.equal(st_a, st_b)
+    assert int(xc_a.abs().max()) > 10 and float(y_a.float().abs().max()) > 0.1
+
+
+def test_decode_step_in_one_launch_refuses_what_it_does_not_cover(dev):
+    ri = lambda *shape: torch.randint(-128, 128, shape, dtype=torch.int8, device=dev)
+    B, D, N = 2, 64, 32                                      # more than sixteen states
+    with pytest.raises(NotImplementedError):
+        ops.mamba1_decode_step(ri(B, D), ri(B, D, 3), 0.04, ri(D, 4), 0.004, 0.03, 0.004, None, True,
+                               torch.zeros(B, D, N, device=dev), ri(B, D), _s(0.02, dev), ri(D, N), _s(0.02, dev), None,
+                               ri(B, N), _s(0.03, dev), ri(B, N), _s(0.03, dev))
+
+
 def test_module_forward_then_update_continue_the_same_sequence(dev):
     B, L, D, N = 2, 64, 96, 16
     d = synth.mamba1_scan_inputs(B, L + 4, D, N, seed=31)
