@@ -67,17 +67,14 @@ __global__ __launch_bounds__(kConvThreads) void conv_fwd_rows_kernel(QaConvParam
         uint32_t o[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            uint32_t packed = 0;
+            float v[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 // window ending at element 4q+j: bytes (4q+j-3 .. 4q+j) of the stream starting at w[k][1]
                 const uint32_t win = j == 3 ? w[k][q + 1] : __builtin_amdgcn_alignbyte(w[k][q + 1], w[k][q], j + 1);
-                const float acc = static_cast<float>(dot4(win, taps));
-                const float v = __builtin_fmaf(s_wx, acc, bias_f);
-                const int r = conv_quant(v, p.scale_out, inv_s_out, SILU, exact_only, kq);
-                packed |= static_cast<uint32_t>(r & 0xff) << (8 * j);
+                v[j] = __builtin_fmaf(s_wx, static_cast<float>(dot4(win, taps)), bias_f);
             }
-            o[q] = packed;
+            o[q] = conv_quant4(v, p.scale_out, inv_s_out, SILU, exact_only, kq);
         }
         if (remaining >= 16) {
             *reinterpret_cast<uint4*>(out + t0) = make_uint4(o[0], o[1], o[2], o[3]);
@@ -128,16 +125,13 @@ __global__ __launch_bounds__(kConvThreads) void conv_fwd_rows_dual_kernel(QaConv
         }
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            uint32_t packed = 0;
+            float v[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const uint32_t win = j == 3 ? w[q + 1] : __builtin_amdgcn_alignbyte(w[q + 1], w[q], j + 1);
-                const float acc = static_cast<float>(dot4(win, taps));
-                const float v = __builtin_fmaf(s_wx, acc, bias_f);
-                const int r = conv_quant(v, p.scale_out, inv_s_out, SILU, exact_only, kq);
-                packed |= static_cast<uint32_t>(r & 0xff) << (8 * j);
+                v[j] = __builtin_fmaf(s_wx, static_cast<float>(dot4(win, taps)), bias_f);
             }
-            o[q] = packed;
+            o[q] = conv_quant4(v, p.scale_out, inv_s_out, SILU, exact_only, kq);
         }
         if (remaining >= 16) {
             *reinterpret_cast<uint4*>(out + t0) = make_uint4(o[0], o[1], o[2], o[3]);

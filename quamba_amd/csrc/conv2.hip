@@ -145,15 +145,14 @@ __global__ __launch_bounds__(kThreads) void conv2_fwd_kernel(QaConv2Params p) {
         for (int i = 0; i < kBatchLoads; ++i) {
             if (tb + i >= t_end) break;
             push(d[i]);
-            uint32_t packed = 0;
+            uint32_t r[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const float acc = static_cast<float>(dot4(win[e], taps[e]));
                 const float v = __builtin_fmaf(part.s_in, acc, bias_f[e]);
-                const int q = conv_quant(v, s_out[e], inv_s_out[e], p.silu_activation, exact_only[e], kq);
-                packed |= static_cast<uint32_t>(q & 0xff) << (8 * e);
+                r[e] = conv_quant_bits(v, s_out[e], inv_s_out[e], p.silu_activation, exact_only[e], kq);
             }
-            *reinterpret_cast<uint32_t*>(out + (tb + i) * out_ls) = packed;
+            *reinterpret_cast<uint32_t*>(out + (tb + i) * out_ls) = pack_low_bytes(r[0], r[1], r[2], r[3]);
         }
     }
 }

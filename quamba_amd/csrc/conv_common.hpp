@@ -26,30 +26,70 @@ __device__ __forceinline__ int8_t conv_epilogue(float v, float s_out, int silu) 
 // through the exact route's ~100 instructions).
 __device__ __forceinline__ bool conv_needs_exact_route(float s_out) { return !(s_out >= 1e-5f); }
 
-// The bounds of the two clamps, held in registers for the life of the thread.  They are not values an
-// instruction can carry inline, and the compiler would otherwise load each of them into a register
-// again for every output (three extra instructions on a path of under thirty).
+// The constants of the cheap route, held in registers for the life of the thread.  They are not values an
+// instruction can carry inline, and the compiler would otherwise load each of them into a register again for
+// every output (three extra instructions on a path of under thirty).
 struct ConvQuantRegs {
-    float clamp_hi, q_hi;
+    float clamp_hi, magic;
     __device__ __forceinline__ ConvQuantRegs() {
-        asm volatile("v_mov_b32 %0, 0x4300c000" : "=v"(clamp_hi));     // 128.75
-        asm volatile("v_mov_b32 %0, 0x42fe0000" : "=v"(q_hi));         // 127.0
+        asm volatile("v_mov_b32 %0, 0x42fe8000" : "=v"(clamp_hi));     // 127.25
+        asm volatile("v_mov_b32 %0, 0x4b400000" : "=v"(magic));        // 1.5 * 2^23
     }
 };
 
-__device__ __forceinline__ int conv_quant(float v, float s_out, float inv_s_out, int silu, bool exact_only,
-                                          const ConvQuantRegs& k) {
+// Returns a word whose low byte is the int8 code (the bytes above it are not meaningful).
+// y is clamped to [-128.25, 127.25] first: beyond +-127.5 / -128.5 both routes saturate to the same code whatever
+// side of the half-integer they fall on, and the clamped value (a quarter away from a half-integer) passes the
+// distance test on its own.  Adding 1.5 * 2^23 rounds to the nearest integer in the addition itself (ties to
+// even; ties are not decided here) and leaves that integer's two's-complement byte in the low 8 bits of the sum.
+// the low bytes of four words, in order
+__device__ __forceinline__ uint32_t pack_low_bytes(uint32_t b0, uint32_t b1, uint32_t b2, uint32_t b3) {
+    const uint32_t lo = __builtin_amdgcn_perm(b1, b0, 0x0c0c0400u);      // bytes: b0.0, b1.0, 0, 0
+    const uint32_t hi = __builtin_amdgcn_perm(b3, b2, 0x0c0c0400u);
+    return __builtin_amdgcn_perm(hi, lo, 0x05040100u);                   // lo.0, lo.1, hi.0, hi.1
+}
+
+// The cheap route alone: the word with the code in its low byte, and whether the exact route must decide instead.
+__device__ __forceinline__ uint32_t conv_quant_cheap(float v, float inv_s_out, int silu, const ConvQuantRegs& k, bool& undecided) {
     float y = v;
     if (silu) {
         const float e = __builtin_amdgcn_exp2f(v * -1.44269504088896341f);
         y = v * __builtin_amdgcn_rcpf(1.0f + e);
     }
-    y = __builtin_amdgcn_fmed3f(y * inv_s_out, -k.clamp_hi, k.clamp_hi);
-    const float yr = __builtin_rintf(y);
-    const float d = __builtin_fabsf(y - yr);
-    int q = static_cast<int>(__builtin_amdgcn_fmed3f(yr, -128.0f, k.q_hi));
-    if (exact_only || !(d <= 0.4995f)) q = conv_epilogue(v, s_out, silu);
+    y = __builtin_amdgcn_fmed3f(y * inv_s_out, -128.25f, k.clamp_hi);
+    const float t = y + k.magic;
+    const float d = __builtin_fabsf(y - (t - k.magic));
+    undecided = !(d <= 0.4995f);
+    return __float_as_uint(t);
+}
+
+__device__ __forceinline__ uint32_t conv_quant_bits(float v, float s_out, float inv_s_out, int silu, bool exact_only,
+                                                   const ConvQuantRegs& k) {
+    bool undecided;
+    uint32_t q = conv_quant_cheap(v, inv_s_out, silu, k, undecided);
+    if (exact_only || undecided) q = static_cast<uint32_t>(static_cast<uint8_t>(conv_epilogue(v, s_out, silu)));
     return q;
+}
+
+// Four outputs at once: the four cheap evaluations are independent and interleave (each is a chain of dependent
+// instructions with two transcendentals), then every output that the cheap route could not decide - rare, so the
+// branch around each is almost never taken - goes through the exact route on its own.
+__device__ __forceinline__ uint32_t conv_quant4(const float (&v)[4], float s_out, float inv_s_out, int silu, bool exact_only,
+                                               const ConvQuantRegs& k) {
+    uint32_t q[4];
+    bool undecided[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) q[j] = conv_quant_cheap(v[j], inv_s_out, silu, k, undecided[j]);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        if (exact_only || undecided[j]) q[j] = static_cast<uint32_t>(static_cast<uint8_t>(conv_epilogue(v[j], s_out, silu)));
+    }
+    return pack_low_bytes(q[0], q[1], q[2], q[3]);
+}
+
+__device__ __forceinline__ int conv_quant(float v, float s_out, float inv_s_out, int silu, bool exact_only,
+                                          const ConvQuantRegs& k) {
+    return static_cast<int8_t>(conv_quant_bits(v, s_out, inv_s_out, silu, exact_only, k) & 0xffu);
 }
 
 // packed taps for sdot4: byte j of the window holds x[t-3+j]; tap for x[t-(k-1-w)] is W[w],
