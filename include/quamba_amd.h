@@ -317,7 +317,8 @@ int qa_mamba1_decode_step(const QaConvParams* conv, const QaSsmUpdateParams* p, 
  * Both operands are K-contiguous: a is (M,K) with row stride lda; w is (N,K) with row stride ldw
  * (the reference's column-major (K,N) "b" operand is the same memory).
  * ---------------------------------------------------------------------------------------- */
-typedef enum QaOutType { QA_OUT_I8 = 0, QA_OUT_F16 = 1 } QaOutType;
+/* BF16 (round to nearest even, csrc/linear/quant_linear_fwd_kernel.cuh:312-316) is an output of the W8A8 GEMM only. */
+typedef enum QaOutType { QA_OUT_I8 = 0, QA_OUT_F16 = 1, QA_OUT_BF16 = 2 } QaOutType;
 /* QA_ROUND_HALF_AWAY selects the rule of w8a8o8_gemv: d = sat8(roundf((s_w[n] * s_a[m|0]) * float(acc))) */
 typedef enum QaRound { QA_ROUND_RNE = 0, QA_ROUND_HALF_AWAY = 1 } QaRound;
 

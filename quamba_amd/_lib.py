@@ -10,7 +10,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libquamba_amd.so")
 
 QA_OK = 0
-QA_OUT_I8, QA_OUT_F16 = 0, 1
+QA_OUT_I8, QA_OUT_F16, QA_OUT_BF16 = 0, 1, 2
 QA_ROUND_RNE, QA_ROUND_HALF_AWAY = 0, 1
 QA_IN_F16, QA_IN_F32 = 0, 1
 

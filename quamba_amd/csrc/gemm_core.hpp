@@ -56,6 +56,25 @@ __device__ __forceinline__ uint32_t pack4_rne_sat8(float v0, float v1, float v2,
     return __builtin_amdgcn_perm(hi, lo, 0x05040100u);                   // lo.0, lo.1, hi.0, hi.1
 }
 
+// Two fp32 values -> two 16-bit floats of the output type (round to nearest even) in one word; bf16 rounds on the
+// bit pattern: add 0x7fff plus the lowest kept bit, keep the high half (NaN payloads are not preserved).
+__device__ __forceinline__ uint32_t bf16_bits(float v) {
+    const uint32_t u = __float_as_uint(v);
+    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+template <int OUT>
+__device__ __forceinline__ uint32_t pack2_f16_or_bf16(float v0, float v1) {
+    if (OUT == QA_OUT_BF16) return bf16_bits(v0) | (bf16_bits(v1) << 16);
+    const __half2 h = __floats2half2_rn(v0, v1);
+    return *reinterpret_cast<const uint32_t*>(&h);
+}
+template <int OUT>
+__device__ __forceinline__ uint16_t one_f16_or_bf16(float v) {
+    if (OUT == QA_OUT_BF16) return static_cast<uint16_t>(bf16_bits(v));
+    const __half h = __float2half(v);
+    return *reinterpret_cast<const uint16_t*>(&h);
+}
+
 struct Epilogue {
     const float* row_scale;   // s_row, numel 1 or M (unused with use_alpha)
     const float* col_scale;   // s_col, numel 1 or N
@@ -79,6 +98,27 @@ struct Cfg {
     static constexpr int kStageBytes = (kBM + kBN) * kBK;
     static constexpr int kLdsBytes = STAGES * kStageBytes;
 };
+
+// Output tile of workgroup `linear`.  Workgroups go to the eight XCDs (each with an L2 of its own) in turn by linear
+// index, and with one workgroup per CU a launch runs in rounds of 256.  The tiles an XCD works on at the same time
+// should share operand panels, so that its L2 fetches each panel once per round: the 32 workgroups an XCD gets in a
+// round take 32 consecutive positions of an order that walks the tile grid in bands of four m-tiles, n-tile by
+// n-tile - a block of 4 x 8 tiles, whatever the tile counts are (the natural m-first order does that only when the
+// number of m-tiles is a multiple of eight).  The workgroups past the last full round keep the band order as it is.
+__device__ __forceinline__ void tile_of_workgroup(int linear, int tiles_m, int tiles_n, int& tm, int& tn) {
+    constexpr int kXcds = 8, kPerXcd = 32, kRound = kXcds * kPerXcd, kBand = 4;
+    const int tiles = tiles_m * tiles_n;
+    int g = linear;
+    if (linear < tiles / kRound * kRound) {
+        const int xcd = linear % kXcds, pos = linear / kXcds;
+        g = ((pos / kPerXcd) * kXcds + xcd) * kPerXcd + pos % kPerXcd;
+    }
+    const int per_band = kBand * tiles_n;
+    const int band = g / per_band, in_band = g % per_band;
+    const int rows = min(kBand, tiles_m - band * kBand);          // the last band may be narrower
+    tm = band * kBand + in_band % rows;
+    tn = in_band / rows;
+}
 
 // Raw buffer descriptor (base, stride 0, num_records bytes) held in four scalar registers.
 __device__ __forceinline__ v4i make_rsrc(const void* base, int num_bytes) {
@@ -302,10 +342,9 @@ __device__ __forceinline__ void epilogue(const Epilogue& e, v16i (&acc)[TN][TM],
                         }
                         *reinterpret_cast<uint32_t*>(stg + frow * kPitch + nl) = word;
                     } else {
-                        __half2 lo = __floats2half2_rn(v0, v1), hi = __floats2half2_rn(v2, v3);
                         uint2 pk;
-                        pk.x = *reinterpret_cast<uint32_t*>(&lo);
-                        pk.y = *reinterpret_cast<uint32_t*>(&hi);
+                        pk.x = pack2_f16_or_bf16<OUT>(v0, v1);
+                        pk.y = pack2_f16_or_bf16<OUT>(v2, v3);
                         *reinterpret_cast<uint2*>(stg + frow * kPitch + nl * 2) = pk;
                     }
                 }
@@ -348,7 +387,7 @@ __device__ __forceinline__ void epilogue(const Epilogue& e, v16i (&acc)[TN][TM],
                             *reinterpret_cast<int8_t*>(stg + nl * kPitch + j * 32 + frow) =
                                 static_cast<int8_t>(quant8(v, round_mode));
                         } else {
-                            *reinterpret_cast<__half*>(stg + nl * kPitch + (j * 32 + frow) * 2) = __float2half(v);
+                            *reinterpret_cast<uint16_t*>(stg + nl * kPitch + (j * 32 + frow) * 2) = one_f16_or_bf16<OUT>(v);
                         }
                     }
                 }
@@ -439,15 +478,14 @@ __device__ __forceinline__ void skinny_reduce_store(const Epilogue& e, v16i (&ac
                 for (int t = 0; t < cols; ++t) dst[t * step] = static_cast<int8_t>(quant8(v[t], round_mode));
             }
         } else {
-            __half* dst = static_cast<__half*>(e.d) + at;
+            uint16_t* dst = static_cast<uint16_t*>(e.d) + at;
             if (vec_ok && cols == 4) {
-                const __half2 lo = __floats2half2_rn(v[0], v[1]), hi = __floats2half2_rn(v[2], v[3]);
                 uint2 pk;
-                pk.x = *reinterpret_cast<const uint32_t*>(&lo);
-                pk.y = *reinterpret_cast<const uint32_t*>(&hi);
+                pk.x = pack2_f16_or_bf16<OUT>(v[0], v[1]);
+                pk.y = pack2_f16_or_bf16<OUT>(v[2], v[3]);
                 *reinterpret_cast<uint2*>(dst) = pk;
             } else {
-                for (int t = 0; t < cols; ++t) dst[t * step] = __float2half(v[t]);
+                for (int t = 0; t < cols; ++t) dst[t * step] = one_f16_or_bf16<OUT>(v[t]);
             }
         }
     }

@@ -24,10 +24,10 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_w8a8_kernel(QaGemmW8A8Par
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave % WGM, wn = wave / WGM;
-    // consecutive workgroups walk down m first so that neighbours share the same weight tile
-    const int tiles_m = (p.m + BM - 1) / BM;
-    const int m0 = (blockIdx.x % tiles_m) * BM;
-    const int n0 = (blockIdx.x / tiles_m) * BN;
+    const int tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
+    int tile_m, tile_n;
+    tile_of_workgroup(blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
 
     const v4i rsrc_a = make_rsrc(p.a, static_cast<int>((static_cast<int64_t>(p.m) - 1) * p.lda + p.k));
     const v4i rsrc_w = make_rsrc(p.w, static_cast<int>((static_cast<int64_t>(p.n) - 1) * p.ldw + p.k));
@@ -105,8 +105,9 @@ int launch_one(const QaGemmW8A8Params& p, hipStream_t stream) {
 
 template <int TM, int TN, int WGM, int WGN, int STAGES, bool FLEX>
 int launch_gemm(const QaGemmW8A8Params& p, hipStream_t stream) {
-    return p.out_type == QA_OUT_I8 ? launch_one<TM, TN, WGM, WGN, STAGES, QA_OUT_I8, FLEX>(p, stream)
-                                   : launch_one<TM, TN, WGM, WGN, STAGES, QA_OUT_F16, FLEX>(p, stream);
+    if (p.out_type == QA_OUT_I8) return launch_one<TM, TN, WGM, WGN, STAGES, QA_OUT_I8, FLEX>(p, stream);
+    if (p.out_type == QA_OUT_BF16) return launch_one<TM, TN, WGM, WGN, STAGES, QA_OUT_BF16, FLEX>(p, stream);
+    return launch_one<TM, TN, WGM, WGN, STAGES, QA_OUT_F16, FLEX>(p, stream);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -233,8 +234,9 @@ int launch_skinny_one(const QaGemmW8A8Params& p, hipStream_t stream) {
 
 template <int TM, int WAVES, bool FLEX>
 int launch_skinny(const QaGemmW8A8Params& p, hipStream_t stream) {
-    return p.out_type == QA_OUT_I8 ? launch_skinny_one<TM, WAVES, QA_OUT_I8, FLEX>(p, stream)
-                                   : launch_skinny_one<TM, WAVES, QA_OUT_F16, FLEX>(p, stream);
+    if (p.out_type == QA_OUT_I8) return launch_skinny_one<TM, WAVES, QA_OUT_I8, FLEX>(p, stream);
+    if (p.out_type == QA_OUT_BF16) return launch_skinny_one<TM, WAVES, QA_OUT_BF16, FLEX>(p, stream);
+    return launch_skinny_one<TM, WAVES, QA_OUT_F16, FLEX>(p, stream);
 }
 
 template <bool FLEX>
@@ -255,7 +257,7 @@ extern "C" int qa_gemm_w8a8(const QaGemmW8A8Params* p, void* stream_) {
     if (!p || !p->a || !p->w || !p->d) return QA_ERR_NULL;
     if (!p->use_alpha && (!p->a_scale || !p->w_scale)) return QA_ERR_NULL;
     if (p->m < 0 || p->n < 0 || p->k < 0) return QA_ERR_SHAPE;
-    if (p->out_type != QA_OUT_I8 && p->out_type != QA_OUT_F16) return QA_ERR_UNSUPPORTED;
+    if (p->out_type != QA_OUT_I8 && p->out_type != QA_OUT_F16 && p->out_type != QA_OUT_BF16) return QA_ERR_UNSUPPORTED;
     if (p->scale_order != 0 && p->scale_order != 1) return QA_ERR_UNSUPPORTED;
     if (p->scale_order == 1 && (p->use_alpha || p->round_mode != QA_ROUND_RNE)) return QA_ERR_UNSUPPORTED;
     if (!p->use_alpha && p->a_scale_numel != 1 && p->a_scale_numel != p->m) return QA_ERR_SHAPE;

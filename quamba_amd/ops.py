@@ -617,7 +617,7 @@ def _gemm_w8a8(c, a, w_nk, a_scales, b_scales, alpha=None, round_half_away=False
     _require(a.dtype == torch.int8 and w_nk.dtype == torch.int8, "a and b must be int8")
     for t, n in ((a, "a"), (w_nk, "b"), (c, "c")):
         _require_gpu(t, n)
-    _require(c.dtype in (torch.int8, torch.float16), "c must be int8 or fp16")
+    _require(c.dtype in (torch.int8, torch.float16, torch.bfloat16), "c must be int8, fp16 or bf16")
     M, K = a.shape
     N = w_nk.shape[0]
     _require(w_nk.shape[1] == K and tuple(c.shape) == (M, N), "shape mismatch: c (M,N) = a (M,K) x b (K,N)")
@@ -627,7 +627,7 @@ def _gemm_w8a8(c, a, w_nk, a_scales, b_scales, alpha=None, round_half_away=False
              "row strides of a and b and K must be multiples of 16")
     p = _lib.QaGemmW8A8Params()
     p.m, p.n, p.k = M, N, K
-    p.out_type = _lib.QA_OUT_I8 if c.dtype == torch.int8 else _lib.QA_OUT_F16
+    p.out_type = {torch.int8: _lib.QA_OUT_I8, torch.float16: _lib.QA_OUT_F16, torch.bfloat16: _lib.QA_OUT_BF16}[c.dtype]
     p.round_mode = _lib.QA_ROUND_HALF_AWAY if round_half_away else _lib.QA_ROUND_RNE
     p.lda, p.ldw, p.ldd = a.stride(0), w_nk.stride(0), c.stride(0)
     p.a, p.w, p.d = ptr(a), ptr(w_nk), ptr(c)
@@ -648,7 +648,7 @@ def _gemm_w8a8(c, a, w_nk, a_scales, b_scales, alpha=None, round_half_away=False
 def scaled_mm_dq(c, a, b, a_scales, b_scales):
     """c = cast(a_scales * (b_scales * (a @ b))) with a int8 (M,K) row-major, b int8 (K,N) column-major
     (b.stride(0) == 1), scales fp32 with 1 or M / 1 or N elements; c int8 (round-half-even,
-    saturating) or fp16, written in place.  Interface of cutlass_scaled_mm_dq."""
+    saturating), fp16 or bf16, written in place.  Interface of cutlass_scaled_mm_dq."""
     _require(b.dim() == 2 and b.stride(0) == 1, "b must be column-major")
     return _gemm_w8a8(c, a, b.t(), a_scales, b_scales)
 

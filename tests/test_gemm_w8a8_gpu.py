@@ -60,6 +60,20 @@ def test_fp16_output_bit_exact(dev, M, N, K):
     np.testing.assert_array_equal(c.cpu().numpy(), f.astype(np.float16))
 
 
+@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (300, 200, 208), (33, 24, 48), (2048, 2560, 512),
+                                   (64, 2560, 5120), (1, 48, 64), (2400, 8100, 80)])
+def test_bf16_output_bit_exact(dev, M, N, K):
+    """bf16 = the oracle's fp32 value rounded to nearest even (the reference's converter); compared as bit patterns."""
+    a, w, sa, sb = _operands(M, N, K, seed=5 * M + K)
+    _, f, _ = oracle.gemm_w8a8(a, w, sa, sb)
+    c = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+    ops.scaled_mm_dq(c, _t(a, dev), _t(w, dev).t(), _t(sa, dev), _t(sb, dev))
+    u = np.ascontiguousarray(f, np.float32).view(np.uint32).astype(np.uint64)
+    want = ((u + 0x7fff + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+    assert np.array_equal(want, torch.from_numpy(f).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16))
+    np.testing.assert_array_equal(c.view(torch.int16).cpu().numpy().view(np.uint16), want)
+
+
 @pytest.mark.parametrize("out_dtype", [torch.int8, torch.float16])
 def test_wide_tile_path_matches_exact_fp32(dev, out_dtype):
     """16384 x 2560 is the shape for which the 256x320 tile is chosen (two full rounds of workgroups).
