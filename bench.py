@@ -554,13 +554,40 @@ def valu_calibration(dev, ops_list=None, launches=4):
 SCAN_MIX = {"four_lane": {"plain": 99, "transcendental": 18}, "eight_lane": {"plain": 58, "transcendental": 9}}
 
 
+def scan_mix_rates(dev):
+    """Issue time of the scan's own instruction mix on live values (probe ops 6 and 7: the recurrence on registers,
+    four plain instructions and one exp2 per chain step, and the same with four more plain instructions): ns per
+    plain and per transcendental wave-instruction per SIMD, and the clock the part settles at under that activity.
+    Constant operands (valu_calibration) leave the part at its highest clock and give lower figures."""
+    from quamba_amd import _lib
+    lib = _probes()
+    wgs, iters = 2048, 10000
+    sink = torch.empty(wgs * 256, dtype=torch.float32, device=dev)
+    ticks = torch.zeros(2, dtype=torch.int64, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    simds = 4 * torch.cuda.get_device_properties(dev).multi_processor_count
+    ns, clock = {}, {}
+    for op in (6, 7):
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            _lib.check(lib.qa_probe_valu(sink.data_ptr(), sink.numel(), ticks.data_ptr(), wgs, iters, op, stream), "diag")
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1)
+        t = ticks.tolist()
+        ns[op] = ms * 1e6 / (wgs * 4.0 / simds * iters * 8)       # per chain step per SIMD
+        clock[op] = 100.0 * t[0] / max(t[1], 1)
+    t_plain = (ns[7] - ns[6]) / 4.0
+    return dict(ns_plain=t_plain, ns_transcendental=ns[6] - 4.0 * t_plain, clock_MHz=clock[6])
+
+
 def scan_issue_bound(dev, B, D, L):
-    """Lower bound of the scan launch from vector-ALU issue alone: every wave's instruction mix priced at the rates a
-    register-only loop reaches on this GPU now (measured here with the probe library), the waves spread evenly over
-    the SIMDs.  Follows the host's choice of the two kinds of workgroup for d_state 16 (qa_sscan_fwd)."""
-    rates = valu_calibration(dev, ("v_mul_f32", "v_exp_f32"), launches=2)
-    t_plain = rates["v_mul_f32"]["ns_per_wave_instruction_per_simd"]
-    t_trans = rates["v_exp_f32"]["ns_per_wave_instruction_per_simd"]
+    """Lower bound of the scan launch from vector-ALU issue alone: every wave's instruction mix priced at the rates
+    the same mix reaches in a register-only loop on live values on this GPU now (scan_mix_rates), the waves spread
+    evenly over the SIMDs.  Follows the host's choice of the two kinds of workgroup for d_state 16 (qa_sscan_fwd)."""
+    rates = scan_mix_rates(dev)
+    t_plain, t_trans = rates["ns_plain"], rates["ns_transcendental"]
     simds = 4 * torch.cuda.get_device_properties(dev).multi_processor_count
     waves4 = B * D // 16
     q, rem = divmod(waves4, simds)
@@ -572,8 +599,8 @@ def scan_issue_bound(dev, B, D, L):
     waves = {"four_lane": B * (D - short) // 16, "eight_lane": B * short // 8}
     groups = (L + 31) // 32 * 8
     ns = sum(waves[k] * groups * (SCAN_MIX[k]["plain"] * t_plain + SCAN_MIX[k]["transcendental"] * t_trans) for k in waves)
-    return dict(issue_bound_us=ns / simds / 1e3, ns_plain=t_plain, ns_transcendental=t_trans, waves=waves,
-                instructions_per_four_steps=SCAN_MIX)
+    return dict(issue_bound_us=ns / simds / 1e3, ns_plain=round(t_plain, 3), ns_transcendental=round(t_trans, 3),
+                clock_MHz=round(rates["clock_MHz"], 1), waves=waves, instructions_per_four_steps=SCAN_MIX)
 
 
 def main():
@@ -642,7 +669,8 @@ def main():
         ib = scan_issue_bound(dev, B, CFG["d_inner"], L)
         roofline["issue_bound_us"] = round(ib["issue_bound_us"], 2)
         roofline["frac_of_issue_bound"] = round(ib["issue_bound_us"] / dom["avg_us"], 4)
-        roofline["issue_bound_inputs"] = {k: ib[k] for k in ("ns_plain", "ns_transcendental", "waves", "instructions_per_four_steps")}
+        roofline["issue_bound_inputs"] = {k: ib[k] for k in ("ns_plain", "ns_transcendental", "clock_MHz", "waves",
+                                                             "instructions_per_four_steps")}
     per_kernel = [dict(kernel=k["name"], bound=k["bound"], avg_us=round(k["avg_us"], 2), achieved=round(k["achieved"], 2),
                        unit=k["unit"], peak=k["peak"], frac=round(k["frac"], 4), traffic=traffic.get(k["name"]))
                   for k in kernels]

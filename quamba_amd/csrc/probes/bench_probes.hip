@@ -51,7 +51,7 @@ __global__ __launch_bounds__(256) void diag_mfma_i8_kernel(int* sink, long long*
     }
 }
 // op 0: v_mul_f32, 1: v_exp_f32, 2: v_rcp_f32, 3: v_log_f32, 4: v_fmac_f32, 5: v_mul_f32 with a quad broadcast (DPP);
-// eight chains per lane
+// eight chains per lane (op 6, 7: diag_scan_mix_kernel below)
 template <int OP>
 __global__ __launch_bounds__(256) void diag_valu_kernel(float* sink, long long* ticks, int iters) {
     const unsigned t = blockIdx.x * 256 + threadIdx.x;
@@ -77,6 +77,48 @@ __global__ __launch_bounds__(256) void diag_valu_kernel(float* sink, long long* 
         ticks[1] = wall_clock64() - w0;
     }
 }
+// The selective scan's recurrence on live values, registers only: per chain and iteration
+//   x = -|h| A;  a = exp2(x);  t = B u;  h = a h + t;  acc = h C + acc      (four plain instructions, one exp2)
+// and, with EXTRA, four more plain instructions on changing values.  The values keep moving (h is bounded: the larger
+// it gets the faster it decays), so the vector ALUs switch as they do in the real kernel and the part settles at the
+// clock it would run the real kernel at; constant operands, as in diag_valu_kernel, leave it at its highest clock.
+template <bool EXTRA>
+__global__ __launch_bounds__(256) void diag_scan_mix_kernel(float* sink, long long* ticks, int iters) {
+    const unsigned t = blockIdx.x * 256 + threadIdx.x;
+    float h[8], acc[8], u[8], e1[8];
+    const float A = 0.05f + 1e-4f * static_cast<float>(mix32(t) & 1023u);
+    const float Bv = 1e-3f * (static_cast<float>(mix32(t + 7u) & 2047u) - 1024.0f);
+    const float Cv = 1e-3f * (static_cast<float>(mix32(t + 13u) & 2047u) - 1024.0f);
+    for (int i = 0; i < 8; ++i) {
+        h[i] = 0.0f; acc[i] = 0.0f; e1[i] = 1.0f;
+        u[i] = 1e-2f * (static_cast<float>(mix32(t * 8 + i) & 255u) - 128.0f);
+    }
+    const long long c0 = clock64(), w0 = wall_clock64();
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float x, a, tt;
+            asm volatile("v_mul_f32 %0, -|%1|, %2" : "=v"(x) : "v"(h[i]), "v"(A));
+            asm volatile("v_exp_f32 %0, %1" : "=v"(a) : "v"(x));
+            asm volatile("v_mul_f32 %0, %1, %2" : "=v"(tt) : "v"(Bv), "v"(u[i]));
+            asm volatile("v_fma_f32 %0, %1, %0, %2" : "+v"(h[i]) : "v"(a), "v"(tt));
+            asm volatile("v_fmac_f32 %0, %1, %2" : "+v"(acc[i]) : "v"(h[i]), "v"(Cv));
+            if (EXTRA) {
+                asm volatile("v_fma_f32 %0, %1, %2, %0" : "+v"(e1[i]) : "v"(a), "v"(Cv));
+                asm volatile("v_mul_f32 %0, %1, %0" : "+v"(e1[i]) : "v"(a));
+                asm volatile("v_fma_f32 %0, %1, %2, %0" : "+v"(e1[i]) : "v"(tt), "v"(A));
+                asm volatile("v_mul_f32 %0, %1, %0" : "+v"(e1[i]) : "v"(a));
+            }
+        }
+    }
+    float s = 0.0f;
+    for (int i = 0; i < 8; ++i) s += acc[i] + e1[i];
+    sink[t] = s;
+    if (t == 0 && ticks) {
+        ticks[0] = clock64() - c0;
+        ticks[1] = wall_clock64() - w0;
+    }
+}
 }  // namespace
 }  // namespace qa
 
@@ -84,7 +126,7 @@ extern "C" int qa_probe_valu(float* sink, int64_t sink_elems, long long* ticks, 
                             void* stream) {
     if (!sink) return QA_ERR_NULL;
     if (workgroups < 1 || iters < 0 || sink_elems < static_cast<int64_t>(workgroups) * 256) return QA_ERR_SHAPE;
-    if (op < 0 || op > 5) return QA_ERR_UNSUPPORTED;
+    if (op < 0 || op > 7) return QA_ERR_UNSUPPORTED;
     const dim3 grid(static_cast<unsigned>(workgroups)), block(256);
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (op == 0) hipLaunchKernelGGL(qa::diag_valu_kernel<0>, grid, block, 0, st, sink, ticks, iters);
@@ -92,7 +134,9 @@ extern "C" int qa_probe_valu(float* sink, int64_t sink_elems, long long* ticks, 
     else if (op == 2) hipLaunchKernelGGL(qa::diag_valu_kernel<2>, grid, block, 0, st, sink, ticks, iters);
     else if (op == 3) hipLaunchKernelGGL(qa::diag_valu_kernel<3>, grid, block, 0, st, sink, ticks, iters);
     else if (op == 4) hipLaunchKernelGGL(qa::diag_valu_kernel<4>, grid, block, 0, st, sink, ticks, iters);
-    else hipLaunchKernelGGL(qa::diag_valu_kernel<5>, grid, block, 0, st, sink, ticks, iters);
+    else if (op == 5) hipLaunchKernelGGL(qa::diag_valu_kernel<5>, grid, block, 0, st, sink, ticks, iters);
+    else if (op == 6) hipLaunchKernelGGL(qa::diag_scan_mix_kernel<false>, grid, block, 0, st, sink, ticks, iters);
+    else hipLaunchKernelGGL(qa::diag_scan_mix_kernel<true>, grid, block, 0, st, sink, ticks, iters);
     return qa::check_launch();
 }
 
