@@ -102,11 +102,13 @@ struct Cfg {
 // Output tile of workgroup `linear`.  Workgroups go to the eight XCDs (each with an L2 of its own) in turn by linear
 // index, and with one workgroup per CU a launch runs in rounds of 256.  The tiles an XCD works on at the same time
 // should share operand panels, so that its L2 fetches each panel once per round: the 32 workgroups an XCD gets in a
-// round take 32 consecutive positions of an order that walks the tile grid in bands of four m-tiles, n-tile by
-// n-tile - a block of 4 x 8 tiles, whatever the tile counts are (the natural m-first order does that only when the
-// number of m-tiles is a multiple of eight).  The workgroups past the last full round keep the band order as it is.
+// round take 32 consecutive positions of an order that walks the tile grid in bands of BAND m-tiles, n-tile by
+// n-tile - a block of BAND x 32/BAND tiles, whatever the tile counts are (the natural m-first order does that only
+// when the number of m-tiles is a multiple of eight).  BAND is 4 or 8, whichever makes the block's operand rows
+// (BAND BM + 32/BAND BN) fewer.  The workgroups past the last full round keep the band order as it is.
+template <int BM, int BN>
 __device__ __forceinline__ void tile_of_workgroup(int linear, int tiles_m, int tiles_n, int& tm, int& tn) {
-    constexpr int kXcds = 8, kPerXcd = 32, kRound = kXcds * kPerXcd, kBand = 4;
+    constexpr int kXcds = 8, kPerXcd = 32, kRound = kXcds * kPerXcd, kBand = BN > BM ? 8 : 4;
     const int tiles = tiles_m * tiles_n;
     int g = linear;
     if (linear < tiles / kRound * kRound) {

@@ -76,7 +76,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_w4a8_kernel(QaGemmW4A8Par
     const int wm = wave % WGM, wn = wave / WGM;
     const int tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
     int tile_m, tile_n;
-    tile_of_workgroup(blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
+    tile_of_workgroup<BM, BN>(blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const bool grouped = p.group_size > 0;
 

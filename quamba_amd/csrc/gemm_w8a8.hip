@@ -26,7 +26,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_w8a8_kernel(QaGemmW8A8Par
     const int wm = wave % WGM, wn = wave / WGM;
     const int tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
     int tile_m, tile_n;
-    tile_of_workgroup(blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
+    tile_of_workgroup<BM, BN>(blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 
     const v4i rsrc_a = make_rsrc(p.a, static_cast<int>((static_cast<int64_t>(p.m) - 1) * p.lda + p.k));
