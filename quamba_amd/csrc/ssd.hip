@@ -505,7 +505,7 @@ __global__ __launch_bounds__(64 * scan_waves_of(Q), 4) void ssd_chunk_scan_kerne
     constexpr int kThreads = 64 * kWaves;
     constexpr int NMT = Q / 16;                                   // 16-row m-tiles of a chunk
     constexpr int TILES = NMT / kWaves;                           // per wave: 4 (Q 256), 2 (Q 128), 1 (Q 64)
-    constexpr int WIN = 4;                                        // pieces of C B^T in flight: a rolling window
+    constexpr int WIN = 2;                                        // pieces of C B^T in flight: a rolling window
     static_assert(Q <= kThreads, "a thread stages at most one share of the x tile");
     constexpr int PPC = kP * N / 8;                               // 16-byte pieces of the entering state
     constexpr int PB = PPC / kThreads;
