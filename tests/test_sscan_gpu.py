@@ -214,6 +214,49 @@ def test_decode_step_in_one_launch_refuses_what_it_does_not_cover(dev):
                                ri(B, N), _s(0.03, dev), ri(B, N), _s(0.03, dev))
 
 
+@pytest.mark.parametrize("s_dt,s_db", [(0.03, 0.05), (0.08, 0.02), (0.2, 0.1)])
+@pytest.mark.parametrize("lanes", [4, 8])
+def test_step_sizes_against_fp64_softplus(dev, s_dt, s_db, lanes):
+    """The step size the forward kernels form, softplus(s_dt q + s_db q_b), read back through dt_sum_out on one-step
+    sequences: every int8 code (one per batch entry) against 256 channels' biases, compared with the fp64 value.  The
+    kernel's softplus is exp2 / log2 on the hardware with one compensated rounding; the arguments reach +-38."""
+    import ctypes as ct
+    from quamba_amd import _lib
+    Bn, D, L, N = 256, 256, 1, 16
+    q = torch.arange(-128, 128, dtype=torch.int8, device=dev).view(Bn, 1, 1).expand(Bn, D, L).contiguous()
+    u = torch.ones(Bn, D, L, dtype=torch.int8, device=dev)
+    A = torch.zeros(D, N, dtype=torch.int8, device=dev)
+    Bm = torch.zeros(Bn, 1, N, L, dtype=torch.int8, device=dev)
+    Cm = Bm.clone()
+    db = torch.randint(-128, 128, (D,), dtype=torch.int8, device=dev, generator=torch.Generator(device=dev).manual_seed(3))
+    out = torch.empty(Bn, L, D, dtype=torch.float16, device=dev)
+    st = torch.empty(Bn, D, 1, N, dtype=torch.float32, device=dev)
+    dts = torch.empty(Bn, D, dtype=torch.float32, device=dev)
+    sc = [_s(v, dev) for v in (0.03, s_dt, 0.02, 0.03, 0.03, s_db)]
+    p = _lib.QaSScanParams()
+    p.batch, p.dim, p.seqlen, p.dstate, p.n_groups = Bn, D, L, N, 1
+    p.delta_softplus = 1
+    p.u_batch_stride, p.u_d_stride = u.stride(0), u.stride(1)
+    p.delta_batch_stride, p.delta_d_stride = q.stride(0), q.stride(1)
+    p.B_batch_stride, p.B_group_stride, p.B_dstate_stride = Bm.stride(0), Bm.stride(1), Bm.stride(2)
+    p.C_batch_stride, p.C_group_stride, p.C_dstate_stride = Cm.stride(0), Cm.stride(1), Cm.stride(2)
+    p.A_d_stride, p.A_dstate_stride = A.stride(0), A.stride(1)
+    p.out_batch_stride, p.out_l_stride, p.out_d_stride = out.stride()
+    p.u, p.delta, p.A_log, p.B, p.C, p.out = (t.data_ptr() for t in (u, q, A, Bm, Cm, out))
+    p.scale_u, p.scale_delta, p.scale_A, p.scale_B, p.scale_C = (t.data_ptr() for t in sc[:5])
+    p.delta_bias, p.scale_delta_bias = db.data_ptr(), sc[5].data_ptr()
+    p.last_state_f32, p.dt_sum_out = st.data_ptr(), dts.data_ptr()
+    p.mapping = ops.sscan_mapping(lanes, 4)
+    _lib.check(_lib.lib().qa_sscan_fwd(ct.byref(p), _lib.current_stream(dev)), "sscan_fwd")
+    torch.cuda.synchronize()
+    x = (np.float32(s_dt) * np.arange(-128, 128, dtype=np.float32)[:, None]
+         + np.float32(s_db) * db.cpu().numpy().astype(np.float32)[None, :])
+    want = np.where(x > 20, x.astype(np.float64), np.log1p(np.exp(x.astype(np.float64))))
+    got = dts.cpu().numpy().astype(np.float64)
+    assert np.abs(got - want).max() > 0                       # hardware exp2 / log2: close, not equal
+    assert (np.abs(got - want) / want).max() <= 1e-5
+
+
 def test_module_forward_then_update_continue_the_same_sequence(dev):
     B, L, D, N = 2, 64, 96, 16
     d = synth.mamba1_scan_inputs(B, L + 4, D, N, seed=31)
