@@ -193,7 +193,7 @@ def _wl_decode(dev):
     conv = QCausalConv1D(D, D, 4, groups=D, device=dev)
     conv.weight, conv.bias = ri(D, 4), ri(D)
     conv.weight_scale, conv.bias_scale, conv.input_scale, conv.output_scale = 0.004, 0.004, 0.04, 0.03
-    conv_state, ssm_state = ri(B, D, 3), torch.randn(B, D, N, device=dev) * 0.1
+    conv_state, ssm_state = ri(B, D, 4), torch.randn(B, D, N, device=dev) * 0.1   # the reference's (B, D, d_conv) conv state
     ring = [(ri(B, D), ri(B, D), ri(B, N), ri(B, N), ri(B, D)) for _ in range(16)]
     A, Dq, db = ri(D, N), ri(D), ri(D)
     it = [0]
@@ -228,7 +228,7 @@ def _wl_decode(dev):
         return _time_fn(graph.replay, 64, 4) / 16
     ms_two = graphed(decode)
     ms = graphed(decode_one_launch)
-    nbytes = 3 * B * D + 2 * B * D * 3 + 2 * B * D * N * 4 + 2 * B * D + D * N
+    nbytes = 3 * B * D + 2 * B * D * 4 + 2 * B * D * N * 4 + 2 * B * D + D * N
     return dict(workload="Mamba1-2.8b decode step (conv update + state update in one launch), batch 64, fp32 state, HIP graph of 16 steps",
                 name="decode_step", us=ms * 1e3, us_two_launches=ms_two * 1e3, us_eager_python=ms_eager * 1e3, tokens_per_s=B / ms * 1e3, bound="hbm",
                 bytes=nbytes, achieved_GBs=nbytes / ms / 1e6, frac=nbytes / ms / 1e6 / HBM_PEAK_GBS)

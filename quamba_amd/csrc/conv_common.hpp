@@ -112,6 +112,9 @@ __device__ __forceinline__ int dot4(uint32_t a, uint32_t b) {
 // on by one step (in place), the window meets the taps, bias, SiLU, requantisation.  Returns the int8 output and,
 // with `store`, writes state and output.  Taps and a four-wide state row are fetched as one word when their layout
 // allows; the requantisation takes the cheap route whenever it provably equals the exact one (conv_quant).
+// W4: four taps with unit stride and a state of four codes (conv_state_len 4, unit stride), each row one aligned
+// word, known at compile time.
+template <bool W4 = false>
 __device__ __forceinline__ int8_t conv_step_row(const QaConvParams& p, int b, int c, bool store) {
     int8_t* st = p.conv_state + b * p.conv_state_batch_stride + c * p.conv_state_c_stride;
     const int8_t* w = p.weight + c * p.weight_c_stride;
@@ -119,6 +122,28 @@ __device__ __forceinline__ int8_t conv_step_row(const QaConvParams& p, int b, in
     const int slen = p.conv_state_len;            // width (slot 0 is dropped) or width-1
     const int drop = slen - (width - 1);          // 1 or 0
     __attribute__((aligned(4))) int8_t xs[4], ws[4] = {0, 0, 0, 0};
+    if constexpr (W4) {
+        // the caller has checked: four taps in one aligned word, a state of four codes in one aligned word.  Every
+        // load is issued at once (the bias through a stand-in address when there is none), no branch in between.
+        const int8_t* x_a = p.x + b * p.x_batch_stride + c * p.x_c_stride;
+        const uint32_t w_word4 = *reinterpret_cast<const uint32_t*>(w);
+        const uint32_t row4 = *reinterpret_cast<const uint32_t*>(st);
+        const int8_t x_new = *x_a;
+        const int8_t bias_q = *(p.bias ? p.bias + c : x_a);
+        const uint32_t win4 = (row4 >> 8) | (static_cast<uint32_t>(static_cast<uint8_t>(x_new)) << 24);
+        if (store) *reinterpret_cast<uint32_t*>(st) = win4;
+        *reinterpret_cast<uint32_t*>(ws) = w_word4;
+        *reinterpret_cast<uint32_t*>(xs) = win4;
+        const float s_wx = p.scale_w * p.scale_x;
+        float v = p.bias ? static_cast<float>(bias_q) * p.scale_b : 0.0f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v = __builtin_fmaf(s_wx * static_cast<float>(ws[i]), static_cast<float>(xs[i]), v);
+        const ConvQuantRegs kq;
+        const int8_t q = static_cast<int8_t>(conv_quant(v, p.scale_out, 1.0f / p.scale_out, p.silu_activation,
+                                                        conv_needs_exact_route(p.scale_out), kq));
+        if (store && p.out) p.out[b * p.out_batch_stride + c * p.out_c_stride] = q;
+        return q;
+    }
     const bool w_word = width == 4 && p.weight_width_stride == 1 && (reinterpret_cast<uintptr_t>(w) & 3u) == 0;
     const bool s_word = slen == 4 && p.conv_state_l_stride == 1 && (reinterpret_cast<uintptr_t>(st) & 3u) == 0;
     if (w_word) {

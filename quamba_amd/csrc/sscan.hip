@@ -46,6 +46,19 @@ __device__ __forceinline__ float softplus20(float x) {
 //   u = fl(1 + e) = 1 + e + r with r = (u - 1) - e exact, so log1p(e) = ln(u - r) = ln u - r / u + ..., and with
 //   u in [1, 2] taking r for r / u is wrong by less than 2^-24 of the result.
 // Above the threshold the second term is below half an ulp of x, so x comes back exactly, as the reference returns it.
+// float(int8 code in byte n of w) in one instruction (the sub-dword operand select converts the byte in place; the
+// compiler, left to itself, shifts and sign-extends the byte out first)
+__device__ __forceinline__ float code_byte_to_float(uint32_t w, int n) {
+    float r;
+    switch (n) {
+        case 0: asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_0" : "=v"(r) : "v"(w)); break;
+        case 1: asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_1" : "=v"(r) : "v"(w)); break;
+        case 2: asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_2" : "=v"(r) : "v"(w)); break;
+        default: asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_3" : "=v"(r) : "v"(w)); break;
+    }
+    return r;
+}
+
 __device__ __forceinline__ float softplus20_flat(float x) {
     const float e = fast_exp2(__builtin_fabsf(x) * -kLog2e);
     const float u = 1.0f + e;
@@ -821,20 +834,25 @@ int launch_fwd_mixed(const QaSScanParams& p, hipStream_t stream, int vec_in, int
 // CONV: the row's input code is not read from p.x but produced here by the causal conv's single-step update on
 // channel d of batch entry b (quant_causal_conv1d_update_kernel.cuh:34-75: shift the conv state, dot product with
 // the taps, bias, SiLU, requantise - the arithmetic of conv_update_kernel, same bits), for one lane per row.
-template <int LPR, bool VEC, bool FP32, bool CONV>
+// FAST: the shape of the Mamba1 decode step is known at compile time (one head, one B/C group, sixteen states whose
+// A_log codes are one aligned 16-byte row, per-tensor scales, no fp16 bias, four taps), so the lane's work is one
+// run of loads, arithmetic and stores without loops or branches on the parameter block.
+template <int LPR, bool VEC, bool FP32, bool CONV, bool FAST = false>
 __device__ __forceinline__ void ssm_update_body(const QaSsmUpdateParams& p, const QaConvParams* cp) {
     static_assert(!CONV || LPR == 1, "the conv step needs one lane per row");
+    static_assert(!FAST || (CONV && VEC), "the fixed shape is the fused decode step's");
+    const int dstate = FAST ? 16 : p.dstate;
     // grid: x over the channels of one head, y = head, z = batch (no integer division on the way in)
     const int gid = blockIdx.x * 256 + threadIdx.x;
     const int sub = gid % LPR;
     const bool row_ok = gid / LPR < p.dim;
     const int d = row_ok ? gid / LPR : p.dim - 1;
-    const int hd = blockIdx.y;
+    const int hd = FAST ? 0 : blockIdx.y;
     const int64_t b = blockIdx.z;
-    const int heads_per_group = p.nheads / p.ngroups;
-    const int g = hd / heads_per_group;
+    const int heads_per_group = FAST ? 1 : p.nheads / p.ngroups;
+    const int g = FAST ? 0 : hd / heads_per_group;
 
-    const bool grouped = p.nhead_groups > 0;
+    const bool grouped = !FAST && p.nhead_groups > 0;
     int sidx = 0;                       // grouped: index of this row's (g, head group, dim group)
     if (grouped) {
         int hg = 0, dg = 0;
@@ -847,9 +865,9 @@ __device__ __forceinline__ void ssm_update_body(const QaSsmUpdateParams& p, cons
         sidx = (g * p.nhead_groups + hg) * p.ndim_groups + dg;
     }
     const float* standin = p.x_scale;   // always readable, four bytes
-    const float* state_scale_row = (grouped && !FP32) ? p.state_scale + static_cast<int64_t>(sidx) * p.dstate : nullptr;
+    const float* state_scale_row = (grouped && !FP32) ? p.state_scale + static_cast<int64_t>(sidx) * dstate : nullptr;
     const bool bias_i8 = p.dt_bias && !p.dt_bias_is_fp16;
-    const bool bias_f16 = p.dt_bias && p.dt_bias_is_fp16;
+    const bool bias_f16 = !FAST && p.dt_bias && p.dt_bias_is_fp16;
     const int64_t bias_i = hd * p.dt_bias_head_stride + d * p.dt_bias_dim_stride;
     const int8_t* x_a = p.x + b * p.x_batch_stride + hd * p.x_head_stride + d * p.x_dim_stride;
     const int8_t* dt_a = p.dt + b * p.dt_batch_stride + hd * p.dt_head_stride + d * p.dt_dim_stride;
@@ -868,15 +886,6 @@ __device__ __forceinline__ void ssm_update_body(const QaSsmUpdateParams& p, cons
     const float D_scale = *(p.D ? p.D_scale : standin);
     const float z_scale = *(p.z ? p.z_scale : standin);
     const float bias_scale = *(bias_i8 ? p.dt_bias_scale : standin);
-    float xq;
-    if constexpr (CONV) {
-        xq = static_cast<float>(conv_step_row(*cp, static_cast<int>(b), d, row_ok));
-    } else {
-        xq = static_cast<float>(*x_a);
-    }
-    const float dtq = static_cast<float>(*dt_a);
-    const float zq = static_cast<float>(*z_a), Dq = static_cast<float>(*D_a);
-    const float b8 = static_cast<float>(*b8_a), b16 = __half2float(*b16_a);
     const float requant_k = grouped ? 1e6f : 1e2f;
 
     const int64_t st_base = b * p.state_batch_stride + hd * p.state_head_stride + d * p.state_dim_stride;
@@ -888,26 +897,48 @@ __device__ __forceinline__ void ssm_update_body(const QaSsmUpdateParams& p, cons
     constexpr int kPieces = 4;
     float hv[kPieces][4], sc[kPieces][4];
     __attribute__((aligned(16))) int8_t a8[kPieces][4];
+    uint32_t a_word[kPieces];               // FAST: the row of A_log as four words
+    // STAGED (FAST with an fp32 state whose rows lie back to back, whole waves of rows): a lane that reads its own
+    // 64-byte row touches one sixteen-byte piece of 64 different rows per load, and the memory system moves such
+    // a wave at about half the rate of one that reads 1 KB in a run.  So the wave moves its 64 rows (4 KB, one run
+    // in memory) with four loads of 1 KB and turns them by way of LDS: piece q of row r sits in slot
+    // 4 r + (q ^ (r / 4 % 4)), which keeps both the run-order and the row-order accesses off each other's banks.
+    constexpr bool STAGED = FAST && FP32;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    float staged[kPieces][4];
+    float4* wave_state = nullptr;
+    const float4* wave_state_in = nullptr;  // a wave past the last row reads the batch entry's first rows, and stores nothing
+    if constexpr (STAGED) {
+        float4* entry = reinterpret_cast<float4*>(static_cast<float*>(p.state) + b * p.state_batch_stride);
+        wave_state = entry + static_cast<int64_t>(gid - lane) * 4;
+        wave_state_in = row_ok ? wave_state : entry;
+    }
     __attribute__((aligned(4))) int8_t b8v[kPieces][4], c8[kPieces][4], s8[kPieces][4];
     // one lane per row with sixteen states in a row of A_log: the lane's sixteen codes come as one 16-byte piece
-    const bool a_row16 = VEC && LPR == 1 && p.dstate == 16 && p.A_dstate_stride == 1 && (reinterpret_cast<uintptr_t>(Ap) & 15u) == 0;
+    const bool a_row16 = FAST || (VEC && LPR == 1 && dstate == 16 && p.A_dstate_stride == 1 && (reinterpret_cast<uintptr_t>(Ap) & 15u) == 0);
 #pragma unroll
     for (int k = 0; k < kPieces; ++k) {
         const int n0 = (sub + k * LPR) * 4;
-        if (n0 >= p.dstate) continue;
+        if (n0 >= dstate) continue;
         if constexpr (VEC) {
             // dstate is a multiple of four here, so the piece is whole.  A_log alone may be a broadcast view
             // (one value per head, stride 0 along the states, as Mamba2 passes it): it is read through its
             // stride, the state and B, C with one load per piece
             if (a_row16) {
-                if (k == 0) *reinterpret_cast<uint4*>(&a8[0][0]) = *reinterpret_cast<const uint4*>(Ap);
+                if (k == 0) {
+                    const uint4 row = *reinterpret_cast<const uint4*>(Ap);
+                    if constexpr (FAST) { a_word[0] = row.x; a_word[1] = row.y; a_word[2] = row.z; a_word[3] = row.w; }
+                    else *reinterpret_cast<uint4*>(&a8[0][0]) = row;
+                }
             } else if (p.A_dstate_stride == 1 && (reinterpret_cast<uintptr_t>(Ap + n0) & 3u) == 0) {
                 *reinterpret_cast<int32_t*>(a8[k]) = *reinterpret_cast<const int32_t*>(Ap + n0);
             } else {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) a8[k][e] = Ap[(n0 + e) * p.A_dstate_stride];
             }
-            if constexpr (LPR == 1) {
+            if constexpr (FAST) {
+                // B and C come as floats through LDS (below)
+            } else if constexpr (LPR == 1) {
                 // every lane of the wave reads the same B and C words (one batch entry per workgroup): scalar loads
                 typedef const __attribute__((address_space(4))) int32_t* const_words;
                 *reinterpret_cast<int32_t*>(b8v[k]) = reinterpret_cast<const_words>(reinterpret_cast<uintptr_t>(Bp))[n0 / 4];
@@ -916,7 +947,11 @@ __device__ __forceinline__ void ssm_update_body(const QaSsmUpdateParams& p, cons
                 *reinterpret_cast<int32_t*>(b8v[k]) = *reinterpret_cast<const int32_t*>(Bp + n0);
                 *reinterpret_cast<int32_t*>(c8[k]) = *reinterpret_cast<const int32_t*>(Cp + n0);
             }
-            if constexpr (FP32) {
+            if constexpr (STAGED) {
+                // piece k of the wave's 4 KB of state, in memory order: lane l brings 16 bytes at (64 k + l) * 16
+                const float4 v = wave_state_in[k * 64 + lane];
+                staged[k][0] = v.x; staged[k][1] = v.y; staged[k][2] = v.z; staged[k][3] = v.w;
+            } else if constexpr (FP32) {
                 const float4 v = *reinterpret_cast<const float4*>(static_cast<const float*>(p.state) + st_base + n0);
                 hv[k][0] = v.x; hv[k][1] = v.y; hv[k][2] = v.z; hv[k][3] = v.w;
             } else {
@@ -927,7 +962,7 @@ __device__ __forceinline__ void ssm_update_body(const QaSsmUpdateParams& p, cons
         } else {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const int n = min(n0 + e, p.dstate - 1);
+                const int n = min(n0 + e, dstate - 1);
                 const int64_t si = st_base + n * p.state_dstate_stride;
                 sc[k][e] = state_scale_row ? state_scale_row[n] : s_state;
                 if constexpr (FP32) hv[k][e] = static_cast<const float*>(p.state)[si];
@@ -938,6 +973,55 @@ __device__ __forceinline__ void ssm_update_body(const QaSsmUpdateParams& p, cons
             }
         }
     }
+    // FAST: B_scale * B[n] and C_scale * C[n] are the same in every lane of the workgroup (one batch entry), and
+    // converting and scaling them in every lane is an eighth of the lane's arithmetic.  Lanes 0-31 of each wave form
+    // one value each (same expression, same bits) and the wave reads all 32 back from LDS as broadcasts.
+    int8_t bc_code = 0;
+    if constexpr (FAST) bc_code = ((lane & 16) ? Cp : Bp)[lane & 15];      // every lane loads: no branch, no wait here
+    // The row's other operands come after the state's pieces are on their way: with CONV the conv step's own loads,
+    // arithmetic and stores then run under the state's round trip instead of before it.
+    const float dtq = static_cast<float>(*dt_a);
+    const float zq = static_cast<float>(*z_a), Dq = static_cast<float>(*D_a);
+    const float b8 = static_cast<float>(*b8_a), b16 = __half2float(*b16_a);
+    float xq;
+    if constexpr (CONV) {
+        xq = static_cast<float>(conv_step_row<FAST>(*cp, static_cast<int>(b), d, row_ok));
+    } else {
+        xq = static_cast<float>(*x_a);
+    }
+    float bvf[kPieces][4], cvf[kPieces][4];
+    if constexpr (FAST) {
+        // a wave writes and reads only its own part of LDS, and a wave's LDS operations complete in order: the
+        // fences keep the compiler from reordering them, no barrier is needed
+        __shared__ __attribute__((aligned(16))) float bc_f32[4][32];
+        if (lane < 32) bc_f32[wv][lane] = (lane < 16 ? B_scale : C_scale) * static_cast<float>(bc_code);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int k = 0; k < kPieces; ++k) {
+            const float4 bq = *reinterpret_cast<const float4*>(&bc_f32[wv][4 * k]);
+            const float4 cq = *reinterpret_cast<const float4*>(&bc_f32[wv][16 + 4 * k]);
+            bvf[k][0] = bq.x; bvf[k][1] = bq.y; bvf[k][2] = bq.z; bvf[k][3] = bq.w;
+            cvf[k][0] = cq.x; cvf[k][1] = cq.y; cvf[k][2] = cq.z; cvf[k][3] = cq.w;
+        }
+    }
+    __shared__ __attribute__((aligned(16))) float4 turn[STAGED ? 4 : 1][STAGED ? 256 : 1];
+    if constexpr (STAGED) {
+#pragma unroll
+        for (int k = 0; k < kPieces; ++k) {
+            const int r = k * 16 + lane / 4, q = lane % 4;
+            turn[wv][4 * r + (q ^ (r / 4 % 4))] = make_float4(staged[k][0], staged[k][1], staged[k][2], staged[k][3]);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int k = 0; k < kPieces; ++k) {
+            const float4 v = turn[wv][4 * lane + (k ^ (lane / 4 % 4))];
+            hv[k][0] = v.x; hv[k][1] = v.y; hv[k][2] = v.z; hv[k][3] = v.w;
+        }
+    }
     const float xv = x_scale * xq;
     float dt = dt_scale * dtq;
     dt += bias_i8 ? bias_scale * b8 : (bias_f16 ? b16 : 0.0f);
@@ -946,19 +1030,22 @@ __device__ __forceinline__ void ssm_update_body(const QaSsmUpdateParams& p, cons
 #pragma unroll
     for (int k = 0; k < kPieces; ++k) {
         const int n0 = (sub + k * LPR) * 4;
-        if (n0 >= p.dstate) continue;
+        if (n0 >= dstate) continue;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             if constexpr (!FP32) hv[k][e] = sc[k][e] * static_cast<float>(s8[k][e]);
-            const float A = -__expf(A_scale * static_cast<float>(a8[k][e]));
+            const float a_code = FAST ? code_byte_to_float(a_word[k], e) : static_cast<float>(a8[k][e]);
+            const float A = -__expf(A_scale * a_code);
             const float dA = __expf(A * dt);
-            const float Bv = B_scale * static_cast<float>(b8v[k][e]);
-            const float Cv = C_scale * static_cast<float>(c8[k][e]);
+            const float Bv = FAST ? bvf[k][e] : B_scale * static_cast<float>(b8v[k][e]);
+            const float Cv = FAST ? cvf[k][e] : C_scale * static_cast<float>(c8[k][e]);
             hv[k][e] = hv[k][e] * dA + (Bv * dt) * xv;
-            if (VEC || n0 + e < p.dstate) acc += hv[k][e] * Cv;
+            if (VEC || n0 + e < dstate) acc += hv[k][e] * Cv;
         }
         if (!row_ok) continue;
-        if constexpr (VEC) {
+        if constexpr (STAGED) {
+            turn[wv][4 * lane + (k ^ (lane / 4 % 4))] = make_float4(hv[k][0], hv[k][1], hv[k][2], hv[k][3]);
+        } else if constexpr (VEC) {
             if constexpr (FP32) {
                 *reinterpret_cast<float4*>(static_cast<float*>(p.state) + st_base + n0) =
                     make_float4(hv[k][0], hv[k][1], hv[k][2], hv[k][3]);
@@ -971,10 +1058,22 @@ __device__ __forceinline__ void ssm_update_body(const QaSsmUpdateParams& p, cons
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int n = n0 + e;
-                if (n >= p.dstate) break;
+                if (n >= dstate) break;
                 const int64_t si = st_base + n * p.state_dstate_stride;
                 if constexpr (FP32) static_cast<float*>(p.state)[si] = hv[k][e];
                 else static_cast<int8_t*>(p.state)[si] = sat8_rne((hv[k][e] * requant_k) / (sc[k][e] * requant_k));
+            }
+        }
+    }
+    if constexpr (STAGED) {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        if (row_ok) {
+#pragma unroll
+            for (int k = 0; k < kPieces; ++k) {
+                const int r = k * 16 + lane / 4, q = lane % 4;
+                wave_state[k * 64 + lane] = turn[wv][4 * r + (q ^ (r / 4 % 4))];
             }
         }
     }
@@ -997,9 +1096,9 @@ __global__ __launch_bounds__(256) void ssm_update_kernel(QaSsmUpdateParams p) {
 }
 
 // conv step + state update of one token in one launch (d_state <= 16, one head)
-template <bool VEC, bool FP32>
+template <bool VEC, bool FP32, bool FAST>
 __global__ __launch_bounds__(256) void decode_step_kernel(QaSsmUpdateParams p, QaConvParams cp) {
-    ssm_update_body<1, VEC, FP32, true>(p, &cp);
+    ssm_update_body<1, VEC, FP32, true, FAST>(p, &cp);
 }
 
 template <int LPR>
@@ -1020,8 +1119,17 @@ int launch_update(const QaSsmUpdateParams& p, hipStream_t stream, const QaConvPa
     if constexpr (LPR == 1) {
         if (conv) {
             auto fused = [&](auto kernel) { hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, p, *conv); };
-            if (p.state_is_fp32) vec ? fused(decode_step_kernel<true, true>) : fused(decode_step_kernel<false, true>);
-            else vec ? fused(decode_step_kernel<true, false>) : fused(decode_step_kernel<false, false>);
+            // the fixed shape of the Mamba1 decode step (see FAST in ssm_update_body)
+            const bool fast = vec && p.dstate == 16 && p.nheads == 1 && p.ngroups == 1 && p.nhead_groups == 0 &&
+                              p.A_dstate_stride == 1 && p.A_dim_stride % 16 == 0 && aligned16(p.A_log) &&
+                              (!p.state_is_fp32 || (p.state_dim_stride == 16 && p.dim % 64 == 0)) &&
+                              !(p.dt_bias && p.dt_bias_is_fp16) && conv->width == 4 && conv->weight_width_stride == 1 &&
+                              aligned4(conv->weight) && conv->weight_c_stride % 4 == 0 && conv->conv_state_len == 4 &&
+                              conv->conv_state_l_stride == 1 && aligned4(conv->conv_state) &&
+                              conv->conv_state_batch_stride % 4 == 0 && conv->conv_state_c_stride % 4 == 0;
+            if (fast) p.state_is_fp32 ? fused(decode_step_kernel<true, true, true>) : fused(decode_step_kernel<true, false, true>);
+            else if (p.state_is_fp32) vec ? fused(decode_step_kernel<true, true, false>) : fused(decode_step_kernel<false, true, false>);
+            else vec ? fused(decode_step_kernel<true, false, false>) : fused(decode_step_kernel<false, false, false>);
             return check_launch();
         }
     }

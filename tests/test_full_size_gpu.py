@@ -119,7 +119,7 @@ def test_decode_1000_steps(dev, one_launch):
     conv = QCausalConv1D(D1, D1, 4, groups=D1, device=dev)
     conv.weight, conv.bias = _ri(dev, D1, 4, seed=40), _ri(dev, D1, seed=41)
     conv.weight_scale, conv.bias_scale, conv.input_scale, conv.output_scale = 0.004, 0.004, 0.04, 0.03
-    conv_state = _ri(dev, Bd, D1, 3, seed=42)
+    conv_state = _ri(dev, Bd, D1, 4, seed=42)         # (B, D, d_conv), as the reference's mixer allocates it
     g = torch.Generator(device=dev).manual_seed(43)
     ssm_state = torch.randn(Bd, D1, N1, device=dev, generator=g) * 0.1
     A, Dq, db = _ri(dev, D1, N1, seed=44), _ri(dev, D1, seed=45), _ri(dev, D1, seed=46)

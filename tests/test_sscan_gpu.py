@@ -180,7 +180,8 @@ def test_update_matches_oracle_over_several_steps(dev, B, D, N, fp32_state):
 
 
 @pytest.mark.parametrize("B,D,N,width,state_len,fp32_state", [(3, 100, 16, 4, 3, True), (64, 1536, 16, 4, 4, False),
-                                                              (2, 257, 8, 3, 2, True), (5, 64, 16, 2, 2, False)])
+                                                              (7, 300, 16, 4, 4, True), (2, 257, 8, 3, 2, True),
+                                                              (5, 64, 16, 2, 2, False)])
 def test_decode_step_in_one_launch_equals_conv_update_then_state_update(dev, B, D, N, width, state_len, fp32_state):
     """qa_mamba1_decode_step against the two calls it stands for, bit for bit (conv output, conv state, y, state),
     over several steps; the two-call path is the one the oracle tests pin."""
