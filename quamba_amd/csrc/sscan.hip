@@ -840,7 +840,7 @@ int launch_fwd_mixed(const QaSScanParams& p, hipStream_t stream, int vec_in, int
 template <int LPR, bool VEC, bool FP32, bool CONV, bool FAST = false>
 __device__ __forceinline__ void ssm_update_body(const QaSsmUpdateParams& p, const QaConvParams* cp) {
     static_assert(!CONV || LPR == 1, "the conv step needs one lane per row");
-    static_assert(!FAST || (CONV && VEC), "the fixed shape is the fused decode step's");
+    static_assert(!FAST || (LPR == 1 && VEC), "the fixed shape has one lane per row and whole pieces");
     const int dstate = FAST ? 16 : p.dstate;
     // grid: x over the channels of one head, y = head, z = batch (no integer division on the way in)
     const int gid = blockIdx.x * 256 + threadIdx.x;
@@ -1090,9 +1090,9 @@ __device__ __forceinline__ void ssm_update_body(const QaSsmUpdateParams& p, cons
     }
 }
 
-template <int LPR, bool VEC, bool FP32>
+template <int LPR, bool VEC, bool FP32, bool FAST = false>
 __global__ __launch_bounds__(256) void ssm_update_kernel(QaSsmUpdateParams p) {
-    ssm_update_body<LPR, VEC, FP32, false>(p, nullptr);
+    ssm_update_body<LPR, VEC, FP32, false, FAST>(p, nullptr);
 }
 
 // conv step + state update of one token in one launch (d_state <= 16, one head)
@@ -1117,13 +1117,19 @@ int launch_update(const QaSsmUpdateParams& p, hipStream_t stream, const QaConvPa
                      aligned4(p.B) && mult(p.B_batch_stride, 4) && mult(p.B_group_stride, 4) &&
                      aligned4(p.C) && mult(p.C_batch_stride, 4) && mult(p.C_group_stride, 4);
     if constexpr (LPR == 1) {
+        // the fixed shape of the Mamba1 decode step (see FAST in ssm_update_body)
+        const bool fast_update = vec && p.dstate == 16 && p.nheads == 1 && p.ngroups == 1 && p.nhead_groups == 0 &&
+                                 p.A_dstate_stride == 1 && p.A_dim_stride % 16 == 0 && aligned16(p.A_log) &&
+                                 (!p.state_is_fp32 || (p.state_dim_stride == 16 && p.dim % 64 == 0)) &&
+                                 !(p.dt_bias && p.dt_bias_is_fp16);
+        if (!conv && fast_update) {
+            auto go = [&](auto kernel) { hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, p); };
+            p.state_is_fp32 ? go(ssm_update_kernel<1, true, true, true>) : go(ssm_update_kernel<1, true, false, true>);
+            return check_launch();
+        }
         if (conv) {
             auto fused = [&](auto kernel) { hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, p, *conv); };
-            // the fixed shape of the Mamba1 decode step (see FAST in ssm_update_body)
-            const bool fast = vec && p.dstate == 16 && p.nheads == 1 && p.ngroups == 1 && p.nhead_groups == 0 &&
-                              p.A_dstate_stride == 1 && p.A_dim_stride % 16 == 0 && aligned16(p.A_log) &&
-                              (!p.state_is_fp32 || (p.state_dim_stride == 16 && p.dim % 64 == 0)) &&
-                              !(p.dt_bias && p.dt_bias_is_fp16) && conv->width == 4 && conv->weight_width_stride == 1 &&
+            const bool fast = fast_update && conv->width == 4 && conv->weight_width_stride == 1 &&
                               aligned4(conv->weight) && conv->weight_c_stride % 4 == 0 && conv->conv_state_len == 4 &&
                               conv->conv_state_l_stride == 1 && aligned4(conv->conv_state) &&
                               conv->conv_state_batch_stride % 4 == 0 && conv->conv_state_c_stride % 4 == 0;

@@ -145,7 +145,7 @@ def test_fwd_unaligned_rows(dev):
 
 
 @pytest.mark.parametrize("B,D,N,fp32_state", [(1, 1536, 16, False), (64, 5120, 16, True), (3, 100, 16, False),
-                                              (2, 64, 128, True), (2, 30, 8, False),
+                                              (2, 192, 16, True), (3, 100, 16, True), (2, 64, 128, True), (2, 30, 8, False),
                                               (4, 5120, 128, False), (4, 8192, 128, True)])
 def test_update_matches_oracle_over_several_steps(dev, B, D, N, fp32_state):
     steps = 5
@@ -180,7 +180,8 @@ def test_update_matches_oracle_over_several_steps(dev, B, D, N, fp32_state):
 
 
 @pytest.mark.parametrize("B,D,N,width,state_len,fp32_state", [(3, 100, 16, 4, 3, True), (64, 1536, 16, 4, 4, False),
-                                                              (7, 300, 16, 4, 4, True), (2, 257, 8, 3, 2, True),
+                                                              (7, 300, 16, 4, 4, True), (3, 320, 16, 4, 4, True),
+                                                              (2, 257, 8, 3, 2, True),
                                                               (5, 64, 16, 2, 2, False)])
 def test_decode_step_in_one_launch_equals_conv_update_then_state_update(dev, B, D, N, width, state_len, fp32_state):
     """qa_mamba1_decode_step against the two calls it stands for, bit for bit (conv output, conv state, y, state),
