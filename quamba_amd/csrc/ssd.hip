@@ -3,12 +3,12 @@
 // Stages and arithmetic follow the reference's Triton pipeline (quamba/triton/quant_ssd_combined.py
 // :61-77, grouped :146-162); see each kernel for the file it restates.  fp16 operands rounded where the
 // reference rounds them, fp32 accumulation, as there; the one pure int8 contraction (C B^T) runs on the
-// int8 matrix cores and stays in fp32.
+// int8 matrix cores inside the chunk scan and stays in fp32 registers.
 //   cumsum      dt = clamp(softplus(s_dt q_dt + dt_bias)), dA_cs = within-chunk cumsum(dt * A)
-//   cb          CB[m,k] = (s_C s_B) * sum_n q_C[m,n] q_B[k,n]                       (int8 MFMA, lower tiles, fp32 out)
 //   state       S_c[p,n] = sum_k f16(x^[k,p]) f16(B^[k,n] exp(dA_last - dA_k) dt_k)   (fp16 MFMA)
 //               P_0 = 0, P_{c+1} = exp(dA_last,c) P_c + S_c in registers; P_c stored in fp16; final state fp32 / int8
-//   chunk_scan  y[m,p] = exp(dA_m) sum_n f16(C^[m,n]) f16(P_c[p,n]) + sum_{k<=m} f16(CB[m,k] e^{dA_m-dA_k} dt_k) f16(x^[k,p])
+//   chunk_scan  CB[m,k] = (s_C s_B) * sum_n q_C[m,n] q_B[k,n]                       (int8 MFMA, at and below the diagonal)
+//               y[m,p] = exp(dA_m) sum_n f16(C^[m,n]) f16(P_c[p,n]) + sum_{k<=m} f16(CB[m,k] e^{dA_m-dA_k} dt_k) f16(x^[k,p])
 //               + D x^[m,p], optional z gate, fp16 out                               (fp16 MFMA)
 // Both fp16 contractions over the time index need x (and B) with time as the fastest-moving index,
 // while memory has channels fastest; the tiles are transposed once on the way into LDS and then read as
@@ -35,21 +35,19 @@ __device__ __forceinline__ float fexp(float x) { return __builtin_amdgcn_exp2f(x
 __device__ __forceinline__ int8_t byte_of(uint32_t w, int j) { return static_cast<int8_t>((w >> (8 * j)) & 0xffu); }
 
 struct Ws {            // workspace sections (byte offsets), see qa_ssd_workspace_bytes
-    int64_t dt, dA, cb, prev, c16, total;
+    int64_t dt, dA, prev, total;
 };
 
 __host__ __device__ inline int64_t align256(int64_t v) { return (v + 255) & ~int64_t(255); }
 
 __host__ __device__ inline Ws ws_layout(const QaSsdParams& p) {
     const int64_t nc = (p.seqlen + p.chunk_size - 1) / p.chunk_size;
-    const int64_t B = p.batch, H = p.nheads, Q = p.chunk_size, G = p.ngroups, N = p.dstate;
+    const int64_t B = p.batch, H = p.nheads, Q = p.chunk_size, N = p.dstate;
     Ws w;
     int64_t off = 0;
     w.dt = off; off = align256(off + B * H * nc * Q * 4);
     w.dA = off; off = align256(off + B * H * nc * Q * 4);
-    w.cb = off; off = align256(off + B * nc * G * Q * Q * 4);
     w.prev = off; off = align256(off + B * nc * H * kP * N * 2);
-    w.c16 = off; off = align256(off + B * static_cast<int64_t>(p.seqlen) * G * N * 2);
     w.total = off;
     return w;
 }
@@ -124,95 +122,6 @@ __global__ __launch_bounds__(256) void ssd_cumsum_kernel(QaSsdParams p, float* d
         dt_row[e] = dtv[e];
         dA_row[e] = before + run[e];
     }
-}
-
-// ---------------------------------------------------------------------------------------------
-// Stage 4 (quamba/triton/quant_bmm_chunk.py:60-66): one wave per 64x64 tile of CB, lower tiles only.
-// Both operands are rows of dstate int8 values, i.e. already MFMA operands.  The diagonal tiles also
-// write their C rows dequantised to fp16 (f16(s_C * q_C)): every head of the group multiplies those
-// rows with its entering state in the chunk scan, which then reads them ready-made.
-// ---------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(64) void ssd_cb_kernel(QaSsdParams p, float* cb_out, __half* c16_out, int nc) {
-    const int Q = p.chunk_size, N = p.dstate, G = p.ngroups;
-    const int nt = Q / 64;
-    // blockIdx.x enumerates lower-triangular tile pairs (mt >= kt)
-    int mt = 0, rem = blockIdx.x;
-    while (rem > mt) { rem -= mt + 1; ++mt; }
-    const int kt = rem;
-    if (mt >= nt) return;
-    const int bcg = blockIdx.y;
-    const int g = bcg % G, c = (bcg / G) % nc, b = bcg / (G * nc);
-    const int lane = threadIdx.x, frow = lane & 31, fhalf = lane >> 5;
-    const int t0 = c * Q;
-    const int lim = min(Q, p.seqlen - t0);
-    const float sC = p.nhead_groups > 0 ? p.C_scale[g] : p.C_scale[0];
-    const float scale = sC * (p.nhead_groups > 0 ? p.B_scale[g] : p.B_scale[0]);
-
-    v16i acc[2][2];
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
-    // every operand piece of the tile pair is requested before the first product: one memory round trip
-    constexpr int KSMAX = 4;                                  // dstate 128
-    const int nks = N / 32;
-    v4i fc[KSMAX][2], fb[KSMAX][2];
-#pragma unroll
-    for (int ks = 0; ks < KSMAX; ++ks) {
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int m = mt * 64 + i * 32 + frow, k = kt * 64 + i * 32 + frow;
-            const bool on = ks < nks;
-            fc[ks][i] = (on && m < lim) ? *reinterpret_cast<const v4i*>(p.C + ((static_cast<int64_t>(b) * p.seqlen + t0 + m) * G + g) * N + ks * 32 + fhalf * 16)
-                                        : v4i{0, 0, 0, 0};
-            fb[ks][i] = (on && k < lim) ? *reinterpret_cast<const v4i*>(p.B + ((static_cast<int64_t>(b) * p.seqlen + t0 + k) * G + g) * N + ks * 32 + fhalf * 16)
-                                        : v4i{0, 0, 0, 0};
-        }
-    }
-#pragma unroll
-    for (int ks = 0; ks < KSMAX; ++ks) {
-        if (ks >= nks) break;
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int m = mt * 64 + i * 32 + frow;
-            if (mt == kt && m < lim) {
-                v8h lo, hi;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    lo[e] = static_cast<_Float16>(sC * static_cast<float>(byte_of(static_cast<uint32_t>(fc[ks][i][e >> 2]), e & 3)));
-                    hi[e] = static_cast<_Float16>(sC * static_cast<float>(byte_of(static_cast<uint32_t>(fc[ks][i][2 + (e >> 2)]), e & 3)));
-                }
-                __half* dst = c16_out + ((static_cast<int64_t>(b) * p.seqlen + t0 + m) * G + g) * N + ks * 32 + fhalf * 16;
-                *reinterpret_cast<v8h*>(dst) = lo;
-                *reinterpret_cast<v8h*>(dst + 8) = hi;
-            }
-        }
-        // B rows as the first operand: the products come out with a lane per row m of C B^T and four
-        // consecutive columns k per register group, which leave as 8-byte pieces
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-            for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[ks][j], fc[ks][i], acc[i][j], 0, 0, 0);
-    }
-    // acc[i][j]: lane holds row m = mt*64 + i*32 + (lane & 31), register r column k = kt*64 + j*32 + 8*(r/4) + 4*(lane/32) + r%4
-    float* tile = cb_out + ((static_cast<int64_t>(b) * nc + c) * G + g) * Q * Q;
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int m = mt * 64 + i * 32 + frow;
-                const int k = kt * 64 + j * 32 + 8 * q + 4 * fhalf;
-                float4 o;
-                o.x = scale * static_cast<float>(acc[i][j][4 * q]);
-                o.y = scale * static_cast<float>(acc[i][j][4 * q + 1]);
-                o.z = scale * static_cast<float>(acc[i][j][4 * q + 2]);
-                o.w = scale * static_cast<float>(acc[i][j][4 * q + 3]);
-                *reinterpret_cast<float4*>(tile + static_cast<int64_t>(m) * Q + k) = o;
-            }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -465,55 +374,75 @@ __global__ __launch_bounds__(256, 3) void ssd_state_kernel(QaSsdParams p, const 
 }
 
 // ---------------------------------------------------------------------------------------------
-// Stage 5 (quamba/triton/quant_chunk_scan.py:96-171): a workgroup of four waves per (batch, chunk, head).  A wave
-// owns whole 16-row m-tiles with all 64 columns p, long and short causal ranges mixed so that the waves carry equal
-// work (with sixteen tiles: 15 - w, 8 + w, 7 - w, w), longest first.  Its A operands are built in registers: rows
-// of f16(C^) come ready-made from the preparation kernel; the weights of term 2 are C B^T (fp32, from the
-// preparation kernel, fetched four 32-step pieces ahead) times the decay.  For the pieces below the diagonal the
-// decay factors into exp(dA_m - R) (one exp per lane and piece) and exp(R - dA_k) dt_k (a table per workgroup)
-// with R = dA at the last step of the piece, so that both exponents are <= 0; on the piece that holds the
-// diagonal it is computed per element, in the reference's order.  The B operands (entering state, transposed
-// x) are read from LDS, both with rows in slot order.  Everything the prologue and the first tile read from
-// global memory is requested before the first LDS write; a tile's operands are requested before the epilogue
-// of the tile before.
+// Stages 4 and 5 (quamba/triton/quant_bmm_chunk.py:60-66, quant_chunk_scan.py:96-171): a workgroup of eight waves
+// per (batch, chunk, head).  A wave owns whole 16-row m-tiles with all 64 channels, a long and a short causal range
+// each (with sixteen tiles: 15 - w and w), the long one first.
+// C B^T never exists in memory: the chunk's B codes sit in LDS, a lane holds 32 codes of its row of C, and
+// v_mfma_i32_16x16x64_i8 forms (C B^T)^T in 16 x 16 blocks - exact integers, times s_C s_B in fp32, the value
+// the reference's bmm kernel stores.  A block comes out with a lane per row m and four consecutive steps k, which
+// is how the next product wants its first operand: two blocks (steps 4 q .. 4 q + 3 and 16 + 4 q .. 16 + 4 q + 3
+// of a 32-step piece, q = lane / 16) are the eight values of a lane, and the x operand is read from LDS in the
+// same order (the order of the summation index is free as long as both operands agree).  The same codes of C,
+// dequantised to fp16, are the first operand of term 1; a lane's codes are states 64 i + 16 q .. + 15, and the
+// entering state is read in that order.  Below the diagonal the decay factors into exp(dA_m - R) (one exp per
+// lane and piece) and exp(R - dA_k) dt_k (a table per workgroup) with R = dA at the last step of the piece, so
+// that both exponents are <= 0; on the piece that holds the diagonal it is computed per element, in the
+// reference's order.  After the prologue a wave reads global memory only for the bytes of the skip term and gate.
+// With 128 states and chunks of 256 steps two workgroups fit a CU's LDS only if the entering state and the upper
+// half of the B codes share their 16 KB: term 1 of both tiles runs first, then the B codes (held in registers
+// since the prologue) take the state's place.
 // ---------------------------------------------------------------------------------------------
 template <int N, int Q>
 struct ScanSmem {
+    static constexpr bool ALIAS = N == 128 && Q == 256;
     static constexpr int XP = Q + 8;        // halves per row of the transposed x tile
     static constexpr int NCH = N / 8;       // 16-byte pieces per row of the entering state
     static constexpr int SWZ = (NCH < 16 ? NCH : 16) - 1;
+    static constexpr int BSWZ = (N / 16 < 8 ? N / 16 : 8) - 1;
+    static constexpr int BROWS = ALIAS ? Q / 2 : Q;
     __attribute__((aligned(16))) _Float16 xt[kP][XP];
     // rows without padding: piece c of row r sits at position c ^ (r & SWZ), so that the sixteen rows of an operand
     // read fall into different banks
     __attribute__((aligned(16))) _Float16 prev[kP][N];
+    __attribute__((aligned(16))) int8_t bq[BROWS][N];   // B codes; 16-byte piece c of row k at position c ^ (k & BSWZ)
     __attribute__((aligned(16))) float dt[Q];
     __attribute__((aligned(16))) float dA[Q];
     __attribute__((aligned(16))) float gk[Q];   // exp(dA[end of the 32-step piece] - dA_k) dt_k
     __attribute__((aligned(16))) float xs[kP];  // x scale per channel
     __attribute__((aligned(16))) float Dv[kP];  // skip weight per channel
+    static_assert(!ALIAS || sizeof(_Float16) * kP * N == static_cast<size_t>(Q / 2) * N, "the upper B rows take exactly the state's place");
+    // row k of the B codes
+    __device__ __forceinline__ int8_t* brow(int k) {
+        if (ALIAS && k >= BROWS) return reinterpret_cast<int8_t*>(&prev[0][0]) + (k - BROWS) * N;
+        return bq[k];
+    }
 };
 
 constexpr int scan_waves_of(int Q) { return Q / 16 < 8 ? Q / 16 : 8; }
 
 template <int N, int Q>
 __global__ __launch_bounds__(64 * scan_waves_of(Q), 4) void ssd_chunk_scan_kernel(QaSsdParams p, const float* dt_ws, const float* dA_ws,
-                                                                                const float* cb_ws, const __half* prev, const __half* c16, int nc) {
+                                                                                const __half* prev, int nc) {
     using S = ScanSmem<N, Q>;
     extern __shared__ __attribute__((aligned(16))) unsigned char ssd_smem_raw[];
     S& sm = *reinterpret_cast<S*>(ssd_smem_raw);
     constexpr int kWaves = scan_waves_of(Q);
     constexpr int kThreads = 64 * kWaves;
     constexpr int NMT = Q / 16;                                   // 16-row m-tiles of a chunk
-    constexpr int TILES = NMT / kWaves;                           // per wave: 4 (Q 256), 2 (Q 128), 1 (Q 64)
-    constexpr int WIN = 2;                                        // pieces of C B^T in flight: a rolling window
-    static_assert(Q <= kThreads, "a thread stages at most one share of the x tile");
+    constexpr int TILES = NMT / kWaves;                           // per wave: 2 (Q 256), 1 (Q 128, 64)
     constexpr int PPC = kP * N / 8;                               // 16-byte pieces of the entering state
     constexpr int PB = PPC / kThreads;
+    constexpr int BPC = Q * N / 16;                               // 16-byte pieces of the B codes
+    constexpr int BB = BPC / kThreads;
+    constexpr int BB_NOW = S::ALIAS ? BB / 2 : BB;                // pieces a thread writes in the prologue
+    static_assert(Q <= kThreads, "a thread stages at most one share of the x tile");
+    static_assert(PPC % kThreads == 0 && BPC % kThreads == 0 && (!S::ALIAS || BB % 2 == 0), "whole shares per thread");
+    static_assert(TILES <= 2, "a long and a short tile per wave");
 
     const int tid = threadIdx.x, lane = tid & 63, l16 = lane & 15, lq = lane >> 4;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);    // the same in every lane: kept in a scalar register
     const int G = p.ngroups, H = p.nheads, L = p.seqlen;
-    // the heads of one (batch, chunk, ssd group) read the same C B^T and C rows: they go to one XCD
+    // the heads of one (batch, chunk, ssd group) read the same B and C codes: they go to one XCD
     int unit, hig, part;
     unit_head_part(blockIdx.x, p.batch * nc * G, H / G, 1, unit, hig, part);
     const int h = (unit % G) * (H / G) + hig;
@@ -521,12 +450,17 @@ __global__ __launch_bounds__(64 * scan_waves_of(Q), 4) void ssd_chunk_scan_kerne
     const int b = unit / (G * nc);
     int g, hg;
     group_of(p, h, g, hg);
+    const bool grouped = p.nhead_groups > 0;
+    const float sC = grouped ? p.C_scale[g] : p.C_scale[0];
+    const float cb_scale = sC * (grouped ? p.B_scale[g] : p.B_scale[0]);
     const int t0 = c * Q;
     const int lim = min(Q, L - t0);
     const uint32_t xrow = static_cast<uint32_t>(H) * kP;          // bytes between steps of x
-    const float* cb = cb_ws + ((static_cast<int64_t>(b) * nc + c) * G + g) * Q * Q;
+    const uint32_t crow = static_cast<uint32_t>(G) * N;           // bytes between steps of B and C
     const int8_t* xbase = p.x + (static_cast<int64_t>(b) * L + t0) * xrow + static_cast<int64_t>(h) * kP;
     const int8_t* zbase = p.z + (static_cast<int64_t>(b) * L + t0) * xrow + static_cast<int64_t>(h) * kP;       // only read if p.z
+    const int8_t* Bbase = p.B + (static_cast<int64_t>(b) * L + t0) * crow + static_cast<int64_t>(g) * N;
+    const int8_t* Cbase = p.C + (static_cast<int64_t>(b) * L + t0) * crow + static_cast<int64_t>(g) * N;
     const float D_scale = p.D ? *p.D_scale : 0.0f;
     const float z_scale = p.z ? *p.z_scale : 0.0f;
     __half* out = static_cast<__half*>(p.out) + (static_cast<int64_t>(b) * L + t0) * xrow + static_cast<int64_t>(h) * kP;
@@ -534,28 +468,10 @@ __global__ __launch_bounds__(64 * scan_waves_of(Q), 4) void ssd_chunk_scan_kerne
     // tile s of this wave
     auto tile_of = [&](int s) { return (s & 1) == 0 ? NMT - 1 - 8 * (s / 2) - wave : 8 * ((TILES - 1 - s) / 2) + wave; };
 
-    // ---- what an m-tile reads from global memory for terms 1 and 2: its rows of f16(C^) and the first pieces of its
-    // rows of C B^T
-    v8h cfr[N / 32];
-    float4 cbr[WIN][2];
-    auto tile_load = [&](int mt) {
-        const int m_row = mt * 16 + l16;
-        const int nks = (mt + 2) / 2;
-        const float* cbp = cb + static_cast<uint32_t>(m_row * Q + 8 * lq);
-        const __half* cp = c16 + ((static_cast<int64_t>(b) * L + t0 + min(m_row, lim - 1)) * G + g) * N + 8 * lq;
-        if (c > 0) {
-#pragma unroll
-            for (int ks = 0; ks < N / 32; ++ks) cfr[ks] = *reinterpret_cast<const v8h*>(cp + 32 * ks);
-        }
-#pragma unroll
-        for (int ks = 0; ks < WIN; ++ks) {
-            if (ks < nks) {
-                cbr[ks][0] = *reinterpret_cast<const float4*>(cbp + 32 * ks);
-                cbr[ks][1] = *reinterpret_cast<const float4*>(cbp + 32 * ks + 4);
-            }
-        }
-    };
-
+    // codes of C of this lane's rows: states 64 i + 16 q .. + 15 (rows past the end of the sequence read the last
+    // row; nothing of theirs is stored)
+    v4i cq[TILES][N / 64];
+    v4i r_b[BB];
     {
         // Prologue: every global read is issued before the first LDS write, so that the workgroup waits for memory
         // once.
@@ -567,11 +483,16 @@ __global__ __launch_bounds__(64 * scan_waves_of(Q), 4) void ssd_chunk_scan_kerne
             r_end = dA_ws[row + (tid | 31)];
         }
         // (the first chunk has no entering state: its slot of the workspace is read all the same and never used)
-        static_assert(PPC % kThreads == 0, "every thread copies the same number of pieces of the entering state");
         v4i r_prev[PB];
         const __half* pst = prev + ((static_cast<int64_t>(b) * nc + c) * H + h) * kP * N;
 #pragma unroll
         for (int i = 0; i < PB; ++i) r_prev[i] = *reinterpret_cast<const v4i*>(pst + (tid + i * kThreads) * 8);
+        // the chunk's B codes
+#pragma unroll
+        for (int i = 0; i < BB; ++i) {
+            const int piece = tid + i * kThreads, k = piece / (N / 16), col = piece % (N / 16);
+            r_b[i] = *reinterpret_cast<const v4i*>(Bbase + static_cast<uint32_t>(min(k, lim - 1)) * crow + 16 * col);
+        }
         // this thread's share of the x tile: steps 4 kb .. 4 kb + 3, channels 16 pb .. 16 pb + 15
         const int pb = tid % 4, kb = tid / 4;
         const bool mine = Q == kThreads || tid < Q;
@@ -591,7 +512,12 @@ __global__ __launch_bounds__(64 * scan_waves_of(Q), 4) void ssd_chunk_scan_kerne
                 }
             }
         }
-        tile_load(tile_of(0));
+#pragma unroll
+        for (int s = 0; s < TILES; ++s) {
+            const int8_t* cp = Cbase + static_cast<uint32_t>(min(tile_of(s) * 16 + l16, lim - 1)) * crow + 16 * lq;
+#pragma unroll
+            for (int i = 0; i < N / 64; ++i) cq[s][i] = *reinterpret_cast<const v4i*>(cp + 64 * i);
+        }
         if (tid < kP) {
             sm.xs[tid] = x_scale_of(p, g, hg, tid);
             sm.Dv[tid] = !p.D ? 0.0f : D_scale * static_cast<float>(p.D_has_hdim ? p.D[h * kP + tid] : p.D[h]);
@@ -608,9 +534,56 @@ __global__ __launch_bounds__(64 * scan_waves_of(Q), 4) void ssd_chunk_scan_kerne
             const int piece = tid + i * kThreads, pr = piece / (N / 8), col = (piece % (N / 8)) * 8;
             *reinterpret_cast<v4i*>(&sm.prev[pr][col ^ ((pr & S::SWZ) * 8)]) = r_prev[i];
         }
+#pragma unroll
+        for (int i = 0; i < BB_NOW; ++i) {
+            const int piece = tid + i * kThreads, k = piece / (N / 16), col = piece % (N / 16);
+            *reinterpret_cast<v4i*>(sm.brow(k) + (col ^ (k & S::BSWZ)) * 16) = r_b[i];
+        }
         if (mine) stage_x_share<S::XP>(sm.xt, xr, sm.xs, pb, kb);
     }
     __syncthreads();
+
+    // term 1 of every tile of the wave: C^ (rows m) x entering state (rows p), zero for the first chunk
+    v4f acc[TILES][4];
+#pragma unroll
+    for (int s = 0; s < TILES; ++s) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[s][j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+        if (c > 0) {
+            const int m0 = tile_of(s) * 16;
+#pragma unroll
+            for (int ks = 0; ks < N / 32; ++ks) {
+                const uint32_t w0 = static_cast<uint32_t>(cq[s][ks / 2][2 * (ks % 2)]), w1 = static_cast<uint32_t>(cq[s][ks / 2][2 * (ks % 2) + 1]);
+                v8h cf;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    cf[e] = static_cast<_Float16>(sC * static_cast<float>(byte_of(w0, e)));
+                    cf[4 + e] = static_cast<_Float16>(sC * static_cast<float>(byte_of(w1, e)));
+                }
+                const int n0 = 64 * (ks / 2) + 16 * lq + 8 * (ks % 2);     // the states of those eight codes
+                v8h fs[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) fs[j] = *reinterpret_cast<const v8h*>(&sm.prev[j * 16 + l16][n0 ^ ((l16 & S::SWZ) * 8)]);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[s][j] = mfma16(cf, fs[j], acc[s][j]);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float em = fexp(sm.dA[m0 + 4 * lq + r]);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[s][j][r] *= em;
+            }
+        }
+    }
+    if constexpr (S::ALIAS) {
+        __syncthreads();                                           // everyone is done with the entering state
+#pragma unroll
+        for (int i = BB_NOW; i < BB; ++i) {
+            const int piece = tid + i * kThreads, k = piece / (N / 16), col = piece % (N / 16);
+            *reinterpret_cast<v4i*>(sm.brow(k) + (col ^ (k & S::BSWZ)) * 16) = r_b[i];
+        }
+        __syncthreads();
+    }
 
 #pragma unroll
     for (int s = 0; s < TILES; ++s) {
@@ -620,8 +593,7 @@ __global__ __launch_bounds__(64 * scan_waves_of(Q), 4) void ssd_chunk_scan_kerne
         const int mt = tile_of(s);
         const int m0 = mt * 16;
         const int nks = (mt + 2) / 2;                               // 32-step pieces that reach row m0 + 15; the last holds the diagonal
-        const int m_row = m0 + l16;                                 // row of this lane's A operands
-        const float* cbp = cb + static_cast<uint32_t>(m_row * Q + 8 * lq);
+        const int m_row = m0 + l16;                                 // row of this lane's first operands
         const float dA_m = sm.dA[m_row];
         // skip-term operands of this lane's four output rows
         // (requested now, used in the epilogue: nothing there waits for memory)
@@ -632,71 +604,67 @@ __global__ __launch_bounds__(64 * scan_waves_of(Q), 4) void ssd_chunk_scan_kerne
             xq[r] = *reinterpret_cast<const uint32_t*>(xbase + at);
             if (p.z) zq[r] = *reinterpret_cast<const uint32_t*>(zbase + at);
         }
-        v4f acc[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
-        // term 1: C^ (rows m) x entering state (rows p), zero for the first chunk
-        if (c > 0) {
-#pragma unroll
-            for (int ks = 0; ks < N / 32; ++ks) {
-                v8h fs[4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) fs[j] = *reinterpret_cast<const v8h*>(&sm.prev[j * 16 + l16][(32 * ks + 8 * lq) ^ ((l16 & S::SWZ) * 8)]);
-#pragma unroll
-                for (int j = 0; j < 4; ++j) acc[j] = mfma16(cfr[ks], fs[j], acc[j]);
-            }
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const float em = fexp(sm.dA[m0 + 4 * lq + r]);
-#pragma unroll
-                for (int j = 0; j < 4; ++j) acc[j][r] *= em;
-            }
-        }
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
             if (ks < max_nks && ks < nks) {
-                const int k0 = 32 * ks + 8 * lq;
+                // steps of this lane's eight values: ka .. ka + 3 and ka + 16 .. ka + 19
+                const int ka = 32 * ks + 4 * lq;
+                // (C B^T)^T for the two 16-step blocks of the piece
+                v4i cbi[2];
+#pragma unroll
+                for (int blk = 0; blk < 2; ++blk) {
+                    const int k = 32 * ks + 16 * blk + l16;
+                    const int8_t* brow = sm.brow(32 * ks + 16 * blk) + l16 * N;
+                    cbi[blk] = v4i{0, 0, 0, 0};
+#pragma unroll
+                    for (int i = 0; i < N / 64; ++i) {
+                        const v4i bo = *reinterpret_cast<const v4i*>(brow + (((4 * i + lq) ^ (k & S::BSWZ)) * 16));
+                        cbi[blk] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bo, cq[s][i], cbi[blk], 0, 0, 0);
+                    }
+                }
                 v8h fx[4];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) fx[j] = *reinterpret_cast<const v8h*>(&sm.xt[j * 16 + l16][k0]);
-                const float4 c0 = cbr[ks % WIN][0], c1 = cbr[ks % WIN][1];
-                const float cv[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
-                if (ks + WIN < max_nks && ks + WIN < nks) {
-                    // the slot is free: the piece WIN ahead takes it
-                    cbr[ks % WIN][0] = *reinterpret_cast<const float4*>(cbp + 32 * (ks + WIN));
-                    cbr[ks % WIN][1] = *reinterpret_cast<const float4*>(cbp + 32 * (ks + WIN) + 4);
+                for (int j = 0; j < 4; ++j) {
+                    const v4h x0 = *reinterpret_cast<const v4h*>(&sm.xt[j * 16 + l16][ka]);
+                    const v4h x1 = *reinterpret_cast<const v4h*>(&sm.xt[j * 16 + l16][ka + 16]);
+                    fx[j] = v8h{x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
                 }
+                float cv[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) cv[e] = cb_scale * static_cast<float>(cbi[e / 4][e % 4]);
                 float wv[8];
                 if (ks + 1 < nks) {
-                    const float4 g0 = *reinterpret_cast<const float4*>(&sm.gk[k0]), g1 = *reinterpret_cast<const float4*>(&sm.gk[k0 + 4]);
+                    const float4 g0 = *reinterpret_cast<const float4*>(&sm.gk[ka]), g1 = *reinterpret_cast<const float4*>(&sm.gk[ka + 16]);
                     const float gk[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
                     const float e_m = fexp(dA_m - sm.dA[32 * ks + 31]);
 #pragma unroll
                     for (int e = 0; e < 8; ++e) wv[e] = cv[e] * (e_m * gk[e]);
                 } else {
                     // the piece with the diagonal: steps after row m do not count
-                    const float4 a0 = *reinterpret_cast<const float4*>(&sm.dA[k0]), a1 = *reinterpret_cast<const float4*>(&sm.dA[k0 + 4]);
-                    const float4 d0 = *reinterpret_cast<const float4*>(&sm.dt[k0]), d1 = *reinterpret_cast<const float4*>(&sm.dt[k0 + 4]);
+                    const float4 a0 = *reinterpret_cast<const float4*>(&sm.dA[ka]), a1 = *reinterpret_cast<const float4*>(&sm.dA[ka + 16]);
+                    const float4 d0 = *reinterpret_cast<const float4*>(&sm.dt[ka]), d1 = *reinterpret_cast<const float4*>(&sm.dt[ka + 16]);
                     const float ak[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
                     const float dk[8] = {d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w};
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) wv[e] = ((k0 + e <= m_row ? cv[e] : 0.0f) * fexp(fminf(dA_m - ak[e], 0.0f))) * dk[e];
+                    for (int e = 0; e < 8; ++e) {
+                        const int k = ka + 16 * (e / 4) + e % 4;
+                        wv[e] = ((k <= m_row ? cv[e] : 0.0f) * fexp(fminf(dA_m - ak[e], 0.0f))) * dk[e];
+                    }
                 }
                 v8h fl;
 #pragma unroll
                 for (int e = 0; e < 8; ++e) fl[e] = static_cast<_Float16>(wv[e]);
 #pragma unroll
-                for (int j = 0; j < 4; ++j) acc[j] = mfma16(fl, fx[j], acc[j]);
+                for (int j = 0; j < 4; ++j) acc[s][j] = mfma16(fl, fx[j], acc[s][j]);
             }
         }
-        if (s + 1 < TILES) tile_load(tile_of(s + 1));              // in flight during the epilogue
-        // Epilogue: acc[j][r] is row m0 + 4 (lane / 16) + r, channel 4 (lane % 16) + j
+        // Epilogue: acc[s][j][r] is row m0 + 4 (lane / 16) + r, channel 4 (lane % 16) + j
         const float4 xs4 = *reinterpret_cast<const float4*>(&sm.xs[4 * l16]), Dv4 = *reinterpret_cast<const float4*>(&sm.Dv[4 * l16]);
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int m = m0 + 4 * lq + r;
             if (m < lim) {
-                float y[4] = {acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
+                float y[4] = {acc[s][0][r], acc[s][1][r], acc[s][2][r], acc[s][3][r]};
                 if (p.D) {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) y[j] += __builtin_fmaf(ubyte_of(xq[r] ^ kBias, j), lane_of(xs4, j), -128.0f * lane_of(xs4, j)) * lane_of(Dv4, j);
@@ -754,8 +722,6 @@ extern "C" int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream_) {
     uint8_t* base = static_cast<uint8_t*>(p->workspace);
     float* dt_ws = reinterpret_cast<float*>(base + ws.dt);
     float* dA_ws = reinterpret_cast<float*>(base + ws.dA);
-    float* cb_ws = reinterpret_cast<float*>(base + ws.cb);
-    __half* c16_ws = reinterpret_cast<__half*>(base + ws.c16);
     const int nc = (p->seqlen + p->chunk_size - 1) / p->chunk_size;
     const int64_t bch = static_cast<int64_t>(p->batch) * nc * p->nheads;
     if (bch > 0x7fffffffLL || static_cast<int64_t>(p->batch) * nc * p->ngroups > 65535) return QA_ERR_SHAPE;
@@ -763,11 +729,8 @@ extern "C" int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream_) {
 
     hipLaunchKernelGGL(ssd_cumsum_kernel, dim3(static_cast<unsigned>((bch + 3) / 4)), dim3(256), 0, stream, *p, dt_ws,
                        dA_ws, nc);
-    const int nt = p->chunk_size / 64;
-    hipLaunchKernelGGL(ssd_cb_kernel, dim3(nt * (nt + 1) / 2, p->batch * nc * p->ngroups), dim3(64), 0, stream, *p, cb_ws, c16_ws, nc);
     __half* prev_ws = reinterpret_cast<__half*>(base + ws.prev);
     const dim3 hgrid(static_cast<unsigned>(p->batch * p->nheads * (p->dstate / 64)));
-    const dim3 sgrid(static_cast<unsigned>(bch));
     int status = QA_OK;
     // more LDS than a kernel gets by default: raise the limit (idempotent)
     auto lds_ok = [&](const void* kernel, size_t lds) {
@@ -779,7 +742,7 @@ extern "C" int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream_) {
     auto launch = [&](auto state_kernel, size_t state_lds, auto scan_kernel, size_t scan_lds, int scan_threads) {
         if (!lds_ok(reinterpret_cast<const void*>(state_kernel), state_lds) || !lds_ok(reinterpret_cast<const void*>(scan_kernel), scan_lds)) return;
         hipLaunchKernelGGL(state_kernel, hgrid, dim3(256), state_lds, stream, *p, dt_ws, dA_ws, prev_ws, nc);
-        hipLaunchKernelGGL(scan_kernel, sgrid, dim3(scan_threads), scan_lds, stream, *p, dt_ws, dA_ws, cb_ws, prev_ws, c16_ws, nc);
+        hipLaunchKernelGGL(scan_kernel, dim3(static_cast<unsigned>(bch)), dim3(scan_threads), scan_lds, stream, *p, dt_ws, dA_ws, prev_ws, nc);
     };
 #define QA_SSD_LAUNCH(N_, Q_) launch(ssd_state_kernel<N_, Q_>, sizeof(StateSmem<Q_>), ssd_chunk_scan_kernel<N_, Q_>, \
                                      sizeof(ScanSmem<N_, Q_>), 64 * scan_waves_of(Q_))

@@ -65,7 +65,8 @@ def test_forward_matches_oracle(dev, B, L, H, N, G, Q):
 
 
 def test_preparation_stages_match_the_oracle(dev):
-    # what the two preparation kernels leave in the workspace: step sizes, their running sums and C B^T
+    # what the preparation kernel leaves in the workspace: step sizes and their running sums (C B^T is formed inside
+    # the chunk scan and never stored; the outputs below depend on every element of it at or below the diagonal)
     B, L, H, N, G, Q = 2, 200, 4, 128, 2, 64
     d = synth.mamba2_ssd_inputs(B, L, H, 64, N, G, seed=77)
     ref = _oracle(d, Q, stages=True)
@@ -73,14 +74,12 @@ def test_preparation_stages_match_the_oracle(dev):
     nc = (L + Q - 1) // Q
     a256 = lambda v: (v + 255) & ~255
     off, parts = 0, {}
-    for name, shape in [("dt", (B, H, nc, Q)), ("dA_cumsum", (B, H, nc, Q)), ("CB", (B, nc, G, Q, Q))]:
+    for name, shape in [("dt", (B, H, nc, Q)), ("dA_cumsum", (B, H, nc, Q))]:
         n = int(np.prod(shape)) * 4
         parts[name] = ws[off:off + n].view(torch.float32).view(shape).cpu().numpy()
         off = a256(off + n)
     np.testing.assert_allclose(parts["dt"], ref["dt"], rtol=1e-5, atol=1e-9)
     np.testing.assert_allclose(parts["dA_cumsum"], ref["dA_cumsum"], rtol=1e-5, atol=1e-8)
-    # exact integer sums times the scale product; Q == 64: one tile, all of it written
-    np.testing.assert_allclose(parts["CB"], ref["CB"], rtol=1e-6, atol=1e-6 * np.abs(ref["CB"]).max())
     _check_y(y, ref["y"])
 
 
