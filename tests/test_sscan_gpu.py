@@ -207,6 +207,29 @@ def test_decode_step_in_one_launch_equals_conv_update_then_state_update(dev, B, 
     assert int(xc_a.abs().max()) > 10 and float(y_a.float().abs().max()) > 0.1
 
 
+@pytest.mark.parametrize("fp32_state", [True, False])
+def test_decode_step_without_optional_operands(dev, fp32_state):
+    """The reference layer's layout (the kernel compiled for that shape) with no skip weight, no gate, no dt bias, no
+    conv bias and no SiLU: one launch against the two calls, bit for bit."""
+    B, D, N = 5, 256, 16
+    g = torch.Generator(device=dev).manual_seed(99)
+    ri = lambda *shape: torch.randint(-128, 128, shape, dtype=torch.int8, device=dev, generator=g)
+    w, A = ri(D, 4), ri(D, N)
+    conv_a = ri(B, D, 4)
+    st_a = (torch.randn(B, D, N, device=dev, generator=g) * 0.1) if fp32_state else ri(B, D, N)
+    conv_b, st_b = conv_a.clone(), st_a.clone()
+    s_dt, s_A, s_B, s_C, s_state = (_s(v, dev) for v in (0.02, 0.02, 0.03, 0.03, 0.004))
+    for _ in range(3):
+        x, dt, Bv, Cv = ri(B, D), ri(B, D), ri(B, N), ri(B, N)
+        xc_a = ops.causal_conv1d_update(x, conv_a, 0.04, w, 0.004, 0.03, 0.004, None, False)
+        y_a = ops.sscan_update(st_a, xc_a, _s(0.03, dev), dt, s_dt, A, s_A, s_state, Bv, s_B, Cv, s_C)
+        xc_b, y_b = ops.mamba1_decode_step(x, conv_b, 0.04, w, 0.004, 0.03, 0.004, None, False, st_b, dt, s_dt, A, s_A, s_state,
+                                           Bv, s_B, Cv, s_C)
+        assert torch.equal(xc_a, xc_b) and torch.equal(conv_a, conv_b)
+        assert torch.equal(y_a, y_b) and torch.equal(st_a, st_b)
+    assert float(y_a.float().abs().max()) > 0.01
+
+
 def test_decode_step_in_one_launch_refuses_what_it_does_not_cover(dev):
     ri = lambda *shape: torch.randint(-128, 128, shape, dtype=torch.int8, device=dev)
     B, D, N = 2, 64, 32                                      # more than sixteen states
