@@ -31,6 +31,19 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
 
+// float(int8 code in byte n of w) in one instruction (the sub-dword operand select converts the byte in place; the
+// compiler, left to itself, shifts and sign-extends the byte out first)
+__device__ __forceinline__ float code_byte_to_float(uint32_t w, int n) {
+    float r;
+    switch (n) {
+        case 0: asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_0" : "=v"(r) : "v"(w)); break;
+        case 1: asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_1" : "=v"(r) : "v"(w)); break;
+        case 2: asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_2" : "=v"(r) : "v"(w)); break;
+        default: asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_3" : "=v"(r) : "v"(w)); break;
+    }
+    return r;
+}
+
 // softplus with the reference's threshold; log1p evaluated so that small exp(x) keeps full
 // relative accuracy (series below 2^-6, log2 above).
 __device__ __forceinline__ float softplus20(float x) {
@@ -46,19 +59,6 @@ __device__ __forceinline__ float softplus20(float x) {
 //   u = fl(1 + e) = 1 + e + r with r = (u - 1) - e exact, so log1p(e) = ln(u - r) = ln u - r / u + ..., and with
 //   u in [1, 2] taking r for r / u is wrong by less than 2^-24 of the result.
 // Above the threshold the second term is below half an ulp of x, so x comes back exactly, as the reference returns it.
-// float(int8 code in byte n of w) in one instruction (the sub-dword operand select converts the byte in place; the
-// compiler, left to itself, shifts and sign-extends the byte out first)
-__device__ __forceinline__ float code_byte_to_float(uint32_t w, int n) {
-    float r;
-    switch (n) {
-        case 0: asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_0" : "=v"(r) : "v"(w)); break;
-        case 1: asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_1" : "=v"(r) : "v"(w)); break;
-        case 2: asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_2" : "=v"(r) : "v"(w)); break;
-        default: asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_3" : "=v"(r) : "v"(w)); break;
-    }
-    return r;
-}
-
 __device__ __forceinline__ float softplus20_flat(float x) {
     const float e = fast_exp2(__builtin_fabsf(x) * -kLog2e);
     const float u = 1.0f + e;
