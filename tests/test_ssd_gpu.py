@@ -49,6 +49,8 @@ def _check_y(y_gpu, y_ref):
 # batch, seqlen, nheads, dstate, ngroups, chunk
 SHAPES = [(1, 64, 2, 128, 1, 64), (2, 33, 4, 128, 1, 64), (1, 89, 4, 64, 2, 64), (2, 300, 8, 64, 2, 128),
           (1, 512, 8, 128, 1, 256), (1, 1024, 4, 128, 1, 256), (1, 130, 4, 128, 4, 128),
+          # chunks of 256 with a ragged last chunk: 128 states (entering state and upper B rows share LDS) and 64
+          (1, 600, 4, 128, 2, 256), (2, 700, 4, 64, 1, 256),
           # fewer states than the kernels are built for (the 16-state row of test_ssd_combined.py:25, and 32, 96)
           (1, 33, 24, 16, 1, 128), (2, 200, 4, 32, 2, 64), (1, 150, 4, 96, 1, 128)]
 
