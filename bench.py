@@ -186,32 +186,22 @@ def _ri(dev):
 
 
 def _wl_decode(dev):
-    """Mamba1-2.8b decode step: conv update + state update, batch 64, fp32 state, sixteen steps in one HIP graph."""
+    """Mamba1-2.8b decode step at batch 64, fp32 state, sixteen steps in one HIP graph.  The row's headline figures
+    (`us`, `tokens_per_s`, `frac`) are the two launches the layer executes - conv update, then state update, with
+    x_proj / dt_proj between them in the full layer - on the benchmark configuration's int8 conv state [64, 5120, 3].
+    `us_one_launch` is the fused kernel (dt, B and C given beforehand), `state_width_4` the same pair of figures on the
+    (B, D, d_conv) buffer the reference's mixer allocates."""
     ri = _ri(dev)
     sc = lambda v: torch.tensor([v], dtype=torch.float32, device=dev)
     B, D, N = 64, 5120, 16
     conv = QCausalConv1D(D, D, 4, groups=D, device=dev)
     conv.weight, conv.bias = ri(D, 4), ri(D)
     conv.weight_scale, conv.bias_scale, conv.input_scale, conv.output_scale = 0.004, 0.004, 0.04, 0.03
-    conv_state, ssm_state = ri(B, D, 4), torch.randn(B, D, N, device=dev) * 0.1   # the reference's (B, D, d_conv) conv state
+    ssm_state = torch.randn(B, D, N, device=dev) * 0.1
     ring = [(ri(B, D), ri(B, D), ri(B, N), ri(B, N), ri(B, D)) for _ in range(16)]
     A, Dq, db = ri(D, N), ri(D), ri(D)
     it = [0]
     s_x, s_dt, s_A, s_B, s_C, s_D, s_z, s_db = (sc(v) for v in (0.03, 0.02, 0.02, 0.03, 0.03, 0.008, 0.04, 0.01))
-
-    def decode():
-        x, dt, Bv, Cv, z = ring[it[0] % 16]
-        it[0] += 1
-        xc = conv.update(x, conv_state)
-        ops.sscan_update(ssm_state, xc, s_x, dt, s_dt, A, s_A, None, Bv, s_B, Cv, s_C, Dq, s_D, z, s_z, db, s_db, True)
-
-    def decode_one_launch():
-        x, dt, Bv, Cv, z = ring[it[0] % 16]
-        it[0] += 1
-        ops.mamba1_decode_step(x, conv_state, conv.input_scale, conv.weight, conv.weight_scale, conv.output_scale,
-                               conv.bias_scale, conv.bias, True, ssm_state, dt, s_dt, A, s_A, None, Bv, s_B, Cv, s_C, Dq, s_D,
-                               z, s_z, db, s_db, True, x_scale=s_x)
-    ms_eager = _time_fn(decode, 208, 16)
 
     # the same 16 steps captured into one HIP graph (how decode loops are run in practice)
     def graphed(step):
@@ -226,12 +216,34 @@ def _wl_decode(dev):
             for _ in range(16):
                 step()
         return _time_fn(graph.replay, 64, 4) / 16
-    ms_two = graphed(decode)
-    ms = graphed(decode_one_launch)
-    nbytes = 3 * B * D + 2 * B * D * 4 + 2 * B * D * N * 4 + 2 * B * D + D * N
-    return dict(workload="Mamba1-2.8b decode step (conv update + state update in one launch), batch 64, fp32 state, HIP graph of 16 steps",
-                name="decode_step", us=ms * 1e3, us_two_launches=ms_two * 1e3, us_eager_python=ms_eager * 1e3, tokens_per_s=B / ms * 1e3, bound="hbm",
-                bytes=nbytes, achieved_GBs=nbytes / ms / 1e6, frac=nbytes / ms / 1e6 / HBM_PEAK_GBS)
+
+    def measure(width):
+        conv_state = ri(B, D, width)
+
+        def decode():
+            x, dt, Bv, Cv, z = ring[it[0] % 16]
+            it[0] += 1
+            xc = conv.update(x, conv_state)
+            ops.sscan_update(ssm_state, xc, s_x, dt, s_dt, A, s_A, None, Bv, s_B, Cv, s_C, Dq, s_D, z, s_z, db, s_db, True)
+
+        def decode_one_launch():
+            x, dt, Bv, Cv, z = ring[it[0] % 16]
+            it[0] += 1
+            ops.mamba1_decode_step(x, conv_state, conv.input_scale, conv.weight, conv.weight_scale, conv.output_scale,
+                                   conv.bias_scale, conv.bias, True, ssm_state, dt, s_dt, A, s_A, None, Bv, s_B, Cv, s_C, Dq,
+                                   s_D, z, s_z, db, s_db, True, x_scale=s_x)
+        ms_eager = _time_fn(decode, 208, 16)
+        return graphed(decode), graphed(decode_one_launch), ms_eager
+
+    ms_two, ms_one, ms_eager = measure(3)
+    ms_two4, ms_one4, _ = measure(4)
+    nbytes = 3 * B * D + 2 * B * D * 3 + 2 * B * D * N * 4 + 2 * B * D + D * N
+    return dict(workload="Mamba1-2.8b decode step (conv update, then state update: two launches), batch 64, fp32 state, "
+                         "int8 conv state [64,5120,3], HIP graph of 16 steps",
+                name="decode_step", us=ms_two * 1e3, us_one_launch=ms_one * 1e3, us_eager_python=ms_eager * 1e3,
+                state_width_4=dict(us=ms_two4 * 1e3, us_one_launch=ms_one4 * 1e3),
+                tokens_per_s=B / ms_two * 1e3, bound="hbm", bytes=nbytes, achieved_GBs=nbytes / ms_two / 1e6,
+                frac=nbytes / ms_two / 1e6 / HBM_PEAK_GBS)
 
 
 def _wl_ssd(dev, steps, warmup, B, L, H, N, G, Q, name, label):
@@ -480,11 +492,11 @@ def other_workloads(dev, steps, warmup):
 
 
 def _probes():
-    """ctypes handle of the bench-only probe library (quamba_amd/libqa_bench_probes.so, built by quamba_amd.build)."""
+    """ctypes handle of the bench-only probe library (bench_probes/libqa_bench_probes.so, built by bench_probes.build)."""
     import ctypes as C
-    path = os.path.join(ROOT, "quamba_amd", "libqa_bench_probes.so")
+    path = os.path.join(ROOT, "bench_probes", "libqa_bench_probes.so")
     if not os.path.exists(path):
-        sys.exit(f"{path} is missing: build it with `python -m quamba_amd.build`")
+        sys.exit(f"{path} is missing: build it with `python -m bench_probes.build`")
     h = C.CDLL(path)
     vp = C.c_void_p
     for name in ("qa_probe_mfma_i8", "qa_probe_valu"):
@@ -494,7 +506,7 @@ def _probes():
     return h
 
 
-def mfma_calibration(dev):
+def mfma_calibration(dev, kinds=(("constant_operands", 0), ("random_operands", 1)), launches=6):
     """Sustained v_mfma_i32_32x32x32_i8 rate of a register-only loop (two waves per SIMD on every CU) for
     constant and for pseudo-random operand bytes, six launches of about 5 ms each; the last one is reported.
     The clock is the ratio of the shader-clock and 100 MHz counters over the loop."""
@@ -505,8 +517,8 @@ def mfma_calibration(dev):
     ticks = torch.zeros(2, dtype=torch.int64, device=dev)
     stream = torch.cuda.current_stream().cuda_stream
     out = {}
-    for name, rnd in (("constant_operands", 0), ("random_operands", 1)):
-        for _ in range(6):
+    for name, rnd in kinds:
+        for _ in range(launches):
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
             _lib.check(lib.qa_probe_mfma_i8(sink.data_ptr(), sink.numel(), ticks.data_ptr(), wgs, iters, rnd, stream), "diag")
@@ -552,6 +564,61 @@ def valu_calibration(dev, ops_list=None, launches=4):
 # (time loop + staging of the next tile + output store, divided by the eight groups of a 32-step tile): the kind with
 # four lanes per channel and four states per lane, and the short kind with eight lanes per channel and two states.
 SCAN_MIX = {"four_lane": {"plain": 99, "transcendental": 18}, "eight_lane": {"plain": 58, "transcendental": 9}}
+
+
+def peaks_measured(dev):
+    """What this GPU sustains right now, beside the published peaks the fractions are quoted against: a plain
+    1 GiB device-to-device copy (read + write bytes per second) and the int8 matrix rate of a register-only loop with
+    pseudo-random operand bytes (the part lowers its clock under the switching activity of live operands)."""
+    src = torch.zeros(1 << 30, dtype=torch.int8, device=dev)
+    dst = torch.empty_like(src)
+    ms = _time_fn(lambda: dst.copy_(src), 5, 2)
+    del src, dst
+    torch.cuda.empty_cache()
+    m = mfma_calibration(dev, kinds=(("random_operands", 1),), launches=4)["random_operands"]
+    return {"copy_GBs": round(2.0 * (1 << 30) / ms / 1e6, 1), "copy_bytes": 1 << 30,
+            "int8_mfma_random_operands_TOPs": m["TOPs"], "int8_mfma_clock_MHz": m["clock_MHz"]}
+
+
+def gemm_phase_clocks(dev, mixer):
+    """Where the two projections spend their time and at what clock: the library built with -DQA_GEMM_CLK
+    (bench_probes/libquamba_amd_clk.so) has every workgroup record the shader clock and the constant 100 MHz clock at
+    the boundaries of its prologue (first operand tiles), main loop and epilogue.  Medians over the workgroups."""
+    import ctypes as C
+    from quamba_amd import _lib
+    path = os.path.join(ROOT, "bench_probes", "libquamba_amd_clk.so")
+    if not os.path.exists(path):
+        sys.exit(f"{path} is missing: build it with `python -m bench_probes.build`")
+    clk = C.CDLL(path)
+    clk.qa_gemm_w8a8.restype = C.c_int
+    clk.qa_gemm_w8a8.argtypes = [C.POINTER(_lib.QaGemmW8A8Params), C.c_void_p]
+    clk.qa_gemm_clk_read.restype = C.c_int
+    clk.qa_gemm_clk_read.argtypes = [C.c_void_p, C.c_int64]
+    prod = _lib.lib()
+    real = prod.qa_gemm_w8a8
+    out = {}
+    try:
+        prod.qa_gemm_w8a8 = clk.qa_gemm_w8a8                       # the modules call through this handle
+        for name, fn, m, n, tile in (("in_proj_w8a8_gemm", lambda: mixer.in_proj.to_seqlen_last(mixer.hidden),
+                                      2 * mixer.D, mixer.B * mixer.L, (320, 256)),
+                                     ("out_proj_w8a8_gemm", lambda: mixer.out_proj(mixer.y_q),
+                                      mixer.B * mixer.L, mixer.dm, (256, 320))):
+            ms = _time_fn(fn, 10, 10)
+            wgs = -(-m // tile[0]) * -(-n // tile[1])
+            buf = np.zeros((8192, 8), np.uint64)
+            if clk.qa_gemm_clk_read(buf.ctypes.data_as(C.c_void_p), buf.nbytes) != 0 or wgs > 8192:
+                continue
+            b = buf[:wgs].astype(np.int64)
+            dc, dw = np.diff(b[:, 0::2], axis=1), np.diff(b[:, 1::2], axis=1)
+            phases = {}
+            for i, ph in enumerate(("prologue", "main_loop", "epilogue")):
+                phases[ph] = {"us": round(float(np.median(dw[:, i])) / 100.0, 2),
+                              "shader_cycles": int(np.median(dc[:, i])),
+                              "clock_MHz": round(float(np.median(dc[:, i] / np.maximum(dw[:, i], 1))) * 100.0, 1)}
+            out[name] = {"us": round(ms * 1e3, 1), "workgroups": wgs, "tile": list(tile), **phases}
+    finally:
+        prod.qa_gemm_w8a8 = real
+    return out
 
 
 def scan_mix_rates(dev):
@@ -603,6 +670,22 @@ def scan_issue_bound(dev, B, D, L):
                 clock_MHz=round(rates["clock_MHz"], 1), waves=waves, instructions_per_four_steps=SCAN_MIX)
 
 
+def load_traffic(path):
+    """HBM bytes per launch from the rocprofv3 counter runs summarised in profiles/hbm_traffic_counters.md: the file
+    names the git head it was measured at and, per entry, the kernels it sums.  An entry whose kernels no longer exist
+    in the library under those names is dropped (its figure would belong to other code)."""
+    if not os.path.exists(path):
+        return {}, None
+    from quamba_amd import _lib
+    doc = json.load(open(path))
+    image = open(_lib.LIB_PATH, "rb").read()
+    out = {}
+    for name, entry in doc.get("entries", {}).items():
+        if all(sym.encode() in image for sym in entry["kernel_symbols"]):
+            out[name] = entry["bytes"]
+    return out, doc.get("head")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -624,8 +707,12 @@ def main():
                          "with random operand bytes (extra key in the JSON line)")
     ap.add_argument("--valu-calibration", action="store_true",
                     help="also measure the issue time of plain and transcendental vector instructions (extra key in the JSON line)")
+    ap.add_argument("--gemm-phase-clocks", action="store_true",
+                    help="also report, for both projections, the time and the clock of a workgroup's prologue, main loop "
+                         "and epilogue (needs bench_probes/libquamba_amd_clk.so)")
     ap.add_argument("--traffic-json", default=os.path.join(ROOT, "profiles", "traffic.json"),
-                    help="HBM bytes per launch measured with rocprofv3 --pmc (written by hand from profiles/)")
+                    help="HBM bytes per launch measured with rocprofv3 --pmc, with the git head and the kernel names they "
+                         "were measured at")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU only: this build has no multi-GPU path (run with --gpus 1)")
@@ -657,13 +744,11 @@ def main():
         else:
             kinfo.update(achieved=kinfo["ops"] / dur_ms / 1e9, peak=INT8_PEAK_TOPS, unit="TOP/s")
         kinfo["frac"] = kinfo["achieved"] / kinfo["peak"]
-    traffic = {}
-    if os.path.exists(args.traffic_json):
-        traffic = json.load(open(args.traffic_json))
+    traffic, traffic_head = load_traffic(args.traffic_json)
     dom = max(kernels, key=lambda k: k["avg_us"])
     roofline = dict(kernel=dom["name"], bound=dom["bound"], achieved=round(dom["achieved"], 2), peak=dom["peak"],
                     unit=dom["unit"], frac=round(dom["frac"], 4), traffic=traffic.get(dom["name"]),
-                    avg_us=round(dom["avg_us"], 2))
+                    traffic_head=traffic_head, avg_us=round(dom["avg_us"], 2))
     if dom["name"] == "sscan_fwd":
         # the bound that binds this kernel is vector-ALU issue, not HBM: how far the launch is from it
         ib = scan_issue_bound(dev, B, CFG["d_inner"], L)
@@ -695,6 +780,9 @@ def main():
         "roofline": roofline,
         "kernels": per_kernel,
     }
+    line["peaks_measured"] = peaks_measured(dev)
+    if args.gemm_phase_clocks:
+        line["gemm_phase_clocks"] = gemm_phase_clocks(dev, mixer)
     if args.copy_calibration:
         src = torch.zeros(1 << 30, dtype=torch.int8, device=dev)
         dst = torch.empty_like(src)

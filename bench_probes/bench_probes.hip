@@ -1,7 +1,7 @@
 // Micro-benchmark probes used by bench.py only (built into libqa_bench_probes.so, never linked into
 // libquamba_amd.so and not part of its C ABI): the rate the matrix cores and the vector ALUs sustain on this part,
 // against which the kernels' own figures are read.
-#include "../qa_common.hpp"
+#include "../quamba_amd/csrc/qa_common.hpp"
 
 namespace qa {
 void set_last_hip_error(int) {}

@@ -10,6 +10,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libquamba_amd.so")
 
 QA_OK = 0
+ABI_VERSION = 2          # what qa_abi_version() of a matching library returns
 QA_OUT_I8, QA_OUT_F16, QA_OUT_BF16 = 0, 1, 2
 QA_ROUND_RNE, QA_ROUND_HALF_AWAY = 0, 1
 QA_IN_F16, QA_IN_F32 = 0, 1
@@ -190,6 +191,9 @@ def lib():
             fn = getattr(handle, name)
             fn.restype = res
             fn.argtypes = args
+        if handle.qa_abi_version() != ABI_VERSION:
+            raise RuntimeError(f"{LIB_PATH} has ABI version {handle.qa_abi_version()}, this binding expects "
+                               f"{ABI_VERSION}: rebuild it with `python -m quamba_amd.build --force`")
         _lib = handle
     return _lib
 

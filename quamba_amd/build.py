@@ -13,9 +13,6 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 BUILD = os.path.join(HERE, "csrc", "build")
 LIB = os.path.join(HERE, "libquamba_amd.so")
-# bench.py's micro-benchmark probes: a library of their own, not part of the product
-PROBES_SRC = os.path.join(CSRC, "probes", "bench_probes.hip")
-PROBES_LIB = os.path.join(HERE, "libqa_bench_probes.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 ARCH = "gfx950"
@@ -64,11 +61,6 @@ def build(force=False, jobs=None):
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError(f"link failed:\n{r.stdout}\n{r.stderr}")
-    if force or _newer(PROBES_SRC, PROBES_LIB):
-        cmd = [HIPCC, *FLAGS, "-shared", PROBES_SRC, "-o", PROBES_LIB]
-        r = subprocess.run(cmd, capture_output=True, text=True)
-        if r.returncode != 0:
-            raise RuntimeError(f"hipcc failed for the bench probes:\n{r.stdout}\n{r.stderr}")
     return LIB
 
 

@@ -21,6 +21,6 @@ extern "C" const char* qa_status_string(int status) {
     }
 }
 
-extern "C" int qa_abi_version(void) { return 1; }
+extern "C" int qa_abi_version(void) { return 2; }
 
 extern "C" int qa_last_hip_error(void) { return qa::g_last_hip_error; }

@@ -44,16 +44,18 @@ __device__ __forceinline__ int quant8(float v, int round_mode) {
 
 // Four values -> four int8 bytes (round half to even, saturating) in one word.  Clamping to the
 // integers -128 and 127 first does not change the rounded result; adding 1.5 * 2^23 then rounds to
-// nearest-even in the addition itself and leaves the two's-complement byte in the low 8 bits.
+// nearest-even in the addition itself and leaves the two's-complement byte in the low 8 bits.  The additions of the
+// second to fourth value write that low byte straight into its place in the word (sub-dword destination select,
+// the other bytes preserved), so no byte permutes are needed.
 __device__ __forceinline__ uint32_t pack4_rne_sat8(float v0, float v1, float v2, float v3) {
-    constexpr float kMagic = 12582912.0f;
-    const uint32_t y0 = __float_as_uint(__builtin_amdgcn_fmed3f(v0, -128.0f, 127.0f) + kMagic);
-    const uint32_t y1 = __float_as_uint(__builtin_amdgcn_fmed3f(v1, -128.0f, 127.0f) + kMagic);
-    const uint32_t y2 = __float_as_uint(__builtin_amdgcn_fmed3f(v2, -128.0f, 127.0f) + kMagic);
-    const uint32_t y3 = __float_as_uint(__builtin_amdgcn_fmed3f(v3, -128.0f, 127.0f) + kMagic);
-    const uint32_t lo = __builtin_amdgcn_perm(y1, y0, 0x0c0c0400u);      // bytes: y0.0, y1.0, 0, 0
-    const uint32_t hi = __builtin_amdgcn_perm(y3, y2, 0x0c0c0400u);
-    return __builtin_amdgcn_perm(hi, lo, 0x05040100u);                   // lo.0, lo.1, hi.0, hi.1
+    const float magic = 12582912.0f;
+    const float c1 = __builtin_amdgcn_fmed3f(v1, -128.0f, 127.0f), c2 = __builtin_amdgcn_fmed3f(v2, -128.0f, 127.0f);
+    const float c3 = __builtin_amdgcn_fmed3f(v3, -128.0f, 127.0f);
+    uint32_t word = __float_as_uint(__builtin_amdgcn_fmed3f(v0, -128.0f, 127.0f) + magic);   // byte 0; bytes 1..3 replaced below
+    asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(word) : "v"(c1), "v"(magic));
+    asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(word) : "v"(c2), "v"(magic));
+    asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(word) : "v"(c3), "v"(magic));
+    return word;
 }
 
 // Two fp32 values -> two 16-bit floats of the output type (round to nearest even) in one word; bf16 rounds on the
@@ -185,37 +187,8 @@ struct TileLoader {
     }
 };
 
-// Accumulates one 128-byte k tile: sa / sw point at this wave's rows of the staged operands.
-// Fragments of step kk+1 are requested before the multiplications of step kk are issued.
-template <int TM, int TN>
-__device__ __forceinline__ void mma_tile(const uint8_t* sa, const uint8_t* sw, int frow, int fhalf,
-                                         v16i (&acc)[TN][TM]) {
-    v4i fa[2][TM], fw[2][TN];
-    auto fetch = [&](int kk, int buf) {
-#pragma unroll
-        for (int i = 0; i < TN; ++i) {
-            const int row = i * 32 + frow;
-            fw[buf][i] = *reinterpret_cast<const v4i*>(sw + row * kBK + swz(row, kk * 2 + fhalf) * 16);
-        }
-#pragma unroll
-        for (int j = 0; j < TM; ++j) {
-            const int row = j * 32 + frow;
-            fa[buf][j] = *reinterpret_cast<const v4i*>(sa + row * kBK + swz(row, kk * 2 + fhalf) * 16);
-        }
-    };
-    fetch(0, 0);
-#pragma unroll
-    for (int kk = 0; kk < kBK / 32; ++kk) {
-        if (kk + 1 < kBK / 32) fetch(kk + 1, (kk + 1) & 1);
-#pragma unroll
-        for (int i = 0; i < TN; ++i)
-#pragma unroll
-            for (int j = 0; j < TM; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fw[kk & 1][i], fa[kk & 1][j], acc[i][j], 0, 0, 0);
-    }
-}
-
-// The same accumulation with the instruction order pinned.  The fragments of step kk+1 are requested
+// Accumulates one 128-byte k tile with the instruction order pinned: sa / sw point at this wave's rows of the
+// staged operands.  The fragments of step kk+1 are requested
 // before the multiplications of step kk are issued, and `hook(slot)` runs after every second
 // multiplication (slot = 0 .. 4*TM*TN/2 - 1): the caller places its global -> LDS requests for the
 // next tile there, one at a time, so that the wave never waits on a full memory queue with
@@ -252,6 +225,57 @@ __device__ __forceinline__ void mma_tile_paced(const uint8_t* sa, const uint8_t*
                     hook(kk * (TM * TN / 2) + (i * TM + j) / 2);
                     __builtin_amdgcn_sched_barrier(0);
                 }
+            }
+    }
+}
+
+// The fragments of k step kk of this wave's rows (sa: TM row blocks of the a operand, sw: TN of the w operand).
+template <int TM, int TN>
+__device__ __forceinline__ void fetch_fragments(const uint8_t* sa, const uint8_t* sw, int kk, int frow, int fhalf,
+                                                v4i (&fa)[TM], v4i (&fw)[TN]) {
+#pragma unroll
+    for (int i = 0; i < TN; ++i) {
+        const int row = i * 32 + frow;
+        fw[i] = *reinterpret_cast<const v4i*>(sw + row * kBK + swz(row, kk * 2 + fhalf) * 16);
+    }
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+        const int row = j * 32 + frow;
+        fa[j] = *reinterpret_cast<const v4i*>(sa + row * kBK + swz(row, kk * 2 + fhalf) * 16);
+    }
+}
+
+// One k tile of a main loop whose workgroup barrier sits before the last k step instead of between tiles.  On entry
+// the fragments of k step 0 of the tile at `sa`/`sw` are in fa[0]/fw[0].  Steps 0..2 fetch the fragments of the step
+// after them; before the multiplications of step 3 the wave waits for its own global -> LDS requests, meets the
+// others at the barrier - every wave then holds all fragments of this tile, so this stage may be overwritten, and
+// the next tile's stage is complete - and fetches step 0 of the next tile from `na`/`nw`.  The matrix pipe has the
+// multiplications of step 3 queued behind the barrier, so it does not drain while the first fragments of the next
+// tile travel.  `hook(idx)` runs after every multiplication, idx counted from the barrier: 0 .. TM*TN-1 during
+// step 3 of this tile, the following 3*TM*TN during steps 0..2 of the next one; the caller places its global ->
+// LDS requests behind the multiplications it chooses (a hook that does nothing costs nothing).
+template <int TM, int TN, class Hook>
+__device__ __forceinline__ void mma_tile_rotated(const uint8_t* sa, const uint8_t* sw, const uint8_t* na, const uint8_t* nw,
+                                                 int frow, int fhalf, v4i (&fa)[2][TM], v4i (&fw)[2][TN],
+                                                 v16i (&acc)[TN][TM], Hook&& hook) {
+#pragma unroll
+    for (int kk = 0; kk < kBK / 32; ++kk) {
+        if (kk + 1 < kBK / 32) {
+            fetch_fragments<TM, TN>(sa, sw, kk + 1, frow, fhalf, fa[(kk + 1) & 1], fw[(kk + 1) & 1]);
+        } else {
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+            __syncthreads();
+            fetch_fragments<TM, TN>(na, nw, 0, frow, fhalf, fa[0], fw[0]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+#pragma unroll
+            for (int j = 0; j < TM; ++j) {
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fw[kk & 1][i], fa[kk & 1][j], acc[i][j], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                hook(((kk + 1) % (kBK / 32)) * (TM * TN) + i * TM + j);
+                __builtin_amdgcn_sched_barrier(0);
             }
     }
 }

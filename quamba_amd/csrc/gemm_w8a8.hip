@@ -8,6 +8,26 @@
 // The tiling, LDS layout and epilogue are in gemm_core.hpp.
 #include "gemm_core.hpp"
 
+// Built with -DQA_GEMM_CLK (bench.py --gemm-phase-clocks, never the product library) thread 0 of every workgroup of
+// the tiled kernel records the shader clock and the constant 100 MHz clock at four points - start, first fragments
+// in registers, end of the main loop, end of the epilogue - and qa_gemm_clk_read copies the table out.
+#ifdef QA_GEMM_CLK
+__device__ unsigned long long g_gemm_clk[8192][8];
+extern "C" int qa_gemm_clk_read(void* dst, int64_t bytes) {
+    if (bytes != static_cast<int64_t>(sizeof(g_gemm_clk))) return QA_ERR_SHAPE;
+    return hipMemcpyFromSymbol(dst, HIP_SYMBOL(g_gemm_clk), sizeof(g_gemm_clk)) == hipSuccess ? QA_OK : QA_ERR_LAUNCH;
+}
+#define CLK_MARK(i)                                                 \
+    do {                                                            \
+        if (threadIdx.x == 0 && blockIdx.x < 8192) {                \
+            g_gemm_clk[blockIdx.x][2 * (i)] = clock64();            \
+            g_gemm_clk[blockIdx.x][2 * (i) + 1] = wall_clock64();   \
+        }                                                           \
+    } while (0)
+#else
+#define CLK_MARK(i)
+#endif
+
 namespace qa {
 namespace {
 
@@ -48,6 +68,41 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_w8a8_kernel(QaGemmW8A8Par
 
     const int k_tiles = (p.k + kBK - 1) / kBK;
     const int frow = lane & 31, fhalf = lane >> 5;
+    CLK_MARK(0);
+    if constexpr (STAGES == 2) {
+        // Two stages, the barrier before the last k step of a tile (mma_tile_rotated).  The requests for a tile go
+        // out one at a time behind every second multiplication, counted from that barrier: the ones that fit into
+        // the last k step of tile t - 2, the rest during the first three steps of tile t - 1.  Past the end of K
+        // every lane is out of range and stores zeros.
+        constexpr int kReq = C::kAInstr + C::kWInstr, kPerStep = TM * TN;
+        constexpr int kEarly = kPerStep / 2 < kReq ? kPerStep / 2 : kReq;      // positions inside the last k step
+        static_assert(kReq <= 4 * kPerStep / 2, "more requests than positions");
+        auto request = [&](int r, int tile) {
+            const uint32_t base = lds_base + (tile & 1) * C::kStageBytes;
+            if (r < C::kAInstr) load_a.template issue_one<WAVES>(r, rsrc_a, tile * kBK, p.k, base, wave);
+            else if (r < kReq) load_w.template issue_one<WAVES>(r - C::kAInstr, rsrc_w, tile * kBK, p.k, base + BM * kBK, wave);
+        };
+#pragma unroll
+        for (int r = 0; r < kReq; ++r) request(r, 0);
+#pragma unroll
+        for (int r = 0; r < kEarly; ++r) request(r, 1);
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(kEarly));
+        __syncthreads();
+        const uint8_t* my_a = lds + (wm * TM * 32) * kBK;
+        const uint8_t* my_w = lds + BM * kBK + (wn * TN * 32) * kBK;
+        v4i fa[2][TM], fw[2][TN];
+        fetch_fragments<TM, TN>(my_a, my_w, 0, frow, fhalf, fa[0], fw[0]);
+        CLK_MARK(1);
+        for (int kt = 0; kt < k_tiles; ++kt) {
+            const int cur = (kt & 1) * C::kStageBytes, nxt = C::kStageBytes - cur;
+            mma_tile_rotated<TM, TN>(my_a + cur, my_w + cur, my_a + nxt, my_w + nxt, frow, fhalf, fa, fw, acc,
+                                     [&](int idx) {
+                                         if (idx % 2 != 1) return;
+                                         const int r = idx / 2;
+                                         request(r, r < kEarly ? kt + 2 : kt + 1);
+                                     });
+        }
+    } else {
     auto issue = [&](int tile) {
         const uint32_t base = lds_base + (tile % STAGES) * C::kStageBytes;
         load_a.template issue<WAVES>(rsrc_a, tile * kBK, p.k, base, wave);
@@ -72,8 +127,10 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_w8a8_kernel(QaGemmW8A8Par
                                        load_w.template issue_one<WAVES>(slot - C::kAInstr, rsrc_w, nt * kBK, p.k, nbase + BM * kBK, wave);
                                });
     }
+    }
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
     __syncthreads();
+    CLK_MARK(2);
 
     Epilogue e;
     e.row_scale = p.a_scale; e.col_scale = p.w_scale;
@@ -81,6 +138,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_w8a8_kernel(QaGemmW8A8Par
     e.use_alpha = p.use_alpha; e.alpha = p.alpha; e.round_mode = p.round_mode; e.col_outer = p.scale_order;
     e.ldd = p.ldd; e.d = p.d;
     epilogue<TM, TN, OUT, FLEX, false, COL_OUTER>(e, acc, lds, p.m, p.n, m0 + wm * TM * 32, n0 + wn * TN * 32, wave, lane);
+    CLK_MARK(3);
 }
 
 template <int TM, int TN, int WGM, int WGN, int STAGES, int OUT, bool FLEX, bool COL_OUTER = false>

@@ -1176,7 +1176,8 @@ extern "C" int qa_sscan_fwd(const QaSScanParams* p, void* stream_) {
     const int per_group = p->dim / p->n_groups;
     if (p->mapping != 0) {
         // a lane mapping named by the caller (tests): only d_state <= 16 has more than one
-        if (N > 16) return QA_ERR_UNSUPPORTED;
+        // a value without the marker bit of QA_SSCAN_MAPPING is not a mapping (an uninitialised field, say)
+        if (!(p->mapping & 0x10000) || (p->mapping & ~0x1ffff) || N > 16) return QA_ERR_UNSUPPORTED;
         const int lanes = (p->mapping >> 8) & 0xff, arg = p->mapping & 0xff;
         if (lanes == 0) {
             // mixed launch: `arg` workgroups of 64 channels with four lanes per channel, the rest with eight

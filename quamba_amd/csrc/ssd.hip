@@ -699,6 +699,10 @@ int validate(const QaSsdParams* p) {
     if (!aligned16(p->x) || !aligned16(p->B) || !aligned16(p->C) || !aligned16(p->out)) return QA_ERR_STRIDE;
     if (p->z && !aligned16(p->z)) return QA_ERR_STRIDE;      // x, the gate and the output are accessed in aligned pieces
     if (p->D && p->D_has_hdim && !aligned16(p->D)) return QA_ERR_STRIDE;
+    // every launch is a one-dimensional grid: one workgroup per (batch, chunk, head) or per (batch, head, 64 states)
+    const int64_t nc = (static_cast<int64_t>(p->seqlen) + p->chunk_size - 1) / p->chunk_size;
+    if (static_cast<int64_t>(p->batch) * nc * p->nheads > 0x7fffffffLL) return QA_ERR_SHAPE;
+    if (static_cast<int64_t>(p->batch) * p->nheads * (p->dstate / 64) > 0x7fffffffLL) return QA_ERR_SHAPE;
     return QA_OK;
 }
 
@@ -724,8 +728,6 @@ extern "C" int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream_) {
     float* dA_ws = reinterpret_cast<float*>(base + ws.dA);
     const int nc = (p->seqlen + p->chunk_size - 1) / p->chunk_size;
     const int64_t bch = static_cast<int64_t>(p->batch) * nc * p->nheads;
-    if (bch > 0x7fffffffLL || static_cast<int64_t>(p->batch) * nc * p->ngroups > 65535) return QA_ERR_SHAPE;
-    if (static_cast<int64_t>(p->batch) * p->nheads * 2 > 0x7fffffffLL) return QA_ERR_SHAPE;
 
     hipLaunchKernelGGL(ssd_cumsum_kernel, dim3(static_cast<unsigned>((bch + 3) / 4)), dim3(256), 0, stream, *p, dt_ws,
                        dA_ws, nc);

@@ -30,24 +30,61 @@ def test_library_exports_every_declared_symbol():
 
 def test_abi_version_and_status_strings():
     l = _lib.lib()
-    assert l.qa_abi_version() == 1
+    assert l.qa_abi_version() == _lib.ABI_VERSION == 2
     assert l.qa_status_string(0) == b"ok"
-    for code in (-1, -2, -3, -4, -5):
+    for code in (-1, -2, -3, -4, -5, -6):
         assert l.qa_status_string(code) not in (b"ok", b"unknown status")
 
 
-def test_struct_sizes_match_the_header(tmp_path):
-    structs = ["QaConvParams", "QaSScanParams", "QaSsmUpdateParams", "QaGemmW8A8Params", "QaGemmW4A8Params",
-               "QaSsdParams"]
-    src = tmp_path / "sz.c"
-    body = "".join(f'printf("{s} %zu\\n", sizeof({s}));' for s in structs)
-    src.write_text(f'#include <stdio.h>\n#include "{HEADER}"\nint main(){{{body}return 0;}}\n')
-    exe = tmp_path / "sz"
+def _param_structs():
+    """Every parameter block the header declares, and its ctypes twin."""
+    text = open(HEADER).read()
+    names = sorted(set(re.findall(r"\}\s*(Qa[A-Za-z0-9]+Params)\s*;", text)))
+    assert len(names) >= 9, names
+    return [(n, getattr(_lib, n)) for n in names]
+
+
+def _layout_from_gcc(tmp_path, structs):
+    """sizeof and the offsetof of every field, as a C compiler lays the header's structs out."""
+    lines = []
+    for name, cls in structs:
+        lines.append(f'printf("{name} . %zu\\n", sizeof({name}));')
+        for field, _ in cls._fields_:
+            lines.append(f'printf("{name} {field} %zu\\n", offsetof({name}, {field}));')
+    src = tmp_path / "layout.c"
+    src.write_text(f'#include <stddef.h>\n#include <stdio.h>\n#include "{HEADER}"\nint main(){{{"".join(lines)}return 0;}}\n')
+    exe = tmp_path / "layout"
     subprocess.run(["gcc", str(src), "-o", str(exe)], check=True)
     out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout
-    sizes = dict(line.split() for line in out.strip().splitlines())
-    for s in structs:
-        assert int(sizes[s]) == C.sizeof(getattr(_lib, s)), s
+    return {(a, b): int(c) for a, b, c in (line.split() for line in out.strip().splitlines())}
+
+
+def test_struct_layouts_match_the_header(tmp_path):
+    """Size and the offset of every field of every Qa*Params block: a field of the binding that the header does not
+    have fails to compile, a missing or reordered one moves an offset or the size."""
+    structs = _param_structs()
+    want = _layout_from_gcc(tmp_path, structs)
+    for name, cls in structs:
+        assert want[(name, ".")] == C.sizeof(cls), name
+        for field, _ in cls._fields_:
+            assert want[(name, field)] == getattr(cls, field).offset, f"{name}.{field}"
+        # the header has no field the binding lacks: the fields tile the struct up to alignment padding
+        covered = sum(C.sizeof(t) for _, t in cls._fields_)
+        assert C.sizeof(cls) - covered < 8 * len(cls._fields_) and covered <= C.sizeof(cls), name
+
+
+def test_a_swapped_pair_of_fields_is_caught(tmp_path):
+    """The check above fails when two neighbouring fields of equal size change places in the binding."""
+    class Swapped(C.Structure):
+        _fields_ = [(n, t) for n, t in _lib.QaGemmW8A8Params._fields_]
+    names = [n for n, _ in Swapped._fields_]
+    i, j = names.index("lda"), names.index("ldw")
+
+    class Swapped2(C.Structure):
+        _fields_ = [f for f in Swapped._fields_[:i]] + [Swapped._fields_[j], Swapped._fields_[i]] + list(Swapped._fields_[j + 1:])
+    want = _layout_from_gcc(tmp_path, [("QaGemmW8A8Params", _lib.QaGemmW8A8Params)])
+    assert C.sizeof(Swapped2) == want[("QaGemmW8A8Params", ".")]
+    assert any(want[("QaGemmW8A8Params", f)] != getattr(Swapped2, f).offset for f, _ in Swapped2._fields_)
 
 
 def test_validation_codes_without_a_gpu():
@@ -75,3 +112,32 @@ def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libquamba_amd.so")
     with pytest.raises(RuntimeError, match="no CPU or PyTorch fallback"):
         _lib.lib()
+
+
+def test_ssd_shape_limits_without_a_gpu():
+    """qa_ssd_workspace_bytes validates the whole parameter block on the host: long problems whose launches are
+    one-dimensional grids are accepted whatever the group count, a grid beyond 2^31 - 1 workgroups is refused."""
+    l = _lib.lib()
+    p = _lib.QaSsdParams()
+    for f in ("x", "dt", "A_log", "B", "C", "out", "x_scale", "dt_scale", "A_log_scale", "B_scale", "C_scale"):
+        setattr(p, f, 256)                                          # never dereferenced by the validation
+    p.batch, p.seqlen, p.nheads, p.headdim, p.dstate, p.ngroups, p.chunk_size = 16, 32768, 128, 64, 128, 8, 64
+    assert l.qa_ssd_workspace_bytes(C.byref(p)) > 0                 # 16 x 512 chunks x 8 groups = 65536 (batch, chunk, group) triples
+    p.batch, p.seqlen = 65536, 65536                                # 65536 x 1024 chunks x 128 heads > 2^31 - 1 workgroups
+    assert l.qa_ssd_workspace_bytes(C.byref(p)) == 0
+    assert l.qa_ssd_chunk_scan_fwd(C.byref(p), None) == -2
+    p.batch, p.seqlen, p.dstate = 2, 512, 256                       # more states than the kernels are built for
+    assert l.qa_ssd_chunk_scan_fwd(C.byref(p), None) == -4
+
+
+def test_the_entry_point_without_allocation_refuses_large_problems_before_any_gpu_call():
+    """The size check of qa_ssd_chunk_scan_fwd_noalloc comes before the first HIP call, so it can be checked here."""
+    l = _lib.lib()
+    p = _lib.QaSsdParams()
+    for f in ("x", "dt", "A_log", "B", "C", "out", "x_scale", "A_log_scale", "B_scale", "C_scale"):
+        setattr(p, f, 256)
+    p.batch, p.seqlen, p.nheads, p.headdim, p.dstate, p.ngroups, p.chunk_size = 4, 4096, 80, 64, 128, 1, 256
+    p.dt_is_fp32 = 1
+    assert l.qa_ssd_workspace_bytes(C.byref(p)) > (64 << 20)
+    assert l.qa_ssd_chunk_scan_fwd_noalloc(C.byref(p), None) == -6
+    assert b"scratch" in l.qa_status_string(-6)

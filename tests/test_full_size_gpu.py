@@ -13,6 +13,7 @@ import pytest
 import torch
 
 import oracle
+from ssd_interval import output_interval
 from quamba_amd import QCausalConv1D, ops
 from quamba_amd import w4a8_utils as wu
 
@@ -113,13 +114,16 @@ def test_w8a8_out_proj_full_size(dev):
 
 
 # ---------------------------------------------------------------- decode: batch 64, 1000 steps
+@pytest.mark.parametrize("state_width", [3, 4], ids=["conv_state_3", "conv_state_4"])
 @pytest.mark.parametrize("one_launch", [False, True], ids=["two_launches", "one_launch"])
-def test_decode_1000_steps(dev, one_launch):
+def test_decode_1000_steps(dev, one_launch, state_width):
+    """conv_state_3 is the benchmark configuration's int8 conv state [64, 5120, 3] (d_conv - 1 columns);
+    conv_state_4 is the (B, D, d_conv) buffer the reference's mixer allocates."""
     Bd, steps = 64, 1000
     conv = QCausalConv1D(D1, D1, 4, groups=D1, device=dev)
     conv.weight, conv.bias = _ri(dev, D1, 4, seed=40), _ri(dev, D1, seed=41)
     conv.weight_scale, conv.bias_scale, conv.input_scale, conv.output_scale = 0.004, 0.004, 0.04, 0.03
-    conv_state = _ri(dev, Bd, D1, 4, seed=42)         # (B, D, d_conv), as the reference's mixer allocates it
+    conv_state = _ri(dev, Bd, D1, state_width, seed=42)
     g = torch.Generator(device=dev).manual_seed(43)
     ssm_state = torch.randn(Bd, D1, N1, device=dev, generator=g) * 0.1
     A, Dq, db = _ri(dev, D1, N1, seed=44), _ri(dev, D1, seed=45), _ri(dev, D1, seed=46)
@@ -165,19 +169,29 @@ def _ssd(dev, x, dt, A, Bm, Cm, Dq, bias, Q, sc, **kw):
                                            final_state_dtype=torch.float32, **kw)
 
 
-def _check_ssd_y(y_gpu, y_ref):
-    """The bar of the fp16 scan outputs on the values themselves, |got - want| <= 1e-2 + 1e-2 |want|.  Both sides round
-    the same operands to fp16 before multiplying; an operand on a rounding tie can fall either way with the last bit
-    of exp, which moves one product by 2^-11 of its size.  With operands drawn from the whole int8 range a single
-    product reaches 10^3 while outputs near zero have a bar of 10^-2, so such outputs exist: they may be one in
-    10 000 and stay inside three times the bar."""
+def _check_ssd_y(y_gpu, ref, interval_of):
+    """The bar of the fp16 scan outputs on the values themselves, |got - want| <= 1e-2 + 1e-2 |want|, for one
+    (batch, head) whose oracle result `ref` carries the stage tensors.  With operands drawn from the whole int8 range
+    a single product reaches 10^3 while an output near zero has a bar of 10^-2, and both sides round the same
+    operands to fp16 before multiplying: an operand on a rounding tie falls either way with the last bit of exp and
+    moves its product by 2^-11 of its size.  Measured on MI355X: between 0 and 11 of 262 144 outputs of a head lie
+    beyond the bar, the farthest at 2.9 times the bar.  The test allows 16 in 262 144 and requires every one of them to
+    lie inside the interval that nudging the fp16-rounded operands of that output by one ulp opens around the float64
+    value (tests/ssd_interval.py): a tie explains it, a dropped or misplaced term would not."""
     got = y_gpu.float().cpu().numpy()
-    want = y_ref.astype(np.float16).astype(np.float32)
+    want = ref["y"].astype(np.float16).astype(np.float32)
     bar = 1e-2 + 1e-2 * np.abs(want)
     err = np.abs(got - want)
-    assert (err > bar).mean() <= 1e-4, f"{(err > bar).sum()} of {err.size} outputs beyond rtol 1e-2 / atol 1e-2"
-    assert (err <= 3 * bar).all(), f"largest error / bar = {(err / bar).max():.2f}"
+    beyond = np.argwhere(err > bar)
+    assert len(beyond) <= max(1, round(16 * err.size / 262144)), f"{len(beyond)} of {err.size} outputs beyond rtol 1e-2 / atol 1e-2"
+    for _, t, _, ch in beyond:
+        lo, hi, y64 = interval_of(int(t), int(ch))
+        g = float(got[0, t, 0, ch])
+        room = 2.0 ** -11 * abs(g) + 1e-6                    # the fp16 rounding of the output itself
+        assert lo - room <= g <= hi + room, f"output (t={t}, p={ch}): {g} outside [{lo}, {hi}] around {y64}"
+        assert hi - lo < 0.25 * max(1.0, np.abs(want).max()), "the interval says nothing"
     assert np.abs(want).max() > 1.0                      # the absolute part of the bar is not what passes the test
+    return len(beyond), float((err / bar).max())
 
 
 def test_ssd_full_size(dev):
@@ -196,10 +210,13 @@ def test_ssd_full_size(dev):
     # oracle on two heads of one batch entry
     for bi, h in ((1, 3), (3, 77)):
         hs = slice(h, h + 1)
+        xq, Cq = _np(x[bi, :, h]), _np(Cm[bi, :, 0])
         ref = oracle.ssd_fwd(_np(x[bi:bi + 1, :, hs]), _np(dt[bi:bi + 1, :, hs]), _np(A[hs]), _np(Bm[bi:bi + 1]), _np(Cm[bi:bi + 1]),
                              _np(Dq[hs]), None, _np(bias[hs]), chunk_size=256, x_scale=0.03, s_dt=0.02, s_A=0.02, s_B=0.03,
-                             s_C=0.03, s_D=0.008)
-        _check_ssd_y(y[bi:bi + 1, :, hs], ref["y"])
+                             s_C=0.03, s_D=0.008, stages=True)
+        D_w = 0.008 * float(_np(Dq[hs])[0])
+        _check_ssd_y(y[bi:bi + 1, :, hs], ref, lambda t, ch: output_interval(
+            ref, t, ch, chunk=256, x_codes=xq, x_scale_p=0.03, C_codes=Cq, s_C=0.03, D_weight=D_w))
         got_f = final[bi:bi + 1, hs].cpu().numpy()
         assert np.abs(got_f - ref["final_f32"]).max() <= 1e-3 * np.abs(ref["final_f32"]).max()
 
@@ -261,7 +278,11 @@ def test_ssd_8b_shape_oracle_heads_and_chunk_independence(dev):
                              _np(Cm[bi:bi + 1, :, gi:gi + 1]), _np(Dq[hs]), None, _np(bias[hs]), chunk_size=256,
                              x_scale=_np(xs[gi, hgi])[None, None], s_dt=0.02, s_A=0.02, s_B=_np(sc["B"][gi:gi + 1]),
                              s_C=_np(sc["C"][gi:gi + 1]), s_D=0.008, head_range=np.ones((1, 1), np.int32),
-                             dim_range=_np(dr[gi, hgi])[None, None])
-        _check_ssd_y(y[bi:bi + 1, :, hs], ref["y"])
+                             dim_range=_np(dr[gi, hgi])[None, None], stages=True)
+        xq, Cq, D_w = _np(x[bi, :, h]), _np(Cm[bi, :, gi]), 0.008 * float(_np(Dq[hs])[0])
+        xs_p = np.repeat(_np(xs[gi, hgi]), 16)               # four dim groups of sixteen channels
+        s_C = float(_np(sc["C"][gi]))
+        _check_ssd_y(y[bi:bi + 1, :, hs], ref, lambda t, ch: output_interval(
+            ref, t, ch, chunk=256, x_codes=xq, x_scale_p=xs_p[ch], C_codes=Cq, s_C=s_C, D_weight=D_w))
         got_f = final[bi:bi + 1, hs].cpu().numpy()
         assert np.abs(got_f - ref["final_f32"]).max() <= 1e-3 * np.abs(ref["final_f32"]).max()

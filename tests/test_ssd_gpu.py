@@ -1,5 +1,5 @@
 """GPU parity of the Mamba2 SSD chunk scan and its single-step update against the CPU oracle.
-fp16 outputs: rtol 1e-2 / atol 1e-2 on the values themselves; fp32 states 1e-3 relative; int8 states at most
+fp16 outputs: rtol 1e-2 / atol 1e-2 on the values themselves, every output; fp32 states 1e-3 relative; int8 states at most
 one step off, and only where the un-rounded quotient lies within 2e-3 of a rounding tie."""
 import numpy as np
 import pytest
@@ -32,17 +32,14 @@ def _gpu(d, dev, chunk, state_scale=None, dt=None, final_dtype=torch.float32, **
 
 
 def _check_y(y_gpu, y_ref):
-    """The bar of the fp16 scan outputs, on the values themselves: |got - want| <= 1e-2 + 1e-2 |want|.
-    Both sides round the same operands to fp16 before multiplying (as the reference does); where a value lies on
-    a rounding tie, the last bit of exp decides which way it goes, and one product of a large operand (outlier
-    channels are 20x the rest) then moves by 2^-11 of its size, which can exceed the bar of an output near zero.
-    Such outputs are allowed for at most two in 100 000, and only up to three times the bar."""
+    """The bar of the fp16 scan outputs, on the values themselves: |got - want| <= 1e-2 + 1e-2 |want| for every output.
+    Measured on MI355X over the cases of this file (synthetic activations with outlier channels): no output beyond the
+    bar, the farthest at 0.9 of it."""
     got = y_gpu.float().cpu().numpy()
     want = y_ref.astype(np.float16).astype(np.float32)
     bar = 1e-2 + 1e-2 * np.abs(want)
     err = np.abs(got - want)
-    assert (err > bar).mean() <= 2e-5, f"{(err > bar).sum()} of {err.size} outputs beyond rtol 1e-2 / atol 1e-2"
-    assert (err <= 3 * bar).all()
+    assert (err <= bar).all(), f"{int((err > bar).sum())} of {err.size} outputs beyond rtol 1e-2 / atol 1e-2, largest error / bar = {(err / bar).max():.2f}"
     assert np.sum((got - y_ref) ** 2) / np.sum(y_ref ** 2) < 1e-6
 
 
