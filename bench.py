@@ -563,7 +563,16 @@ def valu_calibration(dev, ops_list=None, launches=4):
 # Vector instructions a wave of the selective scan issues per group of four steps, counted in the compiled kernel
 # (time loop + staging of the next tile + output store, divided by the eight groups of a 32-step tile): the kind with
 # four lanes per channel and four states per lane, and the short kind with eight lanes per channel and two states.
+# The counts belong to one state of the kernel source: `source_sha256` is the hash of quamba_amd/csrc/sscan.hip they
+# were counted at; when the file has changed since, the line says so (`stale`) instead of passing them off as current.
 SCAN_MIX = {"four_lane": {"plain": 99, "transcendental": 18}, "eight_lane": {"plain": 58, "transcendental": 9}}
+SCAN_MIX_SOURCE_SHA256 = "83b9590278f60f1ac0cab5f6eeaa2a7b6047b7daa4afc33200c7d69c360b8a8c"
+
+
+def scan_mix_is_stale():
+    import hashlib
+    path = os.path.join(ROOT, "quamba_amd", "csrc", "sscan.hip")
+    return hashlib.sha256(open(path, "rb").read()).hexdigest() != SCAN_MIX_SOURCE_SHA256
 
 
 def peaks_measured(dev):
@@ -621,18 +630,20 @@ def gemm_phase_clocks(dev, mixer):
     return out
 
 
-def scan_mix_rates(dev):
+def scan_mix_rates(dev, waves_per_simd=8):
     """Issue time of the scan's own instruction mix on live values (probe ops 6 and 7: the recurrence on registers,
     four plain instructions and one exp2 per chain step, and the same with four more plain instructions): ns per
-    plain and per transcendental wave-instruction per SIMD, and the clock the part settles at under that activity.
-    Constant operands (valu_calibration) leave the part at its highest clock and give lower figures."""
+    plain and per transcendental wave-instruction per SIMD, and the clock the part settles at under that activity,
+    with `waves_per_simd` resident waves on every SIMD (eight: what the vector ALUs sustain; fewer: what that many
+    waves can draw from them).  Constant operands (valu_calibration) leave the part at its highest clock and give
+    lower figures."""
     from quamba_amd import _lib
     lib = _probes()
-    wgs, iters = 2048, 10000
+    simds = 4 * torch.cuda.get_device_properties(dev).multi_processor_count
+    wgs, iters = waves_per_simd * simds // 4, 10000
     sink = torch.empty(wgs * 256, dtype=torch.float32, device=dev)
     ticks = torch.zeros(2, dtype=torch.int64, device=dev)
     stream = torch.cuda.current_stream().cuda_stream
-    simds = 4 * torch.cuda.get_device_properties(dev).multi_processor_count
     ns, clock = {}, {}
     for op in (6, 7):
         for _ in range(3):
@@ -652,22 +663,25 @@ def scan_mix_rates(dev):
 def scan_issue_bound(dev, B, D, L):
     """Lower bound of the scan launch from vector-ALU issue alone: every wave's instruction mix priced at the rates
     the same mix reaches in a register-only loop on live values on this GPU now (scan_mix_rates), the waves spread
-    evenly over the SIMDs.  Follows the host's choice of the two kinds of workgroup for d_state 16 (qa_sscan_fwd)."""
-    rates = scan_mix_rates(dev)
-    t_plain, t_trans = rates["ns_plain"], rates["ns_transcendental"]
+    evenly over the SIMDs.  The split into the two kinds of workgroup is the library's own (qa_sscan_chosen_mapping).
+    `issue_bound_us` uses the rates of eight resident waves per SIMD (what the vector ALUs sustain);
+    `issue_bound_at_launch_occupancy_us` uses the rates the probe reaches with as many waves per SIMD as this launch
+    has - a single wave cannot issue back to back, so few waves draw less from the same ALUs."""
     simds = 4 * torch.cuda.get_device_properties(dev).multi_processor_count
-    waves4 = B * D // 16
-    q, rem = divmod(waves4, simds)
-    short = 0
-    if 2 * waves4 <= 3 * simds:
-        short = D
-    elif q >= 1 and 0 < rem and 2 * rem <= simds and (rem * 16 // B) % 32 == 0 and (D - rem * 16 // B) % 64 == 0:
-        short = rem * 16 // B
+    lanes, arg = ops.sscan_chosen_mapping(B, D, CFG["d_state"])
+    short = D if lanes == 8 else (D - 64 * arg if lanes == 0 else 0)
     waves = {"four_lane": B * (D - short) // 16, "eight_lane": B * short // 8}
     groups = (L + 31) // 32 * 8
-    ns = sum(waves[k] * groups * (SCAN_MIX[k]["plain"] * t_plain + SCAN_MIX[k]["transcendental"] * t_trans) for k in waves)
-    return dict(issue_bound_us=ns / simds / 1e3, ns_plain=round(t_plain, 3), ns_transcendental=round(t_trans, 3),
-                clock_MHz=round(rates["clock_MHz"], 1), waves=waves, instructions_per_four_steps=SCAN_MIX)
+    wps = -(-(waves["four_lane"] + waves["eight_lane"]) // simds)
+    out = dict(waves=waves, waves_per_simd=wps, instructions_per_four_steps=SCAN_MIX, stale=scan_mix_is_stale())
+    for key, n in (("issue_bound_us", 8), ("issue_bound_at_launch_occupancy_us", wps)):
+        rates = scan_mix_rates(dev, n)
+        t_plain, t_trans = rates["ns_plain"], rates["ns_transcendental"]
+        ns = sum(waves[k] * groups * (SCAN_MIX[k]["plain"] * t_plain + SCAN_MIX[k]["transcendental"] * t_trans) for k in waves)
+        out[key] = ns / simds / 1e3
+        out[key.replace("_us", "_rates")] = dict(ns_plain=round(t_plain, 3), ns_transcendental=round(t_trans, 3),
+                                                 clock_MHz=round(rates["clock_MHz"], 1), waves_per_simd=n)
+    return out
 
 
 def load_traffic(path):
@@ -752,10 +766,15 @@ def main():
     if dom["name"] == "sscan_fwd":
         # the bound that binds this kernel is vector-ALU issue, not HBM: how far the launch is from it
         ib = scan_issue_bound(dev, B, CFG["d_inner"], L)
-        roofline["issue_bound_us"] = round(ib["issue_bound_us"], 2)
-        roofline["frac_of_issue_bound"] = round(ib["issue_bound_us"] / dom["avg_us"], 4)
-        roofline["issue_bound_inputs"] = {k: ib[k] for k in ("ns_plain", "ns_transcendental", "clock_MHz", "waves",
-                                                             "instructions_per_four_steps")}
+        if ib["stale"]:
+            roofline["issue_bound_stale"] = "quamba_amd/csrc/sscan.hip has changed since the instruction mix was counted"
+        else:
+            roofline["issue_bound_us"] = round(ib["issue_bound_us"], 2)
+            roofline["frac_of_issue_bound"] = round(ib["issue_bound_us"] / dom["avg_us"], 4)
+            roofline["issue_bound_at_launch_occupancy_us"] = round(ib["issue_bound_at_launch_occupancy_us"], 2)
+            roofline["frac_of_issue_bound_at_launch_occupancy"] = round(ib["issue_bound_at_launch_occupancy_us"] / dom["avg_us"], 4)
+        roofline["issue_bound_inputs"] = {k: ib[k] for k in ("issue_bound_rates", "issue_bound_at_launch_occupancy_rates",
+                                                             "waves", "waves_per_simd", "instructions_per_four_steps")}
     per_kernel = [dict(kernel=k["name"], bound=k["bound"], avg_us=round(k["avg_us"], 2), achieved=round(k["achieved"], 2),
                        unit=k["unit"], peak=k["peak"], frac=round(k["frac"], 4), traffic=traffic.get(k["name"]))
                   for k in kernels]

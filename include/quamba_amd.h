@@ -245,9 +245,16 @@ typedef struct QaSScanParams {
     int32_t mapping;
 } QaSScanParams;
 
-#define QA_SSCAN_MAPPING(lanes, arg) (0x10000 | ((lanes) << 8) | (arg))
+/* marker bit 30, lanes in bits 20..27, the second argument in bits 0..19; a value without the marker is refused */
+#define QA_SSCAN_MAPPING(lanes, arg) (0x40000000 | ((lanes) << 20) | (arg))
 
 int qa_sscan_fwd(const QaSScanParams* p, void* stream);
+/* The mapping qa_sscan_fwd takes for these sizes on the current device, as a QA_SSCAN_MAPPING code (0 for d_state
+ * above 16, which has one mapping per size; p->mapping itself when the caller named one), or a negative QaStatus.
+ * Only batch, dim, dstate, n_groups and mapping are read; nothing is launched.  No counterpart in the reference
+ * (csrc/selective_scan/quant_sscan_fwd_kernel.cuh:296-349 has one launch shape per d_state); bench.py prices the
+ * launch's instruction mix with it. */
+int qa_sscan_chosen_mapping(const QaSScanParams* p);
 
 /* ------------------------------------------------------------------------------------------
  * Single-token recurrent state update (decode step), Mamba1 (nheads == 1, headdim == d_inner)

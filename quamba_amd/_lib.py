@@ -166,6 +166,7 @@ SYMBOLS = {
     "qa_rmsnorm_gated": (C.c_int, [C.POINTER(QaNormGatedParams), vp]),
     "qa_rmsnorm_gated_hadamard_quant": (C.c_int, [C.POINTER(QaNormGatedParams), C.POINTER(QaHadamardParams), vp]),
     "qa_sscan_fwd": (C.c_int, [C.POINTER(QaSScanParams), vp]),
+    "qa_sscan_chosen_mapping": (C.c_int, [C.POINTER(QaSScanParams)]),
     "qa_ssm_state_update": (C.c_int, [C.POINTER(QaSsmUpdateParams), vp]),
     "qa_mamba1_decode_step": (C.c_int, [C.POINTER(QaConvParams), C.POINTER(QaSsmUpdateParams), vp]),
     "qa_gemm_w8a8": (C.c_int, [C.POINTER(QaGemmW8A8Params), vp]),

@@ -1148,6 +1148,53 @@ int launch_update(const QaSsmUpdateParams& p, hipStream_t stream, const QaConvPa
 }  // namespace
 }  // namespace qa
 
+namespace qa {
+namespace {
+// How lanes are laid over channels and states for d_state <= 16, as a QA_SSCAN_MAPPING code.
+// The kernel is bound by vector-ALU issue, so the mapping that wastes the fewest issue slots wins: four lanes per
+// channel and, when the channel count allows, four waves per workgroup sharing one staged B/C tile.  With channel
+// groups a workgroup must stay inside one group.
+int choose_mapping16(const QaSScanParams& p) {
+    const int per_group = p.dim / p.n_groups;
+    int waves = p.dim % 64 == 0 ? 4 : (p.dim % 32 == 0 ? 2 : 1);
+    while (waves > 1 && p.n_groups > 1 && per_group % (16 * waves) != 0) waves >>= 1;
+    if (waves < 4) return QA_SSCAN_MAPPING(4, waves);
+    // Waves per SIMD with four lanes per channel: q + f.  With 0 < f <= 1/2 the last f/(q+f) of the
+    // channels of every batch entry go to the eight-lane kind (see sscan_fwd_mixed_kernel), as long as
+    // both parts stay whole workgroups and, with channel groups, whole groups.
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) {
+        cus = 256;
+    }
+    const int64_t simds = 4LL * cus;
+    const int64_t waves_a = static_cast<int64_t>(p.batch) * p.dim / 16;
+    const int64_t q = waves_a / simds, rem_waves = waves_a % simds;
+    // Few waves (small batches): a launch takes about as long as the busiest SIMD's waves one after the
+    // other, and with so few of them latency, not issue, sets a wave's pace - so twice as many waves
+    // of two thirds the length (eight lanes per channel) finish sooner: up to 1.5 four-lane waves per SIMD.
+    if (2 * waves_a <= 3 * simds && (p.n_groups <= 1 || per_group % 32 == 0)) return QA_SSCAN_MAPPING(8, 4);
+    if (p.n_groups == 1 && q >= 1 && rem_waves > 0 && 2 * rem_waves <= simds) {
+        const int64_t short_channels = rem_waves * 16 / p.batch;      // channels per batch entry for the short kind
+        const int64_t blocks_a = (p.dim - short_channels) / 64;
+        if (short_channels % 32 == 0 && (p.dim - short_channels) % 64 == 0 && blocks_a > 0 && blocks_a <= 0xfffff) {
+            return QA_SSCAN_MAPPING(0, static_cast<int>(blocks_a));
+        }
+    }
+    return QA_SSCAN_MAPPING(4, 4);
+}
+}  // namespace
+}  // namespace qa
+
+extern "C" int qa_sscan_chosen_mapping(const QaSScanParams* p) {
+    if (!p) return QA_ERR_NULL;
+    if (p->batch < 1 || p->dim < 1 || p->dstate < 1 || p->dstate > 256) return QA_ERR_SHAPE;
+    if (p->n_groups < 1 || p->dim % p->n_groups != 0) return QA_ERR_SHAPE;
+    if (p->dstate > 16) return 0;
+    if (p->mapping != 0) return p->mapping;
+    return qa::choose_mapping16(*p);
+}
+
 extern "C" int qa_sscan_fwd(const QaSScanParams* p, void* stream_) {
     using namespace qa;
     if (!p || !p->u || !p->delta || !p->A_log || !p->B || !p->C || !p->out) return QA_ERR_NULL;
@@ -1177,8 +1224,8 @@ extern "C" int qa_sscan_fwd(const QaSScanParams* p, void* stream_) {
     if (p->mapping != 0) {
         // a lane mapping named by the caller (tests): only d_state <= 16 has more than one
         // a value without the marker bit of QA_SSCAN_MAPPING is not a mapping (an uninitialised field, say)
-        if (!(p->mapping & 0x10000) || (p->mapping & ~0x1ffff) || N > 16) return QA_ERR_UNSUPPORTED;
-        const int lanes = (p->mapping >> 8) & 0xff, arg = p->mapping & 0xff;
+        if ((p->mapping & ~0x0fffffff) != 0x40000000 || N > 16) return QA_ERR_UNSUPPORTED;
+        const int lanes = (p->mapping >> 20) & 0xff, arg = p->mapping & 0xfffff;
         if (lanes == 0) {
             // mixed launch: `arg` workgroups of 64 channels with four lanes per channel, the rest with eight
             if (arg < 1 || p->n_groups != 1 || 64LL * arg > p->dim) return QA_ERR_SHAPE;
@@ -1194,39 +1241,12 @@ extern "C" int qa_sscan_fwd(const QaSScanParams* p, void* stream_) {
         return QA_ERR_UNSUPPORTED;
     }
     if (N <= 16) {
-        // The kernel is bound by vector-ALU issue, so the mapping that wastes the fewest issue slots wins: four
-        // lanes per channel and, when the channel count allows, four waves per workgroup sharing one staged
-        // B/C tile.  With channel groups a workgroup must stay inside one group.
-        int waves = p->dim % 64 == 0 ? 4 : (p->dim % 32 == 0 ? 2 : 1);
-        while (waves > 1 && p->n_groups > 1 && per_group % (16 * waves) != 0) waves >>= 1;
-        if (waves == 4) {
-            // Waves per SIMD with four lanes per channel: q + f.  With 0 < f <= 1/2 the last f/(q+f) of the
-            // channels of every batch entry go to the eight-lane kind (see sscan_fwd_mixed_kernel), as long as
-            // both parts stay whole workgroups and, with channel groups, whole groups.
-            int dev = 0, cus = 256;
-            if (hipGetDevice(&dev) != hipSuccess ||
-                hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) {
-                cus = 256;
-            }
-            const int64_t simds = 4LL * cus;
-            const int64_t waves_a = static_cast<int64_t>(p->batch) * p->dim / 16;
-            const int64_t q = waves_a / simds, rem_waves = waves_a % simds;
-            // Few waves (small batches): a launch takes about as long as the busiest SIMD's waves one after the
-            // other, and with so few of them latency, not issue, sets a wave's pace - so twice as many waves
-            // of two thirds the length (eight lanes per channel) finish sooner: up to 1.5 four-lane waves per SIMD.
-            if (2 * waves_a <= 3 * simds && (p->n_groups <= 1 || per_group % 32 == 0)) {
-                return launch_fwd_pre<2, 8, 4>(*p, stream, vec_in, vec_bc, vec_out);
-            }
-            if (p->n_groups == 1 && q >= 1 && rem_waves > 0 && 2 * rem_waves <= simds) {
-                const int64_t short_channels = rem_waves * 16 / p->batch;      // channels per batch entry for the short kind
-                const int blocks_a = static_cast<int>((p->dim - short_channels) / 64);
-                if (short_channels % 32 == 0 && (p->dim - short_channels) % 64 == 0 && blocks_a > 0) {
-                    return launch_fwd_mixed(*p, stream, vec_in, vec_bc, vec_out, blocks_a);
-                }
-            }
-            return launch_fwd_pre<4, 4, 4>(*p, stream, vec_in, vec_bc, vec_out);
-        }
-        if (waves == 2) return launch_fwd_pre<4, 4, 2>(*p, stream, vec_in, vec_bc, vec_out);
+        const int mapping = choose_mapping16(*p);
+        const int lanes = (mapping >> 20) & 0xff, arg = mapping & 0xfffff;
+        if (lanes == 0) return launch_fwd_mixed(*p, stream, vec_in, vec_bc, vec_out, arg);
+        if (lanes == 8) return launch_fwd_pre<2, 8, 4>(*p, stream, vec_in, vec_bc, vec_out);
+        if (arg == 4) return launch_fwd_pre<4, 4, 4>(*p, stream, vec_in, vec_bc, vec_out);
+        if (arg == 2) return launch_fwd_pre<4, 4, 2>(*p, stream, vec_in, vec_bc, vec_out);
         return launch_fwd_pre<4, 4, 1>(*p, stream, vec_in, vec_bc, vec_out);
     }
     // Wider states: eight states per lane, or sixteen.  A workgroup converts its B/C tile once for all of its

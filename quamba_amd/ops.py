@@ -488,7 +488,19 @@ SSCAN_MAPPING = 0
 def sscan_mapping(lanes, arg):
     """QA_SSCAN_MAPPING(lanes per channel, waves per workgroup); lanes == 0: the launch with two kinds of
     workgroup, ``arg`` 64-channel workgroups per batch entry taking four lanes per channel."""
-    return 0x10000 | (int(lanes) << 8) | int(arg)
+    return 0x40000000 | (int(lanes) << 20) | int(arg)
+
+
+def sscan_chosen_mapping(batch, dim, dstate, n_groups=1):
+    """(lanes per channel, argument) of the mapping qa_sscan_fwd takes for these sizes on the current device
+    (qa_sscan_chosen_mapping); lanes == 0 is the launch with two kinds of workgroup, the argument then being the
+    number of 64-channel workgroups per batch entry with four lanes per channel.  None for d_state above 16."""
+    p = _lib.QaSScanParams()
+    p.batch, p.dim, p.dstate, p.n_groups = batch, dim, dstate, n_groups
+    code = _lib.lib().qa_sscan_chosen_mapping(ct.byref(p))
+    if code < 0:
+        _lib.check(code, "sscan_chosen_mapping")
+    return None if code == 0 else ((code >> 20) & 0xff, code & 0xfffff)
 
 
 def _sscan_segments(batch, dim, seqlen):

@@ -141,3 +141,28 @@ def test_the_entry_point_without_allocation_refuses_large_problems_before_any_gp
     assert l.qa_ssd_workspace_bytes(C.byref(p)) > (64 << 20)
     assert l.qa_ssd_chunk_scan_fwd_noalloc(C.byref(p), None) == -6
     assert b"scratch" in l.qa_status_string(-6)
+
+
+def test_scan_mapping_codes_without_a_gpu():
+    """A mapping field without the marker bit of QA_SSCAN_MAPPING is refused before anything is launched, and
+    qa_sscan_chosen_mapping reports the library's own choice (no GPU here: it assumes 256 CUs)."""
+    from quamba_amd import ops
+    l = _lib.lib()
+    p = _lib.QaSScanParams()
+    for f in ("u", "delta", "A_log", "B", "C", "out", "scale_u", "scale_delta", "scale_A", "scale_B", "scale_C"):
+        setattr(p, f, 256)                                          # never dereferenced on these paths
+    p.batch, p.dim, p.seqlen, p.dstate, p.n_groups = 8, 5120, 64, 16, 1
+    for bad in (1, 0x10404, 0x40000000 | (3 << 28)):
+        p.mapping = bad
+        assert l.qa_sscan_fwd(C.byref(p), None) == -4, hex(bad)
+    p.mapping = ops.sscan_mapping(3, 4)                             # well-formed, but no kernel has three lanes per channel
+    assert l.qa_sscan_fwd(C.byref(p), None) == -4
+    p.mapping = 0
+    # 8 x 5120 channels on 1024 SIMDs: 2.5 four-lane waves per SIMD -> the last fifth of the channels takes eight lanes
+    assert ops.sscan_chosen_mapping(8, 5120, 16) == (0, 64)
+    assert ops.sscan_chosen_mapping(1, 5120, 16) == (8, 4)          # few waves: eight lanes per channel
+    assert ops.sscan_chosen_mapping(4, 48, 16) == (4, 1)
+    assert ops.sscan_chosen_mapping(8, 5120, 128) is None
+    p.mapping = ops.sscan_mapping(4, 2)
+    assert l.qa_sscan_chosen_mapping(C.byref(p)) == p.mapping       # a named mapping is reported as it is
+    assert l.qa_sscan_chosen_mapping(None) == -1
