@@ -428,6 +428,9 @@ typedef struct QaSsdParams {
     int64_t workspace_bytes;
 } QaSsdParams;
 
+/* Sizes the kernels are built for: headdim 64, dstate 64 or 128, chunk_size 64, 128 or 256; anything else returns
+ * QA_ERR_UNSUPPORTED (qa_ssd_workspace_bytes: 0).  batch * chunks * nheads and batch * nheads * dstate / 64 must
+ * each fit a one-dimensional grid (2^31 - 1), else QA_ERR_SHAPE. */
 int64_t qa_ssd_workspace_bytes(const QaSsdParams* p);
 int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream);
 
@@ -439,7 +442,10 @@ int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream);
  * library runs on holds it until the process ends.  A problem whose qa_ssd_workspace_bytes() exceeds that size
  * returns QA_ERR_SCRATCH.  The call allocates nothing and frees nothing; same kernels, same results as
  * qa_ssd_chunk_scan_fwd.  All calls on one GPU share the buffer: calls that overlap on one GPU (two streams, two
- * threads) race; calls on one stream, or ordered by events, do not.  Nothing in the buffer has to start at zero. */
+ * threads) race; calls on one stream, or ordered by events, do not.  Nothing in the buffer has to start at zero.
+ * The first call on a device looks the buffer's address up and raises the kernels' LDS limit (two runtime calls
+ * that do not belong under stream capture): make one ordinary call on a device before capturing this entry point
+ * into a HIP graph.  The size check comes before any runtime call. */
 #define QA_SSD_STATIC_SCRATCH_BYTES (64ll << 20)
 int qa_ssd_chunk_scan_fwd_noalloc(const QaSsdParams* p, void* stream);
 
