@@ -29,6 +29,7 @@ from quamba_amd import QCausalConv1D, W8A8B8O8Linear, W8A8B16O16Linear, ops, syn
 
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 INT8_PEAK_TOPS = 5000.0     # MI355X dense int8 MFMA
+F16_PEAK_TFLOPS = 2500.0    # MI355X dense fp16 MFMA
 
 CFG = dict(batch=8, seqlen=2048, d_model=2560, d_inner=5120, d_state=16, dt_rank=160, d_conv=4)
 
@@ -273,8 +274,13 @@ def _wl_ssd(dev, steps, warmup, B, L, H, N, G, Q, name, label):
     # dense multiply-adds: C B^T (lower tiles), chunk states, C x entering state, causal part of (C B^T) x
     nc = (L + Q - 1) // Q
     flops = 2.0 * B * nc * (G * Q * Q * N / 2 + H * Q * 64 * N + H * Q * 64 * N + H * Q * Q * 64 / 2)
+    # fp16 products (chunk states, C x entering state, causal part of (C B^T) x) against the fp16 matrix peak, and the
+    # int8 product C B^T as the kernel forms it - per head, at and below the diagonal in 16 x 32 blocks - against the int8 peak
+    f16_flops = 2.0 * B * nc * H * (2 * Q * 64 * N + Q * Q * 64 / 2)
+    i8_ops = 2.0 * B * nc * H * N * sum(16 * 32 * ((mt + 2) // 2) for mt in range(Q // 16))
     return dict(workload=label, name=name, us=ms * 1e3, tokens_per_s=B * L / ms * 1e3, bound="hbm", bytes=nbytes,
-                achieved_GBs=nbytes / ms / 1e6, frac=nbytes / ms / 1e6 / HBM_PEAK_GBS, dense_TFLOPs=flops / ms / 1e9)
+                achieved_GBs=nbytes / ms / 1e6, frac=nbytes / ms / 1e6 / HBM_PEAK_GBS, dense_TFLOPs=flops / ms / 1e9,
+                mfma_f16_frac=f16_flops / ms / 1e9 / F16_PEAK_TFLOPS, mfma_i8_frac=i8_ops / ms / 1e9 / INT8_PEAK_TOPS)
 
 
 def _wl_w4a8(dev, steps, warmup, M, Nn, K, o8, name):
@@ -625,6 +631,22 @@ def gemm_phase_clocks(dev, mixer):
                               "shader_cycles": int(np.median(dc[:, i])),
                               "clock_MHz": round(float(np.median(dc[:, i] / np.maximum(dw[:, i], 1))) * 100.0, 1)}
             out[name] = {"us": round(ms * 1e3, 1), "workgroups": wgs, "tile": list(tile), **phases}
+        # the same in_proj launch on operands that switch less: the cycles stay, the clock rises
+        zeros = torch.zeros_like(mixer.hidden)
+        weight = mixer.in_proj.weight.clone()
+        for label, zero_w in (("in_proj_zero_activations", False), ("in_proj_all_operands_zero", True)):
+            if zero_w:
+                mixer.in_proj.weight.zero_()
+            ms = _time_fn(lambda: mixer.in_proj.to_seqlen_last(zeros), 10, 10)
+            buf = np.zeros((8192, 8), np.uint64)
+            if clk.qa_gemm_clk_read(buf.ctypes.data_as(C.c_void_p), buf.nbytes) == 0:
+                wgs = out.get("in_proj_w8a8_gemm", {}).get("workgroups", 0)
+                b = buf[:wgs].astype(np.int64)
+                dc, dw = np.diff(b[:, 0::2], axis=1), np.diff(b[:, 1::2], axis=1)
+                out[label] = {"us": round(ms * 1e3, 1),
+                              "main_loop": {"us": round(float(np.median(dw[:, 1])) / 100.0, 2), "shader_cycles": int(np.median(dc[:, 1])),
+                                            "clock_MHz": round(float(np.median(dc[:, 1] / np.maximum(dw[:, 1], 1))) * 100.0, 1)}}
+        mixer.in_proj.weight.copy_(weight)
     finally:
         prod.qa_gemm_w8a8 = real
     return out
