@@ -618,30 +618,42 @@ def gemm_phase_clocks(dev, mixer):
                                       2 * mixer.D, mixer.B * mixer.L, (320, 256)),
                                      ("out_proj_w8a8_gemm", lambda: mixer.out_proj(mixer.y_q),
                                       mixer.B * mixer.L, mixer.dm, (256, 320))):
-            ms = _time_fn(fn, 10, 10)
-            wgs = -(-m // tile[0]) * -(-n // tile[1])
             buf = np.zeros((8192, 8), np.uint64)
-            if clk.qa_gemm_clk_read(buf.ctypes.data_as(C.c_void_p), buf.nbytes) != 0 or wgs > 8192:
+            for _ in range(10):
+                fn()
+            torch.cuda.synchronize()
+            clk.qa_gemm_clk_read(buf.ctypes.data_as(C.c_void_p), buf.nbytes)      # clears the table
+            ms = _time_fn(fn, 10, 0)
+            tiles = -(-m // tile[0]) * -(-n // tile[1])
+            if clk.qa_gemm_clk_read(buf.ctypes.data_as(C.c_void_p), buf.nbytes) != 0:
                 continue
-            b = buf[:wgs].astype(np.int64)
+            b = buf.astype(np.int64)
+            b = b[b[:, 0] != 0]                  # one row per workgroup: the last tile it worked on
+            wgs = len(b)
+            if wgs == 0:
+                continue
             dc, dw = np.diff(b[:, 0::2], axis=1), np.diff(b[:, 1::2], axis=1)
             phases = {}
             for i, ph in enumerate(("prologue", "main_loop", "epilogue")):
                 phases[ph] = {"us": round(float(np.median(dw[:, i])) / 100.0, 2),
                               "shader_cycles": int(np.median(dc[:, i])),
                               "clock_MHz": round(float(np.median(dc[:, i] / np.maximum(dw[:, i], 1))) * 100.0, 1)}
-            out[name] = {"us": round(ms * 1e3, 1), "workgroups": wgs, "tile": list(tile), **phases}
+            out[name] = {"us": round(ms * 1e3, 1), "tiles": tiles, "workgroups": wgs, "tile": list(tile), **phases}
         # the same in_proj launch on operands that switch less: the cycles stay, the clock rises
         zeros = torch.zeros_like(mixer.hidden)
         weight = mixer.in_proj.weight.clone()
         for label, zero_w in (("in_proj_zero_activations", False), ("in_proj_all_operands_zero", True)):
             if zero_w:
                 mixer.in_proj.weight.zero_()
-            ms = _time_fn(lambda: mixer.in_proj.to_seqlen_last(zeros), 10, 10)
             buf = np.zeros((8192, 8), np.uint64)
+            for _ in range(10):
+                mixer.in_proj.to_seqlen_last(zeros)
+            torch.cuda.synchronize()
+            clk.qa_gemm_clk_read(buf.ctypes.data_as(C.c_void_p), buf.nbytes)
+            ms = _time_fn(lambda: mixer.in_proj.to_seqlen_last(zeros), 10, 0)
             if clk.qa_gemm_clk_read(buf.ctypes.data_as(C.c_void_p), buf.nbytes) == 0:
-                wgs = out.get("in_proj_w8a8_gemm", {}).get("workgroups", 0)
-                b = buf[:wgs].astype(np.int64)
+                b = buf.astype(np.int64)
+                b = b[b[:, 0] != 0]
                 dc, dw = np.diff(b[:, 0::2], axis=1), np.diff(b[:, 1::2], axis=1)
                 out[label] = {"us": round(ms * 1e3, 1),
                               "main_loop": {"us": round(float(np.median(dw[:, 1])) / 100.0, 2), "shader_cycles": int(np.median(dc[:, 1])),
