@@ -10,8 +10,7 @@
 
 // Built with -DQA_GEMM_CLK (bench.py --gemm-phase-clocks, never the product library) thread 0 of every workgroup of
 // the tiled kernel records the shader clock and the constant 100 MHz clock at four points - start, first fragments
-// in registers, end of the main loop, end of the epilogue - of the last tile it works on, and qa_gemm_clk_read copies
-// the table out.
+// in registers, end of the main loop, end of the epilogue - and qa_gemm_clk_read copies the table out.
 #ifdef QA_GEMM_CLK
 __device__ unsigned long long g_gemm_clk[8192][8];
 extern "C" int qa_gemm_clk_read(void* dst, int64_t bytes) {     // copies the table out and clears it
@@ -49,16 +48,13 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_w8a8_kernel(QaGemmW8A8Par
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave % WGM, wn = wave / WGM;
     const int tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
+    int tile_m, tile_n;
+    tile_of_workgroup<BM, BN>(blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
     const v4i rsrc_a = make_rsrc(p.a, static_cast<int>((static_cast<int64_t>(p.m) - 1) * p.lda + p.k));
     const v4i rsrc_w = make_rsrc(p.w, static_cast<int>((static_cast<int64_t>(p.n) - 1) * p.ldw + p.k));
     const uint32_t lds_base = lds_offset_of(lds);
-
-    // A launch with fewer workgroups than tiles has every workgroup walk the tiles blockIdx.x, blockIdx.x + gridDim.x,
-    // ... (the positions the hardware's own dispatch order would have given it round after round).
-    for (int tile_linear = blockIdx.x; tile_linear < tiles_m * tiles_n; tile_linear += gridDim.x) {
-    int tile_m, tile_n;
-    tile_of_workgroup<BM, BN>(tile_linear, tiles_m, tiles_n, tile_m, tile_n);
-    const int m0 = tile_m * BM, n0 = tile_n * BN;
 
     TileLoader<C::kAInstr> load_a;
     TileLoader<C::kWInstr> load_w;
@@ -146,8 +142,6 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_w8a8_kernel(QaGemmW8A8Par
     e.ldd = p.ldd; e.d = p.d;
     epilogue<TM, TN, OUT, FLEX, false, COL_OUTER>(e, acc, lds, p.m, p.n, m0 + wm * TM * 32, n0 + wn * TN * 32, wave, lane);
     CLK_MARK(3);
-    __syncthreads();                 // the staging areas of the epilogue are the next tile's operand stages
-    }
 }
 
 template <int TM, int TN, int WGM, int WGN, int STAGES, int OUT, bool FLEX, bool COL_OUTER = false>
@@ -166,18 +160,7 @@ int launch_one(const QaGemmW8A8Params& p, hipStream_t stream) {
             return check_launch();
         }
     }
-    // A kernel whose LDS fills a CU runs one workgroup per CU, i.e. in rounds of as many tiles as there are CUs: it is
-    // launched with one workgroup per CU that walks its tiles, which saves the dispatch of a new workgroup per tile
-    // (0.5 - 2 % of the launch; the tiles a workgroup gets are the ones the round-by-round dispatch would give it).
-    int64_t grid = tiles;
-    if (C::kLdsBytes > 81920) {
-        int dev = 0, cus = 0;
-        if (hipGetDevice(&dev) == hipSuccess &&
-            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0 && tiles > cus) {
-            grid = cus;
-        }
-    }
-    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid)), dim3(C::kThreads), C::kLdsBytes, stream, p);
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(tiles)), dim3(C::kThreads), C::kLdsBytes, stream, p);
     return check_launch();
 }
 
