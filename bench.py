@@ -185,7 +185,22 @@ def cpu_baseline(dev_mixer, seconds_budget=30.0):
                        "conv and scan: C oracle with OpenMP; GEMMs: fp32 torch.matmul on dequantised operands")
 
 
-def _time_fn(fn, steps, warmup):
+SETTLE_MS = 40.0     # untimed repetitions before a measurement (main sets it from --settle-ms)
+
+
+def _time_fn(fn, steps, warmup, settle_ms=None):
+    """Mean time of `steps` calls in ms (HIP events around the whole run), after `warmup` calls and, before them, as many
+    untimed calls as fill `settle_ms`, queued without host synchronisation: the part takes about 30 ms of a new
+    workload to settle its clocks, and an idle gap lets them fall again."""
+    settle_ms = SETTLE_MS if settle_ms is None else settle_ms
+    if settle_ms > 0:
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        fn()
+        torch.cuda.synchronize()
+        est_ms = max((time.perf_counter() - t) * 1e3, 0.02)
+        for _ in range(int(min(2000, settle_ms / est_ms))):
+            fn()
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -587,8 +602,8 @@ def valu_calibration(dev, ops_list=None, launches=4):
 # four lanes per channel and four states per lane, and the short kind with eight lanes per channel and two states.
 # The counts belong to one state of the kernel source: `source_sha256` is the hash of quamba_amd/csrc/sscan.hip they
 # were counted at; when the file has changed since, the line says so (`stale`) instead of passing them off as current.
-SCAN_MIX = {"four_lane": {"plain": 99, "transcendental": 18}, "eight_lane": {"plain": 58, "transcendental": 9}}
-SCAN_MIX_SOURCE_SHA256 = "83b9590278f60f1ac0cab5f6eeaa2a7b6047b7daa4afc33200c7d69c360b8a8c"
+SCAN_MIX = {"four_lane": {"plain": 96, "transcendental": 18}, "eight_lane": {"plain": 57, "transcendental": 9}}
+SCAN_MIX_SOURCE_SHA256 = "ddfccf33dd8fd9759e61dc7f65ac3f2734fc73a1c39900ce0102ae3fabe0406b"
 
 
 def scan_mix_is_stale():
@@ -791,35 +806,37 @@ def main():
         sys.exit("bench.py needs a GPU")
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    global SETTLE_MS
+    SETTLE_MS = min(SETTLE_MS, max(0.0, args.settle_ms))
     mixer = Mixer(dev, args.batch, args.seqlen, input_sets=max(1, args.input_sets))
     B, L = args.batch, args.seqlen
-    # what the part sustains today (copy rate, matrix rate on random operands): measured first, which also takes the
-    # GPU out of the idle state the seconds of host-side input generation above left it in
-    peaks = peaks_measured(dev)
 
     # Settling: the part's power management needs about 30 ms of a new workload to converge (a cold start runs its
     # first steps fast, is throttled below its steady clock for the next ten, and climbs back over twenty more: the scan
     # goes 462, 519, 545, 545, 512, 476 ... 430 (step 14) ... 410 us (step 28)).  The mixer step is therefore repeated,
     # untimed, for --settle-ms before the W warm-up steps; `settle_steps` in the line says how often.
-    settle_steps = 0
+    DOM = 2
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(args.steps)]     # before any GPU work:
+    settle_steps = 0                                                 # creating them later would leave the GPU idle
     if args.settle_ms > 0:
         torch.cuda.synchronize()
         t_settle = time.perf_counter()
-        while (time.perf_counter() - t_settle) * 1e3 < args.settle_ms:
-            mixer.step()
-            settle_steps += 1
-            if settle_steps % 8 == 0:
-                torch.cuda.synchronize()
+        mixer.step()
         torch.cuda.synchronize()
+        est_ms = max((time.perf_counter() - t_settle) * 1e3, 0.05)
+        t_settle = time.perf_counter()
+        mixer.step()
+        torch.cuda.synchronize()
+        est_ms = min(est_ms, max((time.perf_counter() - t_settle) * 1e3, 0.05))
+        settle_steps = 2 + int(min(2000, max(0.0, args.settle_ms / est_ms)))
+        for _ in range(settle_steps - 2):            # queued back to back, no host synchronisation in between
+            mixer.step()
     for _ in range(args.warmup):
         mixer.step()
     torch.cuda.synchronize()
     # The timed region: K steps, with HIP events around the dominant kernel only (the selective scan, position 2..3).
-    # An event between two kernels costs about 7 us of GPU time (the marker waits for the kernel before it and holds the
-    # next one back), so the events around the other three kernels are left to a pass of their own after the timed runs.
-    DOM = 2
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(args.steps)]
-    torch.cuda.synchronize()
+    # An event between two kernels is a marker that waits for the kernel before it, so the events around the other three
+    # kernels are left to a pass of their own after the timed runs.
     t0 = time.perf_counter()
     for i in range(args.steps):
         mixer.step(ev[i], only=(DOM, DOM + 1))
@@ -905,7 +922,9 @@ def main():
         "roofline": roofline,
         "kernels": per_kernel,
     }
-    line["peaks_measured"] = peaks
+    # after the timed runs: a burst of matrix instructions at the power limit right before them depresses the clock of
+    # the steps that follow for longer than the settling phase lasts
+    line["peaks_measured"] = peaks_measured(dev)
     if args.gemm_phase_clocks:
         line["gemm_phase_clocks"] = gemm_phase_clocks(dev, mixer)
     if args.copy_calibration:

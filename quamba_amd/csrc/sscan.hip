@@ -470,6 +470,7 @@ struct PreCfg {
     static constexpr int kStage = T / NSPLIT;              // steps (= bytes per tensor) a lane stages per tile
     static constexpr int kPitch = T + 4;                   // floats per row of per-step values: rows 16-byte
                                                            // aligned, eight rows cover the 32 banks
+    static constexpr int kUzPitch = T + 8;                 // 16-bit (u | z << 8) codes per row: rows 16-byte aligned
     static constexpr int kBcPitch = 2 * kNP + 4;           // floats per step of B | C
     static constexpr int kOutPitch = kCh + 8;              // halves; keeps rows 16-byte aligned
     static constexpr int kBcPieces = (2 * kNP * T / 4 + kThreads - 1) / kThreads;   // dwords of B/C per thread
@@ -479,8 +480,9 @@ template <class Cfg>
 struct PreSmem {
     __attribute__((aligned(16))) float d[Cfg::kCh][Cfg::kPitch];     // step size
     __attribute__((aligned(16))) float du[Cfg::kCh][Cfg::kPitch];    // step size x input
-    float skip[Cfg::kCh][Cfg::kPitch];                               // D x input
-    float gate[Cfg::kCh][Cfg::kPitch];                               // SiLU gate of the step
+    // input and gate codes of a step as they came from memory, u in the low byte and z in the high byte: the lane
+    // that owns the step forms the skip term and looks the gate up itself (two fp32 rows per channel less in LDS)
+    __attribute__((aligned(16))) uint16_t uz[Cfg::kCh][Cfg::kUzPitch];
     __attribute__((aligned(16))) float bc[Cfg::T][Cfg::kBcPitch];    // B (kNP) | C (kNP) of a step, scaled
     __attribute__((aligned(16))) __half out[Cfg::T][Cfg::kOutPitch];
     float gate_table[256];             // SiLU gate per z code (indexed by the raw byte)
@@ -592,7 +594,7 @@ __device__ __forceinline__ void sscan_fwd_pre_body(const QaSScanParams& p, int v
     // Writes the staged tile.  Per step of this lane's share of its channel: step size (bias, softplus), step
     // size x input, skip term and gate - everything the time loop needs that does not depend on the state.
     auto stage = [&](int t0) {
-        float dv[kStage], duv[kStage], sk[kStage], gt[kStage];
+        float dv[kStage], duv[kStage];
 #pragma unroll
         for (int e = 0; e < kStage; ++e) dv[e] = __builtin_fmaf(s_dt, i8_of(r_d[e >> 2], e & 3), db);
         if (softplus) {                  // one uniform branch per tile: the evaluations below overlap
@@ -611,20 +613,19 @@ __device__ __forceinline__ void sscan_fwd_pre_body(const QaSScanParams& p, int v
 #pragma unroll
         for (int e = 0; e < kStage; ++e) {
             // the input scale rides with B and D: (s_B q_B) (dt (s_u q_u)) = ((s_B s_u) q_B) (dt q_u)
-            const float u_q = i8_of(r_u[e >> 2], e & 3);
-            sk[e] = D_u * u_q;
-            duv[e] = dv[e] * u_q;
-            gt[e] = HAS_Z ? sm.gate_table[(r_z[e >> 2] >> (8 * (e & 3))) & 0xffu] : 1.0f;
+            duv[e] = dv[e] * i8_of(r_u[e >> 2], e & 3);
         }
 #pragma unroll
         for (int q = 0; q < kStage / 4; ++q) {
             const int t = slice * kStage + q * 4;
             *reinterpret_cast<float4*>(&sm.d[c_local][t]) = make_float4(dv[q * 4], dv[q * 4 + 1], dv[q * 4 + 2], dv[q * 4 + 3]);
             *reinterpret_cast<float4*>(&sm.du[c_local][t]) = make_float4(duv[q * 4], duv[q * 4 + 1], duv[q * 4 + 2], duv[q * 4 + 3]);
-            *reinterpret_cast<float4*>(&sm.skip[c_local][t]) = make_float4(sk[q * 4], sk[q * 4 + 1], sk[q * 4 + 2], sk[q * 4 + 3]);
-            if constexpr (HAS_Z) {
-                *reinterpret_cast<float4*>(&sm.gate[c_local][t]) = make_float4(gt[q * 4], gt[q * 4 + 1], gt[q * 4 + 2], gt[q * 4 + 3]);
-            }
+            // four steps' codes, interleaved bytewise: (u0 z0 u1 z1) (u2 z2 u3 z3)
+            const uint32_t zw = HAS_Z ? r_z[q] : 0u;
+            uint2 codes;
+            codes.x = __builtin_amdgcn_perm(zw, r_u[q], 0x05010400u);
+            codes.y = __builtin_amdgcn_perm(zw, r_u[q], 0x07030602u);
+            *reinterpret_cast<uint2*>(&sm.uz[c_local][t]) = codes;
         }
 #pragma unroll
         for (int i = 0; i < kBcPieces; ++i) {
@@ -639,7 +640,8 @@ __device__ __forceinline__ void sscan_fwd_pre_body(const QaSScanParams& p, int v
 
     // operands of one group of four steps
     struct Group {
-        float d[4], du[4], B[4][NPL], C[4][NPL], skip, gate;
+        float d[4], du[4], B[4][NPL], C[4][NPL];
+        uint32_t code;                  // of the step this lane owns: u in byte 0, z in byte 1
     };
     auto fetch = [&](Group& o, int tq) {
         const float4 d4 = *reinterpret_cast<const float4*>(&sm.d[c_local][tq * 4]);
@@ -660,8 +662,7 @@ __device__ __forceinline__ void sscan_fwd_pre_body(const QaSScanParams& p, int v
                 o.C[j][0] = Cv.x; o.C[j][1] = Cv.y; o.C[j][2] = Cv.z; o.C[j][3] = Cv.w;
             }
         }
-        o.skip = sm.skip[c_local][tq * 4 + qslice];
-        o.gate = HAS_Z ? sm.gate[c_local][tq * 4 + qslice] : 1.0f;
+        o.code = sm.uz[c_local][tq * 4 + qslice];
     };
 
     const int n_tiles = (L + T - 1) / T;
@@ -690,6 +691,9 @@ __device__ __forceinline__ void sscan_fwd_pre_body(const QaSScanParams& p, int v
             // keep the reads of the next group ahead of this group's arithmetic (the scheduler would sink them
             // to their first use, and a wave would then wait for LDS once per group)
             __builtin_amdgcn_sched_barrier(0);
+            // the gate of the step this lane owns: looked up now, used when the group's sums are complete
+            float gate = 1.0f;
+            if constexpr (HAS_Z) gate = sm.gate_table[(o.code >> 8) & 0xffu];
             float acc[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -710,8 +714,8 @@ __device__ __forceinline__ void sscan_fwd_pre_body(const QaSScanParams& p, int v
             // eight lanes per channel: the other quad holds the other half of the states (both quads then hold
             // the same sums and store the same values)
             if constexpr (NSPLIT == 8) own_sum += __shfl_xor(own_sum, 4);
-            float y = own_sum + o.skip;
-            if constexpr (HAS_Z) y *= o.gate;
+            float y = own_sum + D_u * code_byte_to_float(o.code, 0);
+            if constexpr (HAS_Z) y *= gate;
             sm.out[tq * 4 + qslice][c_local] = __float2half(y);
         }
         __syncthreads();   // out complete; everyone is done reading the staged tile
