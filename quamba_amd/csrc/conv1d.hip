@@ -12,6 +12,7 @@
 // causal halo comes from one extra aligned dword, and the four taps are one packed int8 dot
 // product (exact, so equal to the reference's fp32 accumulation of integer products).
 #include "conv_common.hpp"
+#include <type_traits>
 
 namespace qa {
 namespace {
@@ -20,26 +21,24 @@ constexpr int kConvThreads = 256;
 
 // One thread = 16 consecutive time steps of one (batch, channel) row.  Rows are 16-byte aligned
 // (checked on the host); a ragged tail (seqlen % 16) is handled bytewise by the row's last thread.
-template <bool SILU, int PIECES>
+template <bool SILU, int PIECES, bool BATCH_INNER>
 __global__ __launch_bounds__(kConvThreads) void conv_fwd_rows_kernel(QaConvParams p, int segs) {
     // grid: x over runs of PIECES * 64 segments of a row (one wave each), y over groups of four channels
     // (one per wave), z = batch: no integer division on the way in, and the channel is the same for a
     // whole wave, so its taps and bias are fetched and packed once per wave by scalar instructions.
     // A lane takes segment 64*k + lane of its wave's run, k < PIECES: every load of a wave is 1 KB in one piece.
-    const int c = __builtin_amdgcn_readfirstlane(static_cast<int>(blockIdx.y * 4 + (threadIdx.x >> 6)));
-    const int b = blockIdx.z;
+    // BATCH_INNER, for buffers in which the batch entries of one channel lie next to each other (the layout
+    // in_proj writes): y over groups of four batch entries (one per wave), z = channel, so that the workgroups
+    // sweep the buffer from one end to the other in the order they are dispatched.
+    const int mine = __builtin_amdgcn_readfirstlane(static_cast<int>(blockIdx.y * 4 + (threadIdx.x >> 6)));
+    const int c = BATCH_INNER ? static_cast<int>(blockIdx.z) : mine;
+    const int b = BATCH_INNER ? mine : static_cast<int>(blockIdx.z);
     const int seg0 = blockIdx.x * (64 * PIECES) + (threadIdx.x & 63);
-    if (c >= p.dim || seg0 >= segs) return;
+    if (c >= p.dim || b >= p.batch || seg0 >= segs) return;
     const int8_t* x = p.x + b * p.x_batch_stride + c * p.x_c_stride;
     int8_t* out = p.out + b * p.out_batch_stride + c * p.out_c_stride;
 
-    const uint32_t taps = pack_taps(p.weight + c * p.weight_c_stride, p.weight_width_stride, p.width);
-    const float s_wx = p.scale_w * p.scale_x;
-    const float bias_f = p.bias ? static_cast<float>(p.bias[c]) * p.scale_b : 0.0f;
-    const float inv_s_out = 1.0f / p.scale_out;
-    const bool exact_only = conv_needs_exact_route(p.scale_out);
-    const ConvQuantRegs kq;
-
+    // the row's bytes are requested first; taps, bias and scales arrive while they travel
     uint32_t w[PIECES][5];   // w[k][0] = x[t0-4 .. t0-1], w[k][1..4] = x[t0 .. t0+15]
 #pragma unroll
     for (int k = 0; k < PIECES; ++k) {
@@ -58,6 +57,24 @@ __global__ __launch_bounds__(kConvThreads) void conv_fwd_rows_kernel(QaConvParam
             }
         }
     }
+    // Taps and bias of the wave's channel: one scalar load each when the four taps are an aligned word and the
+    // bias vector consists of whole aligned words (the usual case), else byte by byte.
+    const int8_t* taps_at = p.weight + c * p.weight_c_stride;
+    uint32_t taps;
+    if (p.width == 4 && p.weight_width_stride == 1 && aligned4(taps_at)) taps = *reinterpret_cast<const uint32_t*>(taps_at);
+    else taps = pack_taps(taps_at, p.weight_width_stride, p.width);
+    float bias_f = 0.0f;
+    if (p.bias) {
+        int bias_q;
+        if (aligned4(p.bias) && (p.dim & 3) == 0)
+            bias_q = static_cast<int8_t>(reinterpret_cast<const uint32_t*>(p.bias)[c >> 2] >> (8 * (c & 3)));
+        else bias_q = p.bias[c];
+        bias_f = static_cast<float>(bias_q) * p.scale_b;
+    }
+    const float s_wx = p.scale_w * p.scale_x;
+    const float inv_s_out = 1.0f / p.scale_out;
+    const bool exact_only = conv_needs_exact_route(p.scale_out);
+    const ConvQuantRegs kq(p.scale_out);
 #pragma unroll
     for (int k = 0; k < PIECES; ++k) {
         const int seg = seg0 + 64 * k;
@@ -111,7 +128,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_fwd_rows_dual_kernel(QaConv
         const float bias_f = p.bias ? static_cast<float>(p.bias[c]) * p.scale_b : 0.0f;
         const float inv_s_out = 1.0f / p.scale_out;
     const bool exact_only = conv_needs_exact_route(p.scale_out);
-    const ConvQuantRegs kq;
+    const ConvQuantRegs kq(p.scale_out);
         uint32_t w[5];   // w[0] = x[t0-4 .. t0-1], w[1..4] = x[t0 .. t0+15]
         w[0] = t0 > 0 ? *reinterpret_cast<const uint32_t*>(x + t0 - 4) : 0u;
         if (remaining >= 16) {
@@ -248,11 +265,22 @@ extern "C" int qa_causal_conv1d_fwd(const QaConvParams* p, void* stream_) {
             if (groups > 65535 || p->batch > 65535) return QA_ERR_SHAPE;
             // two segments per lane once a row has at least 128 of them (2048 steps)
             const int pieces = segs >= 128 ? 2 : 1;
-            const dim3 grid(static_cast<unsigned>((segs + 64 * pieces - 1) / (64 * pieces)), static_cast<unsigned>(groups),
-                            static_cast<unsigned>(p->batch));
+            const unsigned runs = static_cast<unsigned>((segs + 64 * pieces - 1) / (64 * pieces));
+            // the batch entries of a channel next to each other, in input and output, and enough of them for a workgroup
+            const bool batch_inner = p->batch >= 4 && p->dim <= 65535 && p->x_batch_stride < p->x_c_stride &&
+                                     p->out_batch_stride < p->out_c_stride;
+            const dim3 grid = batch_inner ? dim3(runs, static_cast<unsigned>((p->batch + 3) / 4), static_cast<unsigned>(p->dim))
+                                          : dim3(runs, static_cast<unsigned>(groups), static_cast<unsigned>(p->batch));
             auto go = [&](auto kernel) { hipLaunchKernelGGL(kernel, grid, dim3(kConvThreads), 0, stream, *p, segs); };
-            if (pieces == 2) p->silu_activation ? go(conv_fwd_rows_kernel<true, 2>) : go(conv_fwd_rows_kernel<false, 2>);
-            else p->silu_activation ? go(conv_fwd_rows_kernel<true, 1>) : go(conv_fwd_rows_kernel<false, 1>);
+            auto pick = [&](auto silu, auto pcs) {
+                constexpr bool S = decltype(silu)::value;
+                constexpr int P = decltype(pcs)::value;
+                batch_inner ? go(conv_fwd_rows_kernel<S, P, true>) : go(conv_fwd_rows_kernel<S, P, false>);
+            };
+            using T = std::true_type; using F = std::false_type;
+            using P1 = std::integral_constant<int, 1>; using P2 = std::integral_constant<int, 2>;
+            if (pieces == 2) p->silu_activation ? pick(T{}, P2{}) : pick(F{}, P2{});
+            else p->silu_activation ? pick(T{}, P1{}) : pick(F{}, P1{});
             return check_launch();
         }
     }

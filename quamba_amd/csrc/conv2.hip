@@ -100,7 +100,6 @@ __global__ __launch_bounds__(kThreads) void conv2_fwd_kernel(QaConv2Params p) {
     uint32_t taps[4];
     float bias_f[4], s_out[4], inv_s_out[4];
     bool exact_only[4];
-    const ConvQuantRegs kq;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         const int ch = ch0 + e;
@@ -110,6 +109,7 @@ __global__ __launch_bounds__(kThreads) void conv2_fwd_kernel(QaConv2Params p) {
         inv_s_out[e] = 1.0f / s_out[e];
         exact_only[e] = conv_needs_exact_route(s_out[e]);
     }
+    const ConvQuantRegs kq(__builtin_fminf(__builtin_fminf(s_out[0], s_out[1]), __builtin_fminf(s_out[2], s_out[3])));
     int64_t out_ls, out_cs;
     int8_t* out = out_ptr(p, part, b, ch0, &out_ls, &out_cs);
     const int8_t* src = p.xBC + b * p.xBC_batch_stride + ch0;
@@ -145,14 +145,10 @@ __global__ __launch_bounds__(kThreads) void conv2_fwd_kernel(QaConv2Params p) {
         for (int i = 0; i < kBatchLoads; ++i) {
             if (tb + i >= t_end) break;
             push(d[i]);
-            uint32_t r[4];
+            float v[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const float acc = static_cast<float>(dot4(win[e], taps[e]));
-                const float v = __builtin_fmaf(part.s_in, acc, bias_f[e]);
-                r[e] = conv_quant_bits(v, s_out[e], inv_s_out[e], p.silu_activation, exact_only[e], kq);
-            }
-            *reinterpret_cast<uint32_t*>(out + (tb + i) * out_ls) = pack_low_bytes(r[0], r[1], r[2], r[3]);
+            for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaf(part.s_in, static_cast<float>(dot4(win[e], taps[e])), bias_f[e]);
+            *reinterpret_cast<uint32_t*>(out + (tb + i) * out_ls) = conv_quant4(v, s_out, inv_s_out, p.silu_activation, exact_only, kq);
         }
     }
 }

@@ -11,80 +11,106 @@ __device__ __forceinline__ int8_t conv_epilogue(float v, float s_out, int silu) 
     return sat8_half_away(v / s_out);
 }
 
-// Requantised output by the cheap route (hardware exp2 / rcp, multiply by 1/s_out, round to nearest)
-// whenever that provably equals the exact route, else by the exact route.  The cheap value y differs
-// from the exactly-evaluated one by less than 3.3e-4 for |y| < 129 and v >= -16: the exponent argument
-// v * log2(e) is rounded twice (a relative error of 1e-7 |v| in the exponential), exp2, rcp and the exact
-// route's own steps are each within 1-1.5 ulp, together below 2.5e-6 relative.  So if y is further than
-// 5e-4 from every half-integer both round to the same integer (a margin proportional to |y| was tried
-// and measured no faster).  y is clamped to +-128.75 first: beyond that both routes saturate, and the
-// clamped value (a quarter away from 129) passes the test on its own.  For v < -16 the bound no longer
-// holds, but there |y| < 1.8e-6 / s_out: with s_out >= 1e-5 both routes give zero, and for smaller
-// output scales the caller sets `exact_only` and every lane takes the exact route.
-// A wave takes the exact route whenever one of its 64 lanes does, which is why the margin is kept as
-// narrow as the error bound allows (at 2e-3, 0.4 % of the lanes, a quarter of all wave-elements went
-// through the exact route's ~100 instructions).
+// Requantised output by the cheap route (hardware exp2 / rcp, round to nearest) whenever that provably equals the
+// exact route, else by the exact route.  The cheap route forms y = v / (s_out (1 + E)), E = 2^(-v log2 e), with one
+// reciprocal: SiLU and the division by the output scale share it.  Relative to the true value, for v >= -16:
+//   cheap route: E carries 7.3e-8 |v| (its argument is rounded twice) + 1.2e-7 (exp2, 1 ulp), which enters 1 + E with
+//                the weight E / (1 + E); then 6e-8 (fused multiply-add), 1.2e-7 (rcp, 1 ulp), 6e-8 (product);
+//   exact route: 1.8e-7 (exp_det, 1.5 ulp) with the same weight; then 6e-8 each for the sum and the two divisions.
+// v >= 0: the weight is at most one half and |v| E / (1 + E) <= 0.28, so the two routes differ by less than 5.9e-7 |y|,
+//         7.6e-5 for |y| <= 128.25.
+// v <  0: they differ by less than (7.3e-8 |v| + 7.2e-7) |y| and |y| = |v| / (s_out (1 + e^|v|)); the product of the
+//         two is at most 2.3e-7 / s_out: 9.2e-5 for s_out >= 2.5e-3.  For smaller output scales |y| can reach 128 at
+//         v = -16, where the difference is below 2.6e-6 |y| = 3.3e-4.
+// So if y is further than the margin - 1.25e-4 for s_out >= 2.5e-3, 5e-4 below - from every half-integer, both
+// routes round to the same integer.  y is clamped to [-128.25, 127.25] first: beyond +-127.5 / -128.5 both routes
+// saturate to the same code whatever side of the half-integer they fall on, and the clamped value (a quarter away
+// from a half-integer) passes the test on its own.  For v < -16 the bounds no longer hold, but there
+// |y| < 1.8e-6 / s_out: with s_out >= 1e-5 both routes give zero, and for smaller output scales the caller sets
+// `exact_only` and every lane takes the exact route.
+// A wave takes the exact route's ~100 instructions for an output whenever one of its 64 lanes needs it, which is
+// why the margin is kept as narrow as the bounds allow: at 5e-4 a wave does so for 6 % of its outputs, a third of
+// the kernel's vector instructions; at 1.25e-4 for 1.6 %.
 __device__ __forceinline__ bool conv_needs_exact_route(float s_out) { return !(s_out >= 1e-5f); }
+__device__ __forceinline__ float conv_cheap_margin(float s_out) { return s_out >= 2.5e-3f ? 1.25e-4f : 5e-4f; }
 
 // The constants of the cheap route, held in registers for the life of the thread.  They are not values an
 // instruction can carry inline, and the compiler would otherwise load each of them into a register again for
-// every output (three extra instructions on a path of under thirty).
+// every output (three extra instructions on a path of under thirty).  `smallest_s_out`: the smallest output scale
+// the thread will requantise with.
 struct ConvQuantRegs {
-    float clamp_hi, magic;
-    __device__ __forceinline__ ConvQuantRegs() {
+    float clamp_hi, magic, margin;
+    __device__ __forceinline__ explicit ConvQuantRegs(float smallest_s_out) : margin(conv_cheap_margin(smallest_s_out)) {
         asm volatile("v_mov_b32 %0, 0x42fe8000" : "=v"(clamp_hi));     // 127.25
         asm volatile("v_mov_b32 %0, 0x4b400000" : "=v"(magic));        // 1.5 * 2^23
     }
 };
 
-// Returns a word whose low byte is the int8 code (the bytes above it are not meaningful).
-// y is clamped to [-128.25, 127.25] first: beyond +-127.5 / -128.5 both routes saturate to the same code whatever
-// side of the half-integer they fall on, and the clamped value (a quarter away from a half-integer) passes the
-// distance test on its own.  Adding 1.5 * 2^23 rounds to the nearest integer in the addition itself (ties to
-// even; ties are not decided here) and leaves that integer's two's-complement byte in the low 8 bits of the sum.
-// the low bytes of four words, in order
-__device__ __forceinline__ uint32_t pack_low_bytes(uint32_t b0, uint32_t b1, uint32_t b2, uint32_t b3) {
-    const uint32_t lo = __builtin_amdgcn_perm(b1, b0, 0x0c0c0400u);      // bytes: b0.0, b1.0, 0, 0
-    const uint32_t hi = __builtin_amdgcn_perm(b3, b2, 0x0c0c0400u);
-    return __builtin_amdgcn_perm(hi, lo, 0x05040100u);                   // lo.0, lo.1, hi.0, hi.1
-}
-
-// The cheap route alone: the word with the code in its low byte, and whether the exact route must decide instead.
-__device__ __forceinline__ uint32_t conv_quant_cheap(float v, float inv_s_out, int silu, const ConvQuantRegs& k, bool& undecided) {
-    float y = v;
+// The cheap route's value in units of the output code, clamped.
+__device__ __forceinline__ float conv_cheap_units(float v, float s_out, float inv_s_out, int silu, const ConvQuantRegs& k) {
+    float y;
     if (silu) {
         const float e = __builtin_amdgcn_exp2f(v * -1.44269504088896341f);
-        y = v * __builtin_amdgcn_rcpf(1.0f + e);
+        y = v * __builtin_amdgcn_rcpf(__builtin_fmaf(e, s_out, s_out));
+    } else {
+        y = v * inv_s_out;
     }
-    y = __builtin_amdgcn_fmed3f(y * inv_s_out, -128.25f, k.clamp_hi);
-    const float t = y + k.magic;
-    const float d = __builtin_fabsf(y - (t - k.magic));
-    undecided = !(d <= 0.4995f);
-    return __float_as_uint(t);
+    return __builtin_amdgcn_fmed3f(y, -128.25f, k.clamp_hi);
 }
+// Signed distance of y's fractional part from one half (exact for the values that matter: the fraction of |y| < 129
+// is exact, and so is the subtraction for fractions of a quarter and more); the cheap route decides when its
+// magnitude is at least the margin.
+__device__ __forceinline__ float conv_cheap_off_half(float y) { return __builtin_amdgcn_fractf(y) - 0.5f; }
 
+// One output: a word whose low byte is the int8 code (the bytes above it are not meaningful).  Adding 1.5 * 2^23
+// rounds to the nearest integer in the addition itself (ties to even; ties are not decided here) and leaves that
+// integer's two's-complement byte in the low 8 bits of the sum.
 __device__ __forceinline__ uint32_t conv_quant_bits(float v, float s_out, float inv_s_out, int silu, bool exact_only,
                                                    const ConvQuantRegs& k) {
-    bool undecided;
-    uint32_t q = conv_quant_cheap(v, inv_s_out, silu, k, undecided);
-    if (exact_only || undecided) q = static_cast<uint32_t>(static_cast<uint8_t>(conv_epilogue(v, s_out, silu)));
+    const float y = conv_cheap_units(v, s_out, inv_s_out, silu, k);
+    uint32_t q = __float_as_uint(y + k.magic);
+    if (exact_only || !(__builtin_fabsf(conv_cheap_off_half(y)) >= k.margin))
+        q = static_cast<uint32_t>(static_cast<uint8_t>(conv_epilogue(v, s_out, silu)));
     return q;
 }
 
-// Four outputs at once: the four cheap evaluations are independent and interleave (each is a chain of dependent
-// instructions with two transcendentals), then every output that the cheap route could not decide - rare, so the
-// branch around each is almost never taken - goes through the exact route on its own.
+// Four outputs at once, as the four bytes of a word: the four cheap evaluations are independent and interleave (each
+// is a chain of dependent instructions with two transcendentals); the rounding additions of the second to fourth
+// output write their low byte straight into its place (sub-dword destination select, the other bytes preserved), so
+// nothing is spent on packing; one comparison on the smallest of the four distances decides whether any output goes
+// through the exact route - rare, so the branch is almost never taken.
+__device__ __forceinline__ uint32_t conv_quant4(const float (&v)[4], const float (&s_out)[4], const float (&inv_s_out)[4], int silu,
+                                               const bool (&exact_only)[4], const ConvQuantRegs& k) {
+    float y[4], off[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) y[j] = conv_cheap_units(v[j], s_out[j], inv_s_out[j], silu, k);
+    uint32_t word = __float_as_uint(y[0] + k.magic);                     // byte 0; bytes 1..3 replaced below
+    asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(word) : "v"(y[1]), "v"(k.magic));
+    asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(word) : "v"(y[2]), "v"(k.magic));
+    asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(word) : "v"(y[3]), "v"(k.magic));
+#pragma unroll
+    for (int j = 0; j < 4; ++j) off[j] = conv_cheap_off_half(y[j]);
+    float nearest;                                                       // min |off[j]|: two instructions
+    asm("v_min3_f32 %0, |%1|, |%2|, |%3|" : "=v"(nearest) : "v"(off[0]), "v"(off[1]), "v"(off[2]));
+    asm("v_min_f32_e64 %0, %1, |%2|" : "=v"(nearest) : "v"(nearest), "v"(off[3]));
+    const bool any_exact = exact_only[0] || exact_only[1] || exact_only[2] || exact_only[3];
+    if (any_exact || !(nearest >= k.margin)) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (exact_only[j] || !(__builtin_fabsf(off[j]) >= k.margin)) {
+                const uint32_t code = static_cast<uint8_t>(conv_epilogue(v[j], s_out[j], silu));
+                word = (word & ~(0xffu << (8 * j))) | (code << (8 * j));
+            }
+        }
+    }
+    return word;
+}
+// the same with one output scale for the four
 __device__ __forceinline__ uint32_t conv_quant4(const float (&v)[4], float s_out, float inv_s_out, int silu, bool exact_only,
                                                const ConvQuantRegs& k) {
-    uint32_t q[4];
-    bool undecided[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) q[j] = conv_quant_cheap(v[j], inv_s_out, silu, k, undecided[j]);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        if (exact_only || undecided[j]) q[j] = static_cast<uint32_t>(static_cast<uint8_t>(conv_epilogue(v[j], s_out, silu)));
-    }
-    return pack_low_bytes(q[0], q[1], q[2], q[3]);
+    const float s[4] = {s_out, s_out, s_out, s_out}, inv[4] = {inv_s_out, inv_s_out, inv_s_out, inv_s_out};
+    const bool ex[4] = {exact_only, exact_only, exact_only, exact_only};
+    return conv_quant4(v, s, inv, silu, ex, k);
 }
 
 __device__ __forceinline__ int conv_quant(float v, float s_out, float inv_s_out, int silu, bool exact_only,
@@ -104,8 +130,11 @@ __device__ __forceinline__ uint32_t pack_taps(const int8_t* w, int64_t wstride, 
     return packed;
 }
 
+// Asked for with the clamp flag (saturation of the 32-bit sum, which four products of bytes never reach): that
+// selects the three-operand form with a literal zero as the addend; without it the compiler picks the accumulating
+// two-operand form, which costs a register clear per product.
 __device__ __forceinline__ int dot4(uint32_t a, uint32_t b) {
-    return __builtin_amdgcn_sdot4(static_cast<int>(a), static_cast<int>(b), 0, false);
+    return __builtin_amdgcn_sdot4(static_cast<int>(a), static_cast<int>(b), 0, true);
 }
 
 // One decode step of channel c of batch entry b (quant_causal_conv1d_update_kernel.cuh:34-75): the conv state moves
@@ -138,7 +167,7 @@ __device__ __forceinline__ int8_t conv_step_row(const QaConvParams& p, int b, in
         float v = p.bias ? static_cast<float>(bias_q) * p.scale_b : 0.0f;
 #pragma unroll
         for (int i = 0; i < 4; ++i) v = __builtin_fmaf(s_wx * static_cast<float>(ws[i]), static_cast<float>(xs[i]), v);
-        const ConvQuantRegs kq;
+        const ConvQuantRegs kq(p.scale_out);
         const int8_t q = static_cast<int8_t>(conv_quant(v, p.scale_out, 1.0f / p.scale_out, p.silu_activation,
                                                         conv_needs_exact_route(p.scale_out), kq));
         if (store && p.out) p.out[b * p.out_batch_stride + c * p.out_c_stride] = q;
@@ -171,7 +200,7 @@ __device__ __forceinline__ int8_t conv_step_row(const QaConvParams& p, int b, in
     const float s_wx = p.scale_w * p.scale_x;
     float v = bias_f;
     for (int i = 0; i < width; ++i) v = __builtin_fmaf(s_wx * static_cast<float>(ws[i]), static_cast<float>(xs[i]), v);
-    const ConvQuantRegs kq;
+    const ConvQuantRegs kq(p.scale_out);
     const int8_t q = static_cast<int8_t>(conv_quant(v, p.scale_out, 1.0f / p.scale_out, p.silu_activation,
                                                     conv_needs_exact_route(p.scale_out), kq));
     if (store && p.out) p.out[b * p.out_batch_stride + c * p.out_c_stride] = q;

@@ -52,6 +52,27 @@ def test_fwd_bit_exact_over_wide_ranges_of_the_pre_activation(dev, s_in, s_out):
     np.testing.assert_array_equal(got.cpu().numpy(), want)
 
 
+@pytest.mark.parametrize("s_out", [0.1, 0.03, 0.0031, 0.0025, 0.0024, 0.0007])
+def test_fwd_bit_exact_with_unsaturated_outputs_on_both_sides_of_the_margin_switch(dev, s_out):
+    """Small taps keep the accumulator within +-4100, and the input scale is chosen so that the requantised value
+    spans about +-150 codes: nearly all of the two million outputs are unsaturated, with up to a million distinct
+    pre-activation values, so thousands of them fall inside the fast epilogue's rounding margin and next to it.  The
+    output scales straddle 2.5e-3, where the margin changes from 1.25e-4 to 5e-4 of a code."""
+    g = np.random.default_rng(int(s_out * 1e5) + 3)
+    B, D, L = 2, 256, 4096
+    qx = g.integers(-128, 128, (B, D, L)).astype(np.int8)
+    qw = g.integers(-8, 9, (D, 4)).astype(np.int8)
+    qb = g.integers(-128, 128, D).astype(np.int8)
+    sw = 0.01
+    s_in = 150.0 * s_out / (4100 * sw)
+    sb = 20.0 * s_out / 128
+    for silu in (True, False):
+        want = oracle.conv1d_fwd(qx, qw, qb, s_in, sw, sb, s_out, silu=silu)
+        assert np.mean(np.abs(want.astype(np.int32)) < 127) > 0.9
+        got = ops.causal_conv1d_fwd(_t(qx, dev), s_in, _t(qw, dev), sw, s_out, sb, _t(qb, dev), None, None, None, silu)
+        np.testing.assert_array_equal(got.cpu().numpy(), want)
+
+
 def test_fwd_no_bias(dev):
     qx, sx, qw, sw, qb, sb, so = _case(2, 128, 256, 4, seed=5, bias=False)
     want = oracle.conv1d_fwd(qx, qw, None, sx, sw, sb, so)
