@@ -410,6 +410,7 @@ struct ScanSmem {
     __attribute__((aligned(16))) float gk[Q];   // exp(dA[end of the 32-step piece] - dA_k) dt_k
     __attribute__((aligned(16))) float xs[kP];  // x scale per channel
     __attribute__((aligned(16))) float Dv[kP];  // skip weight per channel
+    __attribute__((aligned(16))) float gate[256];   // SiLU(z_scale code) of the gate's 256 codes, indexed by the code's byte
     static_assert(!ALIAS || sizeof(_Float16) * kP * N == static_cast<size_t>(Q / 2) * N, "the upper B rows take exactly the state's place");
     // row k of the B codes
     __device__ __forceinline__ int8_t* brow(int k) {
@@ -522,6 +523,13 @@ __global__ __launch_bounds__(64 * scan_waves_of(Q), 4) void ssd_chunk_scan_kerne
             sm.xs[tid] = x_scale_of(p, g, hg, tid);
             sm.Dv[tid] = !p.D ? 0.0f : D_scale * static_cast<float>(p.D_has_hdim ? p.D[h * kP + tid] : p.D[h]);
         }
+        if (p.z) {
+            // the gate has 256 possible values: evaluated once per workgroup, looked up per output
+            for (int i = tid; i < 256; i += kThreads) {
+                const float zv = z_scale * static_cast<float>(static_cast<int8_t>(i));
+                sm.gate[i] = zv * __builtin_amdgcn_rcpf(1.0f + fexp(-zv));
+            }
+        }
         __syncthreads();                                           // the tables per channel (and every load above has landed)
 
         if (tid < Q) {
@@ -631,12 +639,12 @@ __global__ __launch_bounds__(64 * scan_waves_of(Q), 4) void ssd_chunk_scan_kerne
                 }
                 float cv[8];
 #pragma unroll
-                for (int e = 0; e < 8; ++e) cv[e] = cb_scale * static_cast<float>(cbi[e / 4][e % 4]);
+                for (int e = 0; e < 8; ++e) cv[e] = static_cast<float>(cbi[e / 4][e % 4]);
                 float wv[8];
                 if (ks + 1 < nks) {
                     const float4 g0 = *reinterpret_cast<const float4*>(&sm.gk[ka]), g1 = *reinterpret_cast<const float4*>(&sm.gk[ka + 16]);
                     const float gk[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
-                    const float e_m = fexp(dA_m - sm.dA[32 * ks + 31]);
+                    const float e_m = cb_scale * fexp(dA_m - sm.dA[32 * ks + 31]);      // the scale of C B^T rides with the row's decay
 #pragma unroll
                     for (int e = 0; e < 8; ++e) wv[e] = cv[e] * (e_m * gk[e]);
                 } else {
@@ -648,7 +656,7 @@ __global__ __launch_bounds__(64 * scan_waves_of(Q), 4) void ssd_chunk_scan_kerne
 #pragma unroll
                     for (int e = 0; e < 8; ++e) {
                         const int k = ka + 16 * (e / 4) + e % 4;
-                        wv[e] = ((k <= m_row ? cv[e] : 0.0f) * fexp(fminf(dA_m - ak[e], 0.0f))) * dk[e];
+                        wv[e] = ((k <= m_row ? cb_scale * cv[e] : 0.0f) * fexp(fminf(dA_m - ak[e], 0.0f))) * dk[e];
                     }
                 }
                 v8h fl;
@@ -671,10 +679,7 @@ __global__ __launch_bounds__(64 * scan_waves_of(Q), 4) void ssd_chunk_scan_kerne
                 }
                 if (p.z) {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const float zv = z_scale * static_cast<float>(byte_of(zq[r], j));
-                        y[j] *= zv * __builtin_amdgcn_rcpf(1.0f + fexp(-zv));
-                    }
+                    for (int j = 0; j < 4; ++j) y[j] *= sm.gate[(zq[r] >> (8 * j)) & 0xffu];
                 }
                 v4h o;
 #pragma unroll
