@@ -559,11 +559,6 @@ __device__ __forceinline__ void sscan_fwd_pre_body(const QaSScanParams& p, int v
     const int8_t* u_row = p.u + b * p.u_batch_stride + static_cast<int64_t>(cc) * p.u_d_stride;
     const int8_t* d_row = p.delta + b * p.delta_batch_stride + static_cast<int64_t>(cc) * p.delta_d_stride;
     const int8_t* z_row = HAS_Z ? p.z + b * p.z_batch_stride + static_cast<int64_t>(cc) * p.z_d_stride : nullptr;
-    const int8_t* bc_base[2] = {p.B + b * p.B_batch_stride + g * p.B_group_stride,
-                                p.C + b * p.C_batch_stride + g * p.C_group_stride};
-    const int64_t bc_nstride[2] = {p.B_dstate_stride, p.C_dstate_stride};
-    const float bc_scale[2] = {s_B * s_u, s_C};
-
     uint32_t r_u[kStage / 4], r_d[kStage / 4], r_z[kStage / 4];
     uint32_t r_bc[kBcPieces];
 
@@ -574,20 +569,62 @@ __device__ __forceinline__ void sscan_fwd_pre_body(const QaSScanParams& p, int v
         n = piece % kNP;
         col = (piece / kNP) % (T / 4);
     };
+    // this thread's dwords of a tile's B / C codes: the row they come from (states beyond d_state read the last state's
+    // row and are scaled by zero) and the scale they are staged with
+    const int8_t* bc_row[kBcPieces];
+    float bc_factor[kBcPieces];
+#pragma unroll
+    for (int i = 0; i < kBcPieces; ++i) {
+        int which, n, col;
+        bc_piece(tid + i * kThreads, which, n, col);
+        const int nn = min(n, p.dstate - 1);
+        const int8_t* rowB = p.B + b * p.B_batch_stride + g * p.B_group_stride + nn * p.B_dstate_stride;
+        const int8_t* rowC = p.C + b * p.C_batch_stride + g * p.C_group_stride + nn * p.C_dstate_stride;
+        bc_row[i] = which ? rowC : rowB;
+        bc_factor[i] = n < p.dstate ? (which ? s_C : s_B * s_u) : 0.0f;
+    }
 
+    // A tile that lies inside the sequence, of rows that allow vector loads, is requested without a branch per lane: the
+    // requests then stay in flight until stage() needs them.  (With the byte-wise alternative in the same control
+    // flow the compiler waits for every request where the two paths join.)
     auto issue_loads = [&](int t0) {
         const int t = t0 + slice * kStage;
+        const bool whole = t0 + T <= L;
         // rows past the last channel read the last channel's bytes; nothing of theirs is stored
-        load_bytes<kStage>(r_u, u_row, t, L, vec_in);
-        load_bytes<kStage>(r_d, d_row, t, L, vec_in);
-        if constexpr (HAS_Z) load_bytes<kStage>(r_z, z_row, t, L, vec_in);
+        if (vec_in && whole) {
+            if constexpr (kStage == 8) {
+                const uint2 vu = *reinterpret_cast<const uint2*>(u_row + t), vd = *reinterpret_cast<const uint2*>(d_row + t);
+                r_u[0] = vu.x; r_u[1] = vu.y; r_d[0] = vd.x; r_d[1] = vd.y;
+                if constexpr (HAS_Z) {
+                    const uint2 vz = *reinterpret_cast<const uint2*>(z_row + t);
+                    r_z[0] = vz.x; r_z[1] = vz.y;
+                }
+            } else {
+                r_u[0] = *reinterpret_cast<const uint32_t*>(u_row + t);
+                r_d[0] = *reinterpret_cast<const uint32_t*>(d_row + t);
+                if constexpr (HAS_Z) r_z[0] = *reinterpret_cast<const uint32_t*>(z_row + t);
+            }
+        } else {
+            load_bytes<kStage>(r_u, u_row, t, L, false);
+            load_bytes<kStage>(r_d, d_row, t, L, false);
+            if constexpr (HAS_Z) load_bytes<kStage>(r_z, z_row, t, L, false);
+        }
+        if (vec_bc && whole) {
 #pragma unroll
-        for (int i = 0; i < kBcPieces; ++i) {
-            int which, n, col;
-            bc_piece(tid + i * kThreads, which, n, col);
-            uint32_t v[1] = {0u};
-            if (which < 2 && n < p.dstate) load_bytes<4>(v, bc_base[which] + n * bc_nstride[which], t0 + col * 4, L, vec_bc);
-            r_bc[i] = v[0];
+            for (int i = 0; i < kBcPieces; ++i) {
+                int which, n, col;
+                bc_piece(tid + i * kThreads, which, n, col);
+                r_bc[i] = *reinterpret_cast<const uint32_t*>(bc_row[i] + t0 + col * 4);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < kBcPieces; ++i) {
+                int which, n, col;
+                bc_piece(tid + i * kThreads, which, n, col);
+                uint32_t v[1];
+                load_bytes<4>(v, bc_row[i], t0 + col * 4, L, false);
+                r_bc[i] = v[0];
+            }
         }
     };
 
@@ -631,10 +668,8 @@ __device__ __forceinline__ void sscan_fwd_pre_body(const QaSScanParams& p, int v
         for (int i = 0; i < kBcPieces; ++i) {
             int which, n, col;
             bc_piece(tid + i * kThreads, which, n, col);
-            if (which < 2) {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) sm.bc[col * 4 + e][which * kNP + n] = bc_scale[which] * i8_of(r_bc[i], e);
-            }
+            for (int e = 0; e < 4; ++e) sm.bc[col * 4 + e][which * kNP + n] = bc_factor[i] * i8_of(r_bc[i], e);
         }
     };
 
