@@ -235,41 +235,41 @@ __global__ __launch_bounds__(256, 3) void ssd_state_kernel(QaSsdParams p, const 
     if (tid < kP) sm.xs[tid] = x_scale_of(p, g, hg, tid);
     uint4 xr[4], br[4];
     float r_dt = 0.0f, r_dA = 0.0f, r_last = 0.0f;
+    int valid_loaded = Q;                                         // steps of the chunk whose tiles are in xr / br
+    // One path for whole and ragged chunks: rows past the end of the sequence read the last row (the loads stay inside
+    // the tensors) and are zeroed when the chunk is staged.  With a second, ragged path beside it the compiler merges
+    // the two sets of destination registers by copies right behind the loads, i.e. waits for them where they are issued.
     auto load_chunk = [&](int c) {
         const int t0 = c * Q;
         const int valid = min(Q, L - t0);
+        valid_loaded = valid;
         // uniform row addresses plus one per-thread offset: the address arithmetic stays in scalar registers
         const int8_t* xsrc = p.x + (static_cast<int64_t>(b) * L + t0) * xrow + static_cast<int64_t>(h) * kP;
         const int8_t* bsrc = p.B + (static_cast<int64_t>(b) * L + t0) * brow + static_cast<int64_t>(g) * N + part * 64;
         if (mine) {
-            if (valid == Q) {
+            const uint32_t last_x = static_cast<uint32_t>(valid - 1) * xrow + 16 * pb, last_b = static_cast<uint32_t>(valid - 1) * brow + 16 * pb;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    xr[r] = *reinterpret_cast<const uint4*>(xsrc + static_cast<uint32_t>(r) * xrow + static_cast<uint64_t>(voff_x));
-                    br[r] = *reinterpret_cast<const uint4*>(bsrc + static_cast<uint32_t>(r) * brow + static_cast<uint64_t>(voff_b));
-                }
-            } else {
-                // ragged last chunk: steps past the end of the sequence read as zero (the loads stay inside the tensors)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int k = 4 * kb + r;
-                    const uint32_t kk = static_cast<uint32_t>(min(k, valid - 1));
-                    const uint4 xv = *reinterpret_cast<const uint4*>(xsrc + kk * xrow + 16 * pb);
-                    const uint4 bv = *reinterpret_cast<const uint4*>(bsrc + kk * brow + 16 * pb);
-                    xr[r] = k < valid ? xv : make_uint4(0u, 0u, 0u, 0u);
-                    br[r] = k < valid ? bv : make_uint4(0u, 0u, 0u, 0u);
-                }
+            for (int r = 0; r < 4; ++r) {
+                xr[r] = *reinterpret_cast<const uint4*>(xsrc + static_cast<uint64_t>(min(voff_x + static_cast<uint32_t>(r) * xrow, last_x)));
+                br[r] = *reinterpret_cast<const uint4*>(bsrc + static_cast<uint64_t>(min(voff_b + static_cast<uint32_t>(r) * brow, last_b)));
             }
         }
         const float* dA_row = dA_ws + (rows0 + c) * Q;
         r_last = dA_row[Q - 1];
-        if (tid < Q) {
+        if (Q == kThreads || tid < Q) {
             r_dt = dt_ws[(rows0 + c) * Q + tid];
             r_dA = dA_row[tid];
         }
     };
     auto stage_chunk = [&]() {
         if (mine) {
+            if (valid_loaded < Q) {
+                // ragged last chunk: steps past the end of the sequence count as zero
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    if (4 * kb + r >= valid_loaded) xr[r] = br[r] = make_uint4(0u, 0u, 0u, 0u);
+                }
+            }
             stage_x_share<S::XP>(sm.xt, xr, sm.xs, pb, kb);
 #pragma unroll
             for (int d = 0; d < 4; ++d) {
@@ -303,7 +303,11 @@ __global__ __launch_bounds__(256, 3) void ssd_state_kernel(QaSsdParams p, const 
 
     for (int c = 0; c < nc; ++c) {
         const bool more = c + 1 < nc;
-        if (more) load_chunk(c + 1);                               // in flight during the products
+        // in flight during the products.  Unconditional (the last chunk is requested once more and never staged): a
+        // conditional request leaves the tile registers with two possible sources, which the compiler merges by
+        // copies right behind the loads, i.e. by waiting for them where they are issued
+        load_chunk(min(c + 1, nc - 1));
+        __builtin_amdgcn_sched_barrier(0);                         // (the scheduler would sink the requests below the products)
         v4f accs[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) accs[j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
