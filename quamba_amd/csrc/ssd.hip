@@ -498,30 +498,25 @@ __global__ __launch_bounds__(64 * scan_waves_of(Q), 4) void ssd_chunk_scan_kerne
             const int piece = tid + i * kThreads, k = piece / (N / 16), col = piece % (N / 16);
             r_b[i] = *reinterpret_cast<const v4i*>(Bbase + static_cast<uint32_t>(min(k, lim - 1)) * crow + 16 * col);
         }
-        // this thread's share of the x tile: steps 4 kb .. 4 kb + 3, channels 16 pb .. 16 pb + 15
-        const int pb = tid % 4, kb = tid / 4;
-        const bool mine = Q == kThreads || tid < Q;
-        uint4 xr[4];
-        if (mine) {
-            if (lim == Q) {
-                const uint32_t voff_x = static_cast<uint32_t>(4 * kb) * xrow + 16 * pb;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) xr[r] = *reinterpret_cast<const uint4*>(xbase + static_cast<uint32_t>(r) * xrow + static_cast<uint64_t>(voff_x));
-            } else {
-                // ragged last chunk: steps past the end of the sequence read as zero (the loads stay inside the tensor)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int k = 4 * kb + r;
-                    const uint4 xv = *reinterpret_cast<const uint4*>(xbase + static_cast<uint32_t>(min(k, lim - 1)) * xrow + 16 * pb);
-                    xr[r] = k < lim ? xv : make_uint4(0u, 0u, 0u, 0u);
-                }
-            }
-        }
 #pragma unroll
         for (int s = 0; s < TILES; ++s) {
             const int8_t* cp = Cbase + static_cast<uint32_t>(min(tile_of(s) * 16 + l16, lim - 1)) * crow + 16 * lq;
 #pragma unroll
             for (int i = 0; i < N / 64; ++i) cq[s][i] = *reinterpret_cast<const v4i*>(cp + 64 * i);
+        }
+        // (requested last: the compiler moves the loaded words into other registers right behind these loads, i.e.
+        // waits for them here, and everything else is then already on its way)
+        // this thread's share of the x tile: steps 4 kb .. 4 kb + 3, channels 16 pb .. 16 pb + 15
+        const int pb = tid % 4, kb = tid / 4;
+        const bool mine = Q == kThreads || tid < Q;
+        // (one path for whole and ragged chunks: rows past the end of the sequence read the last row and are zeroed
+        // when the tile is staged; with a second path beside it the compiler merges the two sets of destination
+        // registers by copies right behind the loads and so waits for them before the requests below are issued)
+        uint4 xr[4];
+        if (mine) {
+            const uint32_t last_x = static_cast<uint32_t>(lim - 1) * xrow + 16 * pb, voff_x = static_cast<uint32_t>(4 * kb) * xrow + 16 * pb;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) xr[r] = *reinterpret_cast<const uint4*>(xbase + static_cast<uint64_t>(min(voff_x + static_cast<uint32_t>(r) * xrow, last_x)));
         }
         if (tid < kP) {
             sm.xs[tid] = x_scale_of(p, g, hg, tid);
@@ -551,7 +546,16 @@ __global__ __launch_bounds__(64 * scan_waves_of(Q), 4) void ssd_chunk_scan_kerne
             const int piece = tid + i * kThreads, k = piece / (N / 16), col = piece % (N / 16);
             *reinterpret_cast<v4i*>(sm.brow(k) + (col ^ (k & S::BSWZ)) * 16) = r_b[i];
         }
-        if (mine) stage_x_share<S::XP>(sm.xt, xr, sm.xs, pb, kb);
+        if (mine) {
+            if (lim < Q) {
+                // ragged last chunk: steps past the end of the sequence count as zero
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    if (4 * kb + r >= lim) xr[r] = make_uint4(0u, 0u, 0u, 0u);
+                }
+            }
+            stage_x_share<S::XP>(sm.xt, xr, sm.xs, pb, kb);
+        }
     }
     __syncthreads();
 
