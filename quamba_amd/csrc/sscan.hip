@@ -483,8 +483,11 @@ struct PreSmem {
     // input and gate codes of a step as they came from memory, u in the low byte and z in the high byte: the lane
     // that owns the step forms the skip term and looks the gate up itself (two fp32 rows per channel less in LDS)
     __attribute__((aligned(16))) uint16_t uz[Cfg::kCh][Cfg::kUzPitch];
-    __attribute__((aligned(16))) float bc[Cfg::T][Cfg::kBcPitch];    // B (kNP) | C (kNP) of a step, scaled
-    __attribute__((aligned(16))) __half out[Cfg::T][Cfg::kOutPitch];
+    // the two tiles that all waves of the workgroup share, twice each: while tile t is scanned out of one copy the
+    // next tile is staged into the other, so that one barrier per tile is enough (the per-step rows above belong to
+    // the wave that staged them and need none)
+    __attribute__((aligned(16))) float bc[2][Cfg::T][Cfg::kBcPitch];    // B (kNP) | C (kNP) of a step, scaled
+    __attribute__((aligned(16))) __half out[2][Cfg::T][Cfg::kOutPitch];
     float gate_table[256];             // SiLU gate per z code (indexed by the raw byte)
 };
 
@@ -630,7 +633,7 @@ __device__ __forceinline__ void sscan_fwd_pre_body(const QaSScanParams& p, int v
 
     // Writes the staged tile.  Per step of this lane's share of its channel: step size (bias, softplus), step
     // size x input, skip term and gate - everything the time loop needs that does not depend on the state.
-    auto stage = [&](int t0) {
+    auto stage = [&](int t0, int into) {
         float dv[kStage], duv[kStage];
 #pragma unroll
         for (int e = 0; e < kStage; ++e) dv[e] = __builtin_fmaf(s_dt, i8_of(r_d[e >> 2], e & 3), db);
@@ -669,7 +672,7 @@ __device__ __forceinline__ void sscan_fwd_pre_body(const QaSScanParams& p, int v
             int which, n, col;
             bc_piece(tid + i * kThreads, which, n, col);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) sm.bc[col * 4 + e][which * kNP + n] = bc_factor[i] * i8_of(r_bc[i], e);
+            for (int e = 0; e < 4; ++e) sm.bc[into][col * 4 + e][which * kNP + n] = bc_factor[i] * i8_of(r_bc[i], e);
         }
     };
 
@@ -678,14 +681,14 @@ __device__ __forceinline__ void sscan_fwd_pre_body(const QaSScanParams& p, int v
         float d[4], du[4], B[4][NPL], C[4][NPL];
         uint32_t code;                  // of the step this lane owns: u in byte 0, z in byte 1
     };
-    auto fetch = [&](Group& o, int tq) {
+    auto fetch = [&](Group& o, int tq, int from) {
         const float4 d4 = *reinterpret_cast<const float4*>(&sm.d[c_local][tq * 4]);
         const float4 du4 = *reinterpret_cast<const float4*>(&sm.du[c_local][tq * 4]);
         o.d[0] = d4.x; o.d[1] = d4.y; o.d[2] = d4.z; o.d[3] = d4.w;
         o.du[0] = du4.x; o.du[1] = du4.y; o.du[2] = du4.z; o.du[3] = du4.w;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const float* row = sm.bc[tq * 4 + j];
+            const float* row = sm.bc[from][tq * 4 + j];
             if constexpr (NPL == 2) {
                 const float2 Bv = *reinterpret_cast<const float2*>(row + slice * NPL);
                 const float2 Cv = *reinterpret_cast<const float2*>(row + kNP + slice * NPL);
@@ -706,8 +709,9 @@ __device__ __forceinline__ void sscan_fwd_pre_body(const QaSScanParams& p, int v
         for (int i = tid; i < 256; i += kThreads) sm.gate_table[i] = silu_gate(s_z * static_cast<float>(static_cast<int8_t>(i)));
         __syncthreads();
     }
-    stage(0);
+    stage(0, 0);
     __syncthreads();
+    int buf = 0;                          // copy of the shared tiles that holds the tile being scanned
 
     for (int tile = 0; tile < n_tiles; ++tile) {
         const int t0 = tile * T;
@@ -718,11 +722,11 @@ __device__ __forceinline__ void sscan_fwd_pre_body(const QaSScanParams& p, int v
         // the state alone, and their output rows are never stored.  No branch in the body and constant LDS
         // offsets; the operands of a group are fetched while the group before is being computed.
         Group grp[2];
-        fetch(grp[0], 0);
+        fetch(grp[0], 0, buf);
 #pragma unroll
         for (int tq = 0; tq < T / 4; ++tq) {
             Group& o = grp[tq & 1];
-            if (tq + 1 < T / 4) fetch(grp[(tq + 1) & 1], tq + 1);
+            if (tq + 1 < T / 4) fetch(grp[(tq + 1) & 1], tq + 1, buf);
             // keep the reads of the next group ahead of this group's arithmetic (the scheduler would sink them
             // to their first use, and a wave would then wait for LDS once per group)
             __builtin_amdgcn_sched_barrier(0);
@@ -751,9 +755,11 @@ __device__ __forceinline__ void sscan_fwd_pre_body(const QaSScanParams& p, int v
             if constexpr (NSPLIT == 8) own_sum += __shfl_xor(own_sum, 4);
             float y = own_sum + D_u * code_byte_to_float(o.code, 0);
             if constexpr (HAS_Z) y *= gate;
-            sm.out[tq * 4 + qslice][c_local] = __float2half(y);
+            sm.out[buf][tq * 4 + qslice][c_local] = __float2half(y);
         }
-        __syncthreads();   // out complete; everyone is done reading the staged tile
+        // the next tile goes into the other copy (every wave left it at the barrier of the tile before)
+        if (tile + 1 < n_tiles) stage(t0 + T, buf ^ 1);
+        __syncthreads();   // this tile's outputs and the next tile's B / C are complete
 
         // write the tile's output rows: (t, kCh channels) contiguous along channels
         {
@@ -763,16 +769,15 @@ __device__ __forceinline__ void sscan_fwd_pre_body(const QaSScanParams& p, int v
                 const int t = piece / kChunksPerRow, ch8 = (piece % kChunksPerRow) * 8;
                 __half* dst = out_b + (t0 + t) * p.out_l_stride + (c0 + ch8) * p.out_d_stride;
                 if (vec_out && c0 + ch8 + 8 <= p.dim) {
-                    *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(&sm.out[t][ch8]);
+                    *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(&sm.out[buf][t][ch8]);
                 } else {
                     for (int e = 0; e < 8; ++e) {
-                        if (c0 + ch8 + e < p.dim) dst[e * p.out_d_stride] = sm.out[t][ch8 + e];
+                        if (c0 + ch8 + e < p.dim) dst[e * p.out_d_stride] = sm.out[buf][t][ch8 + e];
                     }
                 }
             }
         }
-        if (tile + 1 < n_tiles) stage(t0 + T);
-        __syncthreads();
+        buf ^= 1;
     }
 
     if (p.dt_sum_out) {
