@@ -64,7 +64,9 @@ __device__ __forceinline__ float softplus20_flat(float x) {
     const float u = 1.0f + e;
     const float r = (u - 1.0f) - e;
     const float sp = __builtin_fmaf(fast_log2(u), 0.693147180559945309f, -r);
-    return __builtin_amdgcn_fmed3f(x, 0.0f, __builtin_inff()) + sp;
+    float pos;                                        // max(x, 0): written out, because the builtins put a second
+    asm("v_max_f32 %0, 0, %1" : "=v"(pos) : "v"(x));  // maximum of x with itself in front of it (quieting of NaNs)
+    return pos + sp;
 }
 
 __device__ __forceinline__ float silu_gate(float z) {
@@ -1264,7 +1266,6 @@ extern "C" int qa_sscan_fwd(const QaSScanParams* p, void* stream_) {
                         p->out_l_stride % 8 == 0;
 
     const int N = p->dstate;
-    const int per_group = p->dim / p->n_groups;
     if (p->mapping != 0) {
         // a lane mapping named by the caller (tests): only d_state <= 16 has more than one
         // a value without the marker bit of QA_SSCAN_MAPPING is not a mapping (an uninitialised field, say)
