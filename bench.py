@@ -175,9 +175,7 @@ def cpu_baseline(dev_mixer, seconds_budget=30.0):
         one_pass()
         reps += 1
         el = time.perf_counter() - t0
-        if reps >= 3 and (el > 0.5 * seconds_budget or reps >= 20):
-            break
-        if el > seconds_budget:
+        if (reps >= 3 and el > 0.4 * seconds_budget) or el > seconds_budget:      # about 12 s of CPU work
             break
     per_pass = (time.perf_counter() - t0) / reps
     return dict(value=L / per_pass, unit="tokens/s", cores=threads, kind="port",

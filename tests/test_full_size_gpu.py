@@ -174,7 +174,7 @@ def _check_ssd_y(y_gpu, ref, interval_of):
     (batch, head) whose oracle result `ref` carries the stage tensors.  With operands drawn from the whole int8 range
     a single product reaches 10^3 while an output near zero has a bar of 10^-2, and both sides round the same
     operands to fp16 before multiplying: an operand on a rounding tie falls either way with the last bit of exp and
-    moves its product by 2^-11 of its size.  Measured on MI355X: between 0 and 11 of 262 144 outputs of a head lie
+    moves its product by 2^-11 of its size.  Measured on MI355X: between 0 and 12 of 262 144 outputs of a head lie
     beyond the bar, the farthest at 2.9 times the bar.  The test allows 16 in 262 144 and requires every one of them to
     lie inside the interval that nudging the fp16-rounded operands of that output by one ulp opens around the float64
     value (tests/ssd_interval.py): a tie explains it, a dropped or misplaced term would not."""
