@@ -94,6 +94,19 @@ def test_fwd_on_in_proj_view(dev):
     np.testing.assert_array_equal(got.cpu().numpy(), oracle.conv1d_fwd(qx, qw, qb, sx, sw, sb, so))
 
 
+@pytest.mark.parametrize("B,D,L", [(5, 70, 2048), (7, 64, 96), (3, 33, 2064), (8, 130, 4096), (6, 20, 100)])
+def test_fwd_on_in_proj_view_with_odd_batches_and_channel_counts(dev, B, D, L):
+    """The (B, D, L) view of a [2D][B][L] buffer with batch sizes that do not fill a workgroup of four batch entries,
+    channel counts that leave the bias vector without whole words, rows of two segments per lane and ragged rows."""
+    qx, sx, qw, sw, qb, sb, so = _case(B, D, L, 4, seed=B * 1000 + D)
+    buf = torch.zeros((2 * D, B, L), dtype=torch.int8, device=dev)
+    x = buf.transpose(0, 1)[:, :D]
+    x.copy_(_t(qx, dev))
+    got = ops.causal_conv1d_fwd(x, sx, _t(qw, dev), sw, so, sb, _t(qb, dev))
+    assert got.stride() == x.stride()
+    np.testing.assert_array_equal(got.cpu().numpy(), oracle.conv1d_fwd(qx, qw, qb, sx, sw, sb, so))
+
+
 def test_fwd_unaligned_rows_take_the_generic_path(dev):
     B, D, L, k = 2, 32, 50, 4                   # row stride 50 is not a multiple of 16
     qx, sx, qw, sw, qb, sb, so = _case(B, D, L, k, seed=13)

@@ -49,7 +49,9 @@ SHAPES = [(1, 512, 1536, 16), (2, 33, 1536, 16), (2, 89, 100, 16), (1, 1, 64, 16
           (2, 130, 72, 8), (1, 200, 40, 32), (1, 100, 24, 64), (1, 70, 8, 128), (1, 40, 6, 256),
           (4, 96, 5120, 128), (4, 40, 8192, 128),
           # wide states with many channels (four waves share a B/C tile): ragged channel tails, a padded state count
-          (2, 70, 4170, 32), (2, 50, 2100, 64), (3, 33, 1400, 100)]
+          (2, 70, 4170, 32), (2, 50, 2100, 64), (3, 33, 1400, 100),
+          # aligned rows whose last tile is ragged (whole tiles by vector loads, the last one byte-wise), and one tile only
+          (2, 48, 128, 16), (1, 80, 200, 16), (2, 16, 64, 16), (9, 176, 640, 16)]
 
 
 @pytest.mark.parametrize("B,L,D,N", SHAPES)
