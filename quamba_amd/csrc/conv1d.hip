@@ -123,12 +123,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_fwd_rows_dual_kernel(QaConv
     if (c < p.dim && remaining > 0) {
         const int8_t* x = p.x + b * p.x_batch_stride + c * p.x_c_stride;
         int8_t* out = p.out + b * p.out_batch_stride + c * p.out_c_stride;
-        const uint32_t taps = pack_taps(p.weight + c * p.weight_c_stride, p.weight_width_stride, p.width);
-        const float s_wx = p.scale_w * p.scale_x;
-        const float bias_f = p.bias ? static_cast<float>(p.bias[c]) * p.scale_b : 0.0f;
-        const float inv_s_out = 1.0f / p.scale_out;
-    const bool exact_only = conv_needs_exact_route(p.scale_out);
-    const ConvQuantRegs kq(p.scale_out);
+        // the row's bytes are requested first; taps, bias and scales arrive while they travel
         uint32_t w[5];   // w[0] = x[t0-4 .. t0-1], w[1..4] = x[t0 .. t0+15]
         w[0] = t0 > 0 ? *reinterpret_cast<const uint32_t*>(x + t0 - 4) : 0u;
         if (remaining >= 16) {
@@ -140,6 +135,15 @@ __global__ __launch_bounds__(kConvThreads) void conv_fwd_rows_dual_kernel(QaConv
                 w[1 + (i >> 2)] |= static_cast<uint32_t>(static_cast<uint8_t>(x[t0 + i])) << (8 * (i & 3));
             }
         }
+        const int8_t* taps_at = p.weight + c * p.weight_c_stride;
+        uint32_t taps;
+        if (p.width == 4 && p.weight_width_stride == 1 && aligned4(taps_at)) taps = *reinterpret_cast<const uint32_t*>(taps_at);
+        else taps = pack_taps(taps_at, p.weight_width_stride, p.width);
+        const float s_wx = p.scale_w * p.scale_x;
+        const float bias_f = p.bias ? static_cast<float>(p.bias[c]) * p.scale_b : 0.0f;
+        const float inv_s_out = 1.0f / p.scale_out;
+        const bool exact_only = conv_needs_exact_route(p.scale_out);
+        const ConvQuantRegs kq(p.scale_out);
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             float v[4];
