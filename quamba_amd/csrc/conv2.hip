@@ -21,7 +21,7 @@ namespace qa {
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kRun = 64;          // time steps per wave
+constexpr int kRun = 64;          // time steps per wave unless the launch picks more
 constexpr int kBatchLoads = 8;    // loads in flight per lane
 
 struct Part {
@@ -88,13 +88,16 @@ __device__ __forceinline__ int8_t* out_ptr(const QaConv2Params& p, const Part& p
 }
 
 // grid: x = blocks of 256 channels, y = blocks of 4 runs of kRun steps (one run per wave), z = batch
-__global__ __launch_bounds__(kThreads) void conv2_fwd_kernel(QaConv2Params p) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+template <bool SILU>
+__global__ __launch_bounds__(kThreads) void conv2_fwd_kernel(QaConv2Params p, int run) {
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));   // the same in every lane: the step
+                                                                                          // counters below stay in scalar registers
     const int ch0 = (blockIdx.x * 64 + lane) * 4;
     const int b = blockIdx.z;
-    const int t0 = (blockIdx.y * 4 + wave) * kRun;
+    const int t0 = (blockIdx.y * 4 + wave) * run;
     if (ch0 >= p.dim || t0 >= p.seqlen) return;
-    const int t_end = min(t0 + kRun, p.seqlen);
+    const int t_end = min(t0 + run, p.seqlen);
 
     const Part part = part_of(p, ch0);          // the four channels of a lane never straddle two parts
     uint32_t taps[4];
@@ -137,6 +140,8 @@ __global__ __launch_bounds__(kThreads) void conv2_fwd_kernel(QaConv2Params p) {
         }
     };
     fetch(t0, dn);
+    int8_t* out_at = out + t0 * out_ls;             // walks on by one step's stride (the stride differs from lane to lane: a
+                                                    // product per step would be a 64-bit multiplication in vector registers)
     for (int tb = t0; tb < t_end; tb += kBatchLoads) {
 #pragma unroll
         for (int i = 0; i < kBatchLoads; ++i) d[i] = dn[i];
@@ -148,7 +153,8 @@ __global__ __launch_bounds__(kThreads) void conv2_fwd_kernel(QaConv2Params p) {
             float v[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaf(part.s_in, static_cast<float>(dot4(win[e], taps[e])), bias_f[e]);
-            *reinterpret_cast<uint32_t*>(out + (tb + i) * out_ls) = conv_quant4(v, s_out, inv_s_out, p.silu_activation, exact_only, kq);
+            *reinterpret_cast<uint32_t*>(out_at) = conv_quant4(v, s_out, inv_s_out, SILU, exact_only, kq);
+            out_at += out_ls;
         }
     }
 }
@@ -235,10 +241,24 @@ extern "C" int qa_quamba2_conv1d_fwd(const QaConv2Params* p, void* stream_) {
                      mult4(p->x_batch_stride) && mult4(p->x_l_stride) && mult4(p->B_batch_stride) &&
                      mult4(p->B_l_stride) && mult4(p->C_batch_stride) && mult4(p->C_l_stride);
     if (vec) {
-        const int64_t run_blocks = (p->seqlen + 4 * kRun - 1) / (4 * kRun);
+        // Steps per wave: 64, 128 or 256, whichever needs the fewest rounds of resident waves (seven per SIMD) times its
+        // own length plus a wave's set-up (taps, scales: about 24 steps' worth).  Batch 16 x 1024 steps x 10240 channels
+        // is 10240 waves of 64 steps on 7168 places - a second round at a third of the occupancy - or 5120 of 128.
+        int run = kRun;
+        {
+            const int64_t ch_blocks = (p->dim + 255) / 256, places = 7 * 4 * 256;
+            int64_t best = -1;
+            for (int r = 64; r <= 256; r *= 2) {
+                const int64_t waves = ch_blocks * (((p->seqlen + r - 1) / r + 3) / 4 * 4) * p->batch;
+                const int64_t cost = ((waves + places - 1) / places) * (r + 24);
+                if (best < 0 || cost < best) { best = cost; run = r; }
+            }
+        }
+        const int64_t run_blocks = (p->seqlen + 4 * run - 1) / (4 * run);
         if (run_blocks > 65535) return QA_ERR_SHAPE;
         dim3 grid((p->dim + 255) / 256, static_cast<unsigned>(run_blocks), p->batch);
-        hipLaunchKernelGGL(conv2_fwd_kernel, grid, dim3(kThreads), 0, stream, *p);
+        if (p->silu_activation) hipLaunchKernelGGL(conv2_fwd_kernel<true>, grid, dim3(kThreads), 0, stream, *p, run);
+        else hipLaunchKernelGGL(conv2_fwd_kernel<false>, grid, dim3(kThreads), 0, stream, *p, run);
         return check_launch();
     }
     const int64_t blocks = (total + kThreads - 1) / kThreads;
