@@ -80,11 +80,13 @@ __device__ __forceinline__ float x_scale_of(const QaSsdParams& p, int g, int hg,
 // ---------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void ssd_cumsum_kernel(QaSsdParams p, float* dt_out, float* dA_out, int nc) {
     const int lane = threadIdx.x & 63;
-    const int64_t idx = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
-    if (idx >= static_cast<int64_t>(p.batch) * nc * p.nheads) return;
-    const int h = static_cast<int>(idx % p.nheads);
-    const int c = static_cast<int>((idx / p.nheads) % nc);
-    const int b = static_cast<int>(idx / (static_cast<int64_t>(p.nheads) * nc));
+    // the item is the same for a whole wave and below 2^31 (the host checks): its decomposition is 32-bit arithmetic on
+    // a uniform value instead of 64-bit divisions in every lane
+    const unsigned idx = __builtin_amdgcn_readfirstlane(blockIdx.x * 4u + (threadIdx.x >> 6));
+    if (idx >= static_cast<unsigned>(p.batch) * static_cast<unsigned>(nc) * static_cast<unsigned>(p.nheads)) return;
+    const int h = static_cast<int>(idx % static_cast<unsigned>(p.nheads));
+    const int c = static_cast<int>((idx / static_cast<unsigned>(p.nheads)) % static_cast<unsigned>(nc));
+    const int b = static_cast<int>(idx / (static_cast<unsigned>(p.nheads) * static_cast<unsigned>(nc)));
     const int Q = p.chunk_size, E = Q / 64;            // Q in {64, 128, 256}
     const float A = -expf(*p.A_log_scale * static_cast<float>(p.A_log[h]));
     const float s_dt = p.dt_is_fp32 ? 0.0f : *p.dt_scale;
