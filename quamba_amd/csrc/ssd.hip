@@ -17,6 +17,7 @@
 #include <mutex>
 
 #include "qa_common.hpp"
+#include "ssd_common.hpp"
 
 namespace qa {
 namespace {
@@ -28,51 +29,9 @@ typedef _Float16 v4h __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-constexpr int kP = 64;          // head dimension this build supports
-constexpr float kLog2e = 1.44269504088896341f;
-
-__device__ __forceinline__ float fexp(float x) { return __builtin_amdgcn_exp2f(x * kLog2e); }
+constexpr int kP = 64;          // head dimension of these kernels
+__device__ __forceinline__ float fexp(float x) { return ssd_exp(x); }
 __device__ __forceinline__ int8_t byte_of(uint32_t w, int j) { return static_cast<int8_t>((w >> (8 * j)) & 0xffu); }
-
-struct Ws {            // workspace sections (byte offsets), see qa_ssd_workspace_bytes
-    int64_t dt, dA, prev, total;
-};
-
-__host__ __device__ inline int64_t align256(int64_t v) { return (v + 255) & ~int64_t(255); }
-
-__host__ __device__ inline Ws ws_layout(const QaSsdParams& p) {
-    const int64_t nc = (p.seqlen + p.chunk_size - 1) / p.chunk_size;
-    const int64_t B = p.batch, H = p.nheads, Q = p.chunk_size, N = p.dstate;
-    Ws w;
-    int64_t off = 0;
-    w.dt = off; off = align256(off + B * H * nc * Q * 4);
-    w.dA = off; off = align256(off + B * H * nc * Q * 4);
-    w.prev = off; off = align256(off + B * nc * H * kP * N * 2);
-    w.total = off;
-    return w;
-}
-
-// x scale of channel p of head h (per-tensor, or looked up from the cumulative group ranges,
-// quamba/triton/quant_chunk_state.py:202-214)
-__device__ __forceinline__ void group_of(const QaSsdParams& p, int h, int& g, int& hg) {
-    const int hpg = p.nheads / p.ngroups;
-    g = h / hpg;
-    hg = 0;
-    if (p.nhead_groups > 0) {
-        for (int j = 0; j < p.nhead_groups; ++j) hg += (h % hpg) >= p.x_head_group_range[g * p.nhead_groups + j] ? 1 : 0;
-        hg = min(hg, p.nhead_groups - 1);
-    }
-}
-__device__ __forceinline__ int dim_group_of(const QaSsdParams& p, int g, int hg, int ch) {
-    const int32_t* dr = p.x_dim_group_range + (g * p.nhead_groups + hg) * p.ndim_groups;
-    int dg = 0;
-    for (int j = 0; j < p.ndim_groups; ++j) dg += ch >= dr[j] ? 1 : 0;
-    return min(dg, p.ndim_groups - 1);
-}
-__device__ __forceinline__ float x_scale_of(const QaSsdParams& p, int g, int hg, int ch) {
-    if (p.nhead_groups == 0) return p.x_scale[0];
-    return p.x_scale[(g * p.nhead_groups + hg) * p.ndim_groups + dim_group_of(p, g, hg, ch)];
-}
 
 // ---------------------------------------------------------------------------------------------
 // Stage 1 (quamba/triton/quant_chunk_cumsum.py:56-70).  One wave per (batch, chunk, head): every
@@ -222,7 +181,7 @@ __global__ __launch_bounds__(256, 3) void ssd_state_kernel(QaSsdParams p, const 
     const int h = (unit % G) * (H / G) + hig;
     const int b = unit / G;
     int g, hg;
-    group_of(p, h, g, hg);
+    ssd_group_of(p, h, g, hg);
     const bool grouped = p.nhead_groups > 0;
     const float sB = grouped ? p.B_scale[g] : p.B_scale[0];
     const float nsB = -128.0f * sB;
@@ -234,7 +193,7 @@ __global__ __launch_bounds__(256, 3) void ssd_state_kernel(QaSsdParams p, const 
     const int pb = tid % 4, kb = tid / 4;
     const bool mine = Q == 256 || tid < Q;
     const uint32_t voff_x = static_cast<uint32_t>(4 * kb) * xrow + 16 * pb, voff_b = static_cast<uint32_t>(4 * kb) * brow + 16 * pb;
-    if (tid < kP) sm.xs[tid] = x_scale_of(p, g, hg, tid);
+    if (tid < kP) sm.xs[tid] = ssd_x_scale_of(p, g, hg, tid);
     uint4 xr[4], br[4];
     float r_dt = 0.0f, r_dA = 0.0f, r_last = 0.0f;
     int valid_loaded = Q;                                         // steps of the chunk whose tiles are in xr / br
@@ -365,7 +324,7 @@ __global__ __launch_bounds__(256, 3) void ssd_state_kernel(QaSsdParams p, const 
                 } else {
                     float sc, K;
                     if (grouped) {
-                        const int dg = dim_group_of(p, g, hg, pp);
+                        const int dg = ssd_dim_group_of(p, g, hg, pp);
                         sc = p.state_scale[((g * p.nhead_groups + hg) * p.ndim_groups + dg) * N + n_col];
                         K = 1e6f;
                     } else {
@@ -456,7 +415,7 @@ __global__ __launch_bounds__(64 * scan_waves_of(Q), 4) void ssd_chunk_scan_kerne
     const int c = (unit / G) % nc;
     const int b = unit / (G * nc);
     int g, hg;
-    group_of(p, h, g, hg);
+    ssd_group_of(p, h, g, hg);
     const bool grouped = p.nhead_groups > 0;
     const float sC = grouped ? p.C_scale[g] : p.C_scale[0];
     const float cb_scale = sC * (grouped ? p.B_scale[g] : p.B_scale[0]);
@@ -521,7 +480,7 @@ __global__ __launch_bounds__(64 * scan_waves_of(Q), 4) void ssd_chunk_scan_kerne
             for (int r = 0; r < 4; ++r) xr[r] = *reinterpret_cast<const uint4*>(xbase + static_cast<uint64_t>(min(voff_x + static_cast<uint32_t>(r) * xrow, last_x)));
         }
         if (tid < kP) {
-            sm.xs[tid] = x_scale_of(p, g, hg, tid);
+            sm.xs[tid] = ssd_x_scale_of(p, g, hg, tid);
             sm.Dv[tid] = !p.D ? 0.0f : D_scale * static_cast<float>(p.D_has_hdim ? p.D[h * kP + tid] : p.D[h]);
         }
         if (p.z) {
@@ -708,16 +667,17 @@ int validate(const QaSsdParams* p) {
     if (p->final_states && !p->final_state_is_fp32 && !p->state_scale) return QA_ERR_NULL;
     if (p->nhead_groups > 0 && (!p->x_head_group_range || !p->x_dim_group_range || p->ndim_groups < 1)) return QA_ERR_NULL;
     if (p->batch < 0 || p->seqlen < 0 || p->nheads < 1 || p->ngroups < 1 || p->nheads % p->ngroups != 0) return QA_ERR_SHAPE;
-    if (p->headdim != kP) return QA_ERR_UNSUPPORTED;
-    if (p->dstate != 64 && p->dstate != 128) return QA_ERR_UNSUPPORTED;
-    if (p->chunk_size != 64 && p->chunk_size != 128 && p->chunk_size != 256) return QA_ERR_UNSUPPORTED;
-    if (!aligned16(p->x) || !aligned16(p->B) || !aligned16(p->C) || !aligned16(p->out)) return QA_ERR_STRIDE;
-    if (p->z && !aligned16(p->z)) return QA_ERR_STRIDE;      // x, the gate and the output are accessed in aligned pieces
-    if (p->D && p->D_has_hdim && !aligned16(p->D)) return QA_ERR_STRIDE;
-    // every launch is a one-dimensional grid: one workgroup per (batch, chunk, head) or per (batch, head, 64 states)
+    // what the general kernels take; the matrix-core kernels cover a subset (ssd_fast_shape)
+    if (p->headdim < 1 || p->headdim > 256 || p->dstate < 1 || p->dstate > 1024 || p->chunk_size < 1 || p->chunk_size > 1024) return QA_ERR_UNSUPPORTED;
     const int64_t nc = (static_cast<int64_t>(p->seqlen) + p->chunk_size - 1) / p->chunk_size;
-    if (static_cast<int64_t>(p->batch) * nc * p->nheads > 0x7fffffffLL) return QA_ERR_SHAPE;
-    if (static_cast<int64_t>(p->batch) * p->nheads * (p->dstate / 64) > 0x7fffffffLL) return QA_ERR_SHAPE;
+    if (ssd_fast_shape(*p)) {
+        // every launch is a one-dimensional grid: one workgroup per (batch, chunk, head) or per (batch, head, 64 states)
+        if (static_cast<int64_t>(p->batch) * nc * p->nheads > 0x7fffffffLL) return QA_ERR_SHAPE;
+        if (static_cast<int64_t>(p->batch) * p->nheads * (p->dstate / 64) > 0x7fffffffLL) return QA_ERR_SHAPE;
+    } else {
+        const int st = ssd_general_grid_check(*p);
+        if (st != QA_OK) return st;
+    }
     return QA_OK;
 }
 
@@ -726,7 +686,7 @@ int validate(const QaSsdParams* p) {
 
 extern "C" int64_t qa_ssd_workspace_bytes(const QaSsdParams* p) {
     if (qa::validate(p) != QA_OK) return 0;
-    return qa::ws_layout(*p).total;
+    return qa::ssd_workspace_layout(*p).total;
 }
 
 extern "C" int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream_) {
@@ -734,7 +694,7 @@ extern "C" int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream_) {
     const int st = validate(p);
     if (st != QA_OK) return st;
     if (p->batch == 0 || p->seqlen == 0) return QA_OK;
-    const Ws ws = ws_layout(*p);
+    const SsdWorkspace ws = ssd_workspace_layout(*p);
     if (!p->workspace) return QA_ERR_NULL;
     if (p->workspace_bytes < ws.total || (reinterpret_cast<uintptr_t>(p->workspace) & 255u)) return QA_ERR_STRIDE;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
@@ -744,9 +704,13 @@ extern "C" int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream_) {
     const int nc = (p->seqlen + p->chunk_size - 1) / p->chunk_size;
     const int64_t bch = static_cast<int64_t>(p->batch) * nc * p->nheads;
 
+    __half* prev_ws = reinterpret_cast<__half*>(base + ws.prev);
+    if (!ssd_fast_shape(*p)) {
+        ssd_general_launch(*p, dt_ws, dA_ws, prev_ws, nc, stream);
+        return check_launch();
+    }
     hipLaunchKernelGGL(ssd_cumsum_kernel, dim3(static_cast<unsigned>((bch + 3) / 4)), dim3(256), 0, stream, *p, dt_ws,
                        dA_ws, nc);
-    __half* prev_ws = reinterpret_cast<__half*>(base + ws.prev);
     const dim3 hgrid(static_cast<unsigned>(p->batch * p->nheads * (p->dstate / 64)));
     int status = QA_OK;
     // more LDS than a kernel gets by default: raise the limit (idempotent)
@@ -822,7 +786,7 @@ extern "C" int qa_ssd_chunk_scan_fwd_noalloc(const QaSsdParams* p, void* stream_
     const int st = validate(p);
     if (st != QA_OK) return st;
     if (p->batch == 0 || p->seqlen == 0) return QA_OK;
-    if (ws_layout(*p).total > kStaticScratchBytes) return QA_ERR_SCRATCH;
+    if (ssd_workspace_layout(*p).total > kStaticScratchBytes) return QA_ERR_SCRATCH;
     void* ptr = static_scratch_of_current_device();
     if (!ptr) return QA_ERR_LAUNCH;
     QaSsdParams q = *p;

@@ -775,10 +775,12 @@ def ssd_chunk_scan_combined_fwd(q_x, x_scale, q_dt, dt_scale, q_A_log, A_log_sca
         keep.append(t)
         return ptr(t)
 
-    # The kernels are built for 64 and 128 states.  Fewer (the reference's tests use 16) run as the next of
-    # the two with zero codes in the added B and C columns: those states stay zero and add exactly nothing.
+    # The matrix-core kernels are built for headdim 64, 64 or 128 states and chunks of 64, 128 or 256 steps; the
+    # library runs every other shape on general kernels.  Fewer than 128 states (the reference's tests use 16) with
+    # an otherwise fast shape run as 64 or 128 with zero codes in the added B and C columns: those states stay zero
+    # and add exactly nothing.
     dstate_given = dstate
-    if dstate not in (64, 128) and dstate < 128:
+    if headdim == 64 and chunk_size in (64, 128, 256) and dstate not in (64, 128) and dstate < 128:
         dstate = 64 if dstate < 64 else 128
         q_B = torch.nn.functional.pad(q_B, (0, dstate - dstate_given))
         q_C = torch.nn.functional.pad(q_C, (0, dstate - dstate_given))
@@ -834,7 +836,9 @@ def ssd_chunk_scan_combined_fwd(q_x, x_scale, q_dt, dt_scale, q_A_log, A_log_sca
     lib = _lib.lib()
     nbytes = lib.qa_ssd_workspace_bytes(ct.byref(p))
     if nbytes <= 0:
-        _lib.check(lib.qa_ssd_chunk_scan_fwd(ct.byref(p), None) or -4, "ssd_chunk_scan_fwd")
+        # an invalid request (the call reports which way), or an empty one (nothing to do)
+        _lib.check(lib.qa_ssd_chunk_scan_fwd(ct.byref(p), None), "ssd_chunk_scan_fwd")
+        return (out, final, None) if return_workspace else (out, final)
     if static_scratch:
         _require(not return_workspace, "the library's own scratch buffer cannot be returned")
         with torch.cuda.device(dev):

@@ -126,8 +126,15 @@ def test_ssd_shape_limits_without_a_gpu():
     p.batch, p.seqlen = 65536, 65536                                # 65536 x 1024 chunks x 128 heads > 2^31 - 1 workgroups
     assert l.qa_ssd_workspace_bytes(C.byref(p)) == 0
     assert l.qa_ssd_chunk_scan_fwd(C.byref(p), None) == -2
-    p.batch, p.seqlen, p.dstate = 2, 512, 256                       # more states than the kernels are built for
-    assert l.qa_ssd_chunk_scan_fwd(C.byref(p), None) == -4
+    p.batch, p.seqlen, p.dstate = 2, 512, 256                       # shapes the matrix-core kernels are not built for take the general ones
+    assert l.qa_ssd_workspace_bytes(C.byref(p)) > 0
+    p.headdim, p.chunk_size = 96, 100
+    # 6 chunks: dt and the running sums in fp32 per (batch, head, chunk, step), entering states in fp16 per (batch, chunk, head, channel, state)
+    assert l.qa_ssd_workspace_bytes(C.byref(p)) == 2 * (2 * 128 * 6 * 100 * 4) + 2 * 6 * 128 * 96 * 256 * 2
+    for field, value in (("headdim", 257), ("dstate", 1025), ("chunk_size", 1025), ("chunk_size", 0)):
+        q = _lib.QaSsdParams.from_buffer_copy(p)
+        setattr(q, field, value)
+        assert l.qa_ssd_chunk_scan_fwd(C.byref(q), None) == -4, field
 
 
 def test_the_entry_point_without_allocation_refuses_large_problems_before_any_gpu_call():

@@ -63,6 +63,73 @@ def test_forward_matches_oracle(dev, B, L, H, N, G, Q):
     assert np.abs(got - ref["final_f32"]).max() <= 1e-3 * np.abs(ref["final_f32"]).max()
 
 
+# Shapes outside what the matrix-core kernels are built for (head dimension 64, 64 or 128 states, chunks of 64, 128
+# or 256 steps) run on the library's general kernels, to the same bars.
+# batch, seqlen, nheads, headdim, dstate, ngroups, chunk
+GENERAL_SHAPES = [(1, 100, 4, 128, 128, 1, 64),      # the head dimension of the larger Mamba2 variants
+                  (2, 77, 4, 32, 16, 2, 32),         # small everything
+                  (1, 300, 2, 64, 256, 1, 128),      # more states than one tile pair
+                  (1, 200, 4, 64, 128, 1, 512),      # one chunk longer than the sequence
+                  (1, 700, 2, 64, 64, 2, 512),       # a whole and a ragged chunk of 512
+                  (2, 150, 4, 96, 48, 2, 100),       # nothing a multiple of 64
+                  (1, 130, 6, 40, 24, 3, 48),
+                  (1, 65, 2, 256, 16, 1, 64),        # the largest head dimension
+                  (1, 33, 3, 1, 1, 1, 7)]            # the smallest
+
+
+@pytest.mark.parametrize("B,L,H,P,N,G,Q", GENERAL_SHAPES)
+def test_forward_of_other_shapes_matches_oracle(dev, B, L, H, P, N, G, Q):
+    d = synth.mamba2_ssd_inputs(B, L, H, P, N, G, seed=L + P)
+    ref = _oracle(d, Q)
+    y, final = _gpu(d, dev, Q)
+    assert y.shape == (B, L, H, P) and y.dtype == torch.float16 and final.shape == (B, H, P, N)
+    _check_y(y, ref["y"])
+    got = final.cpu().numpy()
+    assert np.abs(got - ref["final_f32"]).max() <= 1e-3 * np.abs(ref["final_f32"]).max()
+
+
+@pytest.mark.parametrize("with_z,d_has_hdim", [(True, False), (False, True)])
+def test_other_shapes_with_grouped_scales_z_gate_and_int8_state(dev, with_z, d_has_hdim):
+    B, L, H, P, N, G, Q = 2, 150, 8, 96, 80, 2, 96
+    d = synth.mamba2_ssd_inputs(B, L, H, P, N, G, seed=6, grouped=True, nhead_groups=2, ndim_groups=3, with_z=with_z)
+    if d_has_hdim:
+        d["D"] = np.random.default_rng(1).integers(60, 128, (H, P)).astype(np.int8)
+    ref = _oracle(d, Q)
+    g = np.random.default_rng(2)
+    state_scale = (np.abs(ref["final_f32"]).max() / 127 * g.uniform(0.8, 1.2, (G, 2, 3, N))).astype(np.float32)
+    ref = _oracle(d, Q, state_scale=state_scale)
+    y, final = _gpu(d, dev, Q, state_scale=state_scale, final_dtype=torch.int8)
+    _check_y(y, ref["y"])
+    diff = np.abs(final.cpu().numpy().astype(int) - ref["final_i8"].astype(int))
+    assert diff.max() <= 1 and (diff != 0).mean() < 0.02
+    assert np.abs(ref["final_i8"]).max() > 100
+
+
+def test_unaligned_tensors_take_the_general_kernels_with_the_same_result(dev):
+    """The matrix-core kernels read x, B, C and write the output in aligned 16-byte pieces; views that start elsewhere
+    run on the general kernels: same bars against the oracle, and close to the aligned call's own output."""
+    B, L, H, N, G, Q = 1, 200, 4, 128, 1, 128
+    d = synth.mamba2_ssd_inputs(B, L, H, 64, N, G, seed=21)
+    ref = _oracle(d, Q)
+    y0, f0 = _gpu(d, dev, Q)
+
+    def shifted(a):
+        flat = torch.empty(a.size + 1, dtype=torch.int8, device=dev)
+        flat[1:] = torch.from_numpy(np.ascontiguousarray(a)).to(dev).reshape(-1)
+        v = flat[1:].view(a.shape)
+        assert v.data_ptr() % 16 == 1 and v.is_contiguous()
+        return v
+
+    s = lambda v: torch.tensor(np.asarray(v, np.float32)).to(dev)
+    y1, f1 = ops.ssd_chunk_scan_combined_fwd(
+        shifted(d["x"]), s(d["x_scale"]), _t(d["dt"], dev), s(d["s_dt"]), _t(d["A_log"], dev), s(d["s_A"]),
+        shifted(d["B"]), s(d["s_B"]), shifted(d["C"]), s(d["s_C"]), None, Q, q_D=_t(d["D"], dev), D_scale=s(d["s_D"]),
+        dt_bias=_t(d["dt_bias"], dev), dt_softplus=True, final_state_dtype=torch.float32)
+    _check_y(y1, ref["y"])
+    np.testing.assert_allclose(f1.cpu().numpy(), f0.cpu().numpy(), rtol=1e-4, atol=1e-5 * np.abs(ref["final_f32"]).max())
+    assert (y1.float() - y0.float()).abs().max() <= 2e-2 * y0.float().abs().max()
+
+
 def test_preparation_stages_match_the_oracle(dev):
     # what the preparation kernel leaves in the workspace: step sizes and their running sums (C B^T is formed inside
     # the chunk scan and never stored; the outputs below depend on every element of it at or below the diagonal)
@@ -249,9 +316,9 @@ def _oracle_step_noD(d, t, state):
 def test_errors(dev):
     d = synth.mamba2_ssd_inputs(1, 64, 2, 64, 128, 1, seed=1)
     with pytest.raises(NotImplementedError):
-        _gpu(d, dev, 48)                                  # chunk sizes other than 64 / 128 / 256
+        _gpu(d, dev, 2048)                                # chunks of more than 1024 steps
     with pytest.raises(NotImplementedError, match="seq_idx"):
         _gpu(d, dev, 64, seq_idx=torch.zeros(1, 64, device=dev))
-    d2 = synth.mamba2_ssd_inputs(1, 64, 2, 32, 128, 1, seed=1)
+    d2 = synth.mamba2_ssd_inputs(1, 8, 1, 320, 16, 1, seed=1)
     with pytest.raises(NotImplementedError):
-        _gpu(d2, dev, 64)                                 # head dimensions other than 64
+        _gpu(d2, dev, 64)                                 # head dimensions above 256
