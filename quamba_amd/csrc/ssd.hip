@@ -175,25 +175,29 @@ __global__ __launch_bounds__(256, 3) void ssd_state_kernel(QaSsdParams p, const 
 
     const int tid = threadIdx.x, lane = tid & 63, l16 = lane & 15, lq = lane >> 4;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);    // the same in every lane: kept in a scalar register
-    const int G = p.ngroups, H = p.nheads, L = p.seqlen;
+    // a head of 64 s channels runs as s heads of 64 that share the head's step sizes, decay and skip weight: H, h count
+    // those; hp is the head itself and ch0 the first of its channels this workgroup covers
+    const int split = p.headdim / kP;
+    const int G = p.ngroups, H = p.nheads * split, L = p.seqlen;
     int unit, hig, part;
     unit_head_part(blockIdx.x, p.batch * G, H / G, PARTS, unit, hig, part);
     const int h = (unit % G) * (H / G) + hig;
+    const int hp = h / split, ch0 = (h % split) * kP;
     const int b = unit / G;
     int g, hg;
-    ssd_group_of(p, h, g, hg);
+    ssd_group_of(p, hp, g, hg);
     const bool grouped = p.nhead_groups > 0;
     const float sB = grouped ? p.B_scale[g] : p.B_scale[0];
     const float nsB = -128.0f * sB;
     const uint32_t xrow = static_cast<uint32_t>(H) * kP;          // bytes between steps of x
     const uint32_t brow = static_cast<uint32_t>(G) * N;           // bytes between steps of B
-    const int64_t rows0 = (static_cast<int64_t>(b) * H + h) * nc;
+    const int64_t rows0 = (static_cast<int64_t>(b) * p.nheads + hp) * nc;
     // this thread's share of a chunk's tiles: steps 4 kb .. 4 kb + 3, sixteen columns from 16 pb (of x: channels; of
     // B: state columns of this workgroup's part)
     const int pb = tid % 4, kb = tid / 4;
     const bool mine = Q == 256 || tid < Q;
     const uint32_t voff_x = static_cast<uint32_t>(4 * kb) * xrow + 16 * pb, voff_b = static_cast<uint32_t>(4 * kb) * brow + 16 * pb;
-    if (tid < kP) sm.xs[tid] = ssd_x_scale_of(p, g, hg, tid);
+    if (tid < kP) sm.xs[tid] = ssd_x_scale_of(p, g, hg, ch0 + tid);
     uint4 xr[4], br[4];
     float r_dt = 0.0f, r_dA = 0.0f, r_last = 0.0f;
     int valid_loaded = Q;                                         // steps of the chunk whose tiles are in xr / br
@@ -324,7 +328,7 @@ __global__ __launch_bounds__(256, 3) void ssd_state_kernel(QaSsdParams p, const 
                 } else {
                     float sc, K;
                     if (grouped) {
-                        const int dg = ssd_dim_group_of(p, g, hg, pp);
+                        const int dg = ssd_dim_group_of(p, g, hg, ch0 + pp);
                         sc = p.state_scale[((g * p.nhead_groups + hg) * p.ndim_groups + dg) * N + n_col];
                         K = 1e6f;
                     } else {
@@ -407,15 +411,18 @@ __global__ __launch_bounds__(64 * scan_waves_of(Q), 4) void ssd_chunk_scan_kerne
 
     const int tid = threadIdx.x, lane = tid & 63, l16 = lane & 15, lq = lane >> 4;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);    // the same in every lane: kept in a scalar register
-    const int G = p.ngroups, H = p.nheads, L = p.seqlen;
+    // (H, h, hp, ch0 as in the state kernel: heads of 64 s channels run as s heads of 64)
+    const int split = p.headdim / kP;
+    const int G = p.ngroups, H = p.nheads * split, L = p.seqlen;
     // the heads of one (batch, chunk, ssd group) read the same B and C codes: they go to one XCD
     int unit, hig, part;
     unit_head_part(blockIdx.x, p.batch * nc * G, H / G, 1, unit, hig, part);
     const int h = (unit % G) * (H / G) + hig;
+    const int hp = h / split, ch0 = (h % split) * kP;
     const int c = (unit / G) % nc;
     const int b = unit / (G * nc);
     int g, hg;
-    ssd_group_of(p, h, g, hg);
+    ssd_group_of(p, hp, g, hg);
     const bool grouped = p.nhead_groups > 0;
     const float sC = grouped ? p.C_scale[g] : p.C_scale[0];
     const float cb_scale = sC * (grouped ? p.B_scale[g] : p.B_scale[0]);
@@ -443,7 +450,7 @@ __global__ __launch_bounds__(64 * scan_waves_of(Q), 4) void ssd_chunk_scan_kerne
         // once.
         float r_dt = 0.0f, r_dA = 0.0f, r_end = 0.0f;
         if (tid < Q) {
-            const int64_t row = ((static_cast<int64_t>(b) * H + h) * nc + c) * Q;
+            const int64_t row = ((static_cast<int64_t>(b) * p.nheads + hp) * nc + c) * Q;
             r_dt = dt_ws[row + tid];
             r_dA = dA_ws[row + tid];
             r_end = dA_ws[row + (tid | 31)];
@@ -480,8 +487,8 @@ __global__ __launch_bounds__(64 * scan_waves_of(Q), 4) void ssd_chunk_scan_kerne
             for (int r = 0; r < 4; ++r) xr[r] = *reinterpret_cast<const uint4*>(xbase + static_cast<uint64_t>(min(voff_x + static_cast<uint32_t>(r) * xrow, last_x)));
         }
         if (tid < kP) {
-            sm.xs[tid] = ssd_x_scale_of(p, g, hg, tid);
-            sm.Dv[tid] = !p.D ? 0.0f : D_scale * static_cast<float>(p.D_has_hdim ? p.D[h * kP + tid] : p.D[h]);
+            sm.xs[tid] = ssd_x_scale_of(p, g, hg, ch0 + tid);
+            sm.Dv[tid] = !p.D ? 0.0f : D_scale * static_cast<float>(p.D_has_hdim ? p.D[hp * p.headdim + ch0 + tid] : p.D[hp]);
         }
         if (p.z) {
             // the gate has 256 possible values: evaluated once per workgroup, looked up per output
@@ -672,8 +679,9 @@ int validate(const QaSsdParams* p) {
     const int64_t nc = (static_cast<int64_t>(p->seqlen) + p->chunk_size - 1) / p->chunk_size;
     if (ssd_fast_shape(*p)) {
         // every launch is a one-dimensional grid: one workgroup per (batch, chunk, head) or per (batch, head, 64 states)
-        if (static_cast<int64_t>(p->batch) * nc * p->nheads > 0x7fffffffLL) return QA_ERR_SHAPE;
-        if (static_cast<int64_t>(p->batch) * p->nheads * (p->dstate / 64) > 0x7fffffffLL) return QA_ERR_SHAPE;
+        const int64_t heads = static_cast<int64_t>(p->nheads) * (p->headdim / 64);       // heads of 64 channels
+        if (static_cast<int64_t>(p->batch) * nc * heads > 0x7fffffffLL) return QA_ERR_SHAPE;
+        if (static_cast<int64_t>(p->batch) * heads * (p->dstate / 64) > 0x7fffffffLL) return QA_ERR_SHAPE;
     } else {
         const int st = ssd_general_grid_check(*p);
         if (st != QA_OK) return st;
@@ -711,7 +719,8 @@ extern "C" int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream_) {
     }
     hipLaunchKernelGGL(ssd_cumsum_kernel, dim3(static_cast<unsigned>((bch + 3) / 4)), dim3(256), 0, stream, *p, dt_ws,
                        dA_ws, nc);
-    const dim3 hgrid(static_cast<unsigned>(p->batch * p->nheads * (p->dstate / 64)));
+    const int heads64 = p->nheads * (p->headdim / 64);          // the kernels see a head of 64 s channels as s heads of 64
+    const dim3 hgrid(static_cast<unsigned>(p->batch * heads64 * (p->dstate / 64)));
     int status = QA_OK;
     // more LDS than a kernel gets by default: raise the limit (idempotent)
     auto lds_ok = [&](const void* kernel, size_t lds) {
@@ -723,7 +732,7 @@ extern "C" int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream_) {
     auto launch = [&](auto state_kernel, size_t state_lds, auto scan_kernel, size_t scan_lds, int scan_threads) {
         if (!lds_ok(reinterpret_cast<const void*>(state_kernel), state_lds) || !lds_ok(reinterpret_cast<const void*>(scan_kernel), scan_lds)) return;
         hipLaunchKernelGGL(state_kernel, hgrid, dim3(256), state_lds, stream, *p, dt_ws, dA_ws, prev_ws, nc);
-        hipLaunchKernelGGL(scan_kernel, dim3(static_cast<unsigned>(bch)), dim3(scan_threads), scan_lds, stream, *p, dt_ws, dA_ws, prev_ws, nc);
+        hipLaunchKernelGGL(scan_kernel, dim3(static_cast<unsigned>(bch * (p->headdim / 64))), dim3(scan_threads), scan_lds, stream, *p, dt_ws, dA_ws, prev_ws, nc);
     };
 #define QA_SSD_LAUNCH(N_, Q_) launch(ssd_state_kernel<N_, Q_>, sizeof(StateSmem<Q_>), ssd_chunk_scan_kernel<N_, Q_>, \
                                      sizeof(ScanSmem<N_, Q_>), 64 * scan_waves_of(Q_))

@@ -70,7 +70,7 @@ __device__ __forceinline__ int8_t ssd_quantize_state(const QaSsdParams& p, int g
 
 // The shapes the matrix-core kernels are built for (everything else takes the general kernels)
 inline bool ssd_fast_shape(const QaSsdParams& p) {
-    if (p.headdim != 64 || (p.dstate != 64 && p.dstate != 128)) return false;
+    if (p.headdim % 64 != 0 || (p.dstate != 64 && p.dstate != 128)) return false;
     if (p.chunk_size != 64 && p.chunk_size != 128 && p.chunk_size != 256) return false;
     // x, B, C, the gate and the output are accessed in aligned 16-byte pieces there
     if (!aligned16(p.x) || !aligned16(p.B) || !aligned16(p.C) || !aligned16(p.out)) return false;

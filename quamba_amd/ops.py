@@ -775,12 +775,12 @@ def ssd_chunk_scan_combined_fwd(q_x, x_scale, q_dt, dt_scale, q_A_log, A_log_sca
         keep.append(t)
         return ptr(t)
 
-    # The matrix-core kernels are built for headdim 64, 64 or 128 states and chunks of 64, 128 or 256 steps; the
-    # library runs every other shape on general kernels.  Fewer than 128 states (the reference's tests use 16) with
-    # an otherwise fast shape run as 64 or 128 with zero codes in the added B and C columns: those states stay zero
-    # and add exactly nothing.
+    # The matrix-core kernels are built for head dimensions that are multiples of 64, 64 or 128 states and chunks of
+    # 64, 128 or 256 steps; the library runs every other shape on general kernels.  Fewer than 128 states (the
+    # reference's tests use 16) with an otherwise fast shape run as 64 or 128 with zero codes in the added B and C
+    # columns: those states stay zero and add exactly nothing.
     dstate_given = dstate
-    if headdim == 64 and chunk_size in (64, 128, 256) and dstate not in (64, 128) and dstate < 128:
+    if headdim % 64 == 0 and chunk_size in (64, 128, 256) and dstate not in (64, 128) and dstate < 128:
         dstate = 64 if dstate < 64 else 128
         q_B = torch.nn.functional.pad(q_B, (0, dstate - dstate_given))
         q_C = torch.nn.functional.pad(q_C, (0, dstate - dstate_given))

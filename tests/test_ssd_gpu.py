@@ -63,17 +63,22 @@ def test_forward_matches_oracle(dev, B, L, H, N, G, Q):
     assert np.abs(got - ref["final_f32"]).max() <= 1e-3 * np.abs(ref["final_f32"]).max()
 
 
-# Shapes outside what the matrix-core kernels are built for (head dimension 64, 64 or 128 states, chunks of 64, 128
-# or 256 steps) run on the library's general kernels, to the same bars.
+# Heads of 128, 192 and 256 channels run on the matrix-core kernels as two, three and four heads of 64 that share the
+# head's step sizes, decay and skip weight.  Shapes outside what those kernels are built for (head dimensions that are
+# not multiples of 64, state counts other than 64 and 128, chunks other than 64, 128 or 256 steps) run on the
+# library's general kernels, to the same bars.
 # batch, seqlen, nheads, headdim, dstate, ngroups, chunk
 GENERAL_SHAPES = [(1, 100, 4, 128, 128, 1, 64),      # the head dimension of the larger Mamba2 variants
+                  (2, 300, 2, 256, 64, 2, 128),
+                  (1, 520, 3, 192, 128, 1, 256),
+                  (1, 100, 4, 128, 128, 1, 96),      # the same head dimension on the general kernels
                   (2, 77, 4, 32, 16, 2, 32),         # small everything
                   (1, 300, 2, 64, 256, 1, 128),      # more states than one tile pair
                   (1, 200, 4, 64, 128, 1, 512),      # one chunk longer than the sequence
                   (1, 700, 2, 64, 64, 2, 512),       # a whole and a ragged chunk of 512
                   (2, 150, 4, 96, 48, 2, 100),       # nothing a multiple of 64
                   (1, 130, 6, 40, 24, 3, 48),
-                  (1, 65, 2, 256, 16, 1, 64),        # the largest head dimension
+                  (1, 65, 2, 256, 16, 1, 60),        # the largest head dimension
                   (1, 33, 3, 1, 1, 1, 7)]            # the smallest
 
 
@@ -88,15 +93,18 @@ def test_forward_of_other_shapes_matches_oracle(dev, B, L, H, P, N, G, Q):
     assert np.abs(got - ref["final_f32"]).max() <= 1e-3 * np.abs(ref["final_f32"]).max()
 
 
+# (96 channels, 80 states, chunks of 96: the general kernels; 128 channels in dim groups of 32, i.e. two to each half of
+# a head, and 192 channels in dim groups of 48 that straddle the thirds: the matrix-core kernels)
+@pytest.mark.parametrize("P,N,Q,ndg", [(96, 80, 96, 3), (128, 128, 128, 4), (192, 64, 64, 4)])
 @pytest.mark.parametrize("with_z,d_has_hdim", [(True, False), (False, True)])
-def test_other_shapes_with_grouped_scales_z_gate_and_int8_state(dev, with_z, d_has_hdim):
-    B, L, H, P, N, G, Q = 2, 150, 8, 96, 80, 2, 96
-    d = synth.mamba2_ssd_inputs(B, L, H, P, N, G, seed=6, grouped=True, nhead_groups=2, ndim_groups=3, with_z=with_z)
+def test_other_shapes_with_grouped_scales_z_gate_and_int8_state(dev, with_z, d_has_hdim, P, N, Q, ndg):
+    B, L, H, G = 2, 150, 8, 2
+    d = synth.mamba2_ssd_inputs(B, L, H, P, N, G, seed=6, grouped=True, nhead_groups=2, ndim_groups=ndg, with_z=with_z)
     if d_has_hdim:
         d["D"] = np.random.default_rng(1).integers(60, 128, (H, P)).astype(np.int8)
     ref = _oracle(d, Q)
     g = np.random.default_rng(2)
-    state_scale = (np.abs(ref["final_f32"]).max() / 127 * g.uniform(0.8, 1.2, (G, 2, 3, N))).astype(np.float32)
+    state_scale = (np.abs(ref["final_f32"]).max() / 127 * g.uniform(0.8, 1.2, (G, 2, ndg, N))).astype(np.float32)
     ref = _oracle(d, Q, state_scale=state_scale)
     y, final = _gpu(d, dev, Q, state_scale=state_scale, final_dtype=torch.int8)
     _check_y(y, ref["y"])
