@@ -229,9 +229,13 @@ __global__ __launch_bounds__(kConvThreads) void conv_update_kernel(QaConvParams 
     conv_step_row<false>(p, b, c, true);
 }
 
-int validate_common(const QaConvParams* p) {
-    if (!p || !p->x || !p->weight || !p->out) return QA_ERR_NULL;
+// (a call over no elements - no batch entries, no channels, forward: no steps - may pass null tensors)
+int validate_common(const QaConvParams* p, bool update) {
+    if (!p) return QA_ERR_NULL;
     if (p->batch < 0 || p->dim < 0 || p->seqlen < 0) return QA_ERR_SHAPE;
+    const bool empty = p->batch == 0 || p->dim == 0 || (!update && p->seqlen == 0);
+    if (!empty && (!p->x || !p->weight || !p->out)) return QA_ERR_NULL;
+    if (!empty && update && !p->conv_state) return QA_ERR_NULL;
     if (p->width < 2 || p->width > 4) return QA_ERR_SHAPE;
     return QA_OK;
 }
@@ -241,7 +245,7 @@ int validate_common(const QaConvParams* p) {
 
 extern "C" int qa_causal_conv1d_fwd(const QaConvParams* p, void* stream_) {
     using namespace qa;
-    int st = validate_common(p);
+    int st = validate_common(p, false);
     if (st != QA_OK) return st;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const int64_t total = static_cast<int64_t>(p->batch) * p->dim * p->seqlen;
@@ -303,9 +307,8 @@ extern "C" int qa_causal_conv1d_fwd(const QaConvParams* p, void* stream_) {
 
 extern "C" int qa_causal_conv1d_update(const QaConvParams* p, void* stream_) {
     using namespace qa;
-    int st = validate_common(p);
+    int st = validate_common(p, true);
     if (st != QA_OK) return st;
-    if (!p->conv_state) return QA_ERR_NULL;
     if (p->conv_state_len != p->width && p->conv_state_len != p->width - 1) return QA_ERR_SHAPE;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const int64_t total = static_cast<int64_t>(p->batch) * p->dim;

@@ -209,11 +209,14 @@ __global__ __launch_bounds__(kThreads) void conv2_update_kernel(QaConv2Params p)
 }
 
 int validate(const QaConv2Params* p, bool update) {
-    if (!p || !p->xBC || !p->weight || !p->x || !p->B || !p->C) return QA_ERR_NULL;
-    if (!p->x_out_scales || !p->B_out_scales || !p->C_out_scales) return QA_ERR_NULL;
-    if ((p->x_head_group_range == nullptr) != (p->x_dim_group_range == nullptr)) return QA_ERR_NULL;
-    if (update && !p->conv_state) return QA_ERR_NULL;
+    if (!p) return QA_ERR_NULL;
     if (p->batch < 0 || p->dim < 0 || p->seqlen < 0 || p->batch > 65535) return QA_ERR_SHAPE;
+    // (a call over no elements may pass null tensors)
+    const bool empty = p->batch == 0 || p->dim == 0 || (!update && p->seqlen == 0);
+    if (!empty && (!p->xBC || !p->weight || !p->x || !p->B || !p->C)) return QA_ERR_NULL;
+    if (!empty && (!p->x_out_scales || !p->B_out_scales || !p->C_out_scales)) return QA_ERR_NULL;
+    if ((p->x_head_group_range == nullptr) != (p->x_dim_group_range == nullptr)) return QA_ERR_NULL;
+    if (!empty && update && !p->conv_state) return QA_ERR_NULL;
     if (p->width < 2 || p->width > 4) return QA_ERR_SHAPE;
     if (p->x_dim < 0 || p->x_headdim < 1 || p->d_state < 1 || p->n_groups < 1) return QA_ERR_SHAPE;
     if (p->x_dim % p->x_headdim != 0 || p->x_dim % p->n_groups != 0) return QA_ERR_SHAPE;

@@ -6,6 +6,21 @@ namespace {
 thread_local int g_last_hip_error = 0;
 }
 void set_last_hip_error(int code) { g_last_hip_error = code; }
+
+namespace {
+__global__ __launch_bounds__(256) void fill_zero_kernel(uint8_t* dst, int64_t bytes) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i < bytes) dst[i] = 0;
+}
+}  // namespace
+
+int fill_zero(void* dst, int64_t bytes, hipStream_t stream) {
+    if (!dst || bytes <= 0) return QA_OK;
+    const int64_t blocks = (bytes + 255) / 256;
+    if (blocks > 0x7fffffffLL) return QA_ERR_SHAPE;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, static_cast<uint8_t*>(dst), bytes);
+    return check_launch();
+}
 }  // namespace qa
 
 extern "C" const char* qa_status_string(int status) {

@@ -410,10 +410,12 @@ __global__ __launch_bounds__(256) void w4_expand_kernel(QaGemmW4A8Params p, int8
 
 extern "C" int qa_gemm_w4a8(const QaGemmW4A8Params* p, void* stream_) {
     using namespace qa;
-    if (!p || !p->a || !p->w_packed || !p->s_channel || !p->s_token || !p->d) return QA_ERR_NULL;
+    if (!p) return QA_ERR_NULL;
     if (p->m < 0 || p->n < 0 || p->k < 0) return QA_ERR_SHAPE;
+    const bool empty = p->m == 0 || p->n == 0;                      // (an output without elements: tensors may be null)
+    if (!empty && (!p->a || !p->w_packed || !p->s_channel || !p->s_token || !p->d)) return QA_ERR_NULL;
     if (p->group_size != 128 && p->group_size != -1) return QA_ERR_UNSUPPORTED;
-    if (p->group_size == 128 && !p->s_group) return QA_ERR_NULL;
+    if (!empty && p->group_size == 128 && !p->s_group) return QA_ERR_NULL;
     if (p->out_type != QA_OUT_I8 && p->out_type != QA_OUT_F16) return QA_ERR_UNSUPPORTED;
     if (p->tok_scale_numel != 1 && p->tok_scale_numel != p->m) return QA_ERR_SHAPE;
     if (p->k % 128 != 0) return QA_ERR_SHAPE;                       // whole 128-code groups / k tiles

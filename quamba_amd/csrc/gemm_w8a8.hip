@@ -315,9 +315,11 @@ int dispatch_skinny(const QaGemmW8A8Params& p, hipStream_t stream) {
 
 extern "C" int qa_gemm_w8a8(const QaGemmW8A8Params* p, void* stream_) {
     using namespace qa;
-    if (!p || !p->a || !p->w || !p->d) return QA_ERR_NULL;
-    if (!p->use_alpha && (!p->a_scale || !p->w_scale)) return QA_ERR_NULL;
+    if (!p) return QA_ERR_NULL;
     if (p->m < 0 || p->n < 0 || p->k < 0) return QA_ERR_SHAPE;
+    const bool empty = p->m == 0 || p->n == 0;                      // (an output without elements: tensors may be null)
+    if (!empty && (!p->a || !p->w || !p->d)) return QA_ERR_NULL;
+    if (!empty && !p->use_alpha && (!p->a_scale || !p->w_scale)) return QA_ERR_NULL;
     if (p->out_type != QA_OUT_I8 && p->out_type != QA_OUT_F16 && p->out_type != QA_OUT_BF16) return QA_ERR_UNSUPPORTED;
     if (p->scale_order != 0 && p->scale_order != 1) return QA_ERR_UNSUPPORTED;
     if (p->scale_order == 1 && (p->use_alpha || p->round_mode != QA_ROUND_RNE)) return QA_ERR_UNSUPPORTED;

@@ -139,8 +139,9 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) void rmsnorm_gated_kernel(QaNo
 
 extern "C" int qa_rmsnorm_gated(const QaNormGatedParams* p, void* stream_) {
     using namespace qa;
-    if (!p || !p->x || !p->weight || !p->out) return QA_ERR_NULL;
-    if (p->out_mode == QA_NORM_OUT_I8_DYNAMIC && !p->dyn_scale) return QA_ERR_NULL;
+    if (!p) return QA_ERR_NULL;
+    if (p->rows > 0 && (!p->x || !p->weight || !p->out)) return QA_ERR_NULL;      // (no rows: the tensors may be null)
+    if (p->rows > 0 && p->out_mode == QA_NORM_OUT_I8_DYNAMIC && !p->dyn_scale) return QA_ERR_NULL;
     if (p->out_mode < 0 || p->out_mode > 2) return QA_ERR_UNSUPPORTED;
     if (p->rows < 0 || p->dim < 1 || p->group_size < 1 || p->dim % p->group_size != 0) return QA_ERR_SHAPE;
     if (p->group_size % 8 != 0 || p->group_size > kMaxPieces * kWavesPerBlock * 512) return QA_ERR_UNSUPPORTED;

@@ -14,6 +14,10 @@ namespace qa {
 // Records the HIP error of a failed launch for qa_last_hip_error().
 void set_last_hip_error(int code);
 
+// Zeroes `bytes` bytes with a kernel (states after a scan over no steps; a memset node would not survive graph capture
+// on every runtime).  Null or empty: nothing to do.
+int fill_zero(void* dst, int64_t bytes, hipStream_t stream);
+
 inline int check_launch() {
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {

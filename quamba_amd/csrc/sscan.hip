@@ -1243,15 +1243,25 @@ extern "C" int qa_sscan_chosen_mapping(const QaSScanParams* p) {
 
 extern "C" int qa_sscan_fwd(const QaSScanParams* p, void* stream_) {
     using namespace qa;
-    if (!p || !p->u || !p->delta || !p->A_log || !p->B || !p->C || !p->out) return QA_ERR_NULL;
+    if (!p) return QA_ERR_NULL;
+    if (p->batch < 0 || p->dim < 0 || p->seqlen < 0 || p->dstate < 1 || p->dstate > 256) return QA_ERR_SHAPE;
+    if (p->n_groups < 1 || (p->dim > 0 && p->dim % p->n_groups != 0)) return QA_ERR_SHAPE;
+    if (p->batch == 0 || p->dim == 0) return QA_OK;                 // (no channel rows: the tensors may be null)
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (p->seqlen == 0) {
+        // no steps (the step tensors may be null): a scan from the zero state ends in the zero state
+        if (p->carry_state || p->carry_dt_sum) return QA_ERR_SHAPE;
+        const int64_t rows = static_cast<int64_t>(p->batch) * p->dim;
+        int st = fill_zero(p->last_state_i8, rows * p->dstate, stream);
+        if (st == QA_OK) st = fill_zero(p->last_state_f32, rows * p->dstate * 4, stream);
+        if (st == QA_OK) st = fill_zero(p->dt_sum_out, rows * 4, stream);
+        return st;
+    }
+    if (!p->u || !p->delta || !p->A_log || !p->B || !p->C || !p->out) return QA_ERR_NULL;
     if (!p->scale_u || !p->scale_delta || !p->scale_A || !p->scale_B || !p->scale_C) return QA_ERR_NULL;
     if ((p->D && !p->scale_D) || (p->delta_bias && !p->scale_delta_bias) || (p->z && !p->scale_z)) return QA_ERR_NULL;
     if (p->last_state_i8 && !p->scale_ssm_state) return QA_ERR_NULL;
-    if (p->batch < 0 || p->dim < 0 || p->seqlen < 0 || p->dstate < 1 || p->dstate > 256) return QA_ERR_SHAPE;
-    if (p->n_groups < 1 || (p->dim > 0 && p->dim % p->n_groups != 0)) return QA_ERR_SHAPE;
-    if (p->batch == 0 || p->dim == 0) return QA_OK;
     if (p->batch > 65535) return QA_ERR_SHAPE;
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
 
     auto ok16 = [](const void* ptr, std::initializer_list<int64_t> strides) {
         if (!aligned16(ptr)) return 0;
@@ -1319,7 +1329,9 @@ extern "C" int qa_sscan_fwd(const QaSScanParams* p, void* stream_) {
 namespace qa {
 namespace {
 int validate_update(const QaSsmUpdateParams* p, bool needs_x) {
-    if (!p || !p->state || (needs_x && !p->x) || !p->dt || !p->A_log || !p->B || !p->C || !p->out) return QA_ERR_NULL;
+    if (!p) return QA_ERR_NULL;
+    if (p->batch == 0 && p->nheads >= 1 && p->dim >= 0) return QA_OK;      // (no batch entries: the tensors may be null)
+    if (!p->state || (needs_x && !p->x) || !p->dt || !p->A_log || !p->B || !p->C || !p->out) return QA_ERR_NULL;
     if (!p->x_scale || !p->dt_scale || !p->A_log_scale || !p->B_scale || !p->C_scale) return QA_ERR_NULL;
     if (!p->state_is_fp32 && !p->state_scale) return QA_ERR_NULL;
     if ((p->D && !p->D_scale) || (p->z && !p->z_scale)) return QA_ERR_NULL;
@@ -1351,7 +1363,9 @@ extern "C" int qa_mamba1_decode_step(const QaConvParams* conv, const QaSsmUpdate
     using namespace qa;
     const int st = validate_update(p, false);
     if (st != QA_OK) return st;
-    if (!conv || !conv->x || !conv->weight || !conv->conv_state) return QA_ERR_NULL;
+    if (!conv) return QA_ERR_NULL;
+    if (p->batch == 0 && conv->batch == 0) return QA_OK;
+    if (!conv->x || !conv->weight || !conv->conv_state) return QA_ERR_NULL;
     if (conv->width < 2 || conv->width > 4) return QA_ERR_SHAPE;
     if (conv->conv_state_len != conv->width && conv->conv_state_len != conv->width - 1) return QA_ERR_SHAPE;
     if (conv->batch != p->batch || conv->dim != p->dim) return QA_ERR_SHAPE;

@@ -667,13 +667,16 @@ __global__ __launch_bounds__(64 * scan_waves_of(Q), 4) void ssd_chunk_scan_kerne
 }
 
 int validate(const QaSsdParams* p) {
-    if (!p || !p->x || !p->dt || !p->A_log || !p->B || !p->C || !p->out) return QA_ERR_NULL;
-    if (!p->x_scale || !p->A_log_scale || !p->B_scale || !p->C_scale) return QA_ERR_NULL;
-    if (!p->dt_is_fp32 && !p->dt_scale) return QA_ERR_NULL;
-    if ((p->D && !p->D_scale) || (p->z && !p->z_scale)) return QA_ERR_NULL;
-    if (p->final_states && !p->final_state_is_fp32 && !p->state_scale) return QA_ERR_NULL;
-    if (p->nhead_groups > 0 && (!p->x_head_group_range || !p->x_dim_group_range || p->ndim_groups < 1)) return QA_ERR_NULL;
+    if (!p) return QA_ERR_NULL;
     if (p->batch < 0 || p->seqlen < 0 || p->nheads < 1 || p->ngroups < 1 || p->nheads % p->ngroups != 0) return QA_ERR_SHAPE;
+    if (p->batch > 0 && p->seqlen > 0) {                          // (no steps: the tensors may be null)
+        if (!p->x || !p->dt || !p->A_log || !p->B || !p->C || !p->out) return QA_ERR_NULL;
+        if (!p->x_scale || !p->A_log_scale || !p->B_scale || !p->C_scale) return QA_ERR_NULL;
+        if (!p->dt_is_fp32 && !p->dt_scale) return QA_ERR_NULL;
+        if ((p->D && !p->D_scale) || (p->z && !p->z_scale)) return QA_ERR_NULL;
+        if (p->final_states && !p->final_state_is_fp32 && !p->state_scale) return QA_ERR_NULL;
+        if (p->nhead_groups > 0 && (!p->x_head_group_range || !p->x_dim_group_range || p->ndim_groups < 1)) return QA_ERR_NULL;
+    }
     // what the general kernels take; the matrix-core kernels cover a subset (ssd_fast_shape)
     if (p->headdim < 1 || p->headdim > 256 || p->dstate < 1 || p->dstate > 1024 || p->chunk_size < 1 || p->chunk_size > 1024) return QA_ERR_UNSUPPORTED;
     const int64_t nc = (static_cast<int64_t>(p->seqlen) + p->chunk_size - 1) / p->chunk_size;
@@ -701,7 +704,12 @@ extern "C" int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream_) {
     using namespace qa;
     const int st = validate(p);
     if (st != QA_OK) return st;
-    if (p->batch == 0 || p->seqlen == 0) return QA_OK;
+    if (p->batch == 0) return QA_OK;
+    if (p->seqlen == 0) {
+        // no steps: the state after them is the zero state the scan starts from
+        const int64_t states = static_cast<int64_t>(p->batch) * p->nheads * p->headdim * p->dstate;
+        return fill_zero(p->final_states, states * (p->final_state_is_fp32 ? 4 : 1), static_cast<hipStream_t>(stream_));
+    }
     const SsdWorkspace ws = ssd_workspace_layout(*p);
     if (!p->workspace) return QA_ERR_NULL;
     if (p->workspace_bytes < ws.total || (reinterpret_cast<uintptr_t>(p->workspace) & 255u)) return QA_ERR_STRIDE;
@@ -794,7 +802,7 @@ extern "C" int qa_ssd_chunk_scan_fwd_noalloc(const QaSsdParams* p, void* stream_
     using namespace qa;
     const int st = validate(p);
     if (st != QA_OK) return st;
-    if (p->batch == 0 || p->seqlen == 0) return QA_OK;
+    if (p->batch == 0 || p->seqlen == 0) return qa_ssd_chunk_scan_fwd(p, stream_);      // (nothing needs a workspace)
     if (ssd_workspace_layout(*p).total > kStaticScratchBytes) return QA_ERR_SCRATCH;
     void* ptr = static_scratch_of_current_device();
     if (!ptr) return QA_ERR_LAUNCH;

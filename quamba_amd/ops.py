@@ -64,7 +64,7 @@ def causal_conv1d_fwd(x, scale_x, weight, scale_w, scale_out, scale_b, bias=None
     p.scale_x, p.scale_w, p.scale_b, p.scale_out = float(scale_x), float(scale_w), float(scale_b), float(scale_out)
     out_t = None
     if also_channel_last:
-        _require(x.stride(2) == 1 and x.stride(1) % 16 == 0 and x.stride(0) % 16 == 0 and x.data_ptr() % 16 == 0,
+        _require(x.numel() == 0 or (x.stride(2) == 1 and x.stride(1) % 16 == 0 and x.stride(0) % 16 == 0 and x.data_ptr() % 16 == 0),
                  "also_channel_last needs a seqlen-contiguous input with 16-byte aligned rows")
         out_t = torch.empty((batch, seqlen, dim), dtype=torch.int8, device=x.device)
         p.out_t = ptr(out_t)
@@ -837,7 +837,10 @@ def ssd_chunk_scan_combined_fwd(q_x, x_scale, q_dt, dt_scale, q_A_log, A_log_sca
     nbytes = lib.qa_ssd_workspace_bytes(ct.byref(p))
     if nbytes <= 0:
         # an invalid request (the call reports which way), or an empty one (nothing to do)
-        _lib.check(lib.qa_ssd_chunk_scan_fwd(ct.byref(p), None), "ssd_chunk_scan_fwd")
+        with torch.cuda.device(dev):
+            _lib.check(lib.qa_ssd_chunk_scan_fwd(ct.byref(p), _lib.current_stream(dev)), "ssd_chunk_scan_fwd")
+        if dstate != dstate_given:
+            final = final[..., :dstate_given].contiguous()
         return (out, final, None) if return_workspace else (out, final)
     if static_scratch:
         _require(not return_workspace, "the library's own scratch buffer cannot be returned")

@@ -91,20 +91,71 @@ def test_validation_codes_without_a_gpu():
     l = _lib.lib()
     assert l.qa_causal_conv1d_fwd(None, None) == -1
     p = _lib.QaConvParams()
+    p.batch, p.dim, p.seqlen, p.width = 1, 8, 16, 4
     assert l.qa_causal_conv1d_fwd(C.byref(p), None) == -1          # null pointers
     p.x = p.weight = p.out = 16                                     # never dereferenced on these paths
-    p.batch, p.dim, p.seqlen, p.width = 1, 8, 16, 5
+    p.width = 5
     assert l.qa_causal_conv1d_fwd(C.byref(p), None) == -2          # width outside [2,4]
     p.width = 4
     p.x_l_stride, p.x_c_stride = 3, 5
     assert l.qa_causal_conv1d_fwd(C.byref(p), None) == -3          # neither dimension contiguous
     p.seqlen = 0
     assert l.qa_causal_conv1d_fwd(C.byref(p), None) == 0           # empty input: nothing to launch
+    x, p.x, p.out = p.x, 0, 0
+    assert l.qa_causal_conv1d_fwd(C.byref(p), None) == 0           # tensors without elements may be null
+    p.x = p.out = x
     p.seqlen, p.x_l_stride = 1, 1
     assert l.qa_causal_conv1d_update(C.byref(p), None) == -1       # conv_state missing
     p.conv_state = 16
     p.conv_state_len = 7
     assert l.qa_causal_conv1d_update(C.byref(p), None) == -2
+
+
+def test_calls_over_no_elements_need_no_tensors():
+    """Every entry point accepts null tensors when the sizes say there is nothing to read or write (an empty torch
+    tensor has a null data pointer, and so has an empty std::vector), and returns before any HIP call."""
+    l = _lib.lib()
+    conv = _lib.QaConvParams()
+    conv.dim, conv.seqlen, conv.width, conv.conv_state_len = 64, 16, 4, 4
+    assert l.qa_causal_conv1d_fwd(C.byref(conv), None) == 0
+    assert l.qa_causal_conv1d_update(C.byref(conv), None) == 0
+    conv2 = _lib.QaConv2Params()
+    conv2.dim, conv2.seqlen, conv2.width, conv2.x_dim, conv2.x_headdim, conv2.d_state, conv2.n_groups = 96, 16, 4, 64, 64, 16, 1
+    conv2.xBC_c_stride = conv2.x_c_stride = conv2.B_c_stride = conv2.C_c_stride = 1
+    conv2.conv_state_len = 4
+    assert l.qa_quamba2_conv1d_fwd(C.byref(conv2), None) == 0
+    assert l.qa_quamba2_conv1d_update(C.byref(conv2), None) == 0
+    had = _lib.QaHadamardParams()
+    had.dim = had.x_row_stride = had.out_row_stride = 5120
+    assert l.qa_hadamard_quant(C.byref(had), None) == 0
+    norm = _lib.QaNormGatedParams()
+    norm.dim = norm.group_size = norm.x_row_stride = norm.out_row_stride = 256
+    assert l.qa_rmsnorm_gated(C.byref(norm), None) == 0
+    scan = _lib.QaSScanParams()
+    scan.dim, scan.seqlen, scan.dstate, scan.n_groups = 64, 16, 16, 1
+    assert l.qa_sscan_fwd(C.byref(scan), None) == 0
+    upd = _lib.QaSsmUpdateParams()
+    upd.nheads, upd.dim, upd.dstate, upd.ngroups = 1, 64, 16, 1
+    assert l.qa_ssm_state_update(C.byref(upd), None) == 0
+    assert l.qa_mamba1_decode_step(C.byref(conv), C.byref(upd), None) == 0
+    for m, n in ((0, 64), (16, 0)):
+        g8 = _lib.QaGemmW8A8Params()
+        g8.m, g8.n, g8.k, g8.lda, g8.ldw, g8.ldd = m, n, 128, 128, 128, n
+        g8.a_scale_numel = g8.w_scale_numel = 1
+        assert l.qa_gemm_w8a8(C.byref(g8), None) == 0
+        g4 = _lib.QaGemmW4A8Params()
+        g4.m, g4.n, g4.k, g4.lda, g4.ldd, g4.group_size, g4.tok_scale_numel = m, n, 128, 128, n, 128, 1
+        assert l.qa_gemm_w4a8(C.byref(g4), None) == 0
+    ssd = _lib.QaSsdParams()
+    ssd.seqlen, ssd.nheads, ssd.headdim, ssd.dstate, ssd.ngroups, ssd.chunk_size = 100, 4, 64, 128, 1, 64
+    assert l.qa_ssd_chunk_scan_fwd(C.byref(ssd), None) == 0
+    assert l.qa_ssd_chunk_scan_fwd_noalloc(C.byref(ssd), None) == 0
+    # sizes that say there is something to do still need their tensors
+    conv.batch, scan.batch, ssd.batch, had.rows = 1, 1, 1, 1
+    assert l.qa_causal_conv1d_fwd(C.byref(conv), None) == -1
+    assert l.qa_sscan_fwd(C.byref(scan), None) == -1
+    assert l.qa_ssd_chunk_scan_fwd(C.byref(ssd), None) == -1
+    assert l.qa_hadamard_quant(C.byref(had), None) == -1
 
 
 def test_missing_library_fails_loudly(monkeypatch):
