@@ -6,6 +6,8 @@
  * library never allocates, never synchronises and keeps no mutable global state, so calls are
  * re-entrant and can be captured into HIP graphs.  All pointers are device pointers unless said
  * otherwise.  Strides count elements, not bytes.  Return value: QA_OK (0) or a negative QaStatus.
+ * A call whose sizes leave nothing to compute (no batch entries, rows or steps) returns QA_OK without a
+ * launch, and its tensors may then be null; a scan over no steps writes the zero state it starts from.
  *
  * Each entry point names the interface of the reference (enyac-group/Quamba, paths relative to
  * its root) that it replaces.
