@@ -17,6 +17,11 @@
 namespace qa {
 namespace {
 
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
 constexpr int kT = 64;            // tile edge: steps, states, channels of the chunk scan
 constexpr int kTP = 32;           // channels per workgroup of the state kernel
 constexpr int kThreads = 256;
@@ -175,24 +180,35 @@ __global__ __launch_bounds__(kThreads) void ssd_general_state_kernel(QaSsdParams
 }
 
 // ---------------------------------------------------------------------------------------------
-// Stages 4 and 5 (quamba/triton/quant_bmm_chunk.py:60-66, quant_chunk_scan.py:96-171).  A workgroup per (batch,
-// chunk, head, 64 rows m, 64 channels p); a thread owns four rows and four channels.  Term 1 walks the states in
-// tiles of 64; term 2 walks the steps k up to the diagonal in tiles of 64, forming the tile's integer C B^T itself
-// (a thread: four rows m x four steps k, states in tiles of 64) and from it the fp16 weights.
+// Stages 4 and 5 (quamba/triton/quant_bmm_chunk.py:60-66, quant_chunk_scan.py:96-171).  A workgroup of four waves per
+// (batch, chunk, head, 64 rows m, 64 channels p); a wave owns sixteen rows and all 64 channels (four accumulator
+// tiles of v_mfma_f32_16x16x32_f16: a lane holds rows 4 (lane / 16) + r, channel 16 j + lane % 16).
+// Term 1 walks the states in tiles of 64: C^ converted in registers from the codes in LDS, the entering state as rows
+// of channels.  Term 2 walks the steps k up to the diagonal in tiles of 64: v_mfma_i32_16x16x64_i8 forms the tile's
+// integer (C B^T)^T from the codes (exact), a lane turns its four steps of a row into fp16 weights, the wave passes
+// them through its own rows of LDS into operand order, and x^ waits there transposed ([channel][step]).
+// Everything past an edge (rows, steps, states, channels) is zero in LDS, so the products need no bounds.
 // ---------------------------------------------------------------------------------------------
 struct GeneralScanSmem {
-    union {
-        struct { float ct[kT][kT]; float pt[kT][kT]; } one;                                  // [state][row m], [state][channel]
-        struct { float wt[kT][kT]; float xh[kT][kT]; uint32_t cq[kT][17]; uint32_t bq[kT][17]; } two;   // [step][row m], [step][channel]; codes, four to a word
-    };
+    // 16 pad bytes per row: the sixteen rows of an operand read fall into different banks
+    __attribute__((aligned(16))) int8_t cq[kT][kT + 16];         // C codes of the rows m, one tile of 64 states
+    __attribute__((aligned(16))) int8_t bq[kT][kT + 16];         // B codes of the steps k
+    __attribute__((aligned(16))) _Float16 wt[kT][kT + 8];        // weights [row m][step k]
+    __attribute__((aligned(16))) _Float16 xt[kT][kT + 8];        // term 2: x^ [channel][step k]; term 1: entering state [channel][state]
     float dA_m[kT], dA_k[kT], dt_k[kT], xs[kT], Dv[kT];
 };
 
-__global__ __launch_bounds__(kThreads) void ssd_general_chunk_scan_kernel(QaSsdParams p, const float* dt_ws, const float* dA_ws, const __half* prev, int nc) {
-    __shared__ __attribute__((aligned(16))) GeneralScanSmem sm;
+// what the tensors' sizes and addresses allow (chosen on the host)
+constexpr int kVecCodes = 1;      // B, C: rows of 16-byte pieces
+constexpr int kVecX = 2;          // x: four channels per aligned word
+constexpr int kVecState = 4;      // entering state: rows of 16-byte pieces
+
+__global__ __launch_bounds__(kThreads) void ssd_general_chunk_scan_kernel(QaSsdParams p, const float* dt_ws, const float* dA_ws, const __half* prev, int nc, int vec) {
+    __shared__ GeneralScanSmem sm;
     const int P = p.headdim, N = p.dstate, Q = p.chunk_size, H = p.nheads, G = p.ngroups, L = p.seqlen;
     const int ptiles = (P + kT - 1) / kT, mtiles = (Q + kT - 1) / kT;
-    const int tid = threadIdx.x, tm = tid / 16, tq = tid % 16;
+    const int tid = threadIdx.x, lane = tid & 63, l16 = lane & 15, lq = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     unsigned idx = blockIdx.x;
     const int p0 = static_cast<int>(idx % ptiles) * kT; idx /= ptiles;
     const int m0 = static_cast<int>(idx % mtiles) * kT; idx /= mtiles;
@@ -220,51 +236,81 @@ __global__ __launch_bounds__(kThreads) void ssd_general_chunk_scan_kernel(QaSsdP
         sm.Dv[tid] = (!p.D || pp >= P) ? 0.0f : *p.D_scale * static_cast<float>(p.D_has_hdim ? p.D[h * P + pp] : p.D[h]);
         sm.dA_m[tid] = dA_row[min(m0 + tid, Q - 1)];
     }
-    float acc[4][4];
+
+    // 64 rows x 64 codes of B or C (rows from `first`, states from n0) into LDS: a thread moves one 16-byte piece
+    auto stage_codes = [&](int8_t (*dst)[kT + 16], const int8_t* rows0, int first, int n0) {
+        const int r = tid / 4, q = tid % 4, row = first + r, n = n0 + 16 * q;
+        uint4 v = make_uint4(0u, 0u, 0u, 0u);
+        if (row < lim && n < N) {
+            const int8_t* src = rows0 + row * cstep + n;
+            if ((vec & kVecCodes) && n + 16 <= N) {
+                v = *reinterpret_cast<const uint4*>(src);
+            } else {
+                uint32_t w[4] = {0u, 0u, 0u, 0u};
+                for (int e = 0; e < 16 && n + e < N; ++e) w[e / 4] |= static_cast<uint32_t>(static_cast<uint8_t>(src[e])) << (8 * (e % 4));
+                v = make_uint4(w[0], w[1], w[2], w[3]);
+            }
+        }
+        *reinterpret_cast<uint4*>(&dst[r][16 * q]) = v;
+    };
+
+    v4f acc[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = 0.0f;
+    for (int j = 0; j < 4; ++j) acc[j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
 
     // term 1: C^ (rows m) x the state entering the chunk (rows p); zero for the first chunk
     if (c > 0) {
         const __half* pst = prev + ((static_cast<int64_t>(b) * nc + c) * H + h) * P * N;
         for (int n0 = 0; n0 < N; n0 += kT) {
-            __syncthreads();
-            for (int i = tid; i < kT * kT; i += kThreads) {
-                const int r = i / kT, nn = i % kT;
-                float cv = 0.0f, pv = 0.0f;
-                if (n0 + nn < N) {
-                    if (m0 + r < lim) cv = f16r(sC * static_cast<float>(Crow0[(m0 + r) * cstep + n0 + nn]));
-                    if (p0 + r < P) pv = __half2float(pst[static_cast<int64_t>(p0 + r) * N + n0 + nn]);
+            __syncthreads();                                       // the tile before is consumed
+            stage_codes(sm.cq, Crow0, m0, n0);
+            {
+                // the entering state of 64 channels x 64 states: a thread moves sixteen states of one channel
+                const int r = tid / 4, q = tid % 4, pp = p0 + r, n = n0 + 16 * q;
+                uint4 v0 = make_uint4(0u, 0u, 0u, 0u), v1 = v0;
+                if (pp < P && n < N) {
+                    const __half* src = pst + static_cast<int64_t>(pp) * N + n;
+                    if ((vec & kVecState) && n + 16 <= N) {
+                        v0 = *reinterpret_cast<const uint4*>(src);
+                        v1 = *reinterpret_cast<const uint4*>(src + 8);
+                    } else {
+                        uint32_t w[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};
+                        for (int e = 0; e < 16 && n + e < N; ++e) w[e / 2] |= static_cast<uint32_t>(__half_as_ushort(src[e])) << (16 * (e % 2));
+                        v0 = make_uint4(w[0], w[1], w[2], w[3]);
+                        v1 = make_uint4(w[4], w[5], w[6], w[7]);
+                    }
                 }
-                // (a thread's row r is a column here: the 16-byte pieces of a row are exchanged by the state's low bits,
-                // so that the 64 states a wave writes do not all fall into one bank)
-                sm.one.ct[nn][r ^ ((nn & 15) << 2)] = cv;
-                sm.one.pt[nn][r ^ ((nn & 15) << 2)] = pv;
+                *reinterpret_cast<uint4*>(&sm.xt[r][16 * q]) = v0;
+                *reinterpret_cast<uint4*>(&sm.xt[r][16 * q + 8]) = v1;
             }
             __syncthreads();
-            const int states = min(kT, N - n0);
-            for (int nn = 0; nn < states; ++nn) {
-                const float4 cv = *reinterpret_cast<const float4*>(&sm.one.ct[nn][(4 * tm) ^ ((nn & 15) << 2)]);
-                const float4 pv = *reinterpret_cast<const float4*>(&sm.one.pt[nn][(4 * tq) ^ ((nn & 15) << 2)]);
-                const float cvv[4] = {cv.x, cv.y, cv.z, cv.w}, pvv[4] = {pv.x, pv.y, pv.z, pv.w};
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
+            for (int ks = 0; ks < 2; ++ks) {
+                const uint2 cw = *reinterpret_cast<const uint2*>(&sm.cq[16 * wave + l16][32 * ks + 8 * lq]);
+                v8h cf;
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) acc[i][j] += cvv[i] * pvv[j];
+                for (int e = 0; e < 4; ++e) {
+                    cf[e] = static_cast<_Float16>(sC * static_cast<float>(static_cast<int8_t>((cw.x >> (8 * e)) & 0xffu)));
+                    cf[4 + e] = static_cast<_Float16>(sC * static_cast<float>(static_cast<int8_t>((cw.y >> (8 * e)) & 0xffu)));
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const v8h pf = *reinterpret_cast<const v8h*>(&sm.xt[16 * j + l16][32 * ks + 8 * lq]);
+                    acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(cf, pf, acc[j], 0, 0, 0);
+                }
             }
         }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const float em = ssd_exp(sm.dA_m[4 * tm + i]);
+        for (int r = 0; r < 4; ++r) {
+            const float em = ssd_exp(sm.dA_m[16 * wave + 4 * lq + r]);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) acc[i][j] *= em;
+            for (int j = 0; j < 4; ++j) acc[j][r] *= em;
         }
     }
 
     // term 2: steps k <= m, tiles of 64 steps up to the one that holds the last row's diagonal
     const int k_end = min(m0 + kT, lim);
+    const int m_last = m0 + 16 * wave + 15;                        // the wave's last row
     for (int k0 = 0; k0 < k_end; k0 += kT) {
         __syncthreads();                                           // the tiles before are consumed
         if (tid < kT) {
@@ -272,89 +318,92 @@ __global__ __launch_bounds__(kThreads) void ssd_general_chunk_scan_kernel(QaSsdP
             sm.dA_k[tid] = dA_row[min(k, Q - 1)];
             sm.dt_k[tid] = k < lim ? dt_row[k] : 0.0f;
         }
-        // integer C B^T of the tile: rows 4 tm .. + 3, steps 4 tq .. + 3
-        int cb[4][4];
+        {
+            // x^ of 64 steps x 64 channels, transposed: a thread takes four steps of four channels
+            const int kb = tid / 16, pq = tid % 16;
+            uint32_t xw[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) cb[i][j] = 0;
-        for (int n0 = 0; n0 < N; n0 += kT) {
-            if (n0 > 0) __syncthreads();
-            for (int i = tid; i < kT * 16; i += kThreads) {
-                const int r = i / 16, w = i % 16;
-                uint32_t cw = 0u, bwd = 0u;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int nn = n0 + 4 * w + e;
-                    if (nn < N) {
-                        if (m0 + r < lim) cw |= static_cast<uint32_t>(static_cast<uint8_t>(Crow0[(m0 + r) * cstep + nn])) << (8 * e);
-                        if (k0 + r < lim) bwd |= static_cast<uint32_t>(static_cast<uint8_t>(Brow0[(k0 + r) * cstep + nn])) << (8 * e);
+            for (int r = 0; r < 4; ++r) {
+                const int k = k0 + 4 * kb + r, pp = p0 + 4 * pq;
+                xw[r] = 0u;
+                if (k < lim && pp < P) {
+                    const int8_t* src = xrow0 + k * xstep + pp;
+                    if ((vec & kVecX) && pp + 4 <= P) {
+                        xw[r] = *reinterpret_cast<const uint32_t*>(src);
+                    } else {
+                        for (int e = 0; e < 4 && pp + e < P; ++e) xw[r] |= static_cast<uint32_t>(static_cast<uint8_t>(src[e])) << (8 * e);
                     }
                 }
-                sm.two.cq[r][w] = cw;
-                sm.two.bq[r][w] = bwd;
             }
+#pragma unroll
+            for (int cc = 0; cc < 4; ++cc) {
+                const float sc = sm.xs[4 * pq + cc];               // (written before the first barrier of this kernel)
+                v4h v;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) v[r] = static_cast<_Float16>(sc * static_cast<float>(static_cast<int8_t>((xw[r] >> (8 * cc)) & 0xffu)));
+                *reinterpret_cast<v4h*>(&sm.xt[4 * pq + cc][4 * kb]) = v;
+            }
+        }
+        // integer (C B^T)^T of the wave's rows: block kb holds steps 16 kb + 4 (lane / 16) + r of row lane % 16
+        v4i cb[4];
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb) cb[kb] = v4i{0, 0, 0, 0};
+        for (int n0 = 0; n0 < N; n0 += kT) {
+            if (n0 > 0) __syncthreads();
+            stage_codes(sm.cq, Crow0, m0, n0);
+            stage_codes(sm.bq, Brow0, k0, n0);
             __syncthreads();
-#pragma unroll 4
-            for (int w = 0; w < 16; ++w) {
-                uint32_t cw[4], bwd[4];
+            const v4i co = *reinterpret_cast<const v4i*>(&sm.cq[16 * wave + l16][16 * lq]);
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    cw[i] = sm.two.cq[4 * tm + i][w];
-                    bwd[i] = sm.two.bq[4 * tq + i][w];
+            for (int kb = 0; kb < 4; ++kb) {
+                if (k0 + 16 * kb <= m_last) {                      // (blocks wholly above the diagonal stay zero)
+                    const v4i bo = *reinterpret_cast<const v4i*>(&sm.bq[16 * kb + l16][16 * lq]);
+                    cb[kb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bo, co, cb[kb], 0, 0, 0);
                 }
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) cb[i][j] = __builtin_amdgcn_sdot4(static_cast<int>(cw[i]), static_cast<int>(bwd[j]), cb[i][j], false);
             }
         }
-        // the weights, rounded to fp16 where the reference rounds them, as [step][row]; x^ as [step][channel]
+        // the weights, rounded to fp16 where the reference rounds them, into the wave's own rows of LDS
+        {
+            const int m = m0 + 16 * wave + l16;
+            const float dAm = sm.dA_m[16 * wave + l16];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int k = k0 + 4 * tq + j;
-            float wv[4];
+            for (int kb = 0; kb < 4; ++kb) {
+                v4h wv;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int m = m0 + 4 * tm + i;
-                wv[i] = (k <= m && m < lim)
-                            ? f16r(((cb_scale * static_cast<float>(cb[i][j])) * ssd_exp(sm.dA_m[4 * tm + i] - sm.dA_k[4 * tq + j])) * sm.dt_k[4 * tq + j])
-                            : 0.0f;
+                for (int r = 0; r < 4; ++r) {
+                    const int kk = 16 * kb + 4 * lq + r;
+                    const float w = ((cb_scale * static_cast<float>(cb[kb][r])) * ssd_exp(dAm - sm.dA_k[kk])) * sm.dt_k[kk];
+                    wv[r] = (k0 + kk <= m && m < lim) ? static_cast<_Float16>(w) : static_cast<_Float16>(0.0f);
+                }
+                *reinterpret_cast<v4h*>(&sm.wt[16 * wave + l16][16 * kb + 4 * lq]) = wv;
             }
-            *reinterpret_cast<float4*>(&sm.two.wt[4 * tq + j][4 * tm]) = make_float4(wv[0], wv[1], wv[2], wv[3]);
         }
-        for (int i = tid; i < kT * kT; i += kThreads) {
-            const int kk = i / kT, pp = i % kT;
-            float v = 0.0f;
-            if (k0 + kk < lim && p0 + pp < P) v = f16r(sm.xs[pp] * static_cast<float>(xrow0[(k0 + kk) * xstep + p0 + pp]));
-            sm.two.xh[kk][pp] = v;
-        }
-        __syncthreads();
-        const int steps = min(kT, lim - k0);
-        for (int kk = 0; kk < steps; ++kk) {
-            const float4 wv = *reinterpret_cast<const float4*>(&sm.two.wt[kk][4 * tm]);
-            const float4 xv = *reinterpret_cast<const float4*>(&sm.two.xh[kk][4 * tq]);
-            const float wvv[4] = {wv.x, wv.y, wv.z, wv.w}, xvv[4] = {xv.x, xv.y, xv.z, xv.w};
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+        for (int ks = 0; ks < 2; ++ks) {
+            if (k0 + 32 * ks <= m_last) {
+                const v8h wf = *reinterpret_cast<const v8h*>(&sm.wt[16 * wave + l16][32 * ks + 8 * lq]);
 #pragma unroll
-                for (int j = 0; j < 4; ++j) acc[i][j] += wvv[i] * xvv[j];
+                for (int j = 0; j < 4; ++j) {
+                    const v8h xf = *reinterpret_cast<const v8h*>(&sm.xt[16 * j + l16][32 * ks + 8 * lq]);
+                    acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf, xf, acc[j], 0, 0, 0);
+                }
+            }
         }
     }
 
-    // skip term, gate, fp16 out
+    // skip term, gate, fp16 out: acc[j][r] is row 16 wave + 4 (lane / 16) + r, channel 16 j + lane % 16
     const float z_scale = p.z ? *p.z_scale : 0.0f;
     __half* out = static_cast<__half*>(p.out) + ((static_cast<int64_t>(b) * L + t0) * H + h) * P;
     const int8_t* zrow0 = p.z ? p.z + ((static_cast<int64_t>(b) * L + t0) * H + h) * P : nullptr;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int m = m0 + 4 * tm + i;
+    for (int r = 0; r < 4; ++r) {
+        const int m = m0 + 16 * wave + 4 * lq + r;
         if (m >= lim) continue;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const int pl = 4 * tq + j, pp = p0 + pl;
+            const int pl = 16 * j + l16, pp = p0 + pl;
             if (pp >= P) continue;
-            float y = acc[i][j];
+            float y = acc[j][r];
             if (p.D) y += (sm.xs[pl] * static_cast<float>(xrow0[m * xstep + pp])) * sm.Dv[pl];
             if (p.z) {
                 const float zv = z_scale * static_cast<float>(zrow0[m * xstep + pp]);
@@ -382,7 +431,11 @@ void ssd_general_launch(const QaSsdParams& p, float* dt_ws, float* dA_ws, __half
     const int64_t state = static_cast<int64_t>(p.batch) * p.nheads * ((p.headdim + kTP - 1) / kTP) * ((p.dstate + kT - 1) / kT);
     hipLaunchKernelGGL(ssd_general_cumsum_kernel, dim3(static_cast<unsigned>((bch + 3) / 4)), dim3(kThreads), 0, stream, p, dt_ws, dA_ws, nc);
     hipLaunchKernelGGL(ssd_general_state_kernel, dim3(static_cast<unsigned>(state)), dim3(kThreads), 0, stream, p, dt_ws, dA_ws, prev_ws, nc);
-    hipLaunchKernelGGL(ssd_general_chunk_scan_kernel, dim3(static_cast<unsigned>(scan)), dim3(kThreads), 0, stream, p, dt_ws, dA_ws, prev_ws, nc);
+    int vec = 0;
+    if (p.dstate % 16 == 0 && aligned16(p.B) && aligned16(p.C)) vec |= kVecCodes;
+    if (p.headdim % 4 == 0 && aligned4(p.x)) vec |= kVecX;
+    if (p.dstate % 8 == 0) vec |= kVecState;                       // (the workspace itself is 256-byte aligned)
+    hipLaunchKernelGGL(ssd_general_chunk_scan_kernel, dim3(static_cast<unsigned>(scan)), dim3(kThreads), 0, stream, p, dt_ws, dA_ws, prev_ws, nc, vec);
 }
 
 }  // namespace qa
