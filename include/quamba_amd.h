@@ -434,8 +434,8 @@ typedef struct QaSsdParams {
  * (quamba/triton/quant_chunk_scan.py:286-414); beyond that QA_ERR_UNSUPPORTED (qa_ssd_workspace_bytes: 0).
  * Two sets of kernels with the same arithmetic and rounding points: matrix-core kernels for headdim 64, 128, 192 or
  * 256 with dstate 64 or 128, chunk_size 64, 128 or 256 and 16-byte aligned x, B, C, z, out (and D when it has
- * one weight per channel) - the shapes of the released models; general kernels for everything else, an order of
- * magnitude slower.  The workspace has the same size either way.  The launches are one-dimensional grids: batch *
+ * one weight per channel) - the shapes of the released models; general kernels for everything else, three to four
+ * times slower.  The workspace has the same size either way.  The launches are one-dimensional grids: batch *
  * chunks * nheads * headdim / 64 (general kernels: * ceil(chunk_size / 64) as well) must fit 2^31 - 1, else
  * QA_ERR_SHAPE. */
 int64_t qa_ssd_workspace_bytes(const QaSsdParams* p);

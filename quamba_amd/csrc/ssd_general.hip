@@ -23,7 +23,6 @@ typedef _Float16 v4h __attribute__((ext_vector_type(4)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 
 constexpr int kT = 64;            // tile edge: steps, states, channels of the chunk scan
-constexpr int kTP = 32;           // channels per workgroup of the state kernel
 constexpr int kThreads = 256;
 
 __device__ __forceinline__ float f16r(float v) { return static_cast<float>(static_cast<_Float16>(v)); }
@@ -82,31 +81,74 @@ __global__ __launch_bounds__(kThreads) void ssd_general_cumsum_kernel(QaSsdParam
     }
 }
 
+// what the tensors' sizes and addresses allow (chosen on the host)
+constexpr int kVecCodes = 1;      // B, C: rows of 16-byte pieces
+constexpr int kVecX = 2;          // x: four channels per aligned word
+constexpr int kVecState = 4;      // entering state: rows of 16-byte pieces
+constexpr int kVecB4 = 8;         // B: four states per aligned word
+
+// 64 steps x 64 columns of int8 codes (x: channels, B: states; rows `row_step` bytes apart, `width` columns in all,
+// the tile's first column col0) become fp16 values in LDS, transposed to [column][step]: a thread takes four steps
+// of four columns.  value(code, local column, local step) does the arithmetic; steps from `steps` on and columns from
+// `width` on are zero.
+template <typename F>
+__device__ __forceinline__ void stage_transposed(_Float16 (*dst)[kT + 8], const int8_t* rows0, int64_t row_step, int steps, int col0,
+                                                 int width, bool words, int tid, F&& value) {
+    const int kb = tid / 16, cq = tid % 16, col = col0 + 4 * cq;
+    uint32_t w[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int k = 4 * kb + r;
+        w[r] = 0u;
+        if (k < steps && col < width) {
+            const int8_t* src = rows0 + k * row_step + col;
+            if (words && col + 4 <= width) {
+                w[r] = *reinterpret_cast<const uint32_t*>(src);
+            } else {
+                for (int e = 0; e < 4 && col + e < width; ++e) w[r] |= static_cast<uint32_t>(static_cast<uint8_t>(src[e])) << (8 * e);
+            }
+        }
+    }
+#pragma unroll
+    for (int cc = 0; cc < 4; ++cc) {
+        v4h v;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) v[r] = static_cast<_Float16>(value(static_cast<float>(static_cast<int8_t>((w[r] >> (8 * cc)) & 0xffu)), 4 * cq + cc, 4 * kb + r));
+        *reinterpret_cast<v4h*>(&dst[4 * cq + cc][4 * kb]) = v;
+    }
+}
+
 // ---------------------------------------------------------------------------------------------
 // Stages 2, 3 and 6 (quamba/triton/quant_chunk_state.py:76-89, quant_state_passing.py:60-83, quant_ssm_states.py
-// :43,119).  A workgroup per (batch, head, 32 channels, 64 states) walks the chunks in order with its part of the
-// running state in registers (a thread: two channels x four states); the chunk's operands pass through LDS in tiles
-// of 64 steps, already rounded to fp16 and widened again.
+// :43,119).  A workgroup of four waves per (batch, head, 64 channels, 64 states) walks the chunks in order with its
+// part of the running state in registers: a wave owns sixteen states and all 64 channels (four accumulator tiles
+// of v_mfma_f32_16x16x32_f16: a lane holds channels 16 j + 4 (lane / 16) + r, state lane % 16).  The chunk's
+// operands pass through LDS in tiles of 64 steps, rounded to fp16 and transposed to [channel][step] and
+// [state][step]; everything past an edge is zero there.
 // ---------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(kThreads) void ssd_general_state_kernel(QaSsdParams p, const float* dt_ws, const float* dA_ws, __half* prev, int nc) {
-    __shared__ __attribute__((aligned(16))) float xh[kT][kTP];
-    __shared__ __attribute__((aligned(16))) float bw[kT][kT];
+__global__ __launch_bounds__(kThreads) void ssd_general_state_kernel(QaSsdParams p, const float* dt_ws, const float* dA_ws, __half* prev, int nc, int vec) {
+    __shared__ __attribute__((aligned(16))) _Float16 xt[kT][kT + 8];      // x^ [channel][step]
+    __shared__ __attribute__((aligned(16))) _Float16 bt[kT][kT + 8];      // B^ w [state][step]
     __shared__ float wk[kT];
-    __shared__ float xs[kTP];
+    __shared__ float xs[kT];
     const int P = p.headdim, N = p.dstate, Q = p.chunk_size, H = p.nheads, G = p.ngroups, L = p.seqlen;
-    const int ptiles = (P + kTP - 1) / kTP, ntiles = (N + kT - 1) / kT;
-    const int tid = threadIdx.x, tp = tid / 16, tn = tid % 16;
+    const int ptiles = (P + kT - 1) / kT, ntiles = (N + kT - 1) / kT;
+    const int tid = threadIdx.x, lane = tid & 63, l16 = lane & 15, lq = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     unsigned idx = blockIdx.x;
     const int n0 = static_cast<int>(idx % ntiles) * kT; idx /= ntiles;
-    const int p0 = static_cast<int>(idx % ptiles) * kTP; idx /= ptiles;
+    const int p0 = static_cast<int>(idx % ptiles) * kT; idx /= ptiles;
     const int h = static_cast<int>(idx % H);
     const int b = static_cast<int>(idx / H);
     int g, hg;
     ssd_group_of(p, h, g, hg);
     const float sB = p.nhead_groups > 0 ? p.B_scale[g] : p.B_scale[0];
-    if (tid < kTP) xs[tid] = p0 + tid < P ? ssd_x_scale_of(p, g, hg, p0 + tid) : 0.0f;
+    if (tid < kT) xs[tid] = p0 + tid < P ? ssd_x_scale_of(p, g, hg, p0 + tid) : 0.0f;
     const int64_t rows0 = (static_cast<int64_t>(b) * H + h) * nc;
-    float run[2][4] = {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}};
+    const int64_t xstep = static_cast<int64_t>(H) * P, bstep = static_cast<int64_t>(G) * N;
+    v4f run[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) run[j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
 
     for (int c = 0; c < nc; ++c) {
         const int t0 = c * Q;
@@ -114,66 +156,60 @@ __global__ __launch_bounds__(kThreads) void ssd_general_state_kernel(QaSsdParams
         const float* dA_row = dA_ws + (rows0 + c) * Q;
         const float* dt_row = dt_ws + (rows0 + c) * Q;
         const float dA_last = dA_row[Q - 1];
-        float acc[2][4] = {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}};
+        const int8_t* xrow0 = p.x + ((static_cast<int64_t>(b) * L + t0) * H + h) * P;
+        const int8_t* Brow0 = p.B + ((static_cast<int64_t>(b) * L + t0) * G + g) * N;
+        v4f acc[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
         for (int k0 = 0; k0 < lim; k0 += kT) {
             __syncthreads();                                       // the tile before is consumed (first pass: xs is written)
             if (tid < kT) wk[tid] = k0 + tid < lim ? ssd_exp(dA_last - dA_row[k0 + tid]) * dt_row[k0 + tid] : 0.0f;
             __syncthreads();
-            for (int i = tid; i < kT * kTP; i += kThreads) {
-                const int kk = i / kTP, pp = i % kTP;
-                float v = 0.0f;
-                if (k0 + kk < lim && p0 + pp < P) {
-                    const int8_t q = p.x[((static_cast<int64_t>(b) * L + t0 + k0 + kk) * H + h) * P + p0 + pp];
-                    v = f16r(xs[pp] * static_cast<float>(q));
-                }
-                xh[kk][pp] = v;
-            }
-            for (int i = tid; i < kT * kT; i += kThreads) {
-                const int kk = i / kT, nn = i % kT;
-                float v = 0.0f;
-                if (k0 + kk < lim && n0 + nn < N) {
-                    const int8_t q = p.B[((static_cast<int64_t>(b) * L + t0 + k0 + kk) * G + g) * N + n0 + nn];
-                    v = f16r((sB * static_cast<float>(q)) * wk[kk]);
-                }
-                bw[kk][nn] = v;
-            }
+            stage_transposed(xt, xrow0 + k0 * xstep, xstep, lim - k0, p0, P, (vec & kVecX) != 0, tid,
+                             [&](float q, int col, int) { return xs[col] * q; });
+            stage_transposed(bt, Brow0 + k0 * bstep, bstep, lim - k0, n0, N, (vec & kVecB4) != 0, tid,
+                             [&](float q, int, int k) { return (sB * q) * wk[k]; });
             __syncthreads();
-            const int steps = min(kT, lim - k0);
-            for (int kk = 0; kk < steps; ++kk) {
-                const float2 xv = *reinterpret_cast<const float2*>(&xh[kk][2 * tp]);
-                const float4 bv = *reinterpret_cast<const float4*>(&bw[kk][4 * tn]);
-                acc[0][0] += xv.x * bv.x; acc[0][1] += xv.x * bv.y; acc[0][2] += xv.x * bv.z; acc[0][3] += xv.x * bv.w;
-                acc[1][0] += xv.y * bv.x; acc[1][1] += xv.y * bv.y; acc[1][2] += xv.y * bv.z; acc[1][3] += xv.y * bv.w;
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                if (k0 + 32 * ks < lim) {
+                    const v8h bf = *reinterpret_cast<const v8h*>(&bt[16 * wave + l16][32 * ks + 8 * lq]);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const v8h xf = *reinterpret_cast<const v8h*>(&xt[16 * j + l16][32 * ks + 8 * lq]);
+                        acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf, bf, acc[j], 0, 0, 0);
+                    }
+                }
             }
         }
         // P <- exp(dA_last) P + S
         const float decay = ssd_exp(dA_last);
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+        for (int j = 0; j < 4; ++j)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) run[i][j] = decay * run[i][j] + acc[i][j];
+            for (int r = 0; r < 4; ++r) run[j][r] = decay * run[j][r] + acc[j][r];
         if (c + 1 < nc) {
             // the state entering chunk c + 1, in fp16 as the reference keeps it
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+            for (int j = 0; j < 4; ++j)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int pp = p0 + 2 * tp + i, nn = n0 + 4 * tn + j;
-                    if (pp < P && nn < N) prev[(((static_cast<int64_t>(b) * nc + c + 1) * H + h) * P + pp) * N + nn] = __float2half(run[i][j]);
+                for (int r = 0; r < 4; ++r) {
+                    const int pp = p0 + 16 * j + 4 * lq + r, nn = n0 + 16 * wave + l16;
+                    if (pp < P && nn < N) prev[(((static_cast<int64_t>(b) * nc + c + 1) * H + h) * P + pp) * N + nn] = __float2half(run[j][r]);
                 }
         }
     }
 
     if (p.final_states) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+        for (int j = 0; j < 4; ++j)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int pp = p0 + 2 * tp + i, nn = n0 + 4 * tn + j;
+            for (int r = 0; r < 4; ++r) {
+                const int pp = p0 + 16 * j + 4 * lq + r, nn = n0 + 16 * wave + l16;
                 if (pp < P && nn < N) {
                     const int64_t fo = ((static_cast<int64_t>(b) * H + h) * P + pp) * N + nn;
-                    if (p.final_state_is_fp32) static_cast<float*>(p.final_states)[fo] = run[i][j];
-                    else static_cast<int8_t*>(p.final_states)[fo] = ssd_quantize_state(p, g, hg, pp, nn, N, run[i][j]);
+                    if (p.final_state_is_fp32) static_cast<float*>(p.final_states)[fo] = run[j][r];
+                    else static_cast<int8_t*>(p.final_states)[fo] = ssd_quantize_state(p, g, hg, pp, nn, N, run[j][r]);
                 }
             }
     }
@@ -197,11 +233,6 @@ struct GeneralScanSmem {
     __attribute__((aligned(16))) _Float16 xt[kT][kT + 8];        // term 2: x^ [channel][step k]; term 1: entering state [channel][state]
     float dA_m[kT], dA_k[kT], dt_k[kT], xs[kT], Dv[kT];
 };
-
-// what the tensors' sizes and addresses allow (chosen on the host)
-constexpr int kVecCodes = 1;      // B, C: rows of 16-byte pieces
-constexpr int kVecX = 2;          // x: four channels per aligned word
-constexpr int kVecState = 4;      // entering state: rows of 16-byte pieces
 
 __global__ __launch_bounds__(kThreads) void ssd_general_chunk_scan_kernel(QaSsdParams p, const float* dt_ws, const float* dA_ws, const __half* prev, int nc, int vec) {
     __shared__ GeneralScanSmem sm;
@@ -318,32 +349,9 @@ __global__ __launch_bounds__(kThreads) void ssd_general_chunk_scan_kernel(QaSsdP
             sm.dA_k[tid] = dA_row[min(k, Q - 1)];
             sm.dt_k[tid] = k < lim ? dt_row[k] : 0.0f;
         }
-        {
-            // x^ of 64 steps x 64 channels, transposed: a thread takes four steps of four channels
-            const int kb = tid / 16, pq = tid % 16;
-            uint32_t xw[4];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int k = k0 + 4 * kb + r, pp = p0 + 4 * pq;
-                xw[r] = 0u;
-                if (k < lim && pp < P) {
-                    const int8_t* src = xrow0 + k * xstep + pp;
-                    if ((vec & kVecX) && pp + 4 <= P) {
-                        xw[r] = *reinterpret_cast<const uint32_t*>(src);
-                    } else {
-                        for (int e = 0; e < 4 && pp + e < P; ++e) xw[r] |= static_cast<uint32_t>(static_cast<uint8_t>(src[e])) << (8 * e);
-                    }
-                }
-            }
-#pragma unroll
-            for (int cc = 0; cc < 4; ++cc) {
-                const float sc = sm.xs[4 * pq + cc];               // (written before the first barrier of this kernel)
-                v4h v;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) v[r] = static_cast<_Float16>(sc * static_cast<float>(static_cast<int8_t>((xw[r] >> (8 * cc)) & 0xffu)));
-                *reinterpret_cast<v4h*>(&sm.xt[4 * pq + cc][4 * kb]) = v;
-            }
-        }
+        // x^ of 64 steps x 64 channels, transposed (xs was written before the first barrier of this kernel)
+        stage_transposed(sm.xt, xrow0 + k0 * xstep, xstep, lim - k0, p0, P, (vec & kVecX) != 0, tid,
+                         [&](float q, int col, int) { return sm.xs[col] * q; });
         // integer (C B^T)^T of the wave's rows: block kb holds steps 16 kb + 4 (lane / 16) + r of row lane % 16
         v4i cb[4];
 #pragma unroll
@@ -419,7 +427,7 @@ __global__ __launch_bounds__(kThreads) void ssd_general_chunk_scan_kernel(QaSsdP
 int ssd_general_grid_check(const QaSsdParams& p) {
     const int64_t nc = (static_cast<int64_t>(p.seqlen) + p.chunk_size - 1) / p.chunk_size;
     const int64_t scan = static_cast<int64_t>(p.batch) * nc * p.nheads * ((p.chunk_size + kT - 1) / kT) * ((p.headdim + kT - 1) / kT);
-    const int64_t state = static_cast<int64_t>(p.batch) * p.nheads * ((p.headdim + kTP - 1) / kTP) * ((p.dstate + kT - 1) / kT);
+    const int64_t state = static_cast<int64_t>(p.batch) * p.nheads * ((p.headdim + kT - 1) / kT) * ((p.dstate + kT - 1) / kT);
     // one-dimensional grids; the cumsum kernel numbers its (batch, chunk, head) items in 32 bits
     if (scan > 0x7fffffffLL || state > 0x7fffffffLL) return QA_ERR_SHAPE;
     return QA_OK;
@@ -428,13 +436,14 @@ int ssd_general_grid_check(const QaSsdParams& p) {
 void ssd_general_launch(const QaSsdParams& p, float* dt_ws, float* dA_ws, __half* prev_ws, int nc, hipStream_t stream) {
     const int64_t bch = static_cast<int64_t>(p.batch) * nc * p.nheads;
     const int64_t scan = bch * ((p.chunk_size + kT - 1) / kT) * ((p.headdim + kT - 1) / kT);
-    const int64_t state = static_cast<int64_t>(p.batch) * p.nheads * ((p.headdim + kTP - 1) / kTP) * ((p.dstate + kT - 1) / kT);
+    const int64_t state = static_cast<int64_t>(p.batch) * p.nheads * ((p.headdim + kT - 1) / kT) * ((p.dstate + kT - 1) / kT);
     hipLaunchKernelGGL(ssd_general_cumsum_kernel, dim3(static_cast<unsigned>((bch + 3) / 4)), dim3(kThreads), 0, stream, p, dt_ws, dA_ws, nc);
-    hipLaunchKernelGGL(ssd_general_state_kernel, dim3(static_cast<unsigned>(state)), dim3(kThreads), 0, stream, p, dt_ws, dA_ws, prev_ws, nc);
     int vec = 0;
     if (p.dstate % 16 == 0 && aligned16(p.B) && aligned16(p.C)) vec |= kVecCodes;
     if (p.headdim % 4 == 0 && aligned4(p.x)) vec |= kVecX;
     if (p.dstate % 8 == 0) vec |= kVecState;                       // (the workspace itself is 256-byte aligned)
+    if (p.dstate % 4 == 0 && aligned4(p.B)) vec |= kVecB4;
+    hipLaunchKernelGGL(ssd_general_state_kernel, dim3(static_cast<unsigned>(state)), dim3(kThreads), 0, stream, p, dt_ws, dA_ws, prev_ws, nc, vec);
     hipLaunchKernelGGL(ssd_general_chunk_scan_kernel, dim3(static_cast<unsigned>(scan)), dim3(kThreads), 0, stream, p, dt_ws, dA_ws, prev_ws, nc, vec);
 }
 
