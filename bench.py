@@ -312,6 +312,22 @@ def _wl_ssd(dev, steps, warmup, B, L, H, N, G, Q, name, label):
                 mfma_f16_frac=f16_flops / ms / 1e9 / F16_PEAK_TFLOPS, mfma_i8_frac=i8_ops / ms / 1e9 / INT8_PEAK_TOPS)
 
 
+def _wl_ssd_other_shape(dev, steps, warmup, B, L, H, P, N, Q, label):
+    """SSD chunk scan at a shape outside the released models' (other head dimension, state count or chunk length), one
+    group, per-tensor scales, fp32 final states: per-launch time and algorithmic bytes."""
+    ri = _ri(dev)
+    sc = lambda v: torch.tensor([v], dtype=torch.float32, device=dev)
+    x, dt, Bm, Cm, A2, D2 = ri(B, L, H, P), ri(B, L, H), ri(B, L, 1, N), ri(B, L, 1, N), ri(H), ri(H)
+    bias = torch.zeros(H, dtype=torch.float16, device=dev)
+    k_x, k_dt, k_A, k_B, k_C, k_D = (sc(v) for v in (0.03, 0.02, 0.02, 0.03, 0.03, 0.008))
+    ssd = lambda: ops.ssd_chunk_scan_combined_fwd(x, k_x, dt, k_dt, A2, k_A, Bm, k_B, Cm, k_C, None, Q, q_D=D2, D_scale=k_D,
+                                                  dt_bias=bias, dt_softplus=True, final_state_dtype=torch.float32)
+    ms = _time_fn(ssd, steps, warmup)
+    nbytes = B * L * H * P + 2 * B * L * N + B * L * H + 2 * B * L * H * P + 4 * B * H * P * N
+    return dict(workload=label, us=ms * 1e3, tokens_per_s=B * L / ms * 1e3, bound="hbm", bytes=nbytes,
+                achieved_GBs=nbytes / ms / 1e6, frac=nbytes / ms / 1e6 / HBM_PEAK_GBS)
+
+
 def _wl_w4a8(dev, steps, warmup, M, Nn, K, o8, name):
     ri = _ri(dev)
     a = ri(M, K)
@@ -417,6 +433,13 @@ def other_workloads(dev, steps, warmup):
                     tokens_per_s=B * L / ms * 1e3, bound="hbm", achieved_GBs=nbytes / ms / 1e6,
                     frac=nbytes / ms / 1e6 / HBM_PEAK_GBS))
     del xBC
+    # the SSD chunk scan at shapes outside the released models': heads of 128 channels (the matrix-core kernels, a head
+    # as two heads of 64) and 256 states (the general kernels), both with the 2.7b shape's token and channel counts
+    out.append(_wl_ssd_other_shape(dev, min(steps, 10), 2, 4, 4096, 40, 128, 128, 256,
+                                   "SSD chunk scan with heads of 128 channels, batch 4 x 4096, 40 heads, d_state 128, chunk 256"))
+    out.append(_wl_ssd_other_shape(dev, min(steps, 10), 2, 4, 4096, 80, 64, 256, 256,
+                                   "SSD chunk scan with 256 states (general kernels), batch 4 x 4096, 80 heads of 64, chunk 256"))
+    torch.cuda.empty_cache()
     # Hadamard + quantisation of the scan output in front of out_proj: 16384 rows of 5120 (40 x 128) and of 8192
     for dim in (5120, 8192):
         xh = torch.randn(16384, dim, device=dev, dtype=torch.float16)
