@@ -281,7 +281,7 @@ def test_ssd_8b_shape_oracle_heads_and_chunk_independence(dev):
                              dim_range=_np(dr[gi, hgi])[None, None], stages=True)
         xq, Cq, D_w = _np(x[bi, :, h]), _np(Cm[bi, :, gi]), 0.008 * float(_np(Dq[hs])[0])
         xs_p = np.repeat(_np(xs[gi, hgi]), 16)               # four dim groups of sixteen channels
-        s_C = float(_np(sc["C"][gi]))
+        s_C = float(_np(sc["C"][gi]).reshape(-1)[0])
         _check_ssd_y(y[bi:bi + 1, :, hs], ref, lambda t, ch: output_interval(
             ref, t, ch, chunk=256, x_codes=xq, x_scale_p=xs_p[ch], C_codes=Cq, s_C=s_C, D_weight=D_w))
         got_f = final[bi:bi + 1, hs].cpu().numpy()
