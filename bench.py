@@ -273,7 +273,9 @@ def _wl_decode(dev):
                 name="decode_step", us=ms_two * 1e3, us_one_launch=ms_one * 1e3, us_eager_python=ms_eager * 1e3,
                 state_width_4=dict(us=ms_two4 * 1e3, us_one_launch=ms_one4 * 1e3),
                 tokens_per_s=B / ms_two * 1e3, bound="hbm", bytes=nbytes, achieved_GBs=nbytes / ms_two / 1e6,
-                frac=nbytes / ms_two / 1e6 / HBM_PEAK_GBS)
+                frac=nbytes / ms_two / 1e6 / HBM_PEAK_GBS,
+                one_launch=dict(tokens_per_s=B / ms_one * 1e3, achieved_GBs=nbytes / ms_one / 1e6,
+                                frac=nbytes / ms_one / 1e6 / HBM_PEAK_GBS))
 
 
 def _wl_ssd(dev, steps, warmup, B, L, H, N, G, Q, name, label):

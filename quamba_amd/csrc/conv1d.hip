@@ -226,7 +226,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_update_kernel(QaConvParams 
     if (idx >= static_cast<int64_t>(p.batch) * p.dim) return;
     const int c = static_cast<int>(idx % p.dim);
     const int b = static_cast<int>(idx / p.dim);
-    conv_step_row<false>(p, b, c, true);
+    conv_step_row<0>(p, b, c, true);
 }
 
 // (a call over no elements - no batch entries, no channels, forward: no steps - may pass null tensors)

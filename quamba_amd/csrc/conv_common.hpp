@@ -141,9 +141,12 @@ __device__ __forceinline__ int dot4(uint32_t a, uint32_t b) {
 // on by one step (in place), the window meets the taps, bias, SiLU, requantisation.  Returns the int8 output and,
 // with `store`, writes state and output.  Taps and a four-wide state row are fetched as one word when their layout
 // allows; the requantisation takes the cheap route whenever it provably equals the exact one (conv_quant).
-// W4: four taps with unit stride and a state of four codes (conv_state_len 4, unit stride), each row one aligned
-// word, known at compile time.
-template <bool W4 = false>
+// FIXED 4: four taps with unit stride and a state of four codes (conv_state_len 4, unit stride), each row one aligned
+// word, known at compile time.  FIXED 3: four taps in one aligned word and a state of three codes per row, the rows
+// back to back in memory ([batch, dim, 3] contiguous): a row is read with one unaligned word, whose fourth byte
+// belongs to the next row and is not used (the last row of the tensor reads the word that ends with it instead),
+// and written back as three bytes.
+template <int FIXED = 0>
 __device__ __forceinline__ int8_t conv_step_row(const QaConvParams& p, int b, int c, bool store) {
     int8_t* st = p.conv_state + b * p.conv_state_batch_stride + c * p.conv_state_c_stride;
     const int8_t* w = p.weight + c * p.weight_c_stride;
@@ -151,16 +154,33 @@ __device__ __forceinline__ int8_t conv_step_row(const QaConvParams& p, int b, in
     const int slen = p.conv_state_len;            // width (slot 0 is dropped) or width-1
     const int drop = slen - (width - 1);          // 1 or 0
     __attribute__((aligned(4))) int8_t xs[4], ws[4] = {0, 0, 0, 0};
-    if constexpr (W4) {
-        // the caller has checked: four taps in one aligned word, a state of four codes in one aligned word.  Every
-        // load is issued at once (the bias through a stand-in address when there is none), no branch in between.
+    if constexpr (FIXED != 0) {
+        // the caller has checked: four taps in one aligned word, a state of four codes in one aligned word or of
+        // three codes in back-to-back rows.  Every load is issued at once (the bias through a stand-in address when
+        // there is none), no branch in between.
         const int8_t* x_a = p.x + b * p.x_batch_stride + c * p.x_c_stride;
         const uint32_t w_word4 = *reinterpret_cast<const uint32_t*>(w);
-        const uint32_t row4 = *reinterpret_cast<const uint32_t*>(st);
+        uint32_t held;                     // the codes the window keeps, in its low three bytes
+        if constexpr (FIXED == 4) {
+            held = *reinterpret_cast<const uint32_t*>(st) >> 8;
+        } else {
+            const int last = (b == p.batch - 1 && c == p.dim - 1) ? 1 : 0;
+            uint32_t word;
+            __builtin_memcpy(&word, st - last, 4);               // (an unaligned load)
+            held = (last ? word >> 8 : word) & 0x00ffffffu;
+        }
         const int8_t x_new = *x_a;
         const int8_t bias_q = *(p.bias ? p.bias + c : x_a);
-        const uint32_t win4 = (row4 >> 8) | (static_cast<uint32_t>(static_cast<uint8_t>(x_new)) << 24);
-        if (store) *reinterpret_cast<uint32_t*>(st) = win4;
+        const uint32_t win4 = held | (static_cast<uint32_t>(static_cast<uint8_t>(x_new)) << 24);
+        if (store) {
+            if constexpr (FIXED == 4) {
+                *reinterpret_cast<uint32_t*>(st) = win4;
+            } else {
+                st[0] = static_cast<int8_t>(win4 >> 8);
+                st[1] = static_cast<int8_t>(win4 >> 16);
+                st[2] = x_new;
+            }
+        }
         *reinterpret_cast<uint32_t*>(ws) = w_word4;
         *reinterpret_cast<uint32_t*>(xs) = win4;
         const float s_wx = p.scale_w * p.scale_x;

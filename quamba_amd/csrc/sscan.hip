@@ -883,7 +883,8 @@ int launch_fwd_mixed(const QaSScanParams& p, hipStream_t stream, int vec_in, int
 // FAST: the shape of the Mamba1 decode step is known at compile time (one head, one B/C group, sixteen states whose
 // A_log codes are one aligned 16-byte row, per-tensor scales, no fp16 bias, four taps), so the lane's work is one
 // run of loads, arithmetic and stores without loops or branches on the parameter block.
-template <int LPR, bool VEC, bool FP32, bool CONV, bool FAST = false>
+// CONV_STATE: with CONV and FAST, the codes per row of the conv state (4: a word per row; 3: rows back to back).
+template <int LPR, bool VEC, bool FP32, bool CONV, bool FAST = false, int CONV_STATE = 4>
 __device__ __forceinline__ void ssm_update_body(const QaSsmUpdateParams& p, const QaConvParams* cp) {
     static_assert(!CONV || LPR == 1, "the conv step needs one lane per row");
     static_assert(!FAST || (LPR == 1 && VEC), "the fixed shape has one lane per row and whole pieces");
@@ -1031,7 +1032,7 @@ __device__ __forceinline__ void ssm_update_body(const QaSsmUpdateParams& p, cons
     const float b8 = static_cast<float>(*b8_a), b16 = __half2float(*b16_a);
     float xq;
     if constexpr (CONV) {
-        xq = static_cast<float>(conv_step_row<FAST>(*cp, static_cast<int>(b), d, row_ok));
+        xq = static_cast<float>(conv_step_row<FAST ? CONV_STATE : 0>(*cp, static_cast<int>(b), d, row_ok));
     } else {
         xq = static_cast<float>(*x_a);
     }
@@ -1142,9 +1143,9 @@ __global__ __launch_bounds__(256) void ssm_update_kernel(QaSsmUpdateParams p) {
 }
 
 // conv step + state update of one token in one launch (d_state <= 16, one head)
-template <bool VEC, bool FP32, bool FAST>
+template <bool VEC, bool FP32, bool FAST, int CONV_STATE = 4>
 __global__ __launch_bounds__(256) void decode_step_kernel(QaSsmUpdateParams p, QaConvParams cp) {
-    ssm_update_body<1, VEC, FP32, true, FAST>(p, &cp);
+    ssm_update_body<1, VEC, FP32, true, FAST, CONV_STATE>(p, &cp);
 }
 
 template <int LPR>
@@ -1175,11 +1176,16 @@ int launch_update(const QaSsmUpdateParams& p, hipStream_t stream, const QaConvPa
         }
         if (conv) {
             auto fused = [&](auto kernel) { hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, p, *conv); };
-            const bool fast = fast_update && conv->width == 4 && conv->weight_width_stride == 1 &&
-                              aligned4(conv->weight) && conv->weight_c_stride % 4 == 0 && conv->conv_state_len == 4 &&
-                              conv->conv_state_l_stride == 1 && aligned4(conv->conv_state) &&
+            const bool taps4 = fast_update && conv->width == 4 && conv->weight_width_stride == 1 &&
+                               aligned4(conv->weight) && conv->weight_c_stride % 4 == 0 && conv->conv_state_l_stride == 1;
+            const bool fast = taps4 && conv->conv_state_len == 4 && aligned4(conv->conv_state) &&
                               conv->conv_state_batch_stride % 4 == 0 && conv->conv_state_c_stride % 4 == 0;
+            // a state of three codes per row, the rows back to back (the whole tensor has at least two rows)
+            const bool fast3 = taps4 && conv->conv_state_len == 3 && conv->conv_state_c_stride == 3 &&
+                               conv->conv_state_batch_stride == 3 * static_cast<int64_t>(conv->dim) &&
+                               static_cast<int64_t>(conv->batch) * conv->dim >= 2;
             if (fast) p.state_is_fp32 ? fused(decode_step_kernel<true, true, true>) : fused(decode_step_kernel<true, false, true>);
+            else if (fast3) p.state_is_fp32 ? fused(decode_step_kernel<true, true, true, 3>) : fused(decode_step_kernel<true, false, true, 3>);
             else if (p.state_is_fp32) vec ? fused(decode_step_kernel<true, true, false>) : fused(decode_step_kernel<false, true, false>);
             else vec ? fused(decode_step_kernel<true, false, false>) : fused(decode_step_kernel<false, false, false>);
             return check_launch();

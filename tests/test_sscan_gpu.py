@@ -184,7 +184,11 @@ def test_update_matches_oracle_over_several_steps(dev, B, D, N, fp32_state):
 @pytest.mark.parametrize("B,D,N,width,state_len,fp32_state", [(3, 100, 16, 4, 3, True), (64, 1536, 16, 4, 4, False),
                                                               (7, 300, 16, 4, 4, True), (3, 320, 16, 4, 4, True),
                                                               (2, 257, 8, 3, 2, True),
-                                                              (5, 64, 16, 2, 2, False)])
+                                                              (5, 64, 16, 2, 2, False),
+                                                              # a conv state of three codes per row, rows back to back: the
+                                                              # fixed-shape kernel reads a row as one unaligned word
+                                                              (64, 1536, 16, 4, 3, False), (7, 320, 16, 4, 3, True),
+                                                              (1, 64, 16, 4, 3, True), (2, 100, 16, 4, 3, False)])
 def test_decode_step_in_one_launch_equals_conv_update_then_state_update(dev, B, D, N, width, state_len, fp32_state):
     """qa_mamba1_decode_step against the two calls it stands for, bit for bit (conv output, conv state, y, state),
     over several steps; the two-call path is the one the oracle tests pin."""
@@ -209,15 +213,16 @@ def test_decode_step_in_one_launch_equals_conv_update_then_state_update(dev, B, 
     assert int(xc_a.abs().max()) > 10 and float(y_a.float().abs().max()) > 0.1
 
 
+@pytest.mark.parametrize("state_len", [4, 3])
 @pytest.mark.parametrize("fp32_state", [True, False])
-def test_decode_step_without_optional_operands(dev, fp32_state):
-    """The reference layer's layout (the kernel compiled for that shape) with no skip weight, no gate, no dt bias, no
-    conv bias and no SiLU: one launch against the two calls, bit for bit."""
+def test_decode_step_without_optional_operands(dev, fp32_state, state_len):
+    """The reference layer's layout (the kernel compiled for that shape; conv state of four codes per row, or three) with
+    no skip weight, no gate, no dt bias, no conv bias and no SiLU: one launch against the two calls, bit for bit."""
     B, D, N = 5, 256, 16
     g = torch.Generator(device=dev).manual_seed(99)
     ri = lambda *shape: torch.randint(-128, 128, shape, dtype=torch.int8, device=dev, generator=g)
     w, A = ri(D, 4), ri(D, N)
-    conv_a = ri(B, D, 4)
+    conv_a = ri(B, D, state_len)
     st_a = (torch.randn(B, D, N, device=dev, generator=g) * 0.1) if fp32_state else ri(B, D, N)
     conv_b, st_b = conv_a.clone(), st_a.clone()
     s_dt, s_A, s_B, s_C, s_state = (_s(v, dev) for v in (0.02, 0.02, 0.03, 0.03, 0.004))
