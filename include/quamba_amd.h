@@ -319,9 +319,8 @@ int qa_ssm_state_update(const QaSsmUpdateParams* p, void* stream);
  * (may be null) receives the conv output.  One head (p->nheads == 1), d_state <= 16, per-tensor scales.
  * The reference layer's own layout - sixteen states, contiguous (batch, dim, 16) state and (dim, 16) A_log,
  * (batch, dim, 4) or contiguous (batch, dim, 3) conv state, four taps, int8 or no dt bias, dim a multiple of 64 for an
- * fp32 state - takes a kernel
- * compiled for that shape (the state moves in 1 KB runs per wave); any other layout the generic one.  The same
- * holds for qa_ssm_state_update alone. */
+ * fp32 state - takes a kernel compiled for that shape (the state moves in 1 KB runs per wave); any other layout the
+ * generic one.  The same holds for qa_ssm_state_update alone. */
 int qa_mamba1_decode_step(const QaConvParams* conv, const QaSsmUpdateParams* p, void* stream);
 
 /* ------------------------------------------------------------------------------------------
