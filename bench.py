@@ -278,30 +278,31 @@ def _wl_decode(dev):
                                 frac=nbytes / ms_one / 1e6 / HBM_PEAK_GBS))
 
 
-def _wl_ssd(dev, steps, warmup, B, L, H, N, G, Q, name, label):
-    """SSD chunk scan of `label`: per-tensor scales for one group, grouped scales (four head groups x four dim groups
-    per ssd group) otherwise; fp32 final states."""
+def _wl_ssd(dev, steps, warmup, B, L, H, N, G, Q, name, label, fp32_dt=False):
+    """SSD chunk scan of `label`: x scales per (ssd group, four head groups, four dim groups), B and C scales per ssd
+    group; step sizes as int8 codes with bias and softplus in the kernel, or (`fp32_dt`) already processed, fp32 in
+    [1e-3, 1e-1]; fp32 final states."""
     ri = _ri(dev)
     sc = lambda v: torch.tensor([v], dtype=torch.float32, device=dev)
-    x, dt, Bm, Cm = ri(B, L, H, 64), ri(B, L, H), ri(B, L, G, N), ri(B, L, G, N)
+    x, Bm, Cm = ri(B, L, H, 64), ri(B, L, G, N), ri(B, L, G, N)
+    if fp32_dt:
+        dt = torch.exp(torch.rand(B, L, H, device=dev) * (np.log(1e-1) - np.log(1e-3)) + np.log(1e-3)).float()
+    else:
+        dt = ri(B, L, H)
     A2, D2 = ri(H), ri(H)
     bias = torch.zeros(H, dtype=torch.float16, device=dev)
     # scales live on the device before the timed region (creating one is a blocking host-to-device copy)
     k_dt, k_A, k_D = (sc(v) for v in (0.02, 0.02, 0.008))
-    kw = {}
-    if G == 1:
-        k_x, k_B, k_C = sc(0.03), sc(0.03), sc(0.03)
-    else:
-        hpg = H // G
-        k_x = torch.rand(G, 4, 4, device=dev) * 0.02 + 0.02
-        k_B, k_C = torch.rand(G, device=dev) * 0.02 + 0.02, torch.rand(G, device=dev) * 0.02 + 0.02
-        kw = dict(x_head_group_range=(torch.arange(1, 5, dtype=torch.int32, device=dev) * (hpg // 4)).repeat(G, 1),
-                  x_dim_group_range=(torch.arange(1, 5, dtype=torch.int32, device=dev) * 16).repeat(G, 4, 1))
+    hpg = H // G
+    k_x = torch.rand(G, 4, 4, device=dev) * 0.02 + 0.02
+    k_B, k_C = torch.rand(G, device=dev) * 0.02 + 0.02, torch.rand(G, device=dev) * 0.02 + 0.02
+    kw = dict(x_head_group_range=(torch.arange(1, 5, dtype=torch.int32, device=dev) * (hpg // 4)).repeat(G, 1),
+              x_dim_group_range=(torch.arange(1, 5, dtype=torch.int32, device=dev) * 16).repeat(G, 4, 1))
     ssd = lambda: ops.ssd_chunk_scan_combined_fwd(x, k_x, dt, k_dt, A2, k_A, Bm, k_B, Cm, k_C, None, Q,
                                                   q_D=D2, D_scale=k_D, dt_bias=bias, dt_softplus=True,
                                                   final_state_dtype=torch.float32, **kw)
     ms = _time_fn(ssd, steps, warmup)
-    nbytes = B * L * H * 64 + 2 * B * L * G * N + B * L * H + 2 * B * L * H * 64 + 4 * B * H * 64 * N
+    nbytes = B * L * H * 64 + 2 * B * L * G * N + B * L * H * (4 if fp32_dt else 1) + 2 * B * L * H * 64 + 4 * B * H * 64 * N
     # dense multiply-adds: C B^T (lower tiles), chunk states, C x entering state, causal part of (C B^T) x
     nc = (L + Q - 1) // Q
     flops = 2.0 * B * nc * (G * Q * Q * N / 2 + H * Q * 64 * N + H * Q * 64 * N + H * Q * Q * 64 / 2)
@@ -344,7 +345,8 @@ def _wl_w4a8(dev, steps, warmup, M, Nn, K, o8, name):
                 bound="mfma", ops=n_ops, achieved_TOPs=tops, frac=tops / INT8_PEAK_TOPS)
 
 
-SSD_27B = (4, 4096, 80, 128, 1, 256, "ssd_2p7b", "Mamba2-2.7b SSD chunk scan, batch 4 x 4096, 80 heads, d_state 128, chunk 256")
+SSD_27B = (4, 4096, 80, 128, 1, 256, "ssd_2p7b", "Mamba2-2.7b SSD chunk scan, batch 4 x 4096, 80 heads, d_state 128, chunk 256, "
+           "x scales per head group, fp32 step sizes", True)
 SSD_8B = (16, 1024, 128, 128, 8, 256, "ssd_8b", "Mamba2-8b SSD chunk scan, batch 16 x 1024, 128 heads, d_state 128, 8 groups, chunk 256")
 
 

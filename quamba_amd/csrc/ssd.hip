@@ -37,7 +37,7 @@ __device__ __forceinline__ int8_t byte_of(uint32_t w, int j) { return static_cas
 // Stage 1 (quamba/triton/quant_chunk_cumsum.py:56-70).  One wave per (batch, chunk, head): every
 // lane processes chunk_size/64 consecutive steps, then an inclusive scan across the lanes.
 // ---------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void ssd_cumsum_kernel(QaSsdParams p, float* dt_out, float* dA_out, int nc) {
+__global__ __launch_bounds__(256) void ssd_cumsum_kernel(QaSsdParams p, float* dt_out, float* dA_out, float* xs_out, int nc) {
     const int lane = threadIdx.x & 63;
     // the item is the same for a whole wave and below 2^31 (the host checks): its decomposition is 32-bit arithmetic on
     // a uniform value instead of 64-bit divisions in every lane
@@ -47,6 +47,7 @@ __global__ __launch_bounds__(256) void ssd_cumsum_kernel(QaSsdParams p, float* d
     const int c = static_cast<int>((idx / static_cast<unsigned>(p.nheads)) % static_cast<unsigned>(nc));
     const int b = static_cast<int>(idx / (static_cast<unsigned>(p.nheads) * static_cast<unsigned>(nc)));
     const int Q = p.chunk_size, E = Q / 64;            // Q in {64, 128, 256}
+    if (b == 0 && c == 0) ssd_write_x_scales(p, h, lane, xs_out);
     const float A = -expf(*p.A_log_scale * static_cast<float>(p.A_log[h]));
     const float s_dt = p.dt_is_fp32 ? 0.0f : *p.dt_scale;
     const float bias = (!p.dt_is_fp32 && p.dt_bias) ? __half2float(static_cast<const __half*>(p.dt_bias)[h]) : 0.0f;
@@ -165,7 +166,7 @@ struct StateSmem {
 };
 
 template <int N, int Q>
-__global__ __launch_bounds__(256, 3) void ssd_state_kernel(QaSsdParams p, const float* dt_ws, const float* dA_ws, __half* prev, int nc) {
+__global__ __launch_bounds__(256, 3) void ssd_state_kernel(QaSsdParams p, const float* dt_ws, const float* dA_ws, __half* prev, const float* xs_ws, int nc) {
     using S = StateSmem<Q>;
     extern __shared__ __attribute__((aligned(16))) unsigned char ssd_smem_raw[];
     S& sm = *reinterpret_cast<S*>(ssd_smem_raw);
@@ -184,8 +185,7 @@ __global__ __launch_bounds__(256, 3) void ssd_state_kernel(QaSsdParams p, const 
     const int h = (unit % G) * (H / G) + hig;
     const int hp = h / split, ch0 = (h % split) * kP;
     const int b = unit / G;
-    int g, hg;
-    ssd_group_of(p, hp, g, hg);
+    const int g = hp / (p.nheads / G);
     const bool grouped = p.nhead_groups > 0;
     const float sB = grouped ? p.B_scale[g] : p.B_scale[0];
     const float nsB = -128.0f * sB;
@@ -197,7 +197,7 @@ __global__ __launch_bounds__(256, 3) void ssd_state_kernel(QaSsdParams p, const 
     const int pb = tid % 4, kb = tid / 4;
     const bool mine = Q == 256 || tid < Q;
     const uint32_t voff_x = static_cast<uint32_t>(4 * kb) * xrow + 16 * pb, voff_b = static_cast<uint32_t>(4 * kb) * brow + 16 * pb;
-    if (tid < kP) sm.xs[tid] = ssd_x_scale_of(p, g, hg, ch0 + tid);
+    if (tid < kP) sm.xs[tid] = xs_ws[hp * p.headdim + ch0 + tid];
     uint4 xr[4], br[4];
     float r_dt = 0.0f, r_dA = 0.0f, r_last = 0.0f;
     int valid_loaded = Q;                                         // steps of the chunk whose tiles are in xr / br
@@ -328,6 +328,8 @@ __global__ __launch_bounds__(256, 3) void ssd_state_kernel(QaSsdParams p, const 
                 } else {
                     float sc, K;
                     if (grouped) {
+                        int g_, hg;
+                        ssd_group_of(p, hp, g_, hg);
                         const int dg = ssd_dim_group_of(p, g, hg, ch0 + pp);
                         sc = p.state_scale[((g * p.nhead_groups + hg) * p.ndim_groups + dg) * N + n_col];
                         K = 1e6f;
@@ -392,7 +394,7 @@ constexpr int scan_waves_of(int Q) { return Q / 16 < 8 ? Q / 16 : 8; }
 
 template <int N, int Q>
 __global__ __launch_bounds__(64 * scan_waves_of(Q), 4) void ssd_chunk_scan_kernel(QaSsdParams p, const float* dt_ws, const float* dA_ws,
-                                                                                const __half* prev, int nc) {
+                                                                                const __half* prev, const float* xs_ws, int nc) {
     using S = ScanSmem<N, Q>;
     extern __shared__ __attribute__((aligned(16))) unsigned char ssd_smem_raw[];
     S& sm = *reinterpret_cast<S*>(ssd_smem_raw);
@@ -421,8 +423,7 @@ __global__ __launch_bounds__(64 * scan_waves_of(Q), 4) void ssd_chunk_scan_kerne
     const int hp = h / split, ch0 = (h % split) * kP;
     const int c = (unit / G) % nc;
     const int b = unit / (G * nc);
-    int g, hg;
-    ssd_group_of(p, hp, g, hg);
+    const int g = hp / (p.nheads / G);
     const bool grouped = p.nhead_groups > 0;
     const float sC = grouped ? p.C_scale[g] : p.C_scale[0];
     const float cb_scale = sC * (grouped ? p.B_scale[g] : p.B_scale[0]);
@@ -487,7 +488,7 @@ __global__ __launch_bounds__(64 * scan_waves_of(Q), 4) void ssd_chunk_scan_kerne
             for (int r = 0; r < 4; ++r) xr[r] = *reinterpret_cast<const uint4*>(xbase + static_cast<uint64_t>(min(voff_x + static_cast<uint32_t>(r) * xrow, last_x)));
         }
         if (tid < kP) {
-            sm.xs[tid] = ssd_x_scale_of(p, g, hg, ch0 + tid);
+            sm.xs[tid] = xs_ws[hp * p.headdim + ch0 + tid];
             sm.Dv[tid] = !p.D ? 0.0f : D_scale * static_cast<float>(p.D_has_hdim ? p.D[hp * p.headdim + ch0 + tid] : p.D[hp]);
         }
         if (p.z) {
@@ -721,12 +722,13 @@ extern "C" int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream_) {
     const int64_t bch = static_cast<int64_t>(p->batch) * nc * p->nheads;
 
     __half* prev_ws = reinterpret_cast<__half*>(base + ws.prev);
+    float* xs_ws = reinterpret_cast<float*>(base + ws.xs);
     if (!ssd_fast_shape(*p)) {
-        ssd_general_launch(*p, dt_ws, dA_ws, prev_ws, nc, stream);
+        ssd_general_launch(*p, dt_ws, dA_ws, prev_ws, xs_ws, nc, stream);
         return check_launch();
     }
     hipLaunchKernelGGL(ssd_cumsum_kernel, dim3(static_cast<unsigned>((bch + 3) / 4)), dim3(256), 0, stream, *p, dt_ws,
-                       dA_ws, nc);
+                       dA_ws, xs_ws, nc);
     const int heads64 = p->nheads * (p->headdim / 64);          // the kernels see a head of 64 s channels as s heads of 64
     const dim3 hgrid(static_cast<unsigned>(p->batch * heads64 * (p->dstate / 64)));
     int status = QA_OK;
@@ -739,8 +741,8 @@ extern "C" int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream_) {
     };
     auto launch = [&](auto state_kernel, size_t state_lds, auto scan_kernel, size_t scan_lds, int scan_threads) {
         if (!lds_ok(reinterpret_cast<const void*>(state_kernel), state_lds) || !lds_ok(reinterpret_cast<const void*>(scan_kernel), scan_lds)) return;
-        hipLaunchKernelGGL(state_kernel, hgrid, dim3(256), state_lds, stream, *p, dt_ws, dA_ws, prev_ws, nc);
-        hipLaunchKernelGGL(scan_kernel, dim3(static_cast<unsigned>(bch * (p->headdim / 64))), dim3(scan_threads), scan_lds, stream, *p, dt_ws, dA_ws, prev_ws, nc);
+        hipLaunchKernelGGL(state_kernel, hgrid, dim3(256), state_lds, stream, *p, dt_ws, dA_ws, prev_ws, xs_ws, nc);
+        hipLaunchKernelGGL(scan_kernel, dim3(static_cast<unsigned>(bch * (p->headdim / 64))), dim3(scan_threads), scan_lds, stream, *p, dt_ws, dA_ws, prev_ws, xs_ws, nc);
     };
 #define QA_SSD_LAUNCH(N_, Q_) launch(ssd_state_kernel<N_, Q_>, sizeof(StateSmem<Q_>), ssd_chunk_scan_kernel<N_, Q_>, \
                                      sizeof(ScanSmem<N_, Q_>), 64 * scan_waves_of(Q_))
