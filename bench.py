@@ -192,6 +192,7 @@ def _time_fn(fn, steps, warmup, settle_ms=None):
     workload to settle its clocks, and an idle gap lets them fall again."""
     settle_ms = SETTLE_MS if settle_ms is None else settle_ms
     if settle_ms > 0:
+        fn()                                # (the first call may allocate or load code: not a measure of the others)
         torch.cuda.synchronize()
         t = time.perf_counter()
         fn()
@@ -302,6 +303,14 @@ def _wl_ssd(dev, steps, warmup, B, L, H, N, G, Q, name, label, fp32_dt=False):
                                                   q_D=D2, D_scale=k_D, dt_bias=bias, dt_softplus=True,
                                                   final_state_dtype=torch.float32, **kw)
     ms = _time_fn(ssd, steps, warmup)
+    # the same call captured into a HIP graph (how a serving loop would issue it): without the eager launches' work at
+    # every kernel boundary
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ssd()
+    ms_graph = _time_fn(graph.replay, steps, warmup)
+    del graph
     nbytes = B * L * H * 64 + 2 * B * L * G * N + B * L * H * (4 if fp32_dt else 1) + 2 * B * L * H * 64 + 4 * B * H * 64 * N
     # dense multiply-adds: C B^T (lower tiles), chunk states, C x entering state, causal part of (C B^T) x
     nc = (L + Q - 1) // Q
@@ -310,7 +319,7 @@ def _wl_ssd(dev, steps, warmup, B, L, H, N, G, Q, name, label, fp32_dt=False):
     # int8 product C B^T as the kernel forms it - per head, at and below the diagonal in 16 x 32 blocks - against the int8 peak
     f16_flops = 2.0 * B * nc * H * (2 * Q * 64 * N + Q * Q * 64 / 2)
     i8_ops = 2.0 * B * nc * H * N * sum(16 * 32 * ((mt + 2) // 2) for mt in range(Q // 16))
-    return dict(workload=label, name=name, us=ms * 1e3, tokens_per_s=B * L / ms * 1e3, bound="hbm", bytes=nbytes,
+    return dict(workload=label, name=name, us=ms * 1e3, us_hip_graph=ms_graph * 1e3, tokens_per_s=B * L / ms * 1e3, bound="hbm", bytes=nbytes,
                 achieved_GBs=nbytes / ms / 1e6, frac=nbytes / ms / 1e6 / HBM_PEAK_GBS, dense_TFLOPs=flops / ms / 1e9,
                 mfma_f16_frac=f16_flops / ms / 1e9 / F16_PEAK_TFLOPS, mfma_i8_frac=i8_ops / ms / 1e9 / INT8_PEAK_TOPS)
 
