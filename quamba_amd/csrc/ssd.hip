@@ -37,7 +37,7 @@ __device__ __forceinline__ int8_t byte_of(uint32_t w, int j) { return static_cas
 // Stage 1 (quamba/triton/quant_chunk_cumsum.py:56-70).  One wave per (batch, chunk, head): every
 // lane processes chunk_size/64 consecutive steps, then an inclusive scan across the lanes.
 // ---------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void ssd_cumsum_kernel(QaSsdParams p, float* dt_out, float* dA_out, float* xs_out, int nc) {
+__global__ __launch_bounds__(256) void ssd_cumsum_kernel(QaSsdParams p, float* dt_out, float* dA_out, float* xs_out, int32_t* srow_out, int nc) {
     const int lane = threadIdx.x & 63;
     // the item is the same for a whole wave and below 2^31 (the host checks): its decomposition is 32-bit arithmetic on
     // a uniform value instead of 64-bit divisions in every lane
@@ -47,7 +47,7 @@ __global__ __launch_bounds__(256) void ssd_cumsum_kernel(QaSsdParams p, float* d
     const int c = static_cast<int>((idx / static_cast<unsigned>(p.nheads)) % static_cast<unsigned>(nc));
     const int b = static_cast<int>(idx / (static_cast<unsigned>(p.nheads) * static_cast<unsigned>(nc)));
     const int Q = p.chunk_size, E = Q / 64;            // Q in {64, 128, 256}
-    if (b == 0 && c == 0) ssd_write_x_scales(p, h, lane, xs_out);
+    if (b == 0 && c == 0) ssd_write_channel_tables(p, h, lane, xs_out, srow_out);
     const float A = -expf(*p.A_log_scale * static_cast<float>(p.A_log[h]));
     const float s_dt = p.dt_is_fp32 ? 0.0f : *p.dt_scale;
     const float bias = (!p.dt_is_fp32 && p.dt_bias) ? __half2float(static_cast<const __half*>(p.dt_bias)[h]) : 0.0f;
@@ -163,10 +163,12 @@ struct StateSmem {
     __attribute__((aligned(16))) int8_t b8[64][BP];
     __attribute__((aligned(16))) float w[Q];
     __attribute__((aligned(16))) float xs[kP];    // x scale per channel
+    int32_t srow[kP];                             // the channel's row of the grouped state scales
 };
 
 template <int N, int Q>
-__global__ __launch_bounds__(256, 3) void ssd_state_kernel(QaSsdParams p, const float* dt_ws, const float* dA_ws, __half* prev, const float* xs_ws, int nc) {
+__global__ __launch_bounds__(256, 3) void ssd_state_kernel(QaSsdParams p, const float* dt_ws, const float* dA_ws, __half* prev, const float* xs_ws,
+                                                          const int32_t* srow_ws, int nc) {
     using S = StateSmem<Q>;
     extern __shared__ __attribute__((aligned(16))) unsigned char ssd_smem_raw[];
     S& sm = *reinterpret_cast<S*>(ssd_smem_raw);
@@ -197,7 +199,10 @@ __global__ __launch_bounds__(256, 3) void ssd_state_kernel(QaSsdParams p, const 
     const int pb = tid % 4, kb = tid / 4;
     const bool mine = Q == 256 || tid < Q;
     const uint32_t voff_x = static_cast<uint32_t>(4 * kb) * xrow + 16 * pb, voff_b = static_cast<uint32_t>(4 * kb) * brow + 16 * pb;
-    if (tid < kP) sm.xs[tid] = xs_ws[hp * p.headdim + ch0 + tid];
+    if (tid < kP) {
+        sm.xs[tid] = xs_ws[hp * p.headdim + ch0 + tid];
+        sm.srow[tid] = srow_ws[hp * p.headdim + ch0 + tid];
+    }
     uint4 xr[4], br[4];
     float r_dt = 0.0f, r_dA = 0.0f, r_last = 0.0f;
     int valid_loaded = Q;                                         // steps of the chunk whose tiles are in xr / br
@@ -326,19 +331,7 @@ __global__ __launch_bounds__(256, 3) void ssd_state_kernel(QaSsdParams p, const 
                 if (p.final_state_is_fp32) {
                     static_cast<float*>(p.final_states)[fo] = sv;
                 } else {
-                    float sc, K;
-                    if (grouped) {
-                        int g_, hg;
-                        ssd_group_of(p, hp, g_, hg);
-                        const int dg = ssd_dim_group_of(p, g, hg, ch0 + pp);
-                        sc = p.state_scale[((g * p.nhead_groups + hg) * p.ndim_groups + dg) * N + n_col];
-                        K = 1e6f;
-                    } else {
-                        sc = p.state_scale[0];
-                        K = 1e2f;
-                    }
-                    const float s16 = __half2float(__float2half(sv));      // the reference hands fp16 states to the quantiser
-                    static_cast<int8_t*>(p.final_states)[fo] = sat8_rne((s16 * K) / (sc * K));
+                    static_cast<int8_t*>(p.final_states)[fo] = ssd_quantize_state(p, sm.srow[pp], n_col, sv);
                 }
             }
     }
@@ -723,12 +716,13 @@ extern "C" int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream_) {
 
     __half* prev_ws = reinterpret_cast<__half*>(base + ws.prev);
     float* xs_ws = reinterpret_cast<float*>(base + ws.xs);
+    int32_t* srow_ws = reinterpret_cast<int32_t*>(base + ws.srow);
     if (!ssd_fast_shape(*p)) {
-        ssd_general_launch(*p, dt_ws, dA_ws, prev_ws, xs_ws, nc, stream);
+        ssd_general_launch(*p, dt_ws, dA_ws, prev_ws, xs_ws, srow_ws, nc, stream);
         return check_launch();
     }
     hipLaunchKernelGGL(ssd_cumsum_kernel, dim3(static_cast<unsigned>((bch + 3) / 4)), dim3(256), 0, stream, *p, dt_ws,
-                       dA_ws, xs_ws, nc);
+                       dA_ws, xs_ws, srow_ws, nc);
     const int heads64 = p->nheads * (p->headdim / 64);          // the kernels see a head of 64 s channels as s heads of 64
     const dim3 hgrid(static_cast<unsigned>(p->batch * heads64 * (p->dstate / 64)));
     int status = QA_OK;
@@ -741,7 +735,7 @@ extern "C" int qa_ssd_chunk_scan_fwd(const QaSsdParams* p, void* stream_) {
     };
     auto launch = [&](auto state_kernel, size_t state_lds, auto scan_kernel, size_t scan_lds, int scan_threads) {
         if (!lds_ok(reinterpret_cast<const void*>(state_kernel), state_lds) || !lds_ok(reinterpret_cast<const void*>(scan_kernel), scan_lds)) return;
-        hipLaunchKernelGGL(state_kernel, hgrid, dim3(256), state_lds, stream, *p, dt_ws, dA_ws, prev_ws, xs_ws, nc);
+        hipLaunchKernelGGL(state_kernel, hgrid, dim3(256), state_lds, stream, *p, dt_ws, dA_ws, prev_ws, xs_ws, srow_ws, nc);
         hipLaunchKernelGGL(scan_kernel, dim3(static_cast<unsigned>(bch * (p->headdim / 64))), dim3(scan_threads), scan_lds, stream, *p, dt_ws, dA_ws, prev_ws, xs_ws, nc);
     };
 #define QA_SSD_LAUNCH(N_, Q_) launch(ssd_state_kernel<N_, Q_>, sizeof(StateSmem<Q_>), ssd_chunk_scan_kernel<N_, Q_>, \

@@ -12,14 +12,15 @@ constexpr float kSsdLog2e = 1.44269504088896341f;
 __device__ __forceinline__ float ssd_exp(float x) { return __builtin_amdgcn_exp2f(x * kSsdLog2e); }
 
 struct SsdWorkspace {            // sections of the workspace (byte offsets), see qa_ssd_workspace_bytes
-    int64_t dt, dA, prev, xs, total;
+    int64_t dt, dA, prev, xs, srow, total;
 };
 
 __host__ __device__ inline int64_t ssd_align256(int64_t v) { return (v + 255) & ~int64_t(255); }
 
 // dt and the within-chunk cumsum of dt A, fp32 [batch, nheads, chunks, chunk_size]; the states entering the chunks,
-// fp16 [batch, chunks, nheads, headdim, dstate]; the x scale of every channel, fp32 [nheads, headdim] (looked up once
-// from the group ranges by the first kernel: the others read it with one load instead of a chain of dependent ones)
+// fp16 [batch, chunks, nheads, headdim, dstate]; the x scale of every channel, fp32 [nheads, headdim], and the row of
+// the grouped state scales it quantises its final state with, int32 [nheads, headdim] (both looked up once from the
+// group ranges by the first kernel: the others read them with one load instead of a chain of dependent ones)
 __host__ __device__ inline SsdWorkspace ssd_workspace_layout(const QaSsdParams& p) {
     const int64_t nc = (p.seqlen + p.chunk_size - 1) / p.chunk_size;
     const int64_t B = p.batch, H = p.nheads, Q = p.chunk_size, N = p.dstate, P = p.headdim;
@@ -29,6 +30,7 @@ __host__ __device__ inline SsdWorkspace ssd_workspace_layout(const QaSsdParams& 
     w.dA = off; off = ssd_align256(off + B * H * nc * Q * 4);
     w.prev = off; off = ssd_align256(off + B * nc * H * P * N * 2);
     w.xs = off; off = ssd_align256(off + H * P * 4);
+    w.srow = off; off = ssd_align256(off + H * P * 4);
     w.total = off;
     return w;
 }
@@ -55,24 +57,24 @@ __device__ __forceinline__ float ssd_x_scale_of(const QaSsdParams& p, int g, int
     return p.x_scale[(g * p.nhead_groups + hg) * p.ndim_groups + ssd_dim_group_of(p, g, hg, ch)];
 }
 
-// The table of x scales: called by the wave that handles (batch 0, chunk 0, head h) in the first kernel
-__device__ __forceinline__ void ssd_write_x_scales(const QaSsdParams& p, int h, int lane, float* xs_out) {
+// The per-channel tables: called by the wave that handles (batch 0, chunk 0, head h) in the first kernel.
+// srow: index of the first state's scale in state_scale for this channel (0 with one scale for everything)
+__device__ __forceinline__ void ssd_write_channel_tables(const QaSsdParams& p, int h, int lane, float* xs_out, int32_t* srow_out) {
     int g, hg;
     ssd_group_of(p, h, g, hg);
-    for (int ch = lane; ch < p.headdim; ch += 64) xs_out[h * p.headdim + ch] = ssd_x_scale_of(p, g, hg, ch);
+    for (int ch = lane; ch < p.headdim; ch += 64) {
+        xs_out[h * p.headdim + ch] = ssd_x_scale_of(p, g, hg, ch);
+        srow_out[h * p.headdim + ch] = p.nhead_groups > 0 ? ((g * p.nhead_groups + hg) * p.ndim_groups + ssd_dim_group_of(p, g, hg, ch)) * p.dstate : 0;
+    }
 }
 
 // int8 final state of one element (quamba/triton/quant_ssm_states.py:43,119): the reference hands fp16 states to the
 // quantiser; one scale, or one per (ssd group, head group, dim group, state) with the factor 1e6 instead of 1e2
-__device__ __forceinline__ int8_t ssd_quantize_state(const QaSsdParams& p, int g, int hg, int ch, int n, int n_scales, float value) {
-    float sc, K;
-    if (p.nhead_groups > 0) {
-        sc = p.state_scale[((g * p.nhead_groups + hg) * p.ndim_groups + ssd_dim_group_of(p, g, hg, ch)) * n_scales + n];
-        K = 1e6f;
-    } else {
-        sc = p.state_scale[0];
-        K = 1e2f;
-    }
+// (srow: the channel's entry of the table above)
+__device__ __forceinline__ int8_t ssd_quantize_state(const QaSsdParams& p, int srow, int n, float value) {
+    const bool grouped = p.nhead_groups > 0;
+    const float sc = p.state_scale[grouped ? srow + n : 0];
+    const float K = grouped ? 1e6f : 1e2f;
     const float s16 = __half2float(__float2half(value));
     return sat8_rne((s16 * K) / (sc * K));
 }
@@ -90,6 +92,7 @@ inline bool ssd_fast_shape(const QaSsdParams& p) {
 
 // ssd_general.hip
 int ssd_general_grid_check(const QaSsdParams& p);
-void ssd_general_launch(const QaSsdParams& p, float* dt_ws, float* dA_ws, __half* prev_ws, float* xs_ws, int nc, hipStream_t stream);
+void ssd_general_launch(const QaSsdParams& p, float* dt_ws, float* dA_ws, __half* prev_ws, float* xs_ws, int32_t* srow_ws, int nc,
+                        hipStream_t stream);
 
 }  // namespace qa

@@ -32,7 +32,7 @@ __device__ __forceinline__ float f16r(float v) { return static_cast<float>(stati
 // ceil(chunk_size / 64) consecutive steps, then an inclusive scan across the lanes.  Steps past the end of the
 // sequence have dt = 0.
 // ---------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(kThreads) void ssd_general_cumsum_kernel(QaSsdParams p, float* dt_out, float* dA_out, float* xs_out, int nc) {
+__global__ __launch_bounds__(kThreads) void ssd_general_cumsum_kernel(QaSsdParams p, float* dt_out, float* dA_out, float* xs_out, int32_t* srow_out, int nc) {
     const int lane = threadIdx.x & 63;
     const unsigned idx = __builtin_amdgcn_readfirstlane(blockIdx.x * 4u + (threadIdx.x >> 6));
     if (idx >= static_cast<unsigned>(p.batch) * static_cast<unsigned>(nc) * static_cast<unsigned>(p.nheads)) return;
@@ -40,7 +40,7 @@ __global__ __launch_bounds__(kThreads) void ssd_general_cumsum_kernel(QaSsdParam
     const int c = static_cast<int>((idx / static_cast<unsigned>(p.nheads)) % static_cast<unsigned>(nc));
     const int b = static_cast<int>(idx / (static_cast<unsigned>(p.nheads) * static_cast<unsigned>(nc)));
     const int Q = p.chunk_size, E = (Q + 63) / 64;
-    if (b == 0 && c == 0) ssd_write_x_scales(p, h, lane, xs_out);
+    if (b == 0 && c == 0) ssd_write_channel_tables(p, h, lane, xs_out, srow_out);
     const float A = -expf(*p.A_log_scale * static_cast<float>(p.A_log[h]));
     const float s_dt = p.dt_is_fp32 ? 0.0f : *p.dt_scale;
     const float bias = (!p.dt_is_fp32 && p.dt_bias) ? __half2float(static_cast<const __half*>(p.dt_bias)[h]) : 0.0f;
@@ -128,11 +128,12 @@ __device__ __forceinline__ void stage_transposed(_Float16 (*dst)[kT + 8], const 
 // [state][step]; everything past an edge is zero there.
 // ---------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(kThreads) void ssd_general_state_kernel(QaSsdParams p, const float* dt_ws, const float* dA_ws, __half* prev, const float* xs_ws,
-                                                                     int nc, int vec) {
+                                                                     const int32_t* srow_ws, int nc, int vec) {
     __shared__ __attribute__((aligned(16))) _Float16 xt[kT][kT + 8];      // x^ [channel][step]
     __shared__ __attribute__((aligned(16))) _Float16 bt[kT][kT + 8];      // B^ w [state][step]
     __shared__ float wk[kT];
     __shared__ float xs[kT];
+    __shared__ int32_t srow[kT];
     const int P = p.headdim, N = p.dstate, Q = p.chunk_size, H = p.nheads, G = p.ngroups, L = p.seqlen;
     const int ptiles = (P + kT - 1) / kT, ntiles = (N + kT - 1) / kT;
     const int tid = threadIdx.x, lane = tid & 63, l16 = lane & 15, lq = lane >> 4;
@@ -145,7 +146,10 @@ __global__ __launch_bounds__(kThreads) void ssd_general_state_kernel(QaSsdParams
     int g, hg;
     ssd_group_of(p, h, g, hg);
     const float sB = p.nhead_groups > 0 ? p.B_scale[g] : p.B_scale[0];
-    if (tid < kT) xs[tid] = p0 + tid < P ? xs_ws[h * P + p0 + tid] : 0.0f;
+    if (tid < kT) {
+        xs[tid] = p0 + tid < P ? xs_ws[h * P + p0 + tid] : 0.0f;
+        srow[tid] = p0 + tid < P ? srow_ws[h * P + p0 + tid] : 0;
+    }
     const int64_t rows0 = (static_cast<int64_t>(b) * H + h) * nc;
     const int64_t xstep = static_cast<int64_t>(H) * P, bstep = static_cast<int64_t>(G) * N;
     v4f run[4];
@@ -211,7 +215,7 @@ __global__ __launch_bounds__(kThreads) void ssd_general_state_kernel(QaSsdParams
                 if (pp < P && nn < N) {
                     const int64_t fo = ((static_cast<int64_t>(b) * H + h) * P + pp) * N + nn;
                     if (p.final_state_is_fp32) static_cast<float*>(p.final_states)[fo] = run[j][r];
-                    else static_cast<int8_t*>(p.final_states)[fo] = ssd_quantize_state(p, g, hg, pp, nn, N, run[j][r]);
+                    else static_cast<int8_t*>(p.final_states)[fo] = ssd_quantize_state(p, srow[pp - p0], nn, run[j][r]);
                 }
             }
     }
@@ -436,17 +440,19 @@ int ssd_general_grid_check(const QaSsdParams& p) {
     return QA_OK;
 }
 
-void ssd_general_launch(const QaSsdParams& p, float* dt_ws, float* dA_ws, __half* prev_ws, float* xs_ws, int nc, hipStream_t stream) {
+void ssd_general_launch(const QaSsdParams& p, float* dt_ws, float* dA_ws, __half* prev_ws, float* xs_ws, int32_t* srow_ws, int nc,
+                        hipStream_t stream) {
     const int64_t bch = static_cast<int64_t>(p.batch) * nc * p.nheads;
     const int64_t scan = bch * ((p.chunk_size + kT - 1) / kT) * ((p.headdim + kT - 1) / kT);
     const int64_t state = static_cast<int64_t>(p.batch) * p.nheads * ((p.headdim + kT - 1) / kT) * ((p.dstate + kT - 1) / kT);
-    hipLaunchKernelGGL(ssd_general_cumsum_kernel, dim3(static_cast<unsigned>((bch + 3) / 4)), dim3(kThreads), 0, stream, p, dt_ws, dA_ws, xs_ws, nc);
+    hipLaunchKernelGGL(ssd_general_cumsum_kernel, dim3(static_cast<unsigned>((bch + 3) / 4)), dim3(kThreads), 0, stream, p, dt_ws, dA_ws, xs_ws, srow_ws, nc);
     int vec = 0;
     if (p.dstate % 16 == 0 && aligned16(p.B) && aligned16(p.C)) vec |= kVecCodes;
     if (p.headdim % 4 == 0 && aligned4(p.x)) vec |= kVecX;
     if (p.dstate % 8 == 0) vec |= kVecState;                       // (the workspace itself is 256-byte aligned)
     if (p.dstate % 4 == 0 && aligned4(p.B)) vec |= kVecB4;
-    hipLaunchKernelGGL(ssd_general_state_kernel, dim3(static_cast<unsigned>(state)), dim3(kThreads), 0, stream, p, dt_ws, dA_ws, prev_ws, xs_ws, nc, vec);
+    hipLaunchKernelGGL(ssd_general_state_kernel, dim3(static_cast<unsigned>(state)), dim3(kThreads), 0, stream, p, dt_ws, dA_ws, prev_ws, xs_ws, srow_ws,
+                       nc, vec);
     hipLaunchKernelGGL(ssd_general_chunk_scan_kernel, dim3(static_cast<unsigned>(scan)), dim3(kThreads), 0, stream, p, dt_ws, dA_ws, prev_ws, xs_ws, nc, vec);
 }
 

@@ -181,8 +181,8 @@ def test_ssd_shape_limits_without_a_gpu():
     assert l.qa_ssd_workspace_bytes(C.byref(p)) > 0
     p.headdim, p.chunk_size = 96, 100
     # 6 chunks: dt and the running sums in fp32 per (batch, head, chunk, step), entering states in fp16 per (batch, chunk, head,
-    # channel, state), one x scale in fp32 per (head, channel)
-    assert l.qa_ssd_workspace_bytes(C.byref(p)) == 2 * (2 * 128 * 6 * 100 * 4) + 2 * 6 * 128 * 96 * 256 * 2 + 128 * 96 * 4
+    # channel, state), one x scale in fp32 and one row index of the state scales per (head, channel)
+    assert l.qa_ssd_workspace_bytes(C.byref(p)) == 2 * (2 * 128 * 6 * 100 * 4) + 2 * 6 * 128 * 96 * 256 * 2 + 2 * 128 * 96 * 4
     for field, value in (("headdim", 257), ("dstate", 1025), ("chunk_size", 1025), ("chunk_size", 0)):
         q = _lib.QaSsdParams.from_buffer_copy(p)
         setattr(q, field, value)
