@@ -99,6 +99,26 @@ __global__ __launch_bounds__(kThreads) void conv2_fwd_kernel(QaConv2Params p, in
     if (ch0 >= p.dim || t0 >= p.seqlen) return;
     const int t_end = min(t0 + run, p.seqlen);
 
+    // The inputs are requested first: the walk over the group ranges below (dependent loads, four channels) then runs
+    // under their round trip instead of in front of it.
+    const int8_t* src = p.xBC + b * p.xBC_batch_stride + ch0;
+    uint32_t hist[3];
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+        const int t = t0 - 3 + i;
+        hist[i] = *reinterpret_cast<const uint32_t*>(src + max(t, 0) * p.xBC_l_stride);
+    }
+    // the loads of the next batch of steps are in flight while the current batch is worked on
+    uint32_t d[kBatchLoads], dn[kBatchLoads];
+    auto fetch = [&](int tb, uint32_t (&dst)[kBatchLoads]) {
+#pragma unroll
+        for (int i = 0; i < kBatchLoads; ++i) {
+            const int t = min(tb + i, p.seqlen - 1);              // in range for every lane; steps past the end are never used
+            dst[i] = *reinterpret_cast<const uint32_t*>(src + t * p.xBC_l_stride);
+        }
+    };
+    fetch(t0, dn);
+
     const Part part = part_of(p, ch0);          // the four channels of a lane never straddle two parts
     uint32_t taps[4];
     float bias_f[4], s_out[4], inv_s_out[4];
@@ -115,7 +135,6 @@ __global__ __launch_bounds__(kThreads) void conv2_fwd_kernel(QaConv2Params p, in
     const ConvQuantRegs kq(__builtin_fminf(__builtin_fminf(s_out[0], s_out[1]), __builtin_fminf(s_out[2], s_out[3])));
     int64_t out_ls, out_cs;
     int8_t* out = out_ptr(p, part, b, ch0, &out_ls, &out_cs);
-    const int8_t* src = p.xBC + b * p.xBC_batch_stride + ch0;
 
     // byte j of win[e] holds x[t-3+j] of channel ch0+e
     uint32_t win[4] = {0u, 0u, 0u, 0u};
@@ -126,20 +145,7 @@ __global__ __launch_bounds__(kThreads) void conv2_fwd_kernel(QaConv2Params p, in
         win[3] = __builtin_amdgcn_perm(d, win[3], 0x07030201u);
     };
 #pragma unroll
-    for (int i = 0; i < 3; ++i) {
-        const int t = t0 - 3 + i;
-        push(t >= 0 ? *reinterpret_cast<const uint32_t*>(src + t * p.xBC_l_stride) : 0u);
-    }
-    // the loads of the next batch of steps are in flight while the current batch is worked on
-    uint32_t d[kBatchLoads], dn[kBatchLoads];
-    auto fetch = [&](int tb, uint32_t (&dst)[kBatchLoads]) {
-#pragma unroll
-        for (int i = 0; i < kBatchLoads; ++i) {
-            const int t = min(tb + i, p.seqlen - 1);              // in range for every lane; steps past the end are never used
-            dst[i] = *reinterpret_cast<const uint32_t*>(src + t * p.xBC_l_stride);
-        }
-    };
-    fetch(t0, dn);
+    for (int i = 0; i < 3; ++i) push(t0 - 3 + i >= 0 ? hist[i] : 0u);
     int8_t* out_at = out + t0 * out_ls;             // walks on by one step's stride (the stride differs from lane to lane: a
                                                     // product per step would be a 64-bit multiplication in vector registers)
     for (int tb = t0; tb < t_end; tb += kBatchLoads) {
