@@ -199,16 +199,29 @@ __global__ __launch_bounds__(kThreads) void conv2_update_kernel(QaConv2Params p)
     const int width = p.width;
     const int slen = p.conv_state_len;            // width (slot 0 is dropped) or width-1
     const int drop = slen - (width - 1);
-    int8_t xs[4];
-    for (int i = 0; i < width - 1; ++i) xs[i] = st[(i + drop) * p.conv_state_l_stride];
-    xs[width - 1] = p.xBC[b * p.xBC_batch_stride + ch * p.xBC_c_stride];
-    for (int i = 0; i < slen; ++i) st[i * p.conv_state_l_stride] = xs[i + (width - slen)];
+    // four taps and a state of four codes, each in one aligned word (the Mamba2 layer's own buffers): one load and one
+    // store per row instead of one per code
+    const bool w_word = width == 4 && p.weight_width_stride == 1 && aligned4(w);
+    const bool s_word = slen == 4 && p.conv_state_l_stride == 1 && aligned4(st);
+    __attribute__((aligned(4))) int8_t xs[4], ws[4] = {0, 0, 0, 0};
+    const int8_t x_new = p.xBC[b * p.xBC_batch_stride + ch * p.xBC_c_stride];
+    if (w_word) {
+        *reinterpret_cast<uint32_t*>(ws) = *reinterpret_cast<const uint32_t*>(w);
+    } else {
+        for (int i = 0; i < width; ++i) ws[i] = w[i * p.weight_width_stride];
+    }
+    if (s_word) {
+        const uint32_t win = (*reinterpret_cast<const uint32_t*>(st) >> 8) | (static_cast<uint32_t>(static_cast<uint8_t>(x_new)) << 24);
+        *reinterpret_cast<uint32_t*>(st) = win;                    // the whole window is the new state
+        *reinterpret_cast<uint32_t*>(xs) = win;
+    } else {
+        for (int i = 0; i < width - 1; ++i) xs[i] = st[(i + drop) * p.conv_state_l_stride];
+        xs[width - 1] = x_new;
+        for (int i = 0; i < slen; ++i) st[i * p.conv_state_l_stride] = xs[i + (width - slen)];
+    }
     const Part part = part_of(p, ch);
     float v = p.bias ? part.s_bias * static_cast<float>(p.bias[ch]) : 0.0f;
-    for (int i = 0; i < width; ++i) {
-        const float wv = static_cast<float>(w[i * p.weight_width_stride]);
-        v = __builtin_fmaf(part.s_in * wv, static_cast<float>(xs[i]), v);
-    }
+    for (int i = 0; i < width; ++i) v = __builtin_fmaf(part.s_in * static_cast<float>(ws[i]), static_cast<float>(xs[i]), v);
     int64_t out_ls, out_cs;
     int8_t* out = out_ptr(p, part, b, ch, &out_ls, &out_cs);
     out[0] = conv_epilogue(v, out_scale_of(p, part, ch), p.silu_activation);
