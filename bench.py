@@ -637,7 +637,7 @@ def valu_calibration(dev, ops_list=None, launches=4):
 # The counts belong to one state of the kernel source: `source_sha256` is the hash of quamba_amd/csrc/sscan.hip they
 # were counted at; when the file has changed since, the line says so (`stale`) instead of passing them off as current.
 SCAN_MIX = {"four_lane": {"plain": 96, "transcendental": 18}, "eight_lane": {"plain": 57, "transcendental": 9}}
-SCAN_MIX_SOURCE_SHA256 = "332cfb88218c8b9418f1fb23d8f40e3892b09fdaccffbfbab98dcfaacc2530a7"
+SCAN_MIX_SOURCE_SHA256 = "e70cab8ddcf16e14fb332f9d44a854577bfdeee217b5a47359992baa1c18e961"
 
 
 def scan_mix_is_stale():
