@@ -105,7 +105,10 @@ class W8A8QMamba(nn.Module):
             x_rows = x.transpose(1, 2).contiguous()
         x_dbl = self.x_proj(x_rows)                                     # (B, L, dt_rank + 2N)
         dt, B, C = torch.split(x_dbl, [self.dt_rank, self.d_state, self.d_state], dim=-1)
-        dt = self.dt_proj.to_seqlen_last(dt.contiguous())               # (B, D, L)
+        # (the GEMM reads a row-strided operand in place when rows and base are 16-byte aligned)
+        if dt.stride(1) % 16 or dt.stride(0) != seqlen * dt.stride(1) or dt.data_ptr() % 16:
+            dt = dt.contiguous()
+        dt = self.dt_proj.to_seqlen_last(dt)                            # (B, D, L)
         B = B.transpose(1, 2).contiguous()                              # (B, N, L)
         C = C.transpose(1, 2).contiguous()
         want_state = ssm_state is not None
