@@ -2,15 +2,18 @@
 // without 16-byte alignment: the shapes the matrix-core kernels of ssd.hip are not built for.
 //
 // Same stages, same arithmetic and the same fp16 rounding points as there (quamba/triton/quant_ssd_combined.py
-// :61-77, grouped :146-162; the kernels restated are named at each stage), on the vector ALUs with 64-wide tiles in
-// every dimension and byte-wise loads, so that nothing depends on a size being a multiple of anything:
+// :61-77, grouped :146-162; the kernels restated are named at each stage) and the same matrix instructions, on 64-wide
+// tiles in every dimension that pass through LDS with everything past an edge set to zero there; loads are bounded,
+// and byte-wise unless sizes and addresses allow words or 16-byte pieces, so that nothing depends on a size being a
+// multiple of anything:
 //   cumsum      dt = clamp(softplus(s_dt q_dt + dt_bias)), dA_cs = within-chunk cumsum(dt * A)
 //   state       S_c[p,n] = sum_k f16(x^[k,p]) f16(B^[k,n] (exp(dA_last - dA_k) dt_k));  P_{c+1} = exp(dA_last) P_c + S_c,
 //               f16(P_c) stored as the state entering chunk c; final state fp32 / int8
 //   chunk_scan  y[m,p] = exp(dA_m) sum_n f16(C^[m,n]) f16(P_c[p,n])
 //                      + sum_{k<=m} f16(((s_C s_B) (q_C[m,:] . q_B[k,:])) exp(dA_m - dA_k) dt_k) f16(x^[k,p])
 //                      + x^[m,p] D, optional z gate, fp16 out
-// All sums are fp32; the integer contraction of C and B is exact (v_dot4_i32_i8).
+// All sums are fp32 (v_mfma_f32_16x16x32_f16 on fp16-rounded operands); the integer contraction of C and B is exact
+// (v_mfma_i32_16x16x64_i8).
 #include "qa_common.hpp"
 #include "ssd_common.hpp"
 
